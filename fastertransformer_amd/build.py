@@ -1,0 +1,76 @@
+"""Builds the native libraries of the sampling engine in-tree.
+
+  fastertransformer_amd/lib/libftk_sampling.so  HIP kernels + C ABI (include/ftk_sampling.h), gfx950
+  fastertransformer_amd/lib/libft_decode.so     host C++ layers (DynamicDecodeLayer, TopK/TopPSamplingLayer)
+                                                + the handle API used by bindings
+
+Run `python -m fastertransformer_amd.build`. hipcc cross-compiles for gfx950 without a GPU.
+"""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+SRC = os.path.join(PKG, "src")
+LIB = os.path.join(PKG, "lib")
+INCLUDE = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+KERNEL_SOURCES = ["penalty_kernels.hip", "criteria_kernels.hip", "topp_kernels.hip", "topk_kernels.hip",
+                  "fused_kernels.hip"]
+
+# -ffp-contract=off: results must match a plain IEEE evaluation operation by operation.
+# packed-fp32 instructions are disabled on purpose (hardware notes).
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result", "-I", CSRC, "-I", INCLUDE,
+]
+
+
+def _run(cmd):
+    print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def _newer(target, deps):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(force=True, verbose=True):
+    os.makedirs(LIB, exist_ok=True)
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".cuh"))]
+    headers.append(os.path.join(INCLUDE, "ftk_sampling.h"))
+    objs = []
+    for src in KERNEL_SOURCES:
+        path = os.path.join(CSRC, src)
+        if not os.path.exists(path):
+            continue
+        obj = os.path.join(LIB, src.replace(".hip", ".o"))
+        if force or _newer(obj, [path] + headers):
+            _run([HIPCC] + HIP_FLAGS + ["-c", path, "-o", obj])
+        objs.append(obj)
+    kernels_so = os.path.join(LIB, "libftk_sampling.so")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", kernels_so] + objs)
+
+    host_sources = []
+    for d, _, files in os.walk(SRC):
+        host_sources += [os.path.join(d, f) for f in files if f.endswith(".cc")]
+    if host_sources:
+        decode_so = os.path.join(LIB, "libft_decode.so")
+        _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
+              "-D__HIP_PLATFORM_AMD__", "-I", PKG, "-I", INCLUDE, "-I", "/opt/rocm/include", "-o", decode_so]
+             + sorted(host_sources)
+             + ["-L", LIB, "-lftk_sampling", "-L", "/opt/rocm/lib", "-lamdhip64",
+                "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--incremental" not in sys.argv)

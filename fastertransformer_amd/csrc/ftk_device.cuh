@@ -1,0 +1,223 @@
+// Device-side building blocks shared by the sampling kernels (gfx950, 64-lane wavefronts).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ftk_math.h"
+
+namespace ftk {
+
+constexpr int WAVE = 64;
+
+#define FTK_LAUNCH_CHECK()                                                                                             \
+    do {                                                                                                               \
+        hipError_t e_ = hipGetLastError();                                                                             \
+        if (e_ != hipSuccess) {                                                                                        \
+            return (int)e_;                                                                                            \
+        }                                                                                                              \
+    } while (0)
+
+#define FTK_DISPATCH_DTYPE(dtype, ...)                                                                                 \
+    switch (dtype) {                                                                                                   \
+        case DT_F32: {                                                                                                 \
+            constexpr int DT = DT_F32;                                                                                 \
+            __VA_ARGS__;                                                                                               \
+        } break;                                                                                                       \
+        case DT_F16: {                                                                                                 \
+            constexpr int DT = DT_F16;                                                                                 \
+            __VA_ARGS__;                                                                                               \
+        } break;                                                                                                       \
+        case DT_BF16: {                                                                                                \
+            constexpr int DT = DT_BF16;                                                                                \
+            __VA_ARGS__;                                                                                               \
+        } break;                                                                                                       \
+        default:                                                                                                       \
+            return -1;                                                                                                 \
+    }
+
+__device__ __forceinline__ int lane_id()
+{
+    return (int)(threadIdx.x & (WAVE - 1));
+}
+__device__ __forceinline__ int wave_id()
+{
+    return (int)(threadIdx.x >> 6);
+}
+
+// ---- wave / block reductions ----------------------------------------------------------------
+template<typename V>
+__device__ __forceinline__ V wave_max(V v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        V other = __shfl_xor(v, o, WAVE);
+        v       = other > v ? other : v;
+    }
+    return v;
+}
+template<typename V>
+__device__ __forceinline__ V wave_min(V v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        V other = __shfl_xor(v, o, WAVE);
+        v       = other < v ? other : v;
+    }
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        v += __shfl_xor(v, o, WAVE);
+    }
+    return v;
+}
+
+// Block-wide reductions over blockDim.x threads (multiple of 64, <= 1024). `smem` holds >= 16
+// elements of V. The result is returned to every thread. Two barriers.
+template<typename V>
+__device__ __forceinline__ V block_max(V v, V* smem, V identity)
+{
+    v = wave_max(v);
+    if (lane_id() == 0) {
+        smem[wave_id()] = v;
+    }
+    __syncthreads();
+    const int nw = (int)(blockDim.x >> 6);
+    V         r  = (lane_id() < nw) ? smem[lane_id()] : identity;
+    r            = wave_max(r);
+    __syncthreads();
+    return r;
+}
+template<typename V>
+__device__ __forceinline__ V block_min(V v, V* smem, V identity)
+{
+    v = wave_min(v);
+    if (lane_id() == 0) {
+        smem[wave_id()] = v;
+    }
+    __syncthreads();
+    const int nw = (int)(blockDim.x >> 6);
+    V         r  = (lane_id() < nw) ? smem[lane_id()] : identity;
+    r            = wave_min(r);
+    __syncthreads();
+    return r;
+}
+__device__ __forceinline__ int block_sum_i(int v, int* smem)
+{
+    v = wave_sum_i(v);
+    if (lane_id() == 0) {
+        smem[wave_id()] = v;
+    }
+    __syncthreads();
+    const int nw = (int)(blockDim.x >> 6);
+    int       r  = (lane_id() < nw) ? smem[lane_id()] : 0;
+    r            = wave_sum_i(r);
+    __syncthreads();
+    return r;
+}
+
+// Descending bitonic sort of one value per lane across the 64-lane wave: afterwards lane i holds
+// the (i+1)-th largest value.
+__device__ __forceinline__ uint32_t wave_sort_desc(uint32_t v)
+{
+    const int lane = lane_id();
+#pragma unroll
+    for (int k = 2; k <= WAVE; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            const uint32_t other = __shfl_xor(v, j, WAVE);
+            // in a descending sort the lower lane of a pair keeps the larger value inside
+            // "descending" blocks ((lane & k) == 0) and the smaller one otherwise
+            const bool lower     = (lane & j) == 0;
+            const bool desc      = (lane & k) == 0;
+            const bool keep_max  = lower == desc;
+            const uint32_t mx    = other > v ? other : v;
+            const uint32_t mn    = other > v ? v : other;
+            v                    = keep_max ? mx : mn;
+        }
+    }
+    return v;
+}
+
+// In-LDS bitonic sort (ascending) of n 64-bit keys, n a power of two, by all threads of the block.
+__device__ __forceinline__ void block_bitonic_sort_u64(unsigned long long* keys, int n)
+{
+    for (int k = 2; k <= n; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = (int)threadIdx.x; i < (n >> 1); i += (int)blockDim.x) {
+                // i-th compare-exchange pair of this stage
+                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
+                const int hi = lo | j;
+                const bool up = (lo & k) == 0;
+                const unsigned long long a = keys[lo];
+                const unsigned long long b = keys[hi];
+                if ((a > b) == up) {
+                    keys[lo] = b;
+                    keys[hi] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+__device__ __forceinline__ int next_pow2(int n)
+{
+    int p = 1;
+    while (p < n) {
+        p <<= 1;
+    }
+    return p;
+}
+
+// ---- Philox-4x32-10 (counter-based generator; replaces cuRAND's XORWOW) ---------------------
+FTK_HD void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t out[4])
+{
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+        const uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+        const uint32_t n1 = (uint32_t)p1;
+        const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        const uint32_t n3 = (uint32_t)p0;
+        c0 = n0;
+        c1 = n1;
+        c2 = n2;
+        c3 = n3;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    out[0] = c0;
+    out[1] = c1;
+    out[2] = c2;
+    out[3] = c3;
+}
+
+struct RngState {
+    uint64_t seed;
+    uint64_t offset;
+};
+
+// One uniform in (0, 1] (the range of curand_uniform), advancing the row's counter.
+__device__ __forceinline__ float rng_next_uniform(RngState* st)
+{
+    uint32_t       o[4];
+    const uint64_t off = st->offset;
+    philox4x32_10((uint32_t)off, (uint32_t)(off >> 32), 0u, 0u, (uint32_t)st->seed, (uint32_t)(st->seed >> 32), o);
+    st->offset = off + 1;
+    return (float)o[0] * 2.3283064365386963e-10f + 1.16415321826934814453125e-10f;
+}
+
+// The draw of row `b`: injected when the caller supplied one, generated otherwise.
+__device__ __forceinline__ float row_uniform(RngState* rng, const float* injected, int b)
+{
+    if (injected != nullptr) {
+        return injected[b];
+    }
+    return rng_next_uniform(rng + b);
+}
+
+}  // namespace ftk

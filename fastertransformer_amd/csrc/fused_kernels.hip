@@ -1,0 +1,311 @@
+// Fused decode step for rows owned by the top-k layer when no log-prob output is requested.
+//
+// The reference issues, per step, invokeBatchApplyTemperaturePenalty, invokeBatchApplyRepetitionPenalty,
+// invokeMinLengthPenalty, invokeAddBiasEndMask and the two top-k kernels
+// (src/fastertransformer/layers/sampling_layers/BaseSamplingLayer.cc:302-352,
+//  src/fastertransformer/layers/sampling_layers/TopKSamplingLayer.cu:220-266): each is a pass over
+// the [batch, vocab_padded] logits, k+5 reads and 3 writes of every row in total. Here the row is read
+// once and never written: the element arithmetic of those kernels (ftk_transform.cuh) is applied in
+// registers while the chunk streams in, and the result feeds the candidate gather of ftk_topk.cuh.
+//   history_bitmap_kernel - one workgroup per row turns the time-major token history into a bitmap
+//                           over the vocabulary (who gets the repetition / presence penalty)
+//   fused_gather_kernel   - grid (splits, rows): stream, transform, gather candidates
+//   fused_select_kernel   - one workgroup per row: exact tie order, sampling, bookkeeping
+#include "ftk_sampling.h"
+#include "ftk_topk.cuh"
+
+namespace ftk {
+
+struct FusedParams {
+    const void*  logits;
+    const void*  bias;
+    int          V, Vp, batch_size, step, max_input_length;
+    const float* temperatures;
+    const float* penalties;
+    int          penalty_type;
+    const int*   min_lengths;
+    const int*   end_ids;
+    const int*   input_lengths;
+    const int*   output_ids;
+    const int*   sequence_length_in;
+    const int*   top_ks;
+    const float* top_ps;
+    int          max_top_k;
+    const bool*  skip_decode;
+    const bool*  finished_in;
+    const uint32_t* bitmaps;  // [rows][bitmap_words] or null
+    int             bitmap_words;
+};
+
+template<int DT>
+struct FusedRow {
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    const T*              rowp;
+    const T*              bias;
+    const uint32_t*       bitmap;  // this row's history bitmap or null
+    int                   V, Vp;
+    bool                  temp_active, keep_pads;
+    float                 inv;
+    int                   penalty_type;
+    float                 penalty;
+    int                   masked_end_id;  // end id when the min-length mask applies, else -1
+
+    __device__ __forceinline__ FusedRow(const FusedParams& p, int row)
+    {
+        rowp         = (const T*)p.logits + (size_t)row * p.Vp;
+        bias         = (const T*)p.bias;
+        V            = p.V;
+        Vp           = p.Vp;
+        temp_active  = p.temperatures != nullptr;
+        const TemperatureCtx<DT> tc(temp_active ? p.temperatures[row] : 1.0f, V, Vp, false);
+        inv          = tc.inv;
+        keep_pads    = tc.keep_pads;
+        penalty_type = p.penalties != nullptr ? p.penalty_type : 2;
+        penalty      = p.penalties != nullptr ? p.penalties[row] : 0.0f;
+        bitmap       = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
+        masked_end_id = -1;
+        if (p.min_lengths != nullptr
+            && min_length_masks(p.sequence_length_in[row], p.max_input_length, p.min_lengths[row])) {
+            masked_end_id = p.end_ids[row];
+        }
+    }
+    __device__ __forceinline__ const T* data() const
+    {
+        return rowp;
+    }
+    // history-membership bits of columns first .. first+n-1 (n <= 8)
+    __device__ __forceinline__ uint32_t vector_bits(int first, int n) const
+    {
+        if (bitmap == nullptr) {
+            return 0u;
+        }
+        uint32_t bits = 0u;
+        if (first >= 0) {
+            const int w  = first >> 5;
+            const int sh = first & 31;
+            bits         = bitmap[w] >> sh;
+            if (sh + n > 32 && first + n - 1 < Vp) {
+                bits |= bitmap[w + 1] << (32 - sh);
+            }
+        }
+        else {
+            for (int j = 0; j < n; ++j) {
+                const int v = first + j;
+                if (v >= 0 && v < Vp) {
+                    bits |= ((bitmap[v >> 5] >> (v & 31)) & 1u) << j;
+                }
+            }
+        }
+        return bits;
+    }
+    // the value top-k would see for column v, as an order-preserving key
+    __device__ __forceinline__ uint32_t key(int v, T raw, uint32_t in_history) const
+    {
+        float x = S::ld(raw);
+        if (temp_active) {
+            if (v < V) {
+                if (bias != nullptr) {
+                    x = round_t<DT>(x + S::ld(bias[v]));
+                }
+                x = round_t<DT>(x * inv);
+            }
+            else if (!keep_pads) {
+                x = -S::max_t();
+            }
+        }
+        if (in_history) {
+            x = round_t<DT>(repetition_value(x, penalty, penalty_type));
+        }
+        if (v == masked_end_id) {
+            x = -S::max_t();
+        }
+        if (v >= V) {
+            x = -S::max_t();  // addBiasEndMask: pad columns
+        }
+        return order_key(x);
+    }
+    __device__ __forceinline__ uint32_t key_at(int v) const
+    {
+        const uint32_t bit = bitmap != nullptr ? (bitmap[v >> 5] >> (v & 31)) & 1u : 0u;
+        return key(v, rowp[v], bit);
+    }
+};
+
+// Row -> bitmap of the token ids in its history window (skipping prompt padding), built in LDS and
+// written out coalesced. Ids outside [0, Vp) are ignored.
+constexpr int HB_THREADS = 256;
+constexpr int HB_WORDS   = 8192;  // 262144 ids per LDS window
+
+__global__ void __launch_bounds__(HB_THREADS)
+history_bitmap_kernel(uint32_t* __restrict__ bitmaps, int bitmap_words, const int* __restrict__ output_ids,
+                      int batch_size, int Vp, const int* __restrict__ input_lengths, int max_input_length, int step,
+                      const bool* __restrict__ skip_decode, const bool* __restrict__ finished)
+{
+    __shared__ uint32_t bm[HB_WORDS];
+    const int           row = blockIdx.x;
+    if ((skip_decode != nullptr && skip_decode[row]) || (finished != nullptr && finished[row])) {
+        return;
+    }
+    const int input_length = input_lengths != nullptr ? input_lengths[row] : max_input_length;
+    uint32_t* out          = bitmaps + (size_t)row * bitmap_words;
+    for (int base = 0; base < Vp; base += HB_WORDS * 32) {
+        const int words = min(HB_WORDS, bitmap_words - (base >> 5));
+        for (int i = threadIdx.x; i < words; i += HB_THREADS) {
+            bm[i] = 0u;
+        }
+        __syncthreads();
+        for (int t = threadIdx.x; t < step; t += HB_THREADS) {
+            if (t >= input_length && t < max_input_length) {
+                continue;
+            }
+            const int id = output_ids[(size_t)t * batch_size + row];
+            if (id >= base && id < Vp && id < base + HB_WORDS * 32) {
+                atomicOr(&bm[(id - base) >> 5], 1u << ((id - base) & 31));
+            }
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < words; i += HB_THREADS) {
+            out[(base >> 5) + i] = bm[i];
+        }
+        __syncthreads();
+    }
+}
+
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS)
+fused_gather_kernel(FusedParams p, int splits, int nvt, int cap, size_t row_entries,
+                    TopkChunkHeader* __restrict__ headers, TopkEntry* __restrict__ entries)
+{
+    const int row   = blockIdx.y;
+    const int chunk = blockIdx.x;
+    if (p.skip_decode != nullptr && p.skip_decode[row]) {
+        return;
+    }
+    if (p.finished_in != nullptr && p.finished_in[row]) {
+        return;  // a finished row emits its end id without looking at the logits
+    }
+    const int          k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    const FusedRow<DT> r(p, row);
+    topk_gather_chunk<DT>(r, p.Vp, k, chunk, nvt, cap, headers + (size_t)row * splits + chunk,
+                          entries + (size_t)row * row_entries + (size_t)chunk * cap);
+}
+
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS)
+fused_select_kernel(FusedParams p, int* __restrict__ ids, int* __restrict__ sequence_length, bool* __restrict__ finished,
+                    RngState* rng, const float* __restrict__ uniforms, int splits, int cap, size_t row_entries,
+                    const TopkChunkHeader* __restrict__ headers, TopkEntry* __restrict__ entries)
+{
+    __shared__ TopkSelectShared s;
+    const int                   row = blockIdx.x;
+    if (p.skip_decode != nullptr && p.skip_decode[row]) {
+        return;
+    }
+    if (finished != nullptr && finished[row]) {
+        if (threadIdx.x == 0) {
+            ids[row] = p.end_ids[row];
+        }
+        return;
+    }
+    const int   k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    const float tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
+    if (threadIdx.x == 0) {
+        s.misc[0] = __float_as_int(row_uniform(rng, uniforms, row));
+    }
+    __syncthreads();
+    const float        u = __int_as_float(s.misc[0]);
+    const FusedRow<DT> r(p, row);
+    const TopkOutputs  out{ids, sequence_length, finished, nullptr, nullptr};
+    topk_select_row<DT>(r, s, row, p.Vp, k, tp, p.max_top_k, splits, headers + (size_t)row * splits,
+                        entries + (size_t)row * row_entries, cap, false, u, p.end_ids, out);
+}
+
+}  // namespace ftk
+
+using namespace ftk;
+
+extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
+{
+    if (a == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    if (a->dtype < 0 || a->dtype > 2) {
+        return FTK_ERR_DTYPE;
+    }
+    if (a->max_top_k < 1 || a->max_top_k > 1024) {
+        return FTK_ERR_TOPK_DOMAIN;
+    }
+    const int      elem         = a->dtype == FTK_DTYPE_F32 ? 4 : 2;
+    const int      rows         = a->local_batch_size;
+    const TopkPlan plan         = topk_plan(a->vocab_size_padded, rows, a->max_top_k, elem);
+    const int      bitmap_words = (a->vocab_size_padded + 31) / 32 + 1;  // +1: vector_bits may peek one word ahead
+    const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
+    const size_t   need         = bitmap_bytes + plan.bytes;
+    if (a->workspace == nullptr) {
+        a->workspace_size = need;
+        return 0;
+    }
+    if (a->workspace_size < need) {
+        return FTK_ERR_WORKSPACE;
+    }
+    if (rows <= 0) {
+        return 0;
+    }
+    if (a->logits == nullptr || a->ids == nullptr || a->end_ids == nullptr || a->top_ks == nullptr
+        || (a->rng_state == nullptr && a->uniform_draws == nullptr)
+        || (a->min_lengths != nullptr && a->sequence_length == nullptr)) {
+        return FTK_ERR_ARGUMENT;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    FusedParams p{};
+    p.logits             = a->logits;
+    p.bias               = a->embedding_bias;
+    p.V                  = a->vocab_size;
+    p.Vp                 = a->vocab_size_padded;
+    p.batch_size         = a->batch_size;
+    p.step               = a->step;
+    p.max_input_length   = a->max_input_length;
+    p.temperatures       = a->temperatures;
+    p.penalties          = a->penalty_type != FTK_PENALTY_NONE ? a->penalties : nullptr;
+    p.penalty_type       = a->penalty_type;
+    p.min_lengths        = a->min_lengths;
+    p.end_ids            = a->end_ids;
+    p.input_lengths      = a->input_lengths;
+    p.output_ids         = a->output_ids;
+    p.sequence_length_in = a->sequence_length;
+    p.top_ks             = a->top_ks;
+    p.top_ps             = a->top_ps;
+    p.max_top_k          = a->max_top_k;
+    p.skip_decode        = a->skip_decode;
+    p.finished_in        = a->finished;
+    p.bitmaps            = nullptr;
+    p.bitmap_words       = bitmap_words;
+
+    char* ws = (char*)a->workspace;
+    if (p.penalties != nullptr && a->step > 0) {
+        if (a->output_ids == nullptr) {
+            return FTK_ERR_ARGUMENT;
+        }
+        uint32_t* bitmaps = (uint32_t*)ws;
+        history_bitmap_kernel<<<rows, HB_THREADS, 0, st>>>(bitmaps, bitmap_words, a->output_ids, a->batch_size,
+                                                           a->vocab_size_padded, a->input_lengths,
+                                                           a->max_input_length, a->step, a->skip_decode, a->finished);
+        FTK_LAUNCH_CHECK();
+        p.bitmaps = bitmaps;
+    }
+    else {
+        p.penalties = nullptr;
+    }
+    TopkChunkHeader* headers = (TopkChunkHeader*)(ws + bitmap_bytes);
+    TopkEntry*       entries = (TopkEntry*)(headers + (size_t)rows * plan.splits);
+    dim3             grid(plan.splits, rows);
+    FTK_DISPATCH_DTYPE(a->dtype, fused_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(
+                                     p, plan.splits, plan.nvt, plan.cap, plan.row_entries, headers, entries));
+    FTK_LAUNCH_CHECK();
+    FTK_DISPATCH_DTYPE(a->dtype, fused_select_kernel<DT><<<rows, TK_THREADS, 0, st>>>(
+                                     p, a->ids, a->sequence_length, a->finished, (RngState*)a->rng_state,
+                                     a->uniform_draws, plan.splits, plan.cap, plan.row_entries, headers, entries));
+    FTK_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,238 @@
+// C++ launchers with the reference's names and parameter order, forwarding to the C ABI of
+// libftk_sampling.so (include/ftk_sampling.h). They replace the declarations of the reference's
+//   src/fastertransformer/kernels/sampling_topk_kernels.h
+//   src/fastertransformer/kernels/sampling_topp_kernels.h
+//   src/fastertransformer/kernels/sampling_penalty_kernels.h
+//   src/fastertransformer/kernels/ban_bad_words.h
+//   src/fastertransformer/kernels/stop_criteria_kernels.h
+// Differences: hipStream_t for cudaStream_t; ftk_rng_state* for curandState_t* followed by an
+// optional `uniform_draws` device array (defaulted, so reference call sites compile unchanged apart
+// from the state type); C-ABI return codes are re-thrown as the exceptions the reference throws.
+#pragma once
+#include "src/fastertransformer/kernels/penalty_types.h"
+#include "src/fastertransformer/utils/Tensor.h"
+
+namespace fastertransformer {
+
+typedef ftk_rng_state curandState_t;  // call sites keep the reference's spelling
+
+template<typename T>
+struct FtkDType;
+template<>
+struct FtkDType<float> {
+    static constexpr int value = FTK_DTYPE_F32;
+};
+template<>
+struct FtkDType<half> {
+    static constexpr int value = FTK_DTYPE_F16;
+};
+template<>
+struct FtkDType<bfloat16> {
+    static constexpr int value = FTK_DTYPE_BF16;
+};
+
+inline int toFtkPenalty(RepetitionPenaltyType t)
+{
+    return t == RepetitionPenaltyType::Additive ? FTK_PENALTY_ADDITIVE :
+           t == RepetitionPenaltyType::Multiplicative ? FTK_PENALTY_MULTIPLICATIVE : FTK_PENALTY_NONE;
+}
+
+// ---- sampling_topk_kernels.h ----------------------------------------------------------------
+inline void invokeCurandInitialize(curandState_t* state, const size_t batch_size, unsigned long long random_seed,
+                                   hipStream_t stream)
+{
+    check_ftk(ftk_invoke_curand_initialize(state, batch_size, random_seed, stream));
+}
+
+inline void invokeCurandBatchInitialize(curandState_t* states, const size_t batch_size,
+                                        const unsigned long long* random_seeds, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_curand_batch_initialize(states, batch_size, random_seeds, stream));
+}
+
+template<typename T>
+void invokeAddBiasEndMask(T* logits, const T* bias, const int* end_ids, const bool* finished, const int batch_size,
+                          const int vocab_size, const int vocab_size_padded, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_add_bias_end_mask(FtkDType<T>::value, logits, bias, end_ids, finished, batch_size, vocab_size,
+                                           vocab_size_padded, stream));
+}
+
+template<typename T>
+void invokeBatchTopKSampling(void* workspace, size_t& workspace_size, const T* log_probs, int* ids,
+                             int* sequence_length, bool* finished, float* cum_log_probs, float* output_log_probs,
+                             curandState_t* curandstate, const int max_top_k, const int* top_ks, const float top_p,
+                             const float* top_ps, const int vocab_size_padded, const int* end_ids, hipStream_t stream,
+                             const int batch_size, const bool* skip_decode, const float* uniform_draws = nullptr)
+{
+    check_ftk(ftk_invoke_batch_topk_sampling(FtkDType<T>::value, workspace, &workspace_size, log_probs, ids,
+                                             sequence_length, finished, cum_log_probs, output_log_probs, curandstate,
+                                             uniform_draws, max_top_k, top_ks, top_p, top_ps, vocab_size_padded,
+                                             end_ids, stream, batch_size, skip_decode));
+}
+
+template<typename T>
+void invokeTopKSampling(void* workspace, size_t& workspace_size, const T* log_probs, int* ids, int* sequence_length,
+                        bool* finished_buf, float* cum_log_probs, float* output_log_probs, curandState_t* curandstate,
+                        const int top_k, const float top_p, const int vocab_size_padded, const int* end_ids,
+                        hipStream_t stream, const int batch_size, const bool* skip_decode,
+                        const float* uniform_draws = nullptr)
+{
+    invokeBatchTopKSampling(workspace, workspace_size, log_probs, ids, sequence_length, finished_buf, cum_log_probs,
+                            output_log_probs, curandstate, top_k, (const int*)nullptr, top_p, (const float*)nullptr,
+                            vocab_size_padded, end_ids, stream, batch_size, skip_decode, uniform_draws);
+}
+
+template<typename T>
+void invokeTopKTopPSampling(void* workspace, size_t& workspace_size, int* output_ids, const T* logits,
+                            int* sequence_length, bool* finished_buf, float* cum_log_probs, float* output_log_probs,
+                            curandState_t* curandstate, const int batch_size, const int top_k, const float top_p,
+                            const int vocab_size_padded, const int* end_ids, hipStream_t stream,
+                            const float* uniform_draws = nullptr)
+{
+    invokeTopKSampling(workspace, workspace_size, logits, output_ids, sequence_length, finished_buf, cum_log_probs,
+                       output_log_probs, curandstate, top_k, top_p, vocab_size_padded, end_ids, stream, batch_size,
+                       (const bool*)nullptr, uniform_draws);
+}
+
+// ---- sampling_topp_kernels.h ----------------------------------------------------------------
+inline void invokeTopPInitialize(int* topp_id_val_buf, int* topp_offset_buf, int* begin_topp_offset_buf_,
+                                 const size_t batch_size, const int n, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_topp_initialize(topp_id_val_buf, topp_offset_buf, begin_topp_offset_buf_, batch_size, n,
+                                         stream));
+}
+
+template<typename T>
+void invokeAddBiasSoftMax(T* logits, const T* bias, const int* end_ids, const bool* finished, const int m,
+                          const int n_padded, const int n, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_add_bias_softmax(FtkDType<T>::value, logits, bias, end_ids, finished, m, n_padded, n, stream));
+}
+
+template<typename T>
+void invokeBatchTopPSampling(void* workspace, size_t& workspace_size, size_t& cub_temp_storage_size, int* output_ids,
+                             int* sequence_length, bool* finished_buf, float* cum_log_probs, float* output_log_probs,
+                             const T* log_probs, const int* id_vals, int* offset_buf, int* begin_offset_buf,
+                             curandState_t* curandstate, const int batch_size, const size_t vocab_size_padded,
+                             const int* end_ids, const float max_top_p, const float* top_ps, hipStream_t stream,
+                             void* device_prop, const bool* skip_decode, const float* uniform_draws = nullptr)
+{
+    (void)device_prop;
+    check_ftk(ftk_invoke_batch_topp_sampling(FtkDType<T>::value, workspace, &workspace_size, &cub_temp_storage_size,
+                                             output_ids, sequence_length, finished_buf, cum_log_probs,
+                                             output_log_probs, log_probs, id_vals, offset_buf, begin_offset_buf,
+                                             curandstate, uniform_draws, batch_size, vocab_size_padded, end_ids,
+                                             max_top_p, top_ps, stream, skip_decode));
+}
+
+template<typename T>
+void invokeTopPSampling(void* workspace, size_t& workspace_size, size_t& cub_temp_storage_size, int* output_ids,
+                        int* sequence_length, bool* finished_buf, float* cum_log_probs, float* output_log_probs,
+                        const T* log_probs, const int* id_vals, int* offset_buf, int* begin_offset_buf,
+                        curandState_t* curandstate, const int batch_size, const size_t vocab_size_padded,
+                        const int* end_ids, const float top_p, hipStream_t stream, void* device_prop,
+                        const bool* skip_decode, const float* uniform_draws = nullptr)
+{
+    invokeBatchTopPSampling(workspace, workspace_size, cub_temp_storage_size, output_ids, sequence_length,
+                            finished_buf, cum_log_probs, output_log_probs, log_probs, id_vals, offset_buf,
+                            begin_offset_buf, curandstate, batch_size, vocab_size_padded, end_ids, top_p,
+                            (const float*)nullptr, stream, device_prop, skip_decode, uniform_draws);
+}
+
+inline void invokeComputeToppDecay(float* runtime_top_p, const float* runtime_initial_top_p, const int* output_ids,
+                                   const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
+                                   const int local_batch_size, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_compute_topp_decay(runtime_top_p, runtime_initial_top_p, output_ids, top_p_decay, top_p_min,
+                                            top_p_reset_ids, local_batch_size, stream));
+}
+
+// ---- sampling_penalty_kernels.h -------------------------------------------------------------
+template<typename T>
+void invokeApplyRepetitionPenalty(T* logits, const float penalty, const int* start_ids, int* output_ids,
+                                  const int batch_size, const int local_batch_size, const int vocab_size,
+                                  const int vocab_size_padd, const int* input_lengths, const int max_input_len,
+                                  const int step, const RepetitionPenaltyType penalty_type, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_apply_repetition_penalty(FtkDType<T>::value, logits, penalty, start_ids, output_ids,
+                                                  batch_size, local_batch_size, vocab_size, vocab_size_padd,
+                                                  input_lengths, max_input_len, step, toFtkPenalty(penalty_type),
+                                                  stream));
+}
+
+template<typename T>
+void invokeBatchApplyRepetitionPenalty(T* logits, const float* penalties, const int* output_ids, const int batch_size,
+                                       const int local_batch_size, const int vocab_size, const int* input_lengths,
+                                       const int max_input_length, const int step,
+                                       const RepetitionPenaltyType penalty_type, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_batch_apply_repetition_penalty(FtkDType<T>::value, logits, penalties, output_ids, batch_size,
+                                                        local_batch_size, vocab_size, input_lengths,
+                                                        max_input_length, step, toFtkPenalty(penalty_type), stream));
+}
+
+template<typename T>
+void invokeBatchApplyFrequencyPenalty(T* logits, const float* presence, const float* frequency, const int* output_ids,
+                                      const int batch_size, const int local_batch_size, const int vocab_size,
+                                      const int* input_lengths, const int max_input_length, const int step,
+                                      hipStream_t stream)
+{
+    check_ftk(ftk_invoke_batch_apply_frequency_penalty(FtkDType<T>::value, logits, presence, frequency, output_ids,
+                                                       batch_size, local_batch_size, vocab_size, input_lengths,
+                                                       max_input_length, step, stream));
+}
+
+template<typename T>
+void invokeApplyTemperaturePenalty(T* logits, const T* bias, const float temperature, const int batch_size,
+                                   const int vocab_size, const int vocab_size_padd, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_apply_temperature_penalty(FtkDType<T>::value, logits, bias, temperature, batch_size,
+                                                   vocab_size, vocab_size_padd, stream));
+}
+
+template<typename T>
+void invokeBatchApplyTemperaturePenalty(T* logits, const T* bias, const float* temperatures, const int batch_size,
+                                        const int vocab_size, const int vocab_size_padd, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_batch_apply_temperature_penalty(FtkDType<T>::value, logits, bias, temperatures, batch_size,
+                                                         vocab_size, vocab_size_padd, stream));
+}
+
+template<typename T>
+void invokeMinLengthPenalty(T* logits, const int* min_lengths, const int* end_ids, const int* sequnece_lengths,
+                            const int max_input_length, const int batch_size, const int vocab_size_padded,
+                            hipStream_t stream)
+{
+    check_ftk(ftk_invoke_min_length_penalty(FtkDType<T>::value, logits, min_lengths, end_ids, sequnece_lengths,
+                                            max_input_length, batch_size, vocab_size_padded, stream));
+}
+
+// ---- ban_bad_words.h, stop_criteria_kernels.h ---------------------------------------------------
+template<typename T>
+void invokeBanBadWords(T* logits, const int* output_ids_buf, const int* parent_ids_buf, int batch_size,
+                       int local_batch_size, int beam_width, const int* bad_words, bool share_words,
+                       size_t bad_words_len, int id_offset, int vocab_size_padded, size_t step, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_ban_bad_words(FtkDType<T>::value, logits, output_ids_buf, parent_ids_buf, batch_size,
+                                       local_batch_size, beam_width, bad_words, share_words, bad_words_len, id_offset,
+                                       vocab_size_padded, step, stream));
+}
+
+inline void invokeStopWordsCriterion(const int* output_ids, const int* parent_ids, const int* stop_words,
+                                     bool* finished, size_t id_offset, size_t stop_words_len, int batch_size,
+                                     int beam_width, int step, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_stop_words_criterion(output_ids, parent_ids, stop_words, finished, id_offset, stop_words_len,
+                                              batch_size, beam_width, step, stream));
+}
+
+inline void invokeLengthCriterion(bool* finished, bool* should_stop, int* h_pinned_finished_sum_,
+                                  const uint32_t* sequence_limit_length, int batch_size, int beam_width, int step,
+                                  hipStream_t stream)
+{
+    check_ftk(ftk_invoke_length_criterion(finished, should_stop, h_pinned_finished_sum_, sequence_limit_length,
+                                          batch_size, beam_width, step, stream));
+}
+
+}  // namespace fastertransformer

@@ -1,0 +1,42 @@
+// Per-step decode orchestrator: bad words -> top-k / top-p sampling -> stop words -> length criterion.
+// Public surface of the reference's src/fastertransformer/layers/DynamicDecodeLayer.h:29-75.
+// Beam search (beam_width > 1) is outside this engine and raises an error.
+#pragma once
+#include <string>
+#include <unordered_map>
+
+#include "src/fastertransformer/layers/sampling_layers/TopKSamplingLayer.h"
+#include "src/fastertransformer/layers/sampling_layers/TopPSamplingLayer.h"
+
+namespace fastertransformer {
+
+template<typename T>
+class DynamicDecodeLayer: public BaseLayer {
+protected:
+    void allocateBuffer() override;
+    void freeBuffer() override;
+    void initialize();
+
+    TopKSamplingLayer<T>* topk_decode_ = nullptr;
+    TopPSamplingLayer<T>* topp_decode_ = nullptr;
+
+    size_t vocab_size_;
+    size_t vocab_size_padded_;
+    int*   h_pinned_finished_sum_ = nullptr;
+
+public:
+    DynamicDecodeLayer(size_t vocab_size, size_t vocab_size_padded, int end_id, hipStream_t stream,
+                       cublasMMWrapper* cublas_wrapper, IAllocator* allocator, bool is_free_buffer_after_forward,
+                       cudaDeviceProp* cuda_device_prop);
+    ~DynamicDecodeLayer() override;
+    DynamicDecodeLayer(DynamicDecodeLayer const& dynamic_decode_layer);
+
+    void setStream(hipStream_t stream) override;
+
+    void setup(const size_t batch_size, const size_t beam_width, TensorMap* runtime_args);
+    void forward(TensorMap* output_tensors, TensorMap* input_tensors);
+    void forward(std::unordered_map<std::string, Tensor>*       output_tensors,
+                 const std::unordered_map<std::string, Tensor>* input_tensors);
+};
+
+}  // namespace fastertransformer

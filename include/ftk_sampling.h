@@ -1,0 +1,228 @@
+/*
+ * C ABI of the MI355X (gfx950) decode-step sampling engine: libftk_sampling.so.
+ *
+ * Every entry point replaces one `invoke*` kernel launcher of NVIDIA/FasterTransformer's sampling
+ * path (paths below are relative to the FasterTransformer source tree). Parameter order and meaning
+ * follow the reference launcher; the differences are mechanical:
+ *   - the C++ template parameter T becomes the leading `dtype` argument (FTK_DTYPE_*);
+ *   - `cudaStream_t` becomes `ftk_stream_t` (a `hipStream_t` passed as void*);
+ *   - `curandState_t*` becomes `ftk_rng_state*` (counter-based Philox-4x32-10 state) followed by an
+ *     optional `const float* uniform_draws`: when non-null, row b uses uniform_draws[b] in (0, 1]
+ *     instead of drawing, which makes a step reproducible bit for bit;
+ *   - `size_t&` workspace-size out-parameters become `size_t*`;
+ *   - errors are return codes: 0 = success, > 0 = hipError_t, < 0 = FTK_ERR_*.
+ * All pointers are device pointers unless stated otherwise. No entry point allocates memory; all
+ * scratch comes in through `workspace`. Calls are asynchronous on `stream` unless stated otherwise.
+ */
+#ifndef FTK_SAMPLING_H
+#define FTK_SAMPLING_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ftk_stream_t;
+
+enum { FTK_DTYPE_F32 = 0, FTK_DTYPE_F16 = 1, FTK_DTYPE_BF16 = 2 };
+
+/* kernels/penalty_types.h:26-30 (same enumerator order) */
+enum { FTK_PENALTY_ADDITIVE = 0, FTK_PENALTY_MULTIPLICATIVE = 1, FTK_PENALTY_NONE = 2 };
+
+enum {
+    FTK_ERR_DTYPE       = -1, /* unknown dtype */
+    FTK_ERR_TOPK_DOMAIN = -2, /* top-k outside [1, 1024]: std::domain_error in sampling_topk_kernels.cu:393-394 */
+    FTK_ERR_ARGUMENT    = -3, /* null / inconsistent argument */
+    FTK_ERR_WORKSPACE   = -4  /* workspace smaller than the queried size */
+};
+
+/* Per-row generator state; replaces curandState_t (48 bytes) in every signature. Row b draws
+ * Philox-4x32-10(key = seed, counter = {offset, 0, 0, 0}).x mapped to (0, 1], then offset++. */
+typedef struct ftk_rng_state {
+    uint64_t seed;
+    uint64_t offset;
+} ftk_rng_state;
+
+const char* ftk_error_string(int code);
+
+/* ---- kernels/sampling_topk_kernels.h ----------------------------------------------------- */
+
+/* invokeCurandInitialize, kernels/sampling_topk_kernels.cu:39-47 */
+int ftk_invoke_curand_initialize(ftk_rng_state* state, size_t batch_size, unsigned long long random_seed,
+                                 ftk_stream_t stream);
+
+/* invokeCurandBatchInitialize, kernels/sampling_topk_kernels.cu:57-65 */
+int ftk_invoke_curand_batch_initialize(ftk_rng_state* states, size_t batch_size,
+                                       const unsigned long long* random_seeds, ftk_stream_t stream);
+
+/* invokeAddBiasEndMask<T>, kernels/sampling_topk_kernels.cu:96-110 */
+int ftk_invoke_add_bias_end_mask(int dtype, void* logits, const void* bias, const int* end_ids, const bool* finished,
+                                 int batch_size, int vocab_size, int vocab_size_padded, ftk_stream_t stream);
+
+/* invokeBatchTopKSampling<T>, kernels/sampling_topk_kernels.cu:345-396.
+ * workspace == NULL: writes the required size to *workspace_size and launches nothing.
+ * invokeTopKSampling (:438-474) is this call with top_ks == NULL and top_ps == NULL;
+ * invokeTopKTopPSampling (:510-544) additionally passes skip_decode == NULL. */
+int ftk_invoke_batch_topk_sampling(int dtype, void* workspace, size_t* workspace_size, const void* log_probs, int* ids,
+                                   int* sequence_length, bool* finished, float* cum_log_probs,
+                                   float* output_log_probs, ftk_rng_state* rng_state, const float* uniform_draws,
+                                   int max_top_k, const int* top_ks, float top_p, const float* top_ps,
+                                   int vocab_size_padded, const int* end_ids, ftk_stream_t stream, int batch_size,
+                                   const bool* skip_decode);
+
+/* ---- kernels/sampling_topp_kernels.h ----------------------------------------------------- */
+
+/* invokeTopPInitialize, kernels/sampling_topp_kernels.cu:790-799. Kept for callers that own such
+ * buffers; this engine's top-p never reads the id table, so any of the pointers may be NULL. */
+int ftk_invoke_topp_initialize(int* topp_id_val_buf, int* topp_offset_buf, int* begin_topp_offset_buf,
+                               size_t batch_size, int n, ftk_stream_t stream);
+
+/* invokeAddBiasSoftMax<T>, kernels/sampling_topp_kernels.cu:1347-1361 */
+int ftk_invoke_add_bias_softmax(int dtype, void* logits, const void* bias, const int* end_ids, const bool* finished,
+                                int m, int n_padded, int n, ftk_stream_t stream);
+
+/* invokeBatchTopPSampling<T>, kernels/sampling_topp_kernels.cu:1006-1161 (`log_probs` holds
+ * probabilities). workspace == NULL: size query (cub_temp_storage_size is reported as 0).
+ * id_vals / offset_buf / begin_offset_buf are accepted and ignored. invokeTopPSampling
+ * (:1207-1250) is this call with top_ps == NULL. cudaDeviceProp* is dropped (only the reference's
+ * disabled single-pass branch read it). */
+int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace_size, size_t* cub_temp_storage_size,
+                                   int* output_ids, int* sequence_length, bool* finished, float* cum_log_probs,
+                                   float* output_log_probs, const void* log_probs, const int* id_vals,
+                                   int* offset_buf, int* begin_offset_buf, ftk_rng_state* rng_state,
+                                   const float* uniform_draws, int batch_size, size_t vocab_size_padded,
+                                   const int* end_ids, float max_top_p, const float* top_ps, ftk_stream_t stream,
+                                   const bool* skip_decode);
+
+/* invokeComputeToppDecay, kernels/sampling_topp_kernels.cu:1414-1427 */
+int ftk_invoke_compute_topp_decay(float* runtime_top_p, const float* runtime_initial_top_p, const int* output_ids,
+                                  const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
+                                  int local_batch_size, ftk_stream_t stream);
+
+/* ---- kernels/sampling_penalty_kernels.h -------------------------------------------------- */
+
+/* invokeApplyTemperaturePenalty<T>, kernels/sampling_penalty_kernels.cu:75-99 */
+int ftk_invoke_apply_temperature_penalty(int dtype, void* logits, const void* bias, float temperature, int batch_size,
+                                         int vocab_size, int vocab_size_padd, ftk_stream_t stream);
+
+/* invokeBatchApplyTemperaturePenalty<T>, kernels/sampling_penalty_kernels.cu:181-206 */
+int ftk_invoke_batch_apply_temperature_penalty(int dtype, void* logits, const void* bias, const float* temperatures,
+                                               int batch_size, int vocab_size, int vocab_size_padd,
+                                               ftk_stream_t stream);
+
+/* invokeApplyRepetitionPenalty<T>, kernels/sampling_penalty_kernels.cu:288-337 (start_ids is unused there too) */
+int ftk_invoke_apply_repetition_penalty(int dtype, void* logits, float penalty, const int* start_ids,
+                                        const int* output_ids, int batch_size, int local_batch_size, int vocab_size,
+                                        int vocab_size_padd, const int* input_lengths, int max_input_len, int step,
+                                        int penalty_type, ftk_stream_t stream);
+
+/* invokeBatchApplyRepetitionPenalty<T>, kernels/sampling_penalty_kernels.cu:426-459
+ * (`vocab_size` is the row stride, as in the reference) */
+int ftk_invoke_batch_apply_repetition_penalty(int dtype, void* logits, const float* penalties, const int* output_ids,
+                                              int batch_size, int local_batch_size, int vocab_size,
+                                              const int* input_lengths, int max_input_length, int step,
+                                              int penalty_type, ftk_stream_t stream);
+
+/* Extension without a reference counterpart: additive presence + frequency penalty,
+ * logit <- T(float(logit) - presence[b] - frequency[b] * count), count = occurrences of the id in
+ * the non-padding history; with frequency == 0 it equals the additive penalty above. */
+int ftk_invoke_batch_apply_frequency_penalty(int dtype, void* logits, const float* presence, const float* frequency,
+                                             const int* output_ids, int batch_size, int local_batch_size,
+                                             int vocab_size, const int* input_lengths, int max_input_length,
+                                             int step, ftk_stream_t stream);
+
+/* invokeMinLengthPenalty<T>, kernels/sampling_penalty_kernels.cu:502-517 */
+int ftk_invoke_min_length_penalty(int dtype, void* logits, const int* min_lengths, const int* end_ids,
+                                  const int* sequence_lengths, int max_input_length, int batch_size,
+                                  int vocab_size_padded, ftk_stream_t stream);
+
+/* ---- kernels/ban_bad_words.h, kernels/stop_criteria_kernels.h ------------------------------ */
+
+/* invokeBanBadWords<T>, kernels/ban_bad_words.cu:88-120 */
+int ftk_invoke_ban_bad_words(int dtype, void* logits, const int* output_ids_buf, const int* parent_ids_buf,
+                             int batch_size, int local_batch_size, int beam_width, const int* bad_words,
+                             bool share_words, size_t bad_words_len, int id_offset, int vocab_size_padded,
+                             size_t step, ftk_stream_t stream);
+
+/* invokeStopWordsCriterion, kernels/stop_criteria_kernels.cu:83-104 */
+int ftk_invoke_stop_words_criterion(const int* output_ids, const int* parent_ids, const int* stop_words,
+                                    bool* finished, size_t id_offset, size_t stop_words_len, int batch_size,
+                                    int beam_width, int step, ftk_stream_t stream);
+
+/* The same kernel over the first `num_rows` rows only, `batch_size` staying the row stride of
+ * output_ids. DynamicDecodeLayer::forward needs it for micro-batch windows: the reference passes its
+ * window through offset pointers yet still examines `batch_size` rows (layers/DynamicDecodeLayer.cc:451-461),
+ * which runs past the window; this entry point examines the window only. */
+int ftk_invoke_stop_words_criterion_rows(const int* output_ids, const int* parent_ids, const int* stop_words,
+                                         bool* finished, size_t id_offset, size_t stop_words_len, int batch_size,
+                                         int num_rows, int beam_width, int step, ftk_stream_t stream);
+
+/* invokeLengthCriterion, kernels/stop_criteria_kernels.cu:135-157. `should_stop` is a host bool and
+ * `h_pinned_finished_sum` one pinned host int; like the reference the call returns only when
+ * *should_stop is valid. */
+int ftk_invoke_length_criterion(bool* finished, bool* should_stop, int* h_pinned_finished_sum,
+                                const uint32_t* sequence_limit_length, int batch_size, int beam_width, int step,
+                                ftk_stream_t stream);
+
+/* ---- fused decode step ---------------------------------------------------------------------
+ * One call = the kernel sequence BaseSamplingLayer<T>::forward + TopKSamplingLayer<T>::runSampling
+ * issue for the rows a top-k layer owns (layers/sampling_layers/BaseSamplingLayer.cc:255-359,
+ * layers/sampling_layers/TopKSamplingLayer.cu:189-268) when no log-prob output is requested:
+ * bad words, temperature(+bias), repetition/presence penalty, min-length, end/pad mask, top-k
+ * selection and sampling, with the logits read from HBM once and never written. */
+typedef struct ftk_fused_topk_args {
+    int         dtype;
+    const void* logits;         /* [local_batch, vocab_size_padded], not modified */
+    const void* embedding_bias; /* [vocab_size_padded] or NULL */
+    int         vocab_size, vocab_size_padded;
+    int         batch_size;       /* stride of output_ids rows */
+    int         local_batch_size; /* rows in this call */
+    int         step, max_input_length;
+    /* per-row arguments, already offset to the local window */
+    const float* temperatures;   /* NULL = 1.0 */
+    const float* penalties;      /* NULL or [local] */
+    int          penalty_type;   /* FTK_PENALTY_* */
+    const int*   min_lengths;    /* NULL = no min-length mask */
+    const int*   end_ids;        /* [local] */
+    const int*   input_lengths;  /* [local] or NULL */
+    const int*   output_ids;     /* history base + window offset: element (t, row) at output_ids[t*batch_size+row] */
+    const int*   bad_words;      /* [2, L] or [local, 2, L] or NULL */
+    int          bad_words_len;
+    int          bad_words_shared;
+    int          id_offset; /* kept for symmetry with invokeBanBadWords; rows are already windowed */
+    const int*   top_ks;    /* [local] */
+    const float* top_ps;    /* [local] */
+    int          max_top_k;
+    const bool*  skip_decode; /* [local] or NULL */
+    ftk_rng_state* rng_state; /* [local] */
+    const float*   uniform_draws; /* [local] or NULL */
+    /* outputs */
+    int*  ids;             /* [local]: output_ids + step*batch_size + window offset */
+    int*  sequence_length; /* [local] or NULL */
+    bool* finished;        /* [local] or NULL */
+    void*  workspace;
+    size_t workspace_size;
+} ftk_fused_topk_args;
+
+/* workspace == NULL in args: writes the required size into args->workspace_size, launches nothing. */
+int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
+
+/* ---- test hooks (host-side instances of the shared arithmetic, and device probes) ----------- */
+float ftk_host_expf(float x);
+float ftk_host_logf(float x);
+/* kind 0: det_expf, 1: det_logf, 2: float->half->float, 3: float->bf16->float; n elements on device */
+int ftk_test_device_math(int kind, const float* in, float* out, size_t n, ftk_stream_t stream);
+/* draws `n_draws` uniforms per row into out[row*n_draws + i], advancing the states */
+int ftk_test_rng_uniform(ftk_rng_state* states, float* out, int batch_size, int n_draws, ftk_stream_t stream);
+/* non-zero: every top-p row takes the radix-sort fallback (exercises it on small inputs) */
+void ftk_test_set_topp_force_deep(int enable);
+/* raw Philox-4x32-10 block for known-answer tests (host) */
+void ftk_host_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTK_SAMPLING_H */

@@ -1,0 +1,565 @@
+"""GPU parity of every stand-alone kernel entry point against the CPU oracle, through the C ABI.
+
+Integer / id / flag outputs must be bit-exact; penalised logits must match the oracle's bits
+(the contract is 1 ulp in fp32; both sides evaluate the same IEEE operation sequence, so 0 is observed);
+probabilities and log-probs: 1e-5 relative in fp32, 2e-3 in fp16/bf16 (observed: bit-exact).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import ft_oracle as O
+from helpers import DTYPES, DTYPE_NAMES, bits, make_logits, make_word_list, to_numpy, to_torch, ulp_diff_f32, uniforms
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+    assert torch.cuda.is_available()
+    return torch, fa.ftk(), ops
+
+
+def _sync(torch):
+    torch.cuda.synchronize()
+
+
+def test_device_math_matches_host_bitwise(env):
+    torch, lib, ops = env
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.uniform(-104, 89, 400000), rng.uniform(-1, 1, 50000),
+                        -np.abs(rng.standard_normal(200000)) * 10, [0.0, -0.0, -103.9, 88.7, -200.0, 100.0]])
+    x = x.astype(np.float32)
+    d_in = to_torch(x)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(0, d_in.data_ptr(), d_out.data_ptr(), x.size, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), O.expf(x).view(np.uint32))
+    xl = np.abs(np.concatenate([rng.uniform(0, 1, 300000), np.exp(rng.uniform(-100, 88, 300000)),
+                                [0.0, 1.0, 1e-40, 3e38]])).astype(np.float32)
+    d_in = to_torch(xl)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(1, d_in.data_ptr(), d_out.data_ptr(), xl.size, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), O.logf(xl).view(np.uint32))
+
+
+def test_device_conversions_division_subnormals(env):
+    torch, lib, ops = env
+    rng = np.random.default_rng(2)
+    x = np.concatenate([rng.standard_normal(300000) * 100, rng.uniform(-7e4, 7e4, 100000),
+                        rng.standard_normal(100000) * 1e-5, rng.standard_normal(100000) * 1e-7,
+                        [65504.0, 65519.9, 65520.0, -65520.0, 6.0e-8, 2.98e-8, 2.9802322e-8]]).astype(np.float32)
+    d_in = to_torch(x)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(2, d_in.data_ptr(), d_out.data_ptr(), x.size, ops.current_stream()))
+    _sync(torch)
+    ref = O.to_f32(O.to_storage(x, O.F16), O.F16)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), ref.view(np.uint32))
+    ops.check(lib.ftk_test_device_math(3, d_in.data_ptr(), d_out.data_ptr(), x.size, ops.current_stream()))
+    _sync(torch)
+    ref = O.to_f32(O.to_storage(x, O.BF16), O.BF16)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), ref.view(np.uint32))
+    # correctly rounded division and subnormal arithmetic (the softmax relies on both)
+    t = rng.uniform(0.01, 3.0, 200000).astype(np.float32)
+    d_in = to_torch(t)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(4, d_in.data_ptr(), d_out.data_ptr(), t.size, ops.current_stream()))
+    _sync(torch)
+    ref = (np.float32(1.0) / (t + np.float32(1e-6))).astype(np.float32)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), ref.view(np.uint32))
+    s = rng.uniform(0.0, 4.0, 100000).astype(np.float32)
+    d_in = to_torch(s)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(5, d_in.data_ptr(), d_out.data_ptr(), s.size, ops.current_stream()))
+    _sync(torch)
+    tiny = np.float32(1.1754944e-38)
+    ref = (s * tiny + (s * np.float32(0.5)) * tiny).astype(np.float32)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("V,Vp", [(4, 4), (50001, 50001), (50001, 50008), (32000, 32000), (1000, 1024)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_temperature_penalty(env, dt, V, Vp, with_bias):
+    torch, lib, ops = env
+    rng = np.random.default_rng(V + Vp + dt)
+    batch = 6
+    logits = make_logits(rng, dt, batch, V, Vp, scale=3.0)
+    bias = O.to_storage((rng.standard_normal(Vp) * 2).astype(np.float32), dt) if with_bias else None
+    temps = rng.uniform(0.3, 2.0, batch).astype(np.float32)
+    # batch variant
+    ref = logits.copy()
+    O.batch_apply_temperature_penalty(dt, ref, bias, temps, batch, V, Vp)
+    d = to_torch(logits, dt)
+    d_bias = to_torch(bias, dt)
+    d_t = to_torch(temps)
+    ops.check(lib.ftk_invoke_batch_apply_temperature_penalty(dt, d.data_ptr(), ops.ptr(d_bias), d_t.data_ptr(), batch,
+                                                             V, Vp, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+    # scalar variant
+    ref = logits.copy()
+    O.apply_temperature_penalty(dt, ref, bias, 0.53, batch, V, Vp)
+    d = to_torch(logits, dt)
+    ops.check(lib.ftk_invoke_apply_temperature_penalty(dt, d.data_ptr(), ops.ptr(d_bias), 0.53, batch, V, Vp,
+                                                       ops.current_stream()))
+    _sync(torch)
+    got = to_numpy(d, dt)
+    if dt == O.F32:
+        assert ulp_diff_f32(got, ref).max() <= 1
+    assert np.array_equal(bits(got, dt), bits(ref, dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("ptype", [O.PEN_ADDITIVE, O.PEN_MULTIPLICATIVE])
+@pytest.mark.parametrize("V,max_input,step", [(4, 5, 8), (50001, 5, 40), (50001, 1003, 1200), (32000, 0, 2048)])
+def test_repetition_penalty(env, dt, ptype, V, max_input, step):
+    torch, lib, ops = env
+    rng = np.random.default_rng(V + step + ptype)
+    batch, local = 6, 6
+    Vp = V
+    logits = make_logits(rng, dt, batch, V, Vp, scale=3.0)
+    out_ids = rng.integers(0, V, (step, batch)).astype(np.int32)
+    input_lengths = rng.integers(1, max_input + 1, batch).astype(np.int32) if max_input > 0 else np.zeros(batch, np.int32)
+    pens = np.array([1.0, 0.53, 2.01, 1.2, 0.0, 3.0], np.float32) if ptype == O.PEN_ADDITIVE else \
+        np.array([1.0, 0.53, 2.01, 1.2, 0.7, 3.0], np.float32)
+    ref = logits.copy()
+    O.batch_apply_repetition_penalty(dt, ref, pens, out_ids, batch, local, Vp, input_lengths, max_input, step, ptype)
+    d = to_torch(logits, dt)
+    d_ids, d_len, d_pen = to_torch(out_ids), to_torch(input_lengths), to_torch(pens)
+    ops.check(lib.ftk_invoke_batch_apply_repetition_penalty(dt, d.data_ptr(), d_pen.data_ptr(), d_ids.data_ptr(), batch,
+                                                            local, Vp, d_len.data_ptr(), max_input, step, ptype,
+                                                            ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+    # scalar variant, without input_lengths
+    ref = logits.copy()
+    O.apply_repetition_penalty(dt, ref, 1.3, out_ids, batch, local, V, Vp, None, max_input, step, ptype)
+    d = to_torch(logits, dt)
+    ops.check(lib.ftk_invoke_apply_repetition_penalty(dt, d.data_ptr(), 1.3, None, d_ids.data_ptr(), batch, local, V,
+                                                      Vp, None, max_input, step, ptype, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_frequency_penalty_extension(env, dt):
+    torch, lib, ops = env
+    rng = np.random.default_rng(11)
+    batch, V, step, max_input = 4, 32000, 700, 16
+    logits = make_logits(rng, dt, batch, V, V, scale=2.0)
+    out_ids = np.minimum(rng.zipf(1.2, (step, batch)), V - 1).astype(np.int32)
+    input_lengths = rng.integers(1, max_input + 1, batch).astype(np.int32)
+    pres = np.array([0.5, 0.0, 1.0, 0.25], np.float32)
+    freq = np.array([0.3, 0.1, 0.0, 0.0], np.float32)
+    ref = logits.copy()
+    O.batch_apply_frequency_penalty(dt, ref, pres, freq, out_ids, batch, batch, V, input_lengths, max_input, step)
+    d = to_torch(logits, dt)
+    d_ids, d_len, d_pres, d_freq = to_torch(out_ids), to_torch(input_lengths), to_torch(pres), to_torch(freq)
+    ops.check(lib.ftk_invoke_batch_apply_frequency_penalty(dt, d.data_ptr(), d_pres.data_ptr(), d_freq.data_ptr(),
+                                                           d_ids.data_ptr(), batch, batch, V, d_len.data_ptr(),
+                                                           max_input, step, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_min_length_and_end_mask(env, dt):
+    torch, lib, ops = env
+    rng = np.random.default_rng(5)
+    batch, V, Vp = 70, 1000, 1024
+    logits = make_logits(rng, dt, batch, V, Vp)
+    min_lengths = rng.integers(0, 8, batch).astype(np.int32)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    seq = rng.integers(3, 12, batch).astype(np.int32)
+    ref = logits.copy()
+    O.min_length_penalty(dt, ref, min_lengths, end_ids, seq, 4, batch, Vp)
+    d = to_torch(logits, dt)
+    ops.check(lib.ftk_invoke_min_length_penalty(dt, d.data_ptr(), to_torch(min_lengths).data_ptr(),
+                                                to_torch(end_ids).data_ptr(), to_torch(seq).data_ptr(), 4, batch, Vp,
+                                                ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+    finished = (rng.random(batch) < 0.3)
+    for bias in (None, O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt)):
+        ref = logits.copy()
+        O.add_bias_end_mask(dt, ref, bias, end_ids, finished, batch, V, Vp)
+        d = to_torch(logits, dt)
+        ops.check(lib.ftk_invoke_add_bias_end_mask(dt, d.data_ptr(), ops.ptr(to_torch(bias, dt)),
+                                                   to_torch(end_ids).data_ptr(), to_torch(finished).data_ptr(), batch,
+                                                   V, Vp, ops.current_stream()))
+        _sync(torch)
+        assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("V,Vp", [(8, 8), (50, 56), (1000, 1024), (4000, 4000), (50257, 51200)])
+def test_softmax(env, dt, V, Vp):
+    torch, lib, ops = env
+    rng = np.random.default_rng(V * 3 + dt)
+    batch = 5
+    logits = make_logits(rng, dt, batch, V, Vp, scale=3.0)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    finished = np.array([False, True, False, False, True])
+    for bias in (None, O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt)):
+        ref = logits.copy()
+        O.add_bias_softmax(dt, ref, bias, end_ids, finished, batch, Vp, V)
+        d = to_torch(logits, dt)
+        ops.check(lib.ftk_invoke_add_bias_softmax(dt, d.data_ptr(), ops.ptr(to_torch(bias, dt)),
+                                                  to_torch(end_ids).data_ptr(), to_torch(finished).data_ptr(), batch,
+                                                  Vp, V, ops.current_stream()))
+        _sync(torch)
+        got = to_numpy(d, dt)
+        rtol = 1e-5 if dt == O.F32 else 2e-3
+        np.testing.assert_allclose(O.to_f32(got, dt), O.to_f32(ref, dt), rtol=rtol, atol=1e-30)
+        assert np.array_equal(bits(got, dt), bits(ref, dt))  # same IEEE sequence on both sides
+
+
+def _run_topk(env, dt, logits, k_arr, p_arr, max_k, end_ids, u, finished=None, seq=None, skip=None, logprobs=False):
+    torch, lib, ops = env
+    batch, Vp = logits.shape
+    d_logits = to_torch(logits, dt)
+    d_ids = torch.full((batch,), -7, dtype=torch.int32, device="cuda")
+    d_fin = to_torch(finished) if finished is not None else None
+    d_seq = to_torch(seq) if seq is not None else None
+    d_cum = torch.zeros(batch, dtype=torch.float32, device="cuda") if logprobs else None
+    d_out = torch.zeros(batch, dtype=torch.float32, device="cuda") if logprobs else None
+    d_k = to_torch(k_arr) if k_arr is not None else None
+    d_p = to_torch(p_arr) if p_arr is not None else None
+    d_skip = to_torch(skip) if skip is not None else None
+    d_end, d_u = to_torch(end_ids), to_torch(u)
+    ws_size = C.c_size_t(0)
+    ops.check(lib.ftk_invoke_batch_topk_sampling(dt, None, C.addressof(ws_size), None, None, None, None, None, None,
+                                                 None, None, max_k, None, 1.0, None, Vp, None, None, batch, None))
+    ws = torch.empty(max(ws_size.value, 16), dtype=torch.uint8, device="cuda")
+    ops.check(lib.ftk_invoke_batch_topk_sampling(dt, ws.data_ptr(), C.addressof(ws_size), d_logits.data_ptr(),
+                                                 d_ids.data_ptr(), ops.ptr(d_seq), ops.ptr(d_fin), ops.ptr(d_cum),
+                                                 ops.ptr(d_out), None, d_u.data_ptr(), max_k, ops.ptr(d_k), 1.0,
+                                                 ops.ptr(d_p), Vp, d_end.data_ptr(), ops.current_stream(), batch,
+                                                 ops.ptr(d_skip)))
+    _sync(torch)
+    return (to_numpy(d_ids), to_numpy(d_fin) if d_fin is not None else None,
+            to_numpy(d_seq) if d_seq is not None else None, to_numpy(d_cum) if logprobs else None,
+            to_numpy(d_out) if logprobs else None)
+
+
+def _oracle_topk(dt, logits, k_arr, p_arr, max_k, end_ids, u, finished=None, seq=None, skip=None, logprobs=False):
+    batch, Vp = logits.shape
+    ids = np.full(batch, -7, np.int32)
+    fin = finished.copy() if finished is not None else None
+    sq = seq.copy() if seq is not None else None
+    cum = np.zeros(batch, np.float32) if logprobs else None
+    out = np.zeros(batch, np.float32) if logprobs else None
+    rc = O.batch_topk_sampling(dt, logits, ids, sq, fin, cum, out, u, max_k, k_arr, 1.0, p_arr, Vp, end_ids, batch,
+                               skip)
+    assert rc == 0
+    return ids, fin, sq, cum, out
+
+
+def _compare_topk(a, b, dt):
+    assert np.array_equal(a[0], b[0]), "sampled ids differ"
+    for x, y in zip(a[1:3], b[1:3]):
+        if x is not None:
+            assert np.array_equal(x, y)
+    rtol = 1e-5 if dt == O.F32 else 2e-3
+    for x, y in zip(a[3:], b[3:]):
+        if x is not None:
+            np.testing.assert_allclose(x, y, rtol=rtol, atol=1e-6)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("V,batch,ks", [
+    (8, 6, [1, 2, 4, 2, 1, 3]), (4000, 8, [1, 4, 63, 16, 17, 33, 64, 5]), (51200, 6, [1, 4, 16, 40, 64, 1024]),
+    (50257, 4, [40, 40, 7, 1]), (32000, 5, [50, 50, 200, 300, 1000]),
+])
+def test_topk_sampling_logits(env, dt, V, batch, ks):
+    rng = np.random.default_rng(V + batch)
+    logits = make_logits(rng, dt, batch, V, V, scale=3.0, spikes=4 if V > 100 else 0)
+    k_arr = np.array(ks, np.int32)
+    p_arr = rng.uniform(0.3, 1.0, batch).astype(np.float32)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    finished = np.zeros(batch, bool)
+    finished[batch // 2] = True
+    seq = rng.integers(1, 9, batch).astype(np.int32)
+    skip = np.zeros(batch, bool)
+    skip[-1] = V > 8
+    for trial in range(3):
+        u = uniforms(rng, batch)
+        args = (dt, logits, k_arr, p_arr, int(k_arr.max()), end_ids, u, finished, seq, skip)
+        _compare_topk(_run_topk(env, *args), _oracle_topk(*args), dt)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_topk_sampling_tie_stress(env, dt):
+    """rows with few distinct values: the pick order is decided by the reference's tie rules alone"""
+    rng = np.random.default_rng(77)
+    for V, ks in [(5000, [8, 40, 64, 100]), (30000, [16, 33, 1, 500]), (1024, [1024, 700, 3, 64])]:
+        batch = len(ks)
+        levels = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0], np.float32)
+        x = levels[rng.integers(0, len(levels), (batch, V))]
+        x[0, :] = 1.0  # a completely flat row: takes the literal replay
+        logits = O.to_storage(x, dt)
+        k_arr = np.array(ks, np.int32)
+        p_arr = np.ones(batch, np.float32)
+        end_ids = np.zeros(batch, np.int32)
+        for trial in range(2):
+            u = uniforms(rng, batch)
+            args = (dt, logits, k_arr, p_arr, int(k_arr.max()), end_ids, u)
+            _compare_topk(_run_topk(env, *args), _oracle_topk(*args), dt)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_topk_sampling_on_probabilities_with_logprobs(env, dt):
+    rng = np.random.default_rng(9)
+    batch, V = 6, 4000
+    logits = make_logits(rng, dt, batch, V, V, scale=3.0)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    probs = logits.copy()
+    O.add_bias_softmax(dt, probs, None, end_ids, None, batch, V, V)
+    k_arr = np.array([1, 4, 63, 16, 64, 200], np.int32)
+    p_arr = rng.uniform(0.2, 1.0, batch).astype(np.float32)
+    finished = np.zeros(batch, bool)
+    seq = np.ones(batch, np.int32)
+    u = uniforms(rng, batch)
+    args = (dt, probs, k_arr, p_arr, 200, end_ids, u, finished, seq, None, True)
+    _compare_topk(_run_topk(env, *args), _oracle_topk(*args), dt)
+
+
+def test_topk_domain_error(env):
+    torch, lib, ops = env
+    ws = C.c_size_t(0)
+    rc = lib.ftk_invoke_batch_topk_sampling(O.F32, None, C.addressof(ws), None, None, None, None, None, None, None,
+                                            None, 1025, None, 1.0, None, 4000, None, None, 4, None)
+    assert rc == -2  # the reference throws std::domain_error for k = 1025
+
+
+def _run_topp(env, dt, probs, p_arr, end_ids, u, finished=None, seq=None, skip=None, logprobs=False, force_deep=False):
+    torch, lib, ops = env
+    batch, Vp = probs.shape
+    d_probs = to_torch(probs, dt)
+    d_ids = torch.full((batch,), -7, dtype=torch.int32, device="cuda")
+    d_fin = to_torch(finished) if finished is not None else None
+    d_seq = to_torch(seq) if seq is not None else None
+    d_cum = torch.zeros(batch, dtype=torch.float32, device="cuda") if logprobs else None
+    d_out = torch.zeros(batch, dtype=torch.float32, device="cuda") if logprobs else None
+    d_p = to_torch(p_arr)
+    d_skip = to_torch(skip) if skip is not None else None
+    d_end, d_u = to_torch(end_ids), to_torch(u)
+    ws_size, cub = C.c_size_t(0), C.c_size_t(0)
+    ops.check(lib.ftk_invoke_batch_topp_sampling(dt, None, C.addressof(ws_size), C.addressof(cub), None, None, None,
+                                                 None, None, None, None, None, None, None, None, batch, Vp, None, 1.0,
+                                                 None, None, None))
+    ws = torch.empty(max(ws_size.value, 16), dtype=torch.uint8, device="cuda")
+    lib.ftk_test_set_topp_force_deep(int(force_deep))
+    try:
+        ops.check(lib.ftk_invoke_batch_topp_sampling(dt, ws.data_ptr(), C.addressof(ws_size), C.addressof(cub),
+                                                     d_ids.data_ptr(), ops.ptr(d_seq), ops.ptr(d_fin), ops.ptr(d_cum),
+                                                     ops.ptr(d_out), d_probs.data_ptr(), None, None, None, None,
+                                                     d_u.data_ptr(), batch, Vp, d_end.data_ptr(),
+                                                     float(p_arr.max()), d_p.data_ptr(), ops.current_stream(),
+                                                     ops.ptr(d_skip)))
+        _sync(torch)
+    finally:
+        lib.ftk_test_set_topp_force_deep(0)
+    return (to_numpy(d_ids), to_numpy(d_fin) if d_fin is not None else None,
+            to_numpy(d_seq) if d_seq is not None else None, to_numpy(d_cum) if logprobs else None,
+            to_numpy(d_out) if logprobs else None)
+
+
+def _oracle_topp(dt, probs, p_arr, end_ids, u, finished=None, seq=None, skip=None, logprobs=False):
+    batch, Vp = probs.shape
+    ids = np.full(batch, -7, np.int32)
+    fin = finished.copy() if finished is not None else None
+    sq = seq.copy() if seq is not None else None
+    cum = np.zeros(batch, np.float32) if logprobs else None
+    out = np.zeros(batch, np.float32) if logprobs else None
+    O.batch_topp_sampling(dt, probs, ids, sq, fin, cum, out, u, batch, Vp, end_ids, 0.0, p_arr, skip)
+    return ids, fin, sq, cum, out
+
+
+def _zipf_probs(rng, dt, batch, V, s=1.1, noise=0.5):
+    ranks = np.arange(1, V + 1, dtype=np.float64)
+    base = -s * np.log(ranks)
+    x = np.empty((batch, V), np.float32)
+    for b in range(batch):
+        x[b] = (base[rng.permutation(V)] + rng.standard_normal(V) * noise).astype(np.float32)
+    logits = O.to_storage(x, dt)
+    probs = logits.copy()
+    O.add_bias_softmax(dt, probs, None, np.zeros(batch, np.int32), None, batch, V, V)
+    return probs
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("V,batch", [(8, 6), (4000, 8), (51200, 6), (128256, 4)])
+@pytest.mark.parametrize("force_deep", [False, True])
+def test_topp_sampling(env, dt, V, batch, force_deep):
+    rng = np.random.default_rng(V + batch + dt)
+    probs = _zipf_probs(rng, dt, batch, V) if V > 8 else None
+    if probs is None:
+        x = np.log(np.array([0.4, 0.3, 0.2, 0.1, 1e-9, 1e-9, 1e-9, 1e-9], np.float32))
+        logits = O.to_storage(np.tile(x, (batch, 1)), dt)
+        probs = logits.copy()
+        O.add_bias_softmax(dt, probs, None, np.zeros(batch, np.int32), None, batch, V, V)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    finished = np.zeros(batch, bool)
+    seq = rng.integers(1, 9, batch).astype(np.int32)
+    skip = np.zeros(batch, bool)
+    skip[1] = True
+    for trial in range(3):
+        p_arr = rng.uniform(0.2, 1.0, batch).astype(np.float32)
+        if trial == 2:
+            p_arr[:] = 1.0
+        u = uniforms(rng, batch)
+        if trial == 2:
+            u[0] = 1.0  # draw at the very end of the distribution: may never be crossed
+        args = (dt, probs, p_arr, end_ids, u, finished, seq, skip, True)
+        got = _run_topp(env, *args, force_deep=force_deep)
+        _compare_topk(got, _oracle_topp(*args), dt)
+
+
+@pytest.mark.parametrize("dt", [O.F32, O.F16], ids=lambda d: DTYPE_NAMES[d])
+def test_topp_sampling_flat_and_tied_rows(env, dt):
+    """uniform / heavily tied distributions: stable order (ascending id among equals) decides"""
+    rng = np.random.default_rng(21)
+    batch, V = 4, 20000
+    x = np.zeros((batch, V), np.float32)
+    x[1] = rng.integers(0, 3, V).astype(np.float32)
+    x[2, :100] = 5.0
+    x[3] = np.where(rng.random(V) < 0.5, -np.inf, 0.0)
+    logits = O.to_storage(x, dt)
+    probs = logits.copy()
+    O.add_bias_softmax(dt, probs, None, np.zeros(batch, np.int32), None, batch, V, V)
+    end_ids = np.zeros(batch, np.int32)
+    for trial in range(3):
+        p_arr = rng.uniform(0.3, 1.0, batch).astype(np.float32)
+        u = uniforms(rng, batch)
+        args = (dt, probs, p_arr, end_ids, u)
+        _compare_topk(_run_topp(env, *args), _oracle_topp(*args), dt)
+
+
+def test_topp_decay_and_initialize(env):
+    torch, lib, ops = env
+    rng = np.random.default_rng(3)
+    n = 300
+    top_p = rng.uniform(0.1, 1.0, n).astype(np.float32)
+    init = rng.uniform(0.1, 1.0, n).astype(np.float32)
+    ids = rng.integers(0, 20, n).astype(np.int32)
+    reset = rng.integers(0, 20, n).astype(np.int32)
+    decay = rng.uniform(0.5, 1.0, n).astype(np.float32)
+    pmin = rng.uniform(0.05, 0.6, n).astype(np.float32)
+    ref = top_p.copy()
+    O.compute_topp_decay(ref, init, ids, decay, pmin, reset, n)
+    d = to_torch(top_p)
+    ops.check(lib.ftk_invoke_compute_topp_decay(d.data_ptr(), to_torch(init).data_ptr(), to_torch(ids).data_ptr(),
+                                                to_torch(decay).data_ptr(), to_torch(pmin).data_ptr(),
+                                                to_torch(reset).data_ptr(), n, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(to_numpy(d).view(np.uint32), ref.view(np.uint32))
+    batch, V = 5, 77
+    idv = torch.zeros(batch * V, dtype=torch.int32, device="cuda")
+    off = torch.zeros(batch + 1, dtype=torch.int32, device="cuda")
+    boff = torch.zeros(batch + 1, dtype=torch.int32, device="cuda")
+    ops.check(lib.ftk_invoke_topp_initialize(idv.data_ptr(), off.data_ptr(), boff.data_ptr(), batch, V,
+                                             ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(to_numpy(idv), np.tile(np.arange(V, dtype=np.int32), batch))
+    assert np.array_equal(to_numpy(off), np.arange(batch + 1, dtype=np.int32) * V)
+    assert np.array_equal(to_numpy(boff), to_numpy(off))
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("shared", [True, False])
+def test_ban_bad_words(env, dt, shared):
+    torch, lib, ops = env
+    rng = np.random.default_rng(8 + int(shared))
+    batch, local, V, step, ite = 8, 4, 500, 9, 1
+    logits = make_logits(rng, dt, batch, V, V)
+    out_ids = rng.integers(1, V, (step + 1, batch)).astype(np.int32)
+    lists = []
+    for row in range(batch):
+        wl, _ = make_word_list(rng, 12, 4, V, L=48, history=out_ids, step=step, row=row)
+        lists.append(wl)
+    bad = lists[0] if shared else np.stack(lists)
+    ref = logits.copy()
+    off = ite * local
+    bw = bad if shared else bad[off:]
+    O.ban_bad_words(dt, ref[off:], out_ids, batch, local, np.ascontiguousarray(bw), shared, 48, off, V, step)
+    d = to_torch(logits, dt)
+    d_bad, d_ids = to_torch(np.ascontiguousarray(bw)), to_torch(out_ids)
+    elem = 4 if dt == O.F32 else 2
+    ops.check(lib.ftk_invoke_ban_bad_words(dt, d.data_ptr() + off * V * elem, d_ids.data_ptr(), None, batch, local, 1,
+                                           d_bad.data_ptr(), shared, 48, off, V, step, ops.current_stream()))
+    _sync(torch)
+    got = to_numpy(d, dt)
+    assert np.array_equal(bits(got, dt), bits(ref, dt))
+    assert np.isinf(O.to_f32(got, dt)).any()  # the case actually bans something
+
+
+def test_stop_words_and_length_criterion(env):
+    torch, lib, ops = env
+    rng = np.random.default_rng(4)
+    batch, V, step = 16, 50, 7
+    out_ids = rng.integers(1, V, (step + 1, batch)).astype(np.int32)
+    lists = []
+    for row in range(batch):
+        wl, _ = make_word_list(rng, 6, 3, V, L=20)
+        if row % 3 == 0:  # plant a stop word that matches the tail including the token at `step`
+            n = 1 + row % 3 + (row // 3) % 3
+            n = min(n, 3)
+            tail = out_ids[step - n + 1:step + 1, row]
+            wl[0, :n] = tail
+            wl[1, 0] = n
+        lists.append(wl)
+    stop = np.stack(lists)
+    finished = np.zeros(batch, bool)
+    ref = finished.copy()
+    O.stop_words_criterion(out_ids, stop, ref, 0, 20, batch, batch, step)
+    assert ref.any()
+    d_fin = to_torch(finished)
+    ops.check(lib.ftk_invoke_stop_words_criterion(to_torch(out_ids).data_ptr(), None, to_torch(stop).data_ptr(),
+                                                  d_fin.data_ptr(), 0, 20, batch, 1, step, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(to_numpy(d_fin), ref)
+    # length criterion
+    limit = rng.integers(3, 12, batch).astype(np.uint32)
+    for st, pre in [(5, ref), (20, ref)]:
+        fin = pre.copy()
+        should = np.zeros(1, bool)
+        O.length_criterion(fin, should, limit, batch, st)
+        d_fin = to_torch(pre)
+        pinned = torch.zeros(1, dtype=torch.int32).pin_memory()
+        host_flag = np.zeros(1, bool)
+        ops.check(lib.ftk_invoke_length_criterion(d_fin.data_ptr(), host_flag.ctypes.data, pinned.data_ptr(),
+                                                  to_torch(limit).data_ptr(), batch, 1, st, ops.current_stream()))
+        assert np.array_equal(to_numpy(d_fin), fin)
+        assert bool(host_flag[0]) == bool(should[0])
+        assert int(pinned[0]) == int(fin.sum())
+
+
+def test_rng_determinism_and_range(env):
+    torch, lib, ops = env
+    batch, n = 64, 500
+    st = torch.zeros(batch * 2, dtype=torch.int64, device="cuda")
+    ops.check(lib.ftk_invoke_curand_initialize(st.data_ptr(), batch, 1234, ops.current_stream()))
+    out1 = torch.empty(batch * n, dtype=torch.float32, device="cuda")
+    ops.check(lib.ftk_test_rng_uniform(st.data_ptr(), out1.data_ptr(), batch, n, ops.current_stream()))
+    _sync(torch)
+    a = to_numpy(out1).reshape(batch, n)
+    assert (a > 0).all() and (a <= 1).all()
+    assert np.array_equal(a[0], a[17])  # same seed, same stream of draws
+    assert abs(a.mean() - 0.5) < 0.02
+    assert to_numpy(st).reshape(batch, 2)[:, 1].tolist() == [n] * batch  # offsets advanced
+    seeds = to_torch(np.arange(batch, dtype=np.uint64) // 3)
+    ops.check(lib.ftk_invoke_curand_batch_initialize(st.data_ptr(), batch, seeds.data_ptr(), ops.current_stream()))
+    ops.check(lib.ftk_test_rng_uniform(st.data_ptr(), out1.data_ptr(), batch, n, ops.current_stream()))
+    _sync(torch)
+    b = to_numpy(out1).reshape(batch, n)
+    assert np.array_equal(b[0], b[1]) and np.array_equal(b[0], b[2]) and not np.array_equal(b[2], b[3])
+    # known answer: first draw of seed 0 is Philox4x32-10(ctr=0,key=0)[0] = 0x6627e8d5
+    expect = np.float32(np.float32(0x6627e8d5) * np.float32(2.3283064365386963e-10) + np.float32(1.16415321826934814453125e-10))
+    assert b[0, 0] == expect
