@@ -202,9 +202,15 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
     a.ids = output_tensors->at("output_ids").template getPtrWithOffset<int>((size_t)step * batch_size + off);
     a.sequence_length = output_tensors->at("sequence_length", Tensor()).template getPtr<int>();
     a.finished        = output_tensors->at("finished", Tensor()).template getPtr<bool>();
-    ensureWorkspace(local_batch_size);
-    a.workspace       = sampling_workspace_;
-    a.workspace_size  = sampling_workspace_size_;
+    // size query (null workspace), grow if this window needs more than setup() reserved
+    a.workspace = nullptr;
+    check_ftk(ftk_fused_topk_step(&a, stream_));
+    if (a.workspace_size > sampling_workspace_size_) {
+        sampling_workspace_      = allocator_->reMalloc(sampling_workspace_, a.workspace_size, false);
+        sampling_workspace_size_ = a.workspace_size;
+    }
+    a.workspace      = sampling_workspace_;
+    a.workspace_size = sampling_workspace_size_;
     check_ftk(ftk_fused_topk_step(&a, stream_));
     sync_check_hip_error();
     return true;

@@ -180,9 +180,9 @@ def test_min_length_and_end_mask(env, dt):
     ref = logits.copy()
     O.min_length_penalty(dt, ref, min_lengths, end_ids, seq, 4, batch, Vp)
     d = to_torch(logits, dt)
-    ops.check(lib.ftk_invoke_min_length_penalty(dt, d.data_ptr(), to_torch(min_lengths).data_ptr(),
-                                                to_torch(end_ids).data_ptr(), to_torch(seq).data_ptr(), 4, batch, Vp,
-                                                ops.current_stream()))
+    d_min, d_end, d_seq = to_torch(min_lengths), to_torch(end_ids), to_torch(seq)
+    ops.check(lib.ftk_invoke_min_length_penalty(dt, d.data_ptr(), d_min.data_ptr(), d_end.data_ptr(), d_seq.data_ptr(),
+                                                4, batch, Vp, ops.current_stream()))
     _sync(torch)
     assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
     finished = (rng.random(batch) < 0.3)
@@ -190,9 +190,9 @@ def test_min_length_and_end_mask(env, dt):
         ref = logits.copy()
         O.add_bias_end_mask(dt, ref, bias, end_ids, finished, batch, V, Vp)
         d = to_torch(logits, dt)
-        ops.check(lib.ftk_invoke_add_bias_end_mask(dt, d.data_ptr(), ops.ptr(to_torch(bias, dt)),
-                                                   to_torch(end_ids).data_ptr(), to_torch(finished).data_ptr(), batch,
-                                                   V, Vp, ops.current_stream()))
+        d_bias, d_fin = to_torch(bias, dt), to_torch(finished)
+        ops.check(lib.ftk_invoke_add_bias_end_mask(dt, d.data_ptr(), ops.ptr(d_bias), d_end.data_ptr(),
+                                                   d_fin.data_ptr(), batch, V, Vp, ops.current_stream()))
         _sync(torch)
         assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
 
@@ -210,9 +210,9 @@ def test_softmax(env, dt, V, Vp):
         ref = logits.copy()
         O.add_bias_softmax(dt, ref, bias, end_ids, finished, batch, Vp, V)
         d = to_torch(logits, dt)
-        ops.check(lib.ftk_invoke_add_bias_softmax(dt, d.data_ptr(), ops.ptr(to_torch(bias, dt)),
-                                                  to_torch(end_ids).data_ptr(), to_torch(finished).data_ptr(), batch,
-                                                  Vp, V, ops.current_stream()))
+        d_bias, d_end, d_fin = to_torch(bias, dt), to_torch(end_ids), to_torch(finished)
+        ops.check(lib.ftk_invoke_add_bias_softmax(dt, d.data_ptr(), ops.ptr(d_bias), d_end.data_ptr(),
+                                                  d_fin.data_ptr(), batch, Vp, V, ops.current_stream()))
         _sync(torch)
         got = to_numpy(d, dt)
         rtol = 1e-5 if dt == O.F32 else 2e-3
@@ -455,9 +455,9 @@ def test_topp_decay_and_initialize(env):
     ref = top_p.copy()
     O.compute_topp_decay(ref, init, ids, decay, pmin, reset, n)
     d = to_torch(top_p)
-    ops.check(lib.ftk_invoke_compute_topp_decay(d.data_ptr(), to_torch(init).data_ptr(), to_torch(ids).data_ptr(),
-                                                to_torch(decay).data_ptr(), to_torch(pmin).data_ptr(),
-                                                to_torch(reset).data_ptr(), n, ops.current_stream()))
+    d_init, d_ids, d_decay, d_pmin, d_reset = (to_torch(x) for x in (init, ids, decay, pmin, reset))
+    ops.check(lib.ftk_invoke_compute_topp_decay(d.data_ptr(), d_init.data_ptr(), d_ids.data_ptr(), d_decay.data_ptr(),
+                                                d_pmin.data_ptr(), d_reset.data_ptr(), n, ops.current_stream()))
     _sync(torch)
     assert np.array_equal(to_numpy(d).view(np.uint32), ref.view(np.uint32))
     batch, V = 5, 77
@@ -521,8 +521,9 @@ def test_stop_words_and_length_criterion(env):
     O.stop_words_criterion(out_ids, stop, ref, 0, 20, batch, batch, step)
     assert ref.any()
     d_fin = to_torch(finished)
-    ops.check(lib.ftk_invoke_stop_words_criterion(to_torch(out_ids).data_ptr(), None, to_torch(stop).data_ptr(),
-                                                  d_fin.data_ptr(), 0, 20, batch, 1, step, ops.current_stream()))
+    d_ids, d_stop = to_torch(out_ids), to_torch(stop)
+    ops.check(lib.ftk_invoke_stop_words_criterion(d_ids.data_ptr(), None, d_stop.data_ptr(), d_fin.data_ptr(), 0, 20,
+                                                  batch, 1, step, ops.current_stream()))
     _sync(torch)
     assert np.array_equal(to_numpy(d_fin), ref)
     # length criterion
@@ -532,10 +533,11 @@ def test_stop_words_and_length_criterion(env):
         should = np.zeros(1, bool)
         O.length_criterion(fin, should, limit, batch, st)
         d_fin = to_torch(pre)
+        d_limit = to_torch(limit)
         pinned = torch.zeros(1, dtype=torch.int32).pin_memory()
         host_flag = np.zeros(1, bool)
         ops.check(lib.ftk_invoke_length_criterion(d_fin.data_ptr(), host_flag.ctypes.data, pinned.data_ptr(),
-                                                  to_torch(limit).data_ptr(), batch, 1, st, ops.current_stream()))
+                                                  d_limit.data_ptr(), batch, 1, st, ops.current_stream()))
         assert np.array_equal(to_numpy(d_fin), fin)
         assert bool(host_flag[0]) == bool(should[0])
         assert int(pinned[0]) == int(fin.sum())
