@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Headline benchmark: one DynamicDecodeLayer step (top-k + top-p + temperature + repetition penalty)
+over a [256, 128256] fp32 logits batch on one MI355X.
+
+A "step" is one DynamicDecodeLayer::forward over one batch of seeded synthetic logits already resident in
+HBM. The logits cycle through several buffers whose total size exceeds the 256 MB last-level cache, so
+every step streams its logits from HBM. Prints one JSON line (see the keys below).
+
+    python bench.py --gpus 1 --steps 50 --warmup 5
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # the configuration the metric is quoted on (BASELINE.json "metric" / north-star target)
+    "decode_step_b256_v128256_f32_topk64_topp0.9_temp0.8_rep1.1": dict(
+        dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=64, top_p=0.9, temperature=0.8,
+        repetition_penalty=1.1, prompt=64, sigma=2.5),
+}
+
+
+def algorithmic_bytes(w, step):
+    elem = 4 if w["dtype"] == "f32" else 2
+    history = step if w.get("repetition_penalty") else 0
+    return w["batch"] * w["vocab_padded"] * elem + w["batch"] * history * 4 + w["batch"] * 32
+
+
+def run_gpu(name, w, steps, warmup, nbuf=4):
+    import torch
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    dt = {"f32": fa.F32, "f16": fa.F16, "bf16": fa.BF16}[w["dtype"]]
+    B, V, Vp, H = w["batch"], w["vocab"], w["vocab_padded"], w["prompt"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+    bufs = [(torch.randn((B, 1, Vp), generator=gen, device=dev, dtype=torch.float32) * w["sigma"]).to(fa.torch_dtype(dt))
+            for _ in range(nbuf)]
+    total = steps + warmup
+    max_seq = H + total + 1
+    output_ids = torch.zeros((max_seq, B), dtype=torch.int32, device=dev)
+    output_ids[:H] = torch.randint(0, V, (H, B), generator=gen, device=dev, dtype=torch.int32)
+    finished = torch.zeros(B, dtype=torch.bool, device=dev)
+    seq_len = torch.full((B,), H - 1, dtype=torch.int32, device=dev)
+    end_id = torch.full((B,), V - 1, dtype=torch.int32, device=dev)
+    draws = [torch.rand(B, generator=gen, device=dev).clamp_(min=1e-7) for _ in range(nbuf)]
+
+    layer = fa.DynamicDecodeLayer(dt, V, Vp)
+    args = {"runtime_top_k": np.array([w["top_k"]], np.uint32), "runtime_top_p": np.array([w["top_p"]], np.float32),
+            "temperature": np.array([w["temperature"]], np.float32),
+            "repetition_penalty": np.array([w["repetition_penalty"]], np.float32),
+            "random_seed": np.array([7], np.uint64)}
+    layer.setup(B, 1, args)
+    outs = {"output_ids": output_ids, "finished": finished, "sequence_length": seq_len}
+    step_arr = np.zeros(1, np.int32)
+    base = {"step": step_arr, "max_input_length": np.array([H], np.int32), "ite": np.array([0], np.uint32),
+            "local_batch_size": np.array([B], np.int32), "end_id": end_id}
+
+    def one_step(i):
+        step_arr[0] = H + i
+        ins = dict(base, logits=bufs[i % nbuf], uniform_draws=draws[i % nbuf])
+        layer.forward(outs, ins)
+
+    lib = fa.ftk()
+    for i in range(warmup):
+        one_step(i)
+    torch.cuda.synchronize()
+    ops.check(lib.ftk_profile_enable(steps))
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    for i in range(warmup, total):
+        one_step(i)
+    ev1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = ev0.elapsed_time(ev1)
+    kernel_ms = []
+    for k in range(3):
+        tot, n = C.c_double(0.0), C.c_int(0)
+        ops.check(lib.ftk_profile_read(k, C.addressof(tot), C.addressof(n)))
+        kernel_ms.append((tot.value / n.value) if n.value else 0.0)
+    ops.check(lib.ftk_profile_enable(0))
+
+    ms_per_step = wall * 1e3 / steps
+    mid_step = H + warmup + steps // 2
+    alg = algorithmic_bytes(w, mid_step)
+    gather_ms = kernel_ms[1]
+    achieved = alg / (gather_ms * 1e-3) / 1e9 if gather_ms > 0 else 0.0
+    return dict(
+        tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
+        kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2]),
+        roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
+                      traffic=None, kernel="fused_gather_kernel", algorithmic_bytes_per_launch=alg),
+        step_gbs=alg / (gpu_ms / steps * 1e-3) / 1e9,
+        sampled_ids_checksum=int(output_ids[H + warmup:H + total].to(torch.int64).sum().item()),
+    )
+
+
+def run_cpu_baseline(w, budget_s=12.0):
+    """the oracle (a scalar, single-threaded restatement of the reference algorithm) on rows of the same
+    workload, until `budget_s` seconds of CPU work have been spent"""
+    import ft_oracle as O
+    dt = {"f32": O.F32, "f16": O.F16, "bf16": O.BF16}[w["dtype"]]
+    V, Vp, H = w["vocab"], w["vocab_padded"], w["prompt"]
+    rows = 16
+    rng = np.random.default_rng(99)
+    layer = O.OracleDynamicDecodeLayer(dt, V, Vp)
+    layer.setup(rows, [w["top_k"]], [w["top_p"]], [w["temperature"]], [w["repetition_penalty"]])
+    out_ids = np.zeros((H + 64, rows), np.int32)
+    out_ids[:H] = rng.integers(0, V, (H, rows))
+    finished = np.zeros(rows, np.bool_)
+    seq = np.full(rows, H - 1, np.int32)
+    end = np.full(rows, V - 1, np.int32)
+    done, spent, step = 0, 0.0, H
+    while spent < budget_s and step < H + 63:
+        logits = O.to_storage((rng.standard_normal((rows, Vp)) * w["sigma"]).astype(np.float32), dt)
+        u = rng.random(rows).astype(np.float32) * 0.999 + 0.001
+        t0 = time.perf_counter()
+        layer.forward(logits, end, out_ids, step, H, u, finished=finished, sequence_length=seq)
+        spent += time.perf_counter() - t0
+        done += rows
+        step += 1
+    return dict(value=done / spent, unit="tokens/s", cores=1, kind="port",
+                sample="%d rows of the same step (%d decode steps of a %d-row batch), %.1f s of CPU time"
+                       % (done, step - H, rows, spent))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU leg (rows shard across GPUs with no "
+              "exchange, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    name = next(iter(WORKLOADS))
+    w = WORKLOADS[name]
+    r = run_gpu(name, w, a.steps, a.warmup)
+    line = {
+        "metric": "sampled tokens/s, decode step B=256 V=128256 (full top-k+top-p+penalty DynamicDecodeLayer step)",
+        "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"], "top_k": w["top_k"],
+                   "top_p": w["top_p"], "temperature": w["temperature"],
+                   "repetition_penalty": w["repetition_penalty"], "history": w["prompt"]},
+        "roofline": r["roofline"],
+        "gpu_ms_per_step": r["gpu_ms_per_step"], "kernel_ms": r["kernel_ms"], "step_hbm_gbs": r["step_gbs"],
+        "step_hbm_frac": r["step_gbs"] / HBM_PEAK_GBS, "sampled_ids_checksum": r["sampled_ids_checksum"],
+    }
+    if not a.no_cpu_baseline:
+        line["cpu_baseline"] = run_cpu_baseline(w)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

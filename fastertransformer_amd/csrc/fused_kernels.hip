@@ -11,6 +11,8 @@
 //                           over the vocabulary (who gets the repetition / presence penalty)
 //   fused_gather_kernel   - grid (splits, rows): stream, transform, gather candidates
 //   fused_select_kernel   - one workgroup per row: exact tie order, sampling, bookkeeping
+#include <vector>
+
 #include "ftk_sampling.h"
 #include "ftk_topk.cuh"
 
@@ -225,6 +227,92 @@ fused_select_kernel(FusedParams p, int* __restrict__ ids, int* __restrict__ sequ
 
 using namespace ftk;
 
+// ---- optional per-kernel timing (HIP events on the caller's stream) ------------------------------
+namespace {
+struct KernelTimer {
+    std::vector<hipEvent_t> start, stop;
+    int                     used = 0;
+};
+KernelTimer g_timers[3];
+bool        g_profile = false;
+
+struct ScopedKernelTime {
+    KernelTimer* t  = nullptr;
+    hipStream_t  st = nullptr;
+    int          i  = -1;
+    ScopedKernelTime(int which, hipStream_t stream)
+    {
+        if (g_profile && g_timers[which].used < (int)g_timers[which].start.size()) {
+            t  = &g_timers[which];
+            st = stream;
+            i  = t->used++;
+            (void)hipEventRecord(t->start[i], st);
+        }
+    }
+    ~ScopedKernelTime()
+    {
+        if (t != nullptr) {
+            (void)hipEventRecord(t->stop[i], st);
+        }
+    }
+};
+}  // namespace
+
+extern "C" int ftk_profile_enable(int max_launches)
+{
+    for (auto& t : g_timers) {
+        for (auto e : t.start) {
+            (void)hipEventDestroy(e);
+        }
+        for (auto e : t.stop) {
+            (void)hipEventDestroy(e);
+        }
+        t.start.clear();
+        t.stop.clear();
+        t.used = 0;
+        for (int i = 0; i < max_launches; ++i) {
+            hipEvent_t a, b;
+            hipError_t e = hipEventCreate(&a);
+            if (e != hipSuccess) {
+                return (int)e;
+            }
+            e = hipEventCreate(&b);
+            if (e != hipSuccess) {
+                return (int)e;
+            }
+            t.start.push_back(a);
+            t.stop.push_back(b);
+        }
+    }
+    g_profile = max_launches > 0;
+    return 0;
+}
+
+extern "C" int ftk_profile_read(int kernel, double* total_ms, int* launches)
+{
+    if (kernel < 0 || kernel > 2 || total_ms == nullptr || launches == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    KernelTimer& t = g_timers[kernel];
+    double       sum = 0.0;
+    for (int i = 0; i < t.used; ++i) {
+        hipError_t e = hipEventSynchronize(t.stop[i]);
+        if (e != hipSuccess) {
+            return (int)e;
+        }
+        float ms = 0.0f;
+        e        = hipEventElapsedTime(&ms, t.start[i], t.stop[i]);
+        if (e != hipSuccess) {
+            return (int)e;
+        }
+        sum += ms;
+    }
+    *total_ms = sum;
+    *launches = t.used;
+    t.used    = 0;
+    return 0;
+}
+
 extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
 {
     if (a == nullptr) {
@@ -287,7 +375,8 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         if (a->output_ids == nullptr) {
             return FTK_ERR_ARGUMENT;
         }
-        uint32_t* bitmaps = (uint32_t*)ws;
+        uint32_t*        bitmaps = (uint32_t*)ws;
+        ScopedKernelTime timer(0, st);
         history_bitmap_kernel<<<rows, HB_THREADS, 0, st>>>(bitmaps, bitmap_words, a->output_ids, a->batch_size,
                                                            a->vocab_size_padded, a->input_lengths,
                                                            a->max_input_length, a->step, a->skip_decode, a->finished);
@@ -300,12 +389,19 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     TopkChunkHeader* headers = (TopkChunkHeader*)(ws + bitmap_bytes);
     TopkEntry*       entries = (TopkEntry*)(headers + (size_t)rows * plan.splits);
     dim3             grid(plan.splits, rows);
-    FTK_DISPATCH_DTYPE(a->dtype, fused_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(
-                                     p, plan.splits, plan.nvt, plan.cap, plan.row_entries, headers, entries));
+    {
+        ScopedKernelTime timer(1, st);
+        FTK_DISPATCH_DTYPE(a->dtype, fused_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(
+                                         p, plan.splits, plan.nvt, plan.cap, plan.row_entries, headers, entries));
+    }
     FTK_LAUNCH_CHECK();
-    FTK_DISPATCH_DTYPE(a->dtype, fused_select_kernel<DT><<<rows, TK_THREADS, 0, st>>>(
-                                     p, a->ids, a->sequence_length, a->finished, (RngState*)a->rng_state,
-                                     a->uniform_draws, plan.splits, plan.cap, plan.row_entries, headers, entries));
+    {
+        ScopedKernelTime timer(2, st);
+        FTK_DISPATCH_DTYPE(a->dtype, fused_select_kernel<DT><<<rows, TK_THREADS, 0, st>>>(
+                                         p, a->ids, a->sequence_length, a->finished, (RngState*)a->rng_state,
+                                         a->uniform_draws, plan.splits, plan.cap, plan.row_entries, headers,
+                                         entries));
+    }
     FTK_LAUNCH_CHECK();
     return 0;
 }

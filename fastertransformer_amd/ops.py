@@ -55,6 +55,8 @@ _SIGNATURES = {
     "ftk_test_set_topp_force_deep": [_i],
     "ftk_host_philox4x32_10": [_vp, _vp, _vp],
     "ftk_error_string": [_i],
+    "ftk_profile_enable": [_i],
+    "ftk_profile_read": [_i, _vp, _vp],
 }
 _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_char_p,
              "ftk_test_set_topp_force_deep": None, "ftk_host_philox4x32_10": None}

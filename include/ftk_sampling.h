@@ -210,6 +210,14 @@ typedef struct ftk_fused_topk_args {
 /* workspace == NULL in args: writes the required size into args->workspace_size, launches nothing. */
 int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
 
+/* ---- per-kernel timing of the fused step (the reference's counterpart is its CudaTimer / NVTX ranges,
+ * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
+ * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on
+ * the caller's stream (n = 0 switches it off); ftk_profile_read sums them (it synchronises on the
+ * events) and resets the count. kernel: 0 = history bitmap, 1 = gather (the streaming pass), 2 = select. */
+int ftk_profile_enable(int max_launches);
+int ftk_profile_read(int kernel, double* total_ms, int* launches);
+
 /* ---- test hooks (host-side instances of the shared arithmetic, and device probes) ----------- */
 float ftk_host_expf(float x);
 float ftk_host_logf(float x);
