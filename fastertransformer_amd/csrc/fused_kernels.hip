@@ -35,9 +35,17 @@ struct FusedParams {
     int          max_top_k;
     const bool*  skip_decode;
     const bool*  finished_in;
-    const uint32_t* bitmaps;  // [rows][bitmap_words] or null
-    int             bitmap_words;
+    uint32_t*    bitmaps;        // [rows][bitmap_words] scratch, or null when no history penalty applies
+    int          bitmap_words;
+    int          bitmaps_ready;  // history_bitmap_kernel filled `bitmaps` (long histories)
 };
+
+// History bitmaps: bit v set <=> token v occurs in the row's (non-padding) history, i.e. column v gets
+// the repetition / presence penalty. Short histories: every gather workgroup builds the window of the
+// bitmap that covers its own chunk in LDS (a few hundred strided 4-byte reads that overlap the logits
+// loads already in flight). Long histories: history_bitmap_kernel builds whole-row bitmaps once.
+constexpr int FUSED_LOCAL_BITMAP_MAX_STEP = 4096;
+constexpr int FUSED_LDS_BITMAP_WORDS      = TK_ELEMS * TK_THREADS / 32 + 4;
 
 template<int DT>
 struct FusedRow {
@@ -45,27 +53,41 @@ struct FusedRow {
     typedef typename S::T T;
     const T*              rowp;
     const T*              bias;
-    const uint32_t*       bitmap;  // this row's history bitmap or null
     int                   V, Vp;
     bool                  temp_active, keep_pads;
     float                 inv;
-    int                   penalty_type;
+    int                   penalty_type;  // 2 = none
     float                 penalty;
     int                   masked_end_id;  // end id when the min-length mask applies, else -1
+    // history bitmap
+    const uint32_t* bm;         // words in use (global row bitmap or the LDS window), null = none
+    int             bm_origin;  // column of bit 0 of bm[0]
+    uint32_t*       global_bm;  // this row's slice of the scratch bitmaps
+    bool            global_ready;
+    const int*      history;  // output_ids + row, stride batch_size
+    int             batch_size, step, input_length, max_input_length;
 
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row)
     {
-        rowp         = (const T*)p.logits + (size_t)row * p.Vp;
-        bias         = (const T*)p.bias;
-        V            = p.V;
-        Vp           = p.Vp;
-        temp_active  = p.temperatures != nullptr;
+        rowp        = (const T*)p.logits + (size_t)row * p.Vp;
+        bias        = (const T*)p.bias;
+        V           = p.V;
+        Vp          = p.Vp;
+        temp_active = p.temperatures != nullptr;
         const TemperatureCtx<DT> tc(temp_active ? p.temperatures[row] : 1.0f, V, Vp, false);
-        inv          = tc.inv;
-        keep_pads    = tc.keep_pads;
-        penalty_type = p.penalties != nullptr ? p.penalty_type : 2;
-        penalty      = p.penalties != nullptr ? p.penalties[row] : 0.0f;
-        bitmap       = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
+        inv           = tc.inv;
+        keep_pads     = tc.keep_pads;
+        penalty_type  = p.penalties != nullptr ? p.penalty_type : 2;
+        penalty       = p.penalties != nullptr ? p.penalties[row] : 0.0f;
+        global_bm     = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
+        global_ready  = p.bitmaps_ready != 0;
+        bm            = global_ready ? global_bm : nullptr;
+        bm_origin     = 0;
+        history       = p.output_ids != nullptr ? p.output_ids + row : nullptr;
+        batch_size    = p.batch_size;
+        step          = p.step;
+        max_input_length = p.max_input_length;
+        input_length  = p.input_lengths != nullptr ? p.input_lengths[row] : p.max_input_length;
         masked_end_id = -1;
         if (p.min_lengths != nullptr
             && min_length_masks(p.sequence_length_in[row], p.max_input_length, p.min_lengths[row])) {
@@ -76,35 +98,110 @@ struct FusedRow {
     {
         return rowp;
     }
+    __device__ __forceinline__ bool history_position_counts(int t) const
+    {
+        return !(t >= input_length && t < max_input_length);  // skip the padding of short prompts
+    }
+    // called by every thread of the gather workgroup before it touches columns [lo, hi)
+    __device__ __forceinline__ void prepare(int lo, int hi)
+    {
+        if (global_bm == nullptr || global_ready) {
+            return;
+        }
+        __shared__ uint32_t lds_bm[FUSED_LDS_BITMAP_WORDS];
+        const int           origin = lo & ~31;
+        const int           words  = min(FUSED_LDS_BITMAP_WORDS, (hi - origin + 31) / 32 + 1);
+        for (int i = threadIdx.x; i < words; i += blockDim.x) {
+            lds_bm[i] = 0u;
+        }
+        __syncthreads();
+        for (int t = threadIdx.x; t < step; t += blockDim.x) {
+            if (history_position_counts(t)) {
+                const int id = history[(size_t)t * batch_size];
+                if (id >= lo && id < hi) {
+                    atomicOr(&lds_bm[(id - origin) >> 5], 1u << ((id - origin) & 31));
+                }
+            }
+        }
+        __syncthreads();
+        bm        = lds_bm;
+        bm_origin = origin;
+    }
+    // whole-row bitmap in global scratch, for the literal replay of rows the gather could not bound
+    __device__ __forceinline__ void build_global_bitmap()
+    {
+        if (global_bm == nullptr || global_ready) {
+            return;
+        }
+        const int words = (Vp + 31) / 32 + 1;
+        for (int i = threadIdx.x; i < words; i += blockDim.x) {
+            global_bm[i] = 0u;
+        }
+        __threadfence_block();
+        __syncthreads();
+        for (int t = threadIdx.x; t < step; t += blockDim.x) {
+            if (history_position_counts(t)) {
+                const int id = history[(size_t)t * batch_size];
+                if (id >= 0 && id < Vp) {
+                    atomicOr(&global_bm[id >> 5], 1u << (id & 31));
+                }
+            }
+        }
+        __threadfence_block();
+        __syncthreads();
+        bm           = global_bm;
+        bm_origin    = 0;
+        global_ready = true;
+    }
     // history-membership bits of columns first .. first+n-1 (n <= 8)
     __device__ __forceinline__ uint32_t vector_bits(int first, int n) const
     {
-        if (bitmap == nullptr) {
+        if (bm == nullptr) {
             return 0u;
         }
         uint32_t bits = 0u;
-        if (first >= 0) {
-            const int w  = first >> 5;
-            const int sh = first & 31;
-            bits         = bitmap[w] >> sh;
-            if (sh + n > 32 && first + n - 1 < Vp) {
-                bits |= bitmap[w + 1] << (32 - sh);
+        if (first >= bm_origin) {
+            const int rel = first - bm_origin;
+            const int w   = rel >> 5;
+            const int sh  = rel & 31;
+            bits          = bm[w] >> sh;
+            if (sh + n > 32) {
+                bits |= bm[w + 1] << (32 - sh);  // both bitmaps carry one word of slack
             }
+            bits &= (1u << n) - 1u;
         }
         else {
             for (int j = 0; j < n; ++j) {
                 const int v = first + j;
-                if (v >= 0 && v < Vp) {
-                    bits |= ((bitmap[v >> 5] >> (v & 31)) & 1u) << j;
+                if (v >= bm_origin && v < Vp) {
+                    bits |= ((bm[(v - bm_origin) >> 5] >> ((v - bm_origin) & 31)) & 1u) << j;
                 }
             }
         }
         return bits;
     }
-    // the value top-k would see for column v, as an order-preserving key
-    __device__ __forceinline__ uint32_t key(int v, T raw, uint32_t in_history) const
+    __device__ __forceinline__ bool plain_vector(int first, int n) const
     {
-        float x = S::ld(raw);
+        return bias == nullptr && first + n <= V && !(masked_end_id >= first && masked_end_id < first + n);
+    }
+    __device__ __forceinline__ bool has_vector_bits() const
+    {
+        return bm != nullptr;
+    }
+    // pad columns and the masked end id are -MAX_T whatever the logits hold
+    __device__ __forceinline__ bool never_selected(int v) const
+    {
+        return v >= V || v == masked_end_id;
+    }
+    // interior column, no bias, not in the history, not the masked end id
+    __device__ __forceinline__ float fast(float x) const
+    {
+        return temp_active ? round_t<DT>(x * inv) : x;
+    }
+    // the value top-k would see for column v: temperature(+bias) -> history penalty -> min-length mask
+    // -> pad mask, each rounded to T where the reference stores T
+    __device__ __forceinline__ float slow(int v, float x, uint32_t in_history) const
+    {
         if (temp_active) {
             if (v < V) {
                 if (bias != nullptr) {
@@ -125,12 +222,17 @@ struct FusedRow {
         if (v >= V) {
             x = -S::max_t();  // addBiasEndMask: pad columns
         }
-        return order_key(x);
+        return x;
     }
     __device__ __forceinline__ uint32_t key_at(int v) const
     {
-        const uint32_t bit = bitmap != nullptr ? (bitmap[v >> 5] >> (v & 31)) & 1u : 0u;
-        return key(v, rowp[v], bit);
+        const uint32_t bit = bm != nullptr ? (bm[(v - bm_origin) >> 5] >> ((v - bm_origin) & 31)) & 1u : 0u;
+        return order_key(slow(v, S::ld(rowp[v]), bit));
+    }
+    // before key_at() may be used over the whole row
+    __device__ __forceinline__ void prepare_whole_row()
+    {
+        build_global_bitmap();
     }
 };
 
@@ -175,7 +277,7 @@ history_bitmap_kernel(uint32_t* __restrict__ bitmaps, int bitmap_words, const in
 }
 
 template<int DT>
-__global__ void __launch_bounds__(TK_THREADS)
+__global__ void __launch_bounds__(TK_THREADS, 4)
 fused_gather_kernel(FusedParams p, int splits, int nvt, int cap, size_t row_entries,
                     TopkChunkHeader* __restrict__ headers, TopkEntry* __restrict__ entries)
 {
@@ -187,9 +289,9 @@ fused_gather_kernel(FusedParams p, int splits, int nvt, int cap, size_t row_entr
     if (p.finished_in != nullptr && p.finished_in[row]) {
         return;  // a finished row emits its end id without looking at the logits
     }
-    const int          k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    const FusedRow<DT> r(p, row);
-    topk_gather_chunk<DT>(r, p.Vp, k, chunk, nvt, cap, headers + (size_t)row * splits + chunk,
+    const int    k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    FusedRow<DT> r(p, row);
+    topk_gather_chunk<DT>(r, p.Vp, k, chunk, splits, nvt, cap, headers + (size_t)row * splits + chunk,
                           entries + (size_t)row * row_entries + (size_t)chunk * cap);
 }
 
@@ -216,8 +318,8 @@ fused_select_kernel(FusedParams p, int* __restrict__ ids, int* __restrict__ sequ
         s.misc[0] = __float_as_int(row_uniform(rng, uniforms, row));
     }
     __syncthreads();
-    const float        u = __int_as_float(s.misc[0]);
-    const FusedRow<DT> r(p, row);
+    const float  u = __int_as_float(s.misc[0]);
+    FusedRow<DT> r(p, row);
     const TopkOutputs  out{ids, sequence_length, finished, nullptr, nullptr};
     topk_select_row<DT>(r, s, row, p.Vp, k, tp, p.max_top_k, splits, headers + (size_t)row * splits,
                         entries + (size_t)row * row_entries, cap, false, u, p.end_ids, out);
@@ -369,19 +471,23 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     p.finished_in        = a->finished;
     p.bitmaps            = nullptr;
     p.bitmap_words       = bitmap_words;
+    p.bitmaps_ready      = 0;
 
     char* ws = (char*)a->workspace;
     if (p.penalties != nullptr && a->step > 0) {
         if (a->output_ids == nullptr) {
             return FTK_ERR_ARGUMENT;
         }
-        uint32_t*        bitmaps = (uint32_t*)ws;
-        ScopedKernelTime timer(0, st);
-        history_bitmap_kernel<<<rows, HB_THREADS, 0, st>>>(bitmaps, bitmap_words, a->output_ids, a->batch_size,
-                                                           a->vocab_size_padded, a->input_lengths,
-                                                           a->max_input_length, a->step, a->skip_decode, a->finished);
-        FTK_LAUNCH_CHECK();
-        p.bitmaps = bitmaps;
+        p.bitmaps = (uint32_t*)ws;
+        if (a->step > FUSED_LOCAL_BITMAP_MAX_STEP) {
+            ScopedKernelTime timer(0, st);
+            history_bitmap_kernel<<<rows, HB_THREADS, 0, st>>>(p.bitmaps, bitmap_words, a->output_ids, a->batch_size,
+                                                               a->vocab_size_padded, a->input_lengths,
+                                                               a->max_input_length, a->step, a->skip_decode,
+                                                               a->finished);
+            FTK_LAUNCH_CHECK();
+            p.bitmaps_ready = 1;
+        }
     }
     else {
         p.penalties = nullptr;

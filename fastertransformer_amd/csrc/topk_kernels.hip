@@ -13,10 +13,11 @@ struct PlainRowAt: PlainRow<DT> {
     {
         return order_key(Storage<DT>::ld(this->rowp[v]));
     }
+    __device__ __forceinline__ void prepare_whole_row() {}
 };
 
 template<int DT>
-__global__ void __launch_bounds__(TK_THREADS)
+__global__ void __launch_bounds__(TK_THREADS, 4)
 topk_gather_kernel(const typename Storage<DT>::T* __restrict__ log_probs, const bool* __restrict__ finished,
                    const bool* __restrict__ skip_decode, const int* __restrict__ top_ks, int max_top_k, int vocab,
                    int splits, int nvt, int cap, size_t row_entries, TopkChunkHeader* __restrict__ headers,
@@ -33,7 +34,7 @@ topk_gather_kernel(const typename Storage<DT>::T* __restrict__ log_probs, const 
     const int      k = top_ks != nullptr ? top_ks[row] : max_top_k;
     PlainRowAt<DT> r;
     r.rowp = log_probs + (size_t)row * vocab;
-    topk_gather_chunk<DT>(r, vocab, k, chunk, nvt, cap, headers + (size_t)row * splits + chunk,
+    topk_gather_chunk<DT>(r, vocab, k, chunk, splits, nvt, cap, headers + (size_t)row * splits + chunk,
                           entries + (size_t)row * row_entries + (size_t)chunk * cap);
 }
 
