@@ -202,12 +202,19 @@ FTK_HD float bf16_bits_to_float(uint16_t b)
 
 FTK_HD uint16_t float_to_bf16_bits(float f)
 {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const __bf16 v = (__bf16)f;  // v_cvt_pk_bf16_f32, round-to-nearest-even
+    uint16_t     h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+#else
     const uint32_t u = f2u(f);
     if ((u & 0x7FFFFFFFu) > 0x7F800000u) {
         return (uint16_t)((u >> 16) | 0x0040u);
     }
     const uint32_t r = u + 0x7FFFu + ((u >> 16) & 1u);
     return (uint16_t)(r >> 16);
+#endif
 }
 
 // Logits element types. `T` is the storage type; all arithmetic is done on the exact fp32 image

@@ -7,33 +7,59 @@
 // values resolve to the highest thread id, so the picks follow two total orders:
 //   stage 1, inside a slice : value desc, (i mod BS1) desc, i asc
 //   stage 2, over positions : value desc, (pos mod BS2) desc, pos asc,  pos = slice*k + rank
-// The reference reads the row k+2 times. Here the row is read once:
-//   gather kernel  - grid (splits, rows), 256 threads, <= 64 elements per thread held in registers
-//                    as order-preserving keys. A lower bound on the k-th largest value comes from
-//                    the order statistics of the per-thread maxima; everything at or above it
-//                    (typically ~100 elements per chunk) is written to a per-chunk candidate list.
-//   select kernel  - one workgroup per row merges the lists, replays both tie orders on the
-//                    candidates with two LDS bitonic sorts of 64-bit composite keys and samples.
+// The reference reads the row k+2 times. Here the row is read once, as a stream:
+//   stream  - a 256-thread workgroup walks its share of the row tile by tile (16 KB per thread
+//             group of loads in flight, the next tile requested before the current one is examined).
+//             It keeps a lower bound of the row's k-th largest value and an LDS list of everything
+//             at or above it. The bound starts from the order statistics of per-thread maxima of
+//             the first tile and is tightened to the exact k-th largest of the list whenever the
+//             list grows long, so that after the first tile an element costs one multiply, one
+//             maximum and a fraction of a compare.
+//   select  - replays both tie orders on the candidates (ranking by counting for <= 256
+//             candidates, two LDS bitonic sorts of 64-bit composite keys otherwise) and samples.
+// When the batch has at least as many rows as the chip has compute units, one workgroup owns a whole
+// row and runs both phases (no scratch traffic, one launch). Smaller batches split each row over
+// several workgroups that leave their lists in the workspace, and a second launch merges them.
 // Rows whose candidates cannot be bounded (thousands of identical values around the k-th) take a
 // literal, slow replay of the reference's passes.
 #pragma once
 #include "ftk_device.cuh"
 #include "ftk_transform.cuh"
 
+// Optional phase timing for kernel development: FTK_PHASE(i) adds the time since the previous mark of
+// this workgroup to slot i (100 MHz constant clock, thread 0 only). Compiled out by default.
+#ifdef FTK_PHASE_TIMING
+static __device__ unsigned long long g_ftk_phase[32];
+#define FTK_PHASE_BEGIN() unsigned long long ftk_phase_t0_ = wall_clock64()
+#define FTK_PHASE(i)                                                                                                   \
+    do {                                                                                                               \
+        const unsigned long long now_ = wall_clock64();                                                                \
+        if (threadIdx.x == 0) {                                                                                        \
+            atomicAdd(&g_ftk_phase[i], now_ - ftk_phase_t0_);                                                          \
+            atomicAdd(&g_ftk_phase[16 + (i)], 1ull);                                                                   \
+        }                                                                                                              \
+        ftk_phase_t0_ = wall_clock64();                                                                                \
+    } while (0)
+#else
+#define FTK_PHASE_BEGIN()
+#define FTK_PHASE(i)
+#endif
+
 namespace ftk {
 
-constexpr int TK_THREADS = 256;
-constexpr int TK_ELEMS   = 64;    // elements per thread
-constexpr int TK_MAXCAP  = 2048;  // candidates per chunk, upper limit
-constexpr int TK_SELCAP  = 4096;  // candidates per row the select kernel sorts in LDS
+constexpr int TK_THREADS  = 256;
+constexpr int TK_NVT      = 16;    // 16-byte vectors per thread and tile: 64 KB per workgroup in flight
+constexpr int TK_CCAP     = 2048;  // candidates a workgroup can hold
 constexpr int TK_MAXSPLIT = 64;
+constexpr int TK_FILL_WGS = 1024;  // workgroups wanted in flight (4 per compute unit)
 
 struct TopkChunkHeader {
-    uint32_t count;       // entries written
-    uint32_t threshold;   // every element of the chunk with key >= threshold is in the list
-    uint32_t threshold8;  // 0, or a key with >= ceil(k/splits) elements of the chunk at or above it
-    uint32_t flags;       // bit 0: count >= k, `threshold` bounds the row's k-th largest key from below
-                          // bit 1: the chunk could not bound its candidates (row takes the literal replay)
+    uint32_t count;      // entries written
+    uint32_t threshold;  // every element of the chunk with key >= threshold is in the list
+    uint32_t flags;      // bit 0: count >= k, `threshold` bounds the row's k-th largest key from below
+                         // bit 1: the chunk could not bound its candidates (row takes the literal replay)
+    uint32_t share;      // 0, or the chunk's ceil(k/splits)-th largest key: the smallest `share` of a row
+                         // has >= k elements at or above it
 };
 
 struct TopkEntry {
@@ -42,47 +68,42 @@ struct TopkEntry {
 };
 
 struct TopkPlan {
-    int    splits;       // chunks per row
-    int    nvt;          // 16-byte vectors per thread
-    int    cap;          // candidate capacity per chunk
-    size_t row_entries;  // TopkEntry slots per row
-    size_t bytes;        // whole workspace
+    int    splits;         // workgroups per row
+    int    tiles_per_wg;   // tiles each of them streams
+    size_t row_entries;    // TopkEntry slots per row in the workspace
+    size_t bytes;          // whole workspace
 };
 
 inline TopkPlan topk_plan(int vocab_padded, int batch, int max_top_k, int elem_bytes)
 {
     TopkPlan  p;
-    const int epv      = 16 / elem_bytes;
-    const int nvt_max  = TK_ELEMS / epv;
-    const int nvec     = vocab_padded / epv + 2;  // worst case over row misalignments
-    const int s_min    = (nvec + TK_THREADS * nvt_max - 1) / (TK_THREADS * nvt_max);
-    const int s_fill   = (2048 + batch - 1) / (batch > 0 ? batch : 1);  // aim at >= 2048 workgroups
-    const int s_max    = (nvec + TK_THREADS - 1) / TK_THREADS;          // at least one vector per thread
-    int       s        = s_min > s_fill ? s_min : s_fill;
-    if (s > s_max) {
-        s = s_max;
-    }
-    if (s > TK_MAXSPLIT) {
-        s = TK_MAXSPLIT;
-    }
-    if (s < s_min) {
-        s = s_min;  // very large vocabularies: more than TK_MAXSPLIT chunks
-    }
-    p.splits = s;
-    p.nvt    = (nvec + s * TK_THREADS - 1) / (s * TK_THREADS);
-    int cap  = 256;
-    while (cap < 2 * max_top_k && cap < TK_MAXCAP) {
-        cap <<= 1;
-    }
-    p.cap           = cap;
-    size_t entries  = (size_t)s * cap;
-    const size_t lit = (size_t)8 * (max_top_k > 0 ? max_top_k : 1);  // literal replay keeps 8k picks
+    const int epv       = 16 / elem_bytes;
+    const int tile_vecs = TK_THREADS * TK_NVT;
+    const int nvec      = vocab_padded / epv + 2;  // worst case over row misalignments
+    const int tiles     = (nvec + tile_vecs - 1) / tile_vecs;
+    int       s         = (TK_FILL_WGS + batch - 1) / (batch > 0 ? batch : 1);
+    s                   = s > tiles ? tiles : s;
+    s                   = s > TK_MAXSPLIT ? TK_MAXSPLIT : s;
+    s                   = s < 1 ? 1 : s;
+    p.tiles_per_wg      = (tiles + s - 1) / s;
+    p.splits            = (tiles + p.tiles_per_wg - 1) / p.tiles_per_wg;
+    size_t entries      = p.splits > 1 ? (size_t)p.splits * TK_CCAP : 0;
+    const size_t lit    = (size_t)8 * (max_top_k > 0 ? max_top_k : 1);  // the literal replay keeps 8k picks
     if (entries < lit) {
         entries = lit;
     }
     p.row_entries = entries;
-    p.bytes       = (size_t)batch * (s * sizeof(TopkChunkHeader) + entries * sizeof(TopkEntry));
+    p.bytes       = (size_t)batch * (p.splits * sizeof(TopkChunkHeader) + entries * sizeof(TopkEntry));
     return p;
+}
+
+// Workgroup barrier for code that only communicates through LDS: global loads issued earlier stay
+// in flight across it.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 // -------------------------------------------------------------------------------------------
@@ -90,9 +111,11 @@ inline TopkPlan topk_plan(int vocab_padded, int batch, int max_top_k, int elem_b
 // (an fp32 image of a `T`). PlainRow is the identity (stand-alone entry point); the fused decode
 // step supplies one that applies masks and penalties on the fly.
 //   prepare(lo, hi)        - once per workgroup, before streaming columns [lo, hi)
-//   vector_bits(first, n)  - per 16-byte vector: one bit per column that needs the slow path
-//   plain_vector(first, n) - true when every column of the vector takes fast()
+//   has_vector_bits()      - some columns carry a flag (history membership)
+//   vector_bits(first, n)  - one bit per flagged column of a 16-byte vector
+//   plain_vector(first, n) - true when no column of the span needs an index-dependent rule
 //   fast(x)                - index-independent transform of an interior column
+//   flagged(xf)            - fast(x) -> value of a flagged interior column
 //   slow(v, x, bit)        - the full chain for column v
 //   never_selected(v)      - column v is masked to -MAX_T whatever it holds (pad columns)
 // -------------------------------------------------------------------------------------------
@@ -121,7 +144,6 @@ struct PlainRow {
     {
         return false;
     }
-    // columns whose value is -MAX_T by construction need not be looked at
     __device__ __forceinline__ bool never_selected(int v) const
     {
         (void)v;
@@ -130,6 +152,10 @@ struct PlainRow {
     __device__ __forceinline__ float fast(float x) const
     {
         return x;
+    }
+    __device__ __forceinline__ float flagged(float xf) const
+    {
+        return xf;
     }
     __device__ __forceinline__ float slow(int v, float x, uint32_t bit) const
     {
@@ -149,27 +175,61 @@ __device__ __forceinline__ uint32_t min_valid_key()
     return order_key(-Storage<DT>::max_t()) + 1u;  // strict `>` against -MAX_T in TopK_2::insert
 }
 
-// -------------------------------------------------------------------------------------------
-// gather: one chunk of one row.
-// The chunk lives in registers as fp32 values; float comparisons already have the reference's
-// semantics (-0 == +0, NaN never greater), so the streaming part costs a handful of VALU operations
-// per element: transform, running maximum, one compare against the threshold. Order-preserving keys
-// are only built for the ~100 elements that survive.
-// Columns that need individual treatment (row edges, the vocabulary / padding boundary, the masked end
-// id, columns with a history penalty) are evaluated once by a small rolled loop and parked in an LDS
-// list; the unrolled register pass stays branch-free and small. Chunks the fast path cannot bound
-// (fewer than k survivors, thousands of ties, an overfull list) go to topk_gather_rare, which works
-// from memory with rolled loops.
-// -------------------------------------------------------------------------------------------
-constexpr int TK_SLOWCAP = 2048;  // columns per chunk that may take the per-column path
+// tiles of a row, given where it starts relative to 16-byte alignment
+template<int DT>
+__device__ __forceinline__ int topk_row_tiles(const void* rowp, int vocab)
+{
+    typedef typename Storage<DT>::T T;
+    constexpr int                   EPV       = (int)(16 / sizeof(T));
+    constexpr int                   TILE_VECS = TK_NVT * TK_THREADS;
+    const int                       a         = (int)(((uintptr_t)rowp & 15u) / sizeof(T));
+    const int                       nvec      = (a + vocab + EPV - 1) / EPV;
+    return (nvec + TILE_VECS - 1) / TILE_VECS;
+}
 
-struct TopkGatherShared {
-    uint32_t red[16];
-    int      cnt;
-    int      n_slow;
-    int      slow_v[TK_SLOWCAP];
-    float    slow_x[TK_SLOWCAP];
+constexpr int TK_STAGE = 128;  // vectors a wave can park per tile
+
+struct TopkShared {
+    union {
+        struct {
+            uint32_t key[TK_CCAP];
+            uint32_t idx[TK_CCAP];
+        } cand;                            // stream: candidates (order-preserving key, column)
+        unsigned long long keys[TK_CCAP];  // select: composite sort keys
+    };
+    union {
+        struct {
+            uint4 raw[TK_THREADS / WAVE][TK_STAGE];    // stream: vectors with an element at or above the bound,
+            int   first[TK_THREADS / WAVE][TK_STAGE];  // one private list per wave
+        } stage;
+        struct {
+            int                                idx[TK_CCAP];
+            __attribute__((aligned(16))) float w[1024];
+        } sel;  // select: the ordered list
+    };
+    unsigned long long red64[16];
+    uint32_t           red32[16];
+    int                slice_count[8];
+    int                n_cand;
+    uint32_t           thr_new;
+    int                misc[4];
 };
+
+// element j of a 16-byte vector as fp32, extracted with 32-bit operations on the register that holds it
+template<int DT>
+__device__ __forceinline__ float vector_element(const uint4& v, int j)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    if constexpr (DT == DT_F32) {
+        return __uint_as_float(w[j]);
+    }
+    else if constexpr (DT == DT_F16) {
+        return Storage<DT>::ld((uint16_t)(j & 1 ? w[j >> 1] >> 16 : w[j >> 1] & 0xFFFFu));
+    }
+    else {
+        return __uint_as_float(j & 1 ? (w[j >> 1] & 0xFFFF0000u) : (w[j >> 1] << 16));
+    }
+}
 
 // value of column v as top-k sees it, re-read from memory
 template<int DT, class Row>
@@ -178,101 +238,195 @@ __device__ __forceinline__ float topk_value_at(const Row& rowctx, int v)
     return rowctx.slow(v, Storage<DT>::ld(rowctx.data()[v]), rowctx.vector_bits(v, 1));
 }
 
-// Threshold search by bisection on the key over columns [lo_col, hi_col), then compaction; everything is
-// recomputed from memory (the chunk sits in L2), nothing depends on the caller's registers.
-template<int DT, class Row>
-__device__ __noinline__ void topk_gather_rare(const Row& rowctx, TopkGatherShared& s, int k, int lo_col, int hi_col,
-                                              int cap, uint32_t thr, uint32_t thr8, TopkChunkHeader* header,
-                                              TopkEntry* entries)
+// keep the candidates with key >= thr (in place, order not preserved); returns how many
+__device__ __forceinline__ int topk_prune(TopkShared& s, int n, uint32_t thr)
 {
-    const int      t    = threadIdx.x;
-    const uint32_t KMIN = min_valid_key<DT>();
-    auto count_ge = [&](uint32_t thr_key) -> int {
-        const float thr_f = key_to_float(thr_key);
-        int         c     = 0;
-        for (int v = lo_col + t; v < hi_col; v += TK_THREADS) {
-            c += topk_value_at<DT>(rowctx, v) >= thr_f ? 1 : 0;
-        }
-        return block_sum_i(c, (int*)s.red);
-    };
-    uint32_t cmax = 0u;
-    for (int v = lo_col + t; v < hi_col; v += TK_THREADS) {
-        const uint32_t kk = order_key(topk_value_at<DT>(rowctx, v));
-        cmax              = kk > cmax ? kk : cmax;
-    }
-    cmax              = block_max<uint32_t>(cmax, s.red, 0u);
-    const int n_valid = count_ge(KMIN);
-    const int kneed   = k < n_valid ? k : n_valid;
-    int       cnt     = count_ge(thr);
-    bool      ok      = cnt >= kneed && cnt <= cap;
-    if (!ok) {
-        uint32_t lo, hi;  // count(lo) > cap (or lo == KMIN); count(hi) < kneed
-        if (cnt > cap) {
-            lo = thr;
-            hi = cmax + 1u;
-        }
-        else {
-            lo = KMIN;
-            hi = thr;
-            if (n_valid <= cap) {
-                thr = KMIN;
-                ok  = true;
-            }
-        }
-        while (!ok && hi - lo > 1u) {
-            const uint32_t mid = lo + (hi - lo) / 2u;
-            const int      c   = count_ge(mid);
-            if (c > cap) {
-                lo = mid;
-            }
-            else if (c < kneed) {
-                hi = mid;
-            }
-            else {
-                thr = mid;
-                ok  = true;
-            }
-        }
-    }
-    cnt = 0;
-    if (ok) {
-        const float thr_f = key_to_float(thr);
-        if (t == 0) {
-            s.cnt = 0;
-        }
-        __syncthreads();
-        for (int v = lo_col + t; v < hi_col; v += TK_THREADS) {
-            const float xv = topk_value_at<DT>(rowctx, v);
-            if (xv >= thr_f) {
-                const int slot = atomicAdd(&s.cnt, 1);
-                if (slot < cap) {
-                    entries[slot] = TopkEntry{order_key(xv), (uint32_t)v};
-                }
-            }
-        }
-        __syncthreads();
-        cnt = s.cnt;
+    const int t = threadIdx.x;
+    uint32_t  ck[TK_CCAP / TK_THREADS], ci[TK_CCAP / TK_THREADS];
+#pragma unroll
+    for (int r = 0; r < TK_CCAP / TK_THREADS; ++r) {
+        const int i = t + r * TK_THREADS;
+        ck[r]       = i < n ? s.cand.key[i] : 0u;
+        ci[r]       = i < n ? s.cand.idx[i] : 0u;
     }
     if (t == 0) {
-        TopkChunkHeader h;
-        h.count      = ok ? (uint32_t)cnt : 0u;
-        h.threshold  = thr;
-        h.threshold8 = thr8;
-        h.flags      = ((ok && cnt >= k) ? 1u : 0u) | (ok ? 0u : 2u);
-        *header      = h;
+        s.n_cand = 0;
     }
+    lds_barrier();
+#pragma unroll
+    for (int r = 0; r < TK_CCAP / TK_THREADS; ++r) {
+        const int i = t + r * TK_THREADS;
+        if (i < n && ck[r] >= thr) {
+            const int slot   = atomicAdd(&s.n_cand, 1);
+            s.cand.key[slot] = ck[r];
+            s.cand.idx[slot] = ci[r];
+        }
+    }
+    lds_barrier();
+    const int m = s.n_cand;
+    lds_barrier();
+    return m;
 }
 
-template<int DT, class Row>
-__device__ __forceinline__ void topk_gather_chunk(Row& rowctx, int vocab, int k, int chunk, int splits, int nvt,
-                                                  int cap, TopkChunkHeader* header, TopkEntry* entries)
+// The exact k-th largest key of the list (n >= k, every entry >= lower).
+__device__ __forceinline__ uint32_t topk_kth_key(TopkShared& s, int n, int k, uint32_t lower)
 {
-    typedef Storage<DT>         S;
-    typedef typename S::T       T;
-    constexpr int               EPV = (int)(16 / sizeof(T));
-    constexpr int               NVT = TK_ELEMS / EPV;
-    __shared__ TopkGatherShared s;
-    const int                   t = threadIdx.x;
+    const int t = threadIdx.x;
+    uint32_t  nt;
+    if (n <= TK_THREADS) {
+        // rank by counting; ties are ordered by position so exactly one entry has rank k-1
+        const uint32_t k0 = t < n ? s.cand.key[t] : 0u;
+        int            r0 = 0;
+        // entry j precedes entry i when key_j > key_i, or the keys are equal and j < i:
+        //   key_j >= key_i for j < i,  key_j > key_i for j > i   <=>   key_j + (j < i) > key_i
+        // (keys stay below 0xFFFFFFFF, so the increment cannot wrap)
+        const int n4 = (n + 3) & ~3;  // the list is read four entries at a time; the tail is masked
+#pragma unroll 2
+        for (int j = 0; j < n4; j += 4) {
+            const uint4    kk    = *reinterpret_cast<const uint4*>(&s.cand.key[j]);
+            const uint32_t kj[4] = {kk.x, kk.y, kk.z, kk.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int      jj = j + e;
+                const uint32_t kv = jj < n ? kj[e] : 0u;
+                r0 += (kv + (jj < t ? 1u : 0u)) > k0 ? 1 : 0;
+            }
+        }
+        if (t < n && r0 == k - 1) {
+            s.thr_new = k0;
+        }
+        lds_barrier();
+        nt = s.thr_new;
+    }
+    else {
+        // bisection on the key; per step one ballot per held entry, one LDS atomic per wave, one barrier
+        constexpr int PER = TK_CCAP / TK_THREADS;
+        uint32_t      ck[PER];
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int i = t + r * TK_THREADS;
+            ck[r]       = i < n ? s.cand.key[i] : 0u;
+        }
+        if (t < 3) {
+            s.misc[1 + t] = 0;
+        }
+        lds_barrier();
+        uint32_t lo = lower, hi = 0xFFFFFFFFu;  // count(lo) >= k; no key reaches hi
+        int      it = 0;                        // three counters in rotation: add, read, clear
+        while (hi - lo > 1u) {
+            const uint32_t mid = lo + (hi - lo) / 2u;
+            int            c   = 0;
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                if (r * TK_THREADS < n) {
+                    c += __builtin_popcountll(__ballot(ck[r] >= mid));
+                }
+            }
+            int* counter = &s.misc[1 + it % 3];
+            if (lane_id() == 0) {
+                atomicAdd(counter, c);
+            }
+            lds_barrier();
+            c = *counter;
+            if (t == 0) {
+                s.misc[1 + (it + 2) % 3] = 0;  // last read before this step's barrier, next used after the next one
+            }
+            ++it;
+            if (c >= k) {
+                lo = mid;
+            }
+            else {
+                hi = mid;
+            }
+        }
+        nt = lo;
+    }
+    lds_barrier();  // s.thr_new and the counters may be reused right away
+    return nt;
+}
+
+// Raise the bound to the exact k-th largest key of the list (n >= k, every entry >= *thr) and drop
+// what falls below it: k entries plus ties with the k-th remain.
+__device__ __forceinline__ int topk_tighten(TopkShared& s, int n, int k, uint32_t* thr)
+{
+    *thr = topk_kth_key(s, n, k, *thr);
+    return topk_prune(s, n, *thr);
+}
+
+// -------------------------------------------------------------------------------------------
+// stream: tiles [tile_begin, tile_end) of one row -> candidate list in LDS
+// -------------------------------------------------------------------------------------------
+// The recovery path of a tile that overfills the list: everything is recomputed from memory (the tile
+// sits in L2) with rolled loops, nothing depends on the caller's registers. On entry the list holds
+// n_before entries, all >= thr, from earlier tiles. Looks for a higher bound that leaves between k and
+// TK_CCAP candidates; returns the new list length (bound in s.thr_new) or -1 when no bound does.
+template<int DT, class Row>
+__device__ __noinline__ int topk_stream_rare(const Row& rowctx, TopkShared& s, int k, int n_before, int lo_col, int hi_col,
+                                             uint32_t thr)
+{
+    const int t        = threadIdx.x;
+    auto      count_ge = [&](uint32_t key) -> int {
+        const float f = key_to_float(key);
+        int         c = 0;
+        for (int i = t; i < n_before; i += TK_THREADS) {
+            c += s.cand.key[i] >= key ? 1 : 0;
+        }
+        for (int v = lo_col + t; v < hi_col; v += TK_THREADS) {
+            c += topk_value_at<DT>(rowctx, v) >= f ? 1 : 0;
+        }
+        return block_sum_i(c, (int*)s.red32);
+    };
+    uint32_t lo = thr, hi = 0xFFFFFFFFu;  // count(lo) > TK_CCAP, count(hi) == 0
+    bool     ok = count_ge(thr) <= TK_CCAP;  // (a wave ran out of parking space, the list itself fits)
+    while (!ok && hi - lo > 1u) {
+        const uint32_t mid = lo + (hi - lo) / 2u;
+        const int      c   = count_ge(mid);
+        if (c > TK_CCAP) {
+            lo = mid;
+        }
+        else if (c < k) {
+            hi = mid;
+        }
+        else {
+            thr = mid;
+            ok  = true;
+        }
+    }
+    if (!ok) {
+        return -1;
+    }
+    (void)topk_prune(s, n_before, thr);
+    const float thr_f = key_to_float(thr);
+    for (int v = lo_col + t; v < hi_col; v += TK_THREADS) {
+        const float xv = topk_value_at<DT>(rowctx, v);
+        if (xv >= thr_f) {
+            const int slot   = atomicAdd(&s.n_cand, 1);
+            s.cand.key[slot] = order_key(xv);
+            s.cand.idx[slot] = (uint32_t)v;
+        }
+    }
+    if (t == 0) {
+        s.thr_new = thr;
+    }
+    lds_barrier();
+    const int n = s.n_cand;
+    lds_barrier();
+    return n;
+}
+
+// Returns the number of candidates left in s.cand (all elements of the tiles with key >= *thr_out), or
+// -1 when the range could not be bounded. When the result is >= k, *thr_out bounds the k-th largest key
+// of the range from below; otherwise the list holds every selectable element of the range.
+template<int DT, class Row>
+__device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab, int k, int tile_begin, int tile_end,
+                                           uint32_t* thr_out)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         EPV       = (int)(16 / sizeof(T));
+    constexpr int         NVT       = TK_NVT;
+    constexpr int         TILE_VECS = NVT * TK_THREADS;
+    const int             t         = threadIdx.x;
 
     const T*       rowp     = rowctx.data();
     const int      a        = (int)(((uintptr_t)rowp & 15u) / sizeof(T));  // columns between the aligned base and column 0
@@ -281,214 +435,343 @@ __device__ __forceinline__ void topk_gather_chunk(Row& rowctx, int vocab, int k,
     const int      vfull_lo = (a + EPV - 1) / EPV;  // vectors [vfull_lo, vfull_hi) lie entirely inside the row
     const int      vfull_hi = (a + vocab) / EPV;
     const bool     any_full = vfull_hi > vfull_lo;
-    const int      vec0     = chunk * nvt * TK_THREADS;
     const uint32_t KMIN     = min_valid_key<DT>();
     const float    NEG_INF  = -__builtin_inff();
-    const int      lo_col   = max(0, vec0 * EPV - a);
-    const int      hi_col   = max(lo_col, min(vocab, (vec0 + nvt * TK_THREADS) * EPV - a));
+    const int      lo_col   = max(0, tile_begin * TILE_VECS * EPV - a);
+    const int      hi_col   = max(lo_col, min(vocab, tile_end * TILE_VECS * EPV - a));
 
-    // A chunk is "plain" when every one of its vectors lies inside the row and no column needs an
-    // index-dependent rule (pads, masked end id, bias): true for all but a handful of chunks per row.
-    // Plain chunks run a loop without per-vector index checks.
-    const bool chunk_plain = any_full && nvt == NVT && vec0 >= vfull_lo && vec0 + NVT * TK_THREADS <= vfull_hi
-                             && rowctx.plain_vector(lo_col, hi_col - lo_col);
-
-    // ---- load: every vector load is issued before the first use. Lanes whose vector is not entirely
-    // inside the row read a harmless in-row vector instead and visit their columns one by one.
+    // A tile is "plain" when every one of its vectors lies inside the row and no column needs an
+    // index-dependent rule (pads, masked end id, bias): true for all but a handful of tiles per row.
+    auto tile_plain = [&](int tile) -> bool {
+        const int vec0 = tile * TILE_VECS;
+        return any_full && vec0 >= vfull_lo && vec0 + TILE_VECS <= vfull_hi
+               && rowctx.plain_vector(vec0 * EPV - a, TILE_VECS * EPV);
+    };
+    // Every vector load of a tile is issued back to back. Lanes whose vector is not entirely inside the
+    // row read a harmless in-row vector instead and visit their columns one by one.
     uint4 raw[NVT];
-    if (chunk_plain) {
-        const uint4* p0 = base + vec0 + t;
+    auto  load_tile = [&](int tile) {
+        const int vec0 = tile * TILE_VECS;
+        if (tile_plain(tile)) {
+            const uint4* p0 = base + vec0 + t;
 #pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            raw[it] = p0[it * TK_THREADS];
-        }
-    }
-    else if (any_full) {
-#pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            const int  vi   = vec0 + it * TK_THREADS + t;
-            const bool full = it < nvt && vi >= vfull_lo && vi < vfull_hi;
-            raw[it]         = base[full ? vi : vfull_lo];
-        }
-    }
-    else {
-#pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            raw[it] = make_uint4(0, 0, 0, 0);
-        }
-    }
-    // per-workgroup side data of the row (e.g. the history bitmap) while the loads are in flight
-    if (t == 0) {
-        s.n_slow = 0;
-    }
-    rowctx.prepare(lo_col, hi_col);
-    __syncthreads();
-
-    float    x[TK_ELEMS];
-    float    tmax     = NEG_INF;
-    uint32_t slowmask = 0u;  // bit `it`: vector `it` of this thread takes the per-column path
-    if (chunk_plain && !rowctx.has_vector_bits()) {
-#pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            const T* e = reinterpret_cast<const T*>(&raw[it]);
-#pragma unroll
-            for (int j = 0; j < EPV; ++j) {
-                x[it * EPV + j] = rowctx.fast(S::ld(e[j]));
-                tmax            = __builtin_fmaxf(tmax, x[it * EPV + j]);  // NaN never becomes the maximum
+            for (int it = 0; it < NVT; ++it) {
+                raw[it] = p0[it * TK_THREADS];
             }
         }
-    }
-    else if (chunk_plain) {
-        const int first0 = (vec0 + t) * EPV - a;
+        else if (any_full) {
 #pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            const T*   e     = reinterpret_cast<const T*>(&raw[it]);
-            const bool fastv = rowctx.vector_bits(first0 + it * TK_THREADS * EPV, EPV) == 0u;
-            slowmask |= fastv ? 0u : (1u << it);
-#pragma unroll
-            for (int j = 0; j < EPV; ++j) {
-                const float v   = rowctx.fast(S::ld(e[j]));
-                x[it * EPV + j] = fastv ? v : NEG_INF;
-                tmax            = __builtin_fmaxf(tmax, x[it * EPV + j]);
+            for (int it = 0; it < NVT; ++it) {
+                const int vi = vec0 + it * TK_THREADS + t;
+                raw[it]      = base[(vi >= vfull_lo && vi < vfull_hi) ? vi : vfull_lo];
             }
         }
-    }
-    else {
+        else {
 #pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            const int  vi    = vec0 + it * TK_THREADS + t;
-            const int  first = vi * EPV - a;
-            const T*   e     = reinterpret_cast<const T*>(&raw[it]);
-            const bool live  = it < nvt && vi < nvec;
-            const bool fastv = live && any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV)
-                               && rowctx.vector_bits(first, EPV) == 0u;
-            slowmask |= (live && !fastv) ? (1u << it) : 0u;
-#pragma unroll
-            for (int j = 0; j < EPV; ++j) {
-                const float v   = rowctx.fast(S::ld(e[j]));
-                x[it * EPV + j] = fastv ? v : NEG_INF;
-                tmax            = __builtin_fmaxf(tmax, x[it * EPV + j]);
+            for (int it = 0; it < NVT; ++it) {
+                raw[it] = make_uint4(0, 0, 0, 0);
             }
-        }
-    }
-    // per-column path: evaluate once, park in LDS
-    bool slow_overflow = false;
-    for (uint32_t m = slowmask; m != 0u; m &= m - 1u) {
-        const int it    = __builtin_ctz(m);
-        const int first = (vec0 + it * TK_THREADS + t) * EPV - a;
-        for (int j = 0; j < EPV; ++j) {
-            const int v = first + j;
-            if (v >= 0 && v < vocab && !rowctx.never_selected(v)) {
-                const float xv   = topk_value_at<DT>(rowctx, v);
-                tmax             = __builtin_fmaxf(tmax, xv);
-                const int   slot = atomicAdd(&s.n_slow, 1);
-                if (slot < TK_SLOWCAP) {
-                    s.slow_v[slot] = v;
-                    s.slow_x[slot] = xv;
-                }
-                else {
-                    slow_overflow = true;
-                }
-            }
-        }
-    }
-
-    // ---- lower bounds from thread maxima. Each wave sorts its 64 maxima; the q-th largest of each wave,
-    // minimised over the 4 waves, has >= 4q elements of the chunk at or above it.
-    //   thr  (q  = ceil(k/4))          : >= k elements        -> everything >= thr goes to the candidate list
-    //   thr8 (qs = ceil(k/(4*splits))) : >= k/splits elements -> the smallest one over the row's chunks has
-    //                                    >= k elements above it; lets the select kernel tighten its bound
-    const uint32_t sorted = wave_sort_desc(order_key(tmax));
-    const int      q      = k <= 4 * WAVE ? (k + 3) / 4 : WAVE;
-    int            qs     = (k + 4 * splits - 1) / (4 * splits);
-    qs                    = qs < 1 ? 1 : qs;
-    uint32_t thr  = block_min<uint32_t>(__shfl(sorted, q - 1, WAVE), s.red, 0xFFFFFFFFu);
-    uint32_t thr8 = block_min<uint32_t>(__shfl(sorted, (qs <= WAVE ? qs : WAVE) - 1, WAVE), s.red, 0xFFFFFFFFu);
-    if (thr < KMIN) {
-        thr = KMIN;
-    }
-    if (thr8 < KMIN || qs > WAVE) {
-        thr8 = 0u;  // no guarantee
-    }
-
-    // ---- compaction. x >= key_to_float(thr)  <=>  order_key(x) >= thr (NaN fails both)
-    const float thr_f = key_to_float(thr);
-    if (t == 0) {
-        s.cnt = 0;
-    }
-    __syncthreads();  // also publishes the slow list
-    auto push = [&](int v, float xv) {
-        const int slot = atomicAdd(&s.cnt, 1);
-        if (slot < cap) {
-            entries[slot] = TopkEntry{order_key(xv), (uint32_t)v};
         }
     };
-    // survivors of the register pass: one bit per vector whose maximum reaches the threshold, then a
-    // rolled loop that re-reads those few vectors column by column
-    uint32_t hits = 0u;
+
+    if (t == 0) {
+        s.n_cand = 0;
+    }
+    load_tile(tile_begin);
+    // per-workgroup side data of the row (e.g. the history bitmap) while the loads are in flight
+    rowctx.prepare(lo_col, hi_col);
+    lds_barrier();
+    const bool bitsv = rowctx.has_vector_bits();
+    FTK_PHASE(1);
+
+    // ---- initial bound from the first tile: maxima over the vectors that take the fast transform
+    // (leaving the others out only lowers the bound).
+    uint32_t thr;
+    {
+        const int vec0    = tile_begin * TILE_VECS;
+        auto      vec_max = [&](int it) -> float {
+            const int  vi    = vec0 + it * TK_THREADS + t;
+            const int  first = vi * EPV - a;
+            const bool fastv = any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV)
+                               && (!bitsv || rowctx.vector_bits(first, EPV) == 0u);
+            float vmax = NEG_INF;
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) {
+                vmax = __builtin_fmaxf(vmax, rowctx.fast(vector_element<DT>(raw[it], j)));  // NaN never wins
+            }
+            return fastv ? vmax : NEG_INF;
+        };
+        // maxima of four groups of this thread's vectors: four distinct elements per thread
+        float gm[4] = {NEG_INF, NEG_INF, NEG_INF, NEG_INF};
+#pragma unroll
+        for (int it = 0; it < NVT; ++it) {
+            gm[it / (NVT / 4)] = __builtin_fmaxf(gm[it / (NVT / 4)], vec_max(it));
+        }
+        if (k <= 4 * WAVE) {
+            // each wave sorts its 64 thread maxima; the q-th largest of each wave, minimised over the 4
+            // waves, has >= 4q >= k elements of the tile at or above it
+            const float    tmax   = __builtin_fmaxf(__builtin_fmaxf(gm[0], gm[1]), __builtin_fmaxf(gm[2], gm[3]));
+            const uint32_t sorted = wave_sort_desc(order_key(tmax));
+            const int      q      = (k + 3) / 4;
+            thr = block_min<uint32_t>(__shfl(sorted, q - 1, WAVE), s.red32, 0xFFFFFFFFu);
+        }
+        else {
+            // the same with the group maxima: 16 sorted sequences, >= 16q >= k elements
+            const int q = (k + 15) / 16;
+            uint32_t  m = 0xFFFFFFFFu;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t sorted = wave_sort_desc(order_key(gm[g]));
+                const uint32_t qth    = __shfl(sorted, q - 1, WAVE);
+                m                     = qth < m ? qth : m;
+            }
+            thr = block_min<uint32_t>(m, s.red32, 0xFFFFFFFFu);
+        }
+        if (thr < KMIN) {
+            thr = KMIN;  // fewer than k usable maxima: take every selectable element
+        }
+    }
+    FTK_PHASE(2);
+    float thr_f = key_to_float(thr);  // x >= thr_f  <=>  order_key(x) >= thr (NaN fails both)
+    // The first tile is examined a second time below. Keep the compiler from carrying the converted
+    // values of the first pass along in registers: make the tile opaque here (no instructions).
 #pragma unroll
     for (int it = 0; it < NVT; ++it) {
-        float vmax = x[it * EPV];
-#pragma unroll
-        for (int j = 1; j < EPV; ++j) {
-            vmax = __builtin_fmaxf(vmax, x[it * EPV + j]);
-        }
-        hits |= vmax >= thr_f ? (1u << it) : 0u;
+        asm volatile("" : "+v"(raw[it].x), "+v"(raw[it].y), "+v"(raw[it].z), "+v"(raw[it].w));
     }
-    for (; hits != 0u; hits &= hits - 1u) {
-        const int it    = __builtin_ctz(hits);
-        const int first = (vec0 + it * TK_THREADS + t) * EPV - a;
+
+    auto push = [&](int v, float xv) {
+        const int slot = atomicAdd(&s.n_cand, 1);
+        if (slot < TK_CCAP) {
+            s.cand.key[slot] = order_key(xv);
+            s.cand.idx[slot] = (uint32_t)v;
+        }
+    };
+    // the elements of one vector at or above the bound: one slot allocation for all of them
+    auto push_vector = [&](int first, const float* x) {
+        uint32_t m = 0u;
+#pragma unroll
         for (int j = 0; j < EPV; ++j) {
-            const float xv = rowctx.fast(S::ld(rowp[first + j]));
-            if (xv >= thr_f) {
-                push(first + j, xv);
+            m |= x[j] >= thr_f ? (1u << j) : 0u;
+        }
+        int slot = atomicAdd(&s.n_cand, __builtin_popcount(m));
+#pragma unroll
+        for (int j = 0; j < EPV; ++j) {
+            if ((m >> j) & 1u) {
+                if (slot < TK_CCAP) {
+                    s.cand.key[slot] = order_key(x[j]);
+                    s.cand.idx[slot] = (uint32_t)(first + j);
+                }
+                ++slot;
             }
         }
-    }
-    const int n_slow = s.n_slow < TK_SLOWCAP ? s.n_slow : TK_SLOWCAP;
-    for (int i = t; i < n_slow; i += TK_THREADS) {
-        if (s.slow_x[i] >= thr_f) {
-            push(s.slow_v[i], s.slow_x[i]);
+    };
+    // Vectors with an element at or above the bound are parked in the wave's private LDS list (slot from
+    // a ballot, no atomics, nothing to wait for) and expanded into candidates after the tile's last vector.
+    const int wv     = wave_id();
+    int       wcount = 0;  // wave-uniform
+    auto      park   = [&](bool hit, const uint4& v, int first) {
+        const unsigned long long m = __ballot(hit);
+        if (m != 0ull) {
+            if (hit) {
+                const int slot =
+                    wcount + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                if (slot < TK_STAGE) {
+                    s.stage.raw[wv][slot]   = v;
+                    s.stage.first[wv][slot] = first;
+                }
+            }
+            wcount += __builtin_popcountll(m);
         }
-    }
-    const int any_overflow = __syncthreads_or(slow_overflow ? 1 : 0);
-    const int cnt          = s.cnt;
-    if (cnt >= k && cnt <= cap && !any_overflow) {
-        if (t == 0) {
-            TopkChunkHeader h;
-            h.count      = (uint32_t)cnt;
-            h.threshold  = thr;
-            h.threshold8 = thr8;
-            h.flags      = 1u;
-            *header      = h;
+    };
+    auto drain = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        const int staged = wcount < TK_STAGE ? wcount : TK_STAGE;
+        for (int e = lane_id(); e < staged; e += WAVE) {
+            const uint4 v     = s.stage.raw[wv][e];
+            const int   first = s.stage.first[wv][e];
+            float       x[EPV];
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) {
+                x[j] = rowctx.fast(vector_element<DT>(v, j));
+            }
+            if (bitsv) {
+                const uint32_t bits = rowctx.vector_bits(first, EPV);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    if ((bits >> j) & 1u) {
+                        x[j] = rowctx.flagged(x[j]);
+                    }
+                }
+            }
+            push_vector(first, x);
         }
-        return;
+        if (wcount > TK_STAGE && lane_id() == 0) {
+            atomicAdd(&s.n_cand, TK_CCAP + 1);  // out of parking space: the tile takes the recovery path
+        }
+        wcount = 0;
+    };
+    const int tighten_at = min(max(256, 2 * k), 3 * TK_CCAP / 4);
+    int       n          = 0;
+
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        const int vec0     = tile * TILE_VECS;
+        const int first0   = (vec0 + t) * EPV - a;
+        uint32_t  slowmask = 0u;  // bit `it`: vector `it` of this thread takes the per-column path
+        if (tile_plain(tile)) {
+#pragma unroll
+            for (int it = 0; it < NVT; ++it) {
+                const int first = first0 + it * TK_THREADS * EPV;
+                float     x[EPV];
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    x[j] = rowctx.fast(vector_element<DT>(raw[it], j));
+                }
+                if (bitsv) {
+                    const uint32_t bits = rowctx.vector_bits(first, EPV);
+                    if (bits != 0u) {
+#pragma unroll
+                        for (int j = 0; j < EPV; ++j) {
+                            if ((bits >> j) & 1u) {
+                                x[j] = rowctx.flagged(x[j]);
+                            }
+                        }
+                    }
+                }
+                float vmax = x[0];
+#pragma unroll
+                for (int j = 1; j < EPV; ++j) {
+                    vmax = __builtin_fmaxf(vmax, x[j]);
+                }
+                park(vmax >= thr_f, raw[it], first);
+            }
+        }
+        else {
+#pragma unroll
+            for (int it = 0; it < NVT; ++it) {
+                const int  vi    = vec0 + it * TK_THREADS + t;
+                const int  first = first0 + it * TK_THREADS * EPV;
+                const bool fastv = any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV)
+                                   && (!bitsv || rowctx.vector_bits(first, EPV) == 0u);
+                slowmask |= (vi < nvec && !fastv) ? (1u << it) : 0u;
+                float vmax = NEG_INF;
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    vmax = __builtin_fmaxf(vmax, rowctx.fast(vector_element<DT>(raw[it], j)));
+                }
+                park(fastv && vmax >= thr_f, raw[it], first);
+            }
+            for (; slowmask != 0u; slowmask &= slowmask - 1u) {
+                const int first = first0 + __builtin_ctz(slowmask) * TK_THREADS * EPV;
+                for (int j = 0; j < EPV; ++j) {
+                    const int v = first + j;
+                    if (v >= 0 && v < vocab && !rowctx.never_selected(v)) {
+                        const float xv = topk_value_at<DT>(rowctx, v);
+                        if (xv >= thr_f) {
+                            push(v, xv);
+                        }
+                    }
+                }
+            }
+        }
+        drain();
+        FTK_PHASE(3);
+        // the next tile is requested before the bookkeeping of this one
+        if (tile + 1 < tile_end) {
+            load_tile(tile + 1);
+        }
+        lds_barrier();
+        const int n_now = s.n_cand;
+        lds_barrier();
+        if (n_now > TK_CCAP) {
+            const int tlo = max(0, vec0 * EPV - a);
+            const int thi = max(tlo, min(vocab, (vec0 + TILE_VECS) * EPV - a));
+#ifdef FTK_NO_RARE
+            (void)tlo; (void)thi;
+            n = -1;
+#else
+            n             = topk_stream_rare<DT, Row>(rowctx, s, k, n, tlo, thi, thr);
+#endif
+            if (n < 0) {
+                return -1;
+            }
+            thr   = s.thr_new;
+            thr_f = key_to_float(thr);
+            if (tile + 1 < tile_end) {
+                load_tile(tile + 1);  // again, so that no tile data has to survive the call
+            }
+        }
+        else if (n_now > tighten_at && n_now > k && tile + 1 < tile_end) {
+            n     = topk_tighten(s, n_now, k, &thr);
+            thr_f = key_to_float(thr);
+        }
+        else {
+            n = n_now;
+        }
+        FTK_PHASE(4);
     }
-    __syncthreads();
-    topk_gather_rare<DT, Row>(rowctx, s, k, lo_col, hi_col, cap, thr, thr8, header, entries);
+    *thr_out = thr;
+    return n;
+}
+
+// a workgroup's list -> workspace, for rows that are split over several workgroups
+__device__ __forceinline__ void topk_dump_list(TopkShared& s, int n, int k, int splits, uint32_t thr,
+                                               TopkChunkHeader* header, TopkEntry* entries)
+{
+    const int t = threadIdx.x;
+    FTK_PHASE_BEGIN();
+    if (n > k) {
+        n = topk_tighten(s, n, k, &thr);  // exact k-th largest of the chunk: keeps the merge short
+    }
+    const int kshare = (k + splits - 1) / splits;
+    uint32_t  share  = 0u;
+    if (n >= kshare && n > 0) {
+        share = topk_kth_key(s, n, kshare, thr);
+    }
+    for (int i = t; i < n; i += TK_THREADS) {
+        entries[i] = TopkEntry{s.cand.key[i], s.cand.idx[i]};
+    }
+    if (t == 0) {
+        TopkChunkHeader h;
+        h.count     = n < 0 ? 0u : (uint32_t)n;
+        h.threshold = thr;
+        h.flags     = n < 0 ? 2u : (n >= k ? 1u : 0u);
+        h.share     = share;
+        *header     = h;
+    }
+    FTK_PHASE(5);
 }
 
 // -------------------------------------------------------------------------------------------
-// select: merge, replay the reference's two tie orders, sample
+// sampling and the literal replay
 // -------------------------------------------------------------------------------------------
-struct TopkSelectShared {
-    unsigned long long keys[TK_SELCAP];  // 32 KB
-    int                idx[TK_SELCAP];   // 16 KB
-    __attribute__((aligned(16))) float w[1024];
-    unsigned long long red64[16];
-    uint32_t           red32[16];
-    int                slice_count[8];
-    int                counter;
-    int                misc[4];
-};
-
 struct TopkOutputs {
     int*   ids;
     int*   sequence_length;
     bool*  finished;
     float* cum_log_probs;
     float* output_log_probs;
+    // values of the row read when the kernel starts, so that the last thread standing does not wait for
+    // memory again; rows that are already finished never get here
+    int   sequence_length_in;
+    float cum_log_prob_in;
 };
+
+__device__ __forceinline__ TopkOutputs topk_outputs(int* ids, int* sequence_length, bool* finished,
+                                                    float* cum_log_probs, float* output_log_probs, int row)
+{
+    TopkOutputs o;
+    o.ids                = ids;
+    o.sequence_length    = sequence_length;
+    o.finished           = finished;
+    o.cum_log_probs      = cum_log_probs;
+    o.output_log_probs   = output_log_probs;
+    o.sequence_length_in = sequence_length != nullptr ? sequence_length[row] : 0;
+    o.cum_log_prob_in    = cum_log_probs != nullptr ? cum_log_probs[row] : 0.0f;
+    return o;
+}
 
 // thread 0 only: weights w[0..n) in selection order -> sampled position (sampling_topk_kernels.cu:282-311).
 // `w` is 16-byte aligned LDS, zero padded to a multiple of 4 (adding +0 to a non-negative sum is exact),
@@ -526,14 +809,14 @@ __device__ __forceinline__ void topk_emit(const TopkOutputs& o, int row, int id,
     if (probs_in && any_valid) {
         const float lp = det_logf(w);
         if (o.cum_log_probs != nullptr) {
-            o.cum_log_probs[row] += lp;
+            o.cum_log_probs[row] = o.cum_log_prob_in + lp;
         }
         if (o.output_log_probs != nullptr) {
             o.output_log_probs[row] = lp - det_logf(s_sum);
         }
     }
     if (o.sequence_length != nullptr && o.finished != nullptr) {
-        o.sequence_length[row] = o.finished[row] ? o.sequence_length[row] : o.sequence_length[row] + 1;
+        o.sequence_length[row] = o.sequence_length_in + 1;  // the row was not finished (:317-320)
         o.finished[row]        = id == end_ids[row];
     }
 }
@@ -542,7 +825,7 @@ __device__ __forceinline__ void topk_emit(const TopkOutputs& o, int row, int id,
 // Every pick is the smallest composite key strictly greater than the previous pick, where the
 // composite encodes the reference's order; picks of stage 1 go to `picks` (8k entries, global).
 template<int DT, class Row>
-__device__ void topk_literal(Row& rowctx, TopkSelectShared& s, int vocab, int k, int BS1, int BS2,
+__device__ void topk_literal(Row& rowctx, TopkShared& s, int vocab, int k, int BS1, int BS2,
                              TopkEntry* picks, int* n_list_out)
 {
     const int      t    = threadIdx.x;
@@ -620,7 +903,7 @@ __device__ void topk_literal(Row& rowctx, TopkSelectShared& s, int vocab, int k,
         if (t == 0) {
             const int pos = (int)(best & 0xFFFFFFull);
             s.keys[ite]   = (unsigned long long)(~picks[pos].key) << 32;
-            s.idx[ite]    = (int)picks[pos].idx;
+            s.sel.idx[ite]    = (int)picks[pos].idx;
         }
         last      = best;
         have_last = true;
@@ -630,110 +913,55 @@ __device__ void topk_literal(Row& rowctx, TopkSelectShared& s, int vocab, int k,
     *n_list_out = n_list;
 }
 
+// -------------------------------------------------------------------------------------------
+// select: replay the reference's two tie orders on the candidates in s.cand, sample, emit.
+// `n` < 0 asks for the literal replay.
+// -------------------------------------------------------------------------------------------
 template<int DT, class Row>
-__device__ __forceinline__ void topk_select_row(Row& rowctx, TopkSelectShared& s, int row, int vocab, int k,
-                                                float p, int max_top_k, int splits, const TopkChunkHeader* headers,
-                                                TopkEntry* entries, int cap, bool probs_in, float u,
-                                                const int* end_ids, const TopkOutputs& out)
+__device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int n, uint32_t thr, int row, int vocab,
+                                                int k, float p, int max_top_k, TopkEntry* picks, bool probs_in,
+                                                float u, const int* end_ids, const TopkOutputs& out)
 {
-    const int t   = threadIdx.x;
-    const int BS1 = max_top_k <= 16 ? 128 : 256;
-    const int BS2 = max_top_k <= 32 ? 128 : 256;
+    const int t       = threadIdx.x;
+    const int bs1_log = max_top_k <= 16 ? 7 : 8;
+    const int BS1     = 1 << bs1_log;
+    const int BS2     = max_top_k <= 32 ? 128 : 256;
+    int       n_list  = 0;  // length of the final ordered list: values in s.w (as fp32), ids in s.idx
+    FTK_PHASE_BEGIN();
 
-    // ---- merge chunk headers
-    // Row-wide lower bound T0 of the k-th largest key. Two valid bounds, take the larger:
-    //   any chunk's `threshold` with >= k elements above it;
-    //   the smallest `threshold8` when every chunk has one (splits x ceil(k/splits) >= k elements).
-    // A list is complete above its own `threshold` (lists of chunks with fewer than k valid elements
-    // hold all of them), and T0 is never below the threshold of a list that was cut.
-    uint32_t T0       = min_valid_key<DT>();
-    uint32_t min8     = 0xFFFFFFFFu;
-    bool     overflow = false;
-    for (int c = 0; c < splits; ++c) {
-        const TopkChunkHeader h = headers[c];
-        overflow                = overflow || (h.flags & 2u) != 0u;
-        min8                    = h.threshold8 < min8 ? h.threshold8 : min8;
-        if ((h.flags & 1u) && h.threshold > T0) {
-            T0 = h.threshold;
+    if (n >= 0) {
+        if (n > TK_THREADS && n > k) {
+            n = topk_tighten(s, n, k, &thr);
         }
-    }
-    if (min8 > T0) {
-        T0 = min8;  // min8 == 0 when some chunk has no threshold8
-    }
-    int  n_list  = 0;  // length of the final ordered list: values in s.w (as fp32), ids in s.idx
-    bool literal = overflow;
-    int  n       = 0;
-
-    // candidates at or above a threshold over all chunk lists -> LDS with the stage-1 composite key
-    //   slice(3) | ~key(32) | BS1-1-t (8) | j (21),   i = (j*8 + slice)*BS1 + t
-    auto gather = [&](uint32_t thr) -> int {
+        FTK_PHASE(9);
+        // candidates -> stage-1 composite keys, in place
+        //   slice(3) | ~key(32) | BS1-1-t (8) | j (21),   i = (j*8 + slice)*BS1 + t
+        constexpr int PER = TK_CCAP / TK_THREADS;
+        uint32_t      ck[PER], ci[PER];
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int i = t + r * TK_THREADS;
+            ck[r]       = i < n ? s.cand.key[i] : 0u;
+            ci[r]       = i < n ? s.cand.idx[i] : 0u;
+        }
         if (t < 8) {
             s.slice_count[t] = 0;
         }
-        if (t == 0) {
-            s.counter = 0;
-        }
-        __syncthreads();
-        for (int ch = 0; ch < splits; ++ch) {
-            const int        cnt = (int)headers[ch].count;
-            const TopkEntry* e   = entries + (size_t)ch * cap;
-            for (int i = t; i < cnt; i += TK_THREADS) {
-                const TopkEntry en = e[i];
-                if (en.key >= thr) {
-                    const int idx   = (int)en.idx;
-                    const int blk   = idx / BS1;
-                    const int tt    = idx - blk * BS1;
-                    const int slice = blk & 7;
-                    const int slot  = atomicAdd(&s.counter, 1);
-                    if (slot < TK_SELCAP) {
-                        atomicAdd(&s.slice_count[slice], 1);
-                        s.keys[slot] = ((unsigned long long)slice << 61) | ((unsigned long long)(~en.key) << 29)
-                                       | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
-                    }
-                }
+        lds_barrier();
+#pragma unroll
+        for (int r = 0; r < PER; ++r) {
+            const int i = t + r * TK_THREADS;
+            if (i < n) {
+                const int blk   = (int)(ci[r] >> bs1_log);
+                const int tt    = (int)(ci[r] & (uint32_t)(BS1 - 1));
+                const int slice = blk & 7;
+                atomicAdd(&s.slice_count[slice], 1);
+                s.keys[i] = ((unsigned long long)slice << 61) | ((unsigned long long)(~ck[r]) << 29)
+                            | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
             }
         }
-        __syncthreads();
-        const int total = s.counter;
-        __syncthreads();
-        return total;
-    };
-
-    if (!literal) {
-        n = gather(T0);
-        if (n > TK_SELCAP) {
-            // every chunk had to keep >= k candidates (k in the hundreds): find the exact k-th largest
-            // key by bisection over the lists, then gather again
-            auto count_ge = [&](uint32_t thr) -> int {
-                int c = 0;
-                for (int ch = 0; ch < splits; ++ch) {
-                    const int        cnt = (int)headers[ch].count;
-                    const TopkEntry* e   = entries + (size_t)ch * cap;
-                    for (int i = t; i < cnt; i += TK_THREADS) {
-                        c += e[i].key >= thr ? 1 : 0;
-                    }
-                }
-                return block_sum_i(c, (int*)s.red32);
-            };
-            uint32_t lo = T0, hi = 0xFFFFFFFFu;  // count(lo) >= k always holds
-            while (hi - lo > 1u) {
-                const uint32_t mid = lo + (hi - lo) / 2u;
-                if (count_ge(mid) >= k) {
-                    lo = mid;
-                }
-                else {
-                    hi = mid;
-                }
-            }
-            T0 = lo;
-            n  = gather(T0);
-        }
-        if (n > TK_SELCAP) {
-            literal = true;  // thousands of identical values around the k-th
-        }
-    }
-
-    if (!literal) {
+        lds_barrier();
+        FTK_PHASE(10);
         int slice_start[8];
         {
             int acc = 0;
@@ -768,26 +996,36 @@ __device__ __forceinline__ void topk_select_row(Row& rowctx, TopkSelectShared& s
         if (n <= TK_THREADS) {
             // ---- small candidate sets (the usual case): rank by counting, one candidate per thread.
             // Composite keys are unique, so "number of smaller keys" is the sorted position.
+            // (keys are read two at a time; an odd list is padded with a key that never counts)
             const unsigned long long mine = t < n ? s.keys[t] : ~0ull;
-            int                      q    = 0;
-            for (int j = 0; j < n; ++j) {
-                q += s.keys[j] < mine ? 1 : 0;
+            const int                n2   = (n + 1) & ~1;
+            auto                     rank = [&](unsigned long long key) -> int {
+                int q = 0;
+#pragma unroll 4
+                for (int j = 0; j < n2; j += 2) {
+                    const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&s.keys[j]);
+                    q += kk.x < key ? 1 : 0;
+                    q += kk.y < key ? 1 : 0;
+                }
+                return q;
+            };
+            if (t == 0 && n2 != n) {
+                s.keys[n] = ~0ull;
             }
+            lds_barrier();
+            const int                q      = rank(mine);
             int                      my_idx = 0;
             const unsigned long long k2     = t < n ? stage2_key(mine, q, 0, &my_idx) : ~0ull;
-            __syncthreads();
+            lds_barrier();
             s.keys[t] = k2;
-            __syncthreads();
-            int q2 = 0;
-            for (int j = 0; j < n; ++j) {
-                q2 += s.keys[j] < k2 ? 1 : 0;
-            }
+            lds_barrier();
+            const int q2 = rank(k2);
             const bool kept = k2 != ~0ull;
             n_list          = block_sum_i(kept ? 1 : 0, (int*)s.red32);
             n_list          = n_list < k ? n_list : k;
             if (kept && q2 < n_list) {
-                s.w[q2]   = key_to_float(~(uint32_t)(k2 >> 32));
-                s.idx[q2] = my_idx;
+                s.sel.w[q2]   = key_to_float(~(uint32_t)(k2 >> 32));
+                s.sel.idx[q2] = my_idx;
             }
             __syncthreads();
         }
@@ -804,7 +1042,7 @@ __device__ __forceinline__ void topk_select_row(Row& rowctx, TopkSelectShared& s
                 if (qi < n) {
                     int idx;
                     nk        = stage2_key(s.keys[qi], qi, qi, &idx);
-                    s.idx[qi] = idx;
+                    s.sel.idx[qi] = idx;
                 }
                 s.keys[qi] = nk;
             }
@@ -823,7 +1061,7 @@ __device__ __forceinline__ void topk_select_row(Row& rowctx, TopkSelectShared& s
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = t + r * TK_THREADS;
-                my_idx[r]   = i < n_list ? s.idx[(int)(s.keys[i] & 0xFFFull)] : 0;
+                my_idx[r]   = i < n_list ? s.sel.idx[(int)(s.keys[i] & 0xFFFull)] : 0;
                 my_val[r]   = i < n_list ? key_to_float(~(uint32_t)(s.keys[i] >> 32)) : 0.0f;
             }
             __syncthreads();
@@ -831,40 +1069,134 @@ __device__ __forceinline__ void topk_select_row(Row& rowctx, TopkSelectShared& s
             for (int r = 0; r < 4; ++r) {
                 const int i = t + r * TK_THREADS;
                 if (i < n_list) {
-                    s.idx[i] = my_idx[r];
-                    s.w[i]   = my_val[r];
+                    s.sel.idx[i] = my_idx[r];
+                    s.sel.w[i]   = my_val[r];
                 }
             }
             __syncthreads();
         }
     }
     else {
-        topk_literal<DT, Row>(rowctx, s, vocab, k, BS1, BS2, entries, &n_list);
+        topk_literal<DT, Row>(rowctx, s, vocab, k, BS1, BS2, picks, &n_list);
         for (int i = t; i < n_list; i += TK_THREADS) {
-            s.w[i] = key_to_float(~(uint32_t)(s.keys[i] >> 32));
+            s.sel.w[i] = key_to_float(~(uint32_t)(s.keys[i] >> 32));
         }
         __syncthreads();
     }
 
+    FTK_PHASE(11);
     // ---- weights (sampling_topk_kernels.cu:264-279): exp(x - max) on logits, the value itself on
     // probabilities; the list is padded with zero weights to a multiple of 4 for the vectorised walk
-    const float x0 = n_list > 0 ? s.w[0] : 0.0f;
+    const float x0 = n_list > 0 ? s.sel.w[0] : 0.0f;
     __syncthreads();
     for (int i = t; i < ((n_list + 3) & ~3); i += TK_THREADS) {
-        const float x = i < n_list ? s.w[i] : 0.0f;
-        s.w[i]        = i < n_list ? (probs_in ? x : det_expf(x - x0)) : 0.0f;
+        const float x = i < n_list ? s.sel.w[i] : 0.0f;
+        s.sel.w[i]        = i < n_list ? (probs_in ? x : det_expf(x - x0)) : 0.0f;
     }
     __syncthreads();
+    FTK_PHASE(12);
     if (t == 0) {
         if (n_list == 0) {
             topk_emit(out, row, 0, probs_in, 0.0f, 0.0f, end_ids, false);
         }
         else {
             float     s_sum;
-            const int pick = topk_sample_walk(s.w, n_list, u, p, &s_sum);
-            topk_emit(out, row, s.idx[pick] % vocab, probs_in, s.w[pick], s_sum, end_ids, true);
+            const int pick = topk_sample_walk(s.sel.w, n_list, u, p, &s_sum);
+            topk_emit(out, row, s.sel.idx[pick] % vocab, probs_in, s.sel.w[pick], s_sum, end_ids, true);
         }
     }
+    FTK_PHASE(13);
+}
+
+// Rows split over several workgroups: merge their lists from the workspace into s.cand.
+// Returns the candidate count, or -1 for the literal replay; *thr_out is a valid bound when the result
+// is >= k.
+template<int DT>
+__device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits, const TopkChunkHeader* headers,
+                                                const TopkEntry* entries, uint32_t* thr_out)
+{
+    const int t = threadIdx.x;
+    FTK_PHASE_BEGIN();
+    // Row-wide lower bound T0 of the k-th largest key, the larger of two valid ones: the largest
+    // `threshold` of a chunk that holds >= k elements, and the smallest `share` when every chunk has one.
+    // A list is complete above its own threshold (lists of chunks with fewer than k selectable elements
+    // hold all of them), and T0 is never below the threshold of a list that was cut.
+    uint32_t T0        = min_valid_key<DT>();
+    uint32_t min_share = 0xFFFFFFFFu;
+    bool     overflow  = false;
+    for (int c = 0; c < splits; ++c) {
+        const TopkChunkHeader h = headers[c];
+        overflow                = overflow || (h.flags & 2u) != 0u;
+        min_share               = h.share < min_share ? h.share : min_share;
+        if ((h.flags & 1u) && h.threshold > T0) {
+            T0 = h.threshold;
+        }
+    }
+    if (overflow) {
+        return -1;
+    }
+    if (min_share > T0) {
+        T0 = min_share;  // 0 when some chunk has no share bound
+    }
+    FTK_PHASE(7);
+    // one wave per chunk list
+    auto gather = [&](uint32_t thr) -> int {
+        if (t == 0) {
+            s.n_cand = 0;
+        }
+        __syncthreads();
+        for (int ch = wave_id(); ch < splits; ch += TK_THREADS / WAVE) {
+            const int        cnt = (int)headers[ch].count;
+            const TopkEntry* e   = entries + (size_t)ch * TK_CCAP;
+            for (int i = lane_id(); i < cnt; i += WAVE) {
+                const TopkEntry en = e[i];
+                if (en.key >= thr) {
+                    const int slot = atomicAdd(&s.n_cand, 1);
+                    if (slot < TK_CCAP) {
+                        s.cand.key[slot] = en.key;
+                        s.cand.idx[slot] = en.idx;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int total = s.n_cand;
+        __syncthreads();
+        return total;
+    };
+    int n = gather(T0);
+    FTK_PHASE(8);
+    if (n > TK_CCAP) {
+        // large k over many chunks: find the exact k-th largest key by bisection over the lists
+        auto count_ge = [&](uint32_t thr) -> int {
+            int c = 0;
+            for (int ch = 0; ch < splits; ++ch) {
+                const int        cnt = (int)headers[ch].count;
+                const TopkEntry* e   = entries + (size_t)ch * TK_CCAP;
+                for (int i = t; i < cnt; i += TK_THREADS) {
+                    c += e[i].key >= thr ? 1 : 0;
+                }
+            }
+            return block_sum_i(c, (int*)s.red32);
+        };
+        uint32_t lo = T0, hi = 0xFFFFFFFFu;  // count(lo) >= k always holds
+        while (hi - lo > 1u) {
+            const uint32_t mid = lo + (hi - lo) / 2u;
+            if (count_ge(mid) >= k) {
+                lo = mid;
+            }
+            else {
+                hi = mid;
+            }
+        }
+        T0 = lo;
+        n  = gather(T0);
+    }
+    if (n > TK_CCAP) {
+        return -1;  // thousands of identical values around the k-th
+    }
+    *thr_out = T0;
+    return n;
 }
 
 }  // namespace ftk

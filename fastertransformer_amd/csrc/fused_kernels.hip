@@ -7,10 +7,11 @@
 // the [batch, vocab_padded] logits, k+5 reads and 3 writes of every row in total. Here the row is read
 // once and never written: the element arithmetic of those kernels (ftk_transform.cuh) is applied in
 // registers while the chunk streams in, and the result feeds the candidate gather of ftk_topk.cuh.
-//   history_bitmap_kernel - one workgroup per row turns the time-major token history into a bitmap
-//                           over the vocabulary (who gets the repetition / presence penalty)
-//   fused_gather_kernel   - grid (splits, rows): stream, transform, gather candidates
-//   fused_select_kernel   - one workgroup per row: exact tie order, sampling, bookkeeping
+//   fused_row_kernel      - one workgroup per row: stream, transform, select, sample, bookkeeping
+//   fused_gather_kernel / fused_select_kernel - the same in two launches for small batches, whose rows
+//                           are split over several workgroups
+//   history_bitmap_kernel - very large vocabularies only: turns the time-major token history into a
+//                           bitmap over the vocabulary (who gets the repetition / presence penalty)
 #include <vector>
 
 #include "ftk_sampling.h"
@@ -37,18 +38,34 @@ struct FusedParams {
     const bool*  finished_in;
     uint32_t*    bitmaps;        // [rows][bitmap_words] scratch, or null when no history penalty applies
     int          bitmap_words;
-    int          bitmaps_ready;  // history_bitmap_kernel filled `bitmaps` (long histories)
+    int          bitmaps_ready;  // history_bitmap_kernel filled `bitmaps`
+    int          lds_window;        // 0: none, 1: small LDS bitmap window, 2: large
 };
 
 // History bitmaps: bit v set <=> token v occurs in the row's (non-padding) history, i.e. column v gets
-// the repetition / presence penalty. Short histories: every gather workgroup builds the window of the
-// bitmap that covers its own chunk in LDS (a few hundred strided 4-byte reads that overlap the logits
-// loads already in flight). Long histories: history_bitmap_kernel builds whole-row bitmaps once.
-constexpr int FUSED_LOCAL_BITMAP_MAX_STEP = 4096;
-constexpr int FUSED_LDS_BITMAP_WORDS      = TK_ELEMS * TK_THREADS / 32 + 4;
+// the repetition / presence penalty. A streaming workgroup builds the window of the bitmap that covers
+// its own columns in LDS (strided 4-byte reads of the history that overlap the logits loads already in
+// flight). When the window does not fit, or many workgroups per row would each scan a long history,
+// history_bitmap_kernel builds whole-row bitmaps in the workspace first.
+constexpr int FUSED_BITMAP_WORDS_SMALL     = 2048 + 4;  // LDS window of 64 Ki columns: four workgroups per compute unit
+constexpr int FUSED_BITMAP_WORDS_LARGE     = 5120 + 4;  // 160 Ki columns: three
+constexpr int FUSED_BITMAP_WORDS_GLOBAL    = 0;         // no window: bitmaps in global memory
+constexpr int FUSED_SPLIT_BITMAP_MAX_STEP  = 8192;
 
-template<int DT>
+// the LDS window of the history bitmap (one per workgroup)
+template<int BMW>
+__device__ __forceinline__ uint32_t* fused_lds_bitmap()
+{
+    __shared__ uint32_t words[BMW];
+    return words;
+}
+
+// BMW > 0: the history bitmap is a window of BMW words in LDS, built by prepare().
+// BMW == 0: whole-row bitmaps in global memory (built by history_bitmap_kernel, or by
+//           prepare_whole_row() for the literal replay).
+template<int DT, int BMW>
 struct FusedRow {
+    static constexpr int  LDS_WORDS = BMW > 0 ? BMW : 1;
     typedef Storage<DT>   S;
     typedef typename S::T T;
     const T*              rowp;
@@ -60,8 +77,8 @@ struct FusedRow {
     float                 penalty;
     int                   masked_end_id;  // end id when the min-length mask applies, else -1
     // history bitmap
-    const uint32_t* bm;         // words in use (global row bitmap or the LDS window), null = none
-    int             bm_origin;  // column of bit 0 of bm[0]
+    int             bm_mode;    // 0: no history penalty, otherwise the bitmap is in place
+    int             bm_origin;  // column of bit 0 of word 0
     uint32_t*       global_bm;  // this row's slice of the scratch bitmaps
     bool            global_ready;
     const int*      history;  // output_ids + row, stride batch_size
@@ -81,7 +98,7 @@ struct FusedRow {
         penalty       = p.penalties != nullptr ? p.penalties[row] : 0.0f;
         global_bm     = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
         global_ready  = p.bitmaps_ready != 0;
-        bm            = global_ready ? global_bm : nullptr;
+        bm_mode       = (BMW == 0 && global_bm != nullptr && global_ready) ? 1 : 0;
         bm_origin     = 0;
         history       = p.output_ids != nullptr ? p.output_ids + row : nullptr;
         batch_size    = p.batch_size;
@@ -105,33 +122,40 @@ struct FusedRow {
     // called by every thread of the gather workgroup before it touches columns [lo, hi)
     __device__ __forceinline__ void prepare(int lo, int hi)
     {
-        if (global_bm == nullptr || global_ready) {
+        if (BMW == 0 || global_bm == nullptr) {
             return;
         }
-        __shared__ uint32_t lds_bm[FUSED_LDS_BITMAP_WORDS];
-        const int           origin = lo & ~31;
-        const int           words  = min(FUSED_LDS_BITMAP_WORDS, (hi - origin + 31) / 32 + 1);
+        uint32_t* window = fused_lds_bitmap<LDS_WORDS>();
+        const int origin = lo & ~31;
+        const int words  = min(LDS_WORDS, (hi - origin + 31) / 32 + 1);
         for (int i = threadIdx.x; i < words; i += blockDim.x) {
-            lds_bm[i] = 0u;
+            window[i] = 0u;
         }
         __syncthreads();
         for (int t = threadIdx.x; t < step; t += blockDim.x) {
             if (history_position_counts(t)) {
                 const int id = history[(size_t)t * batch_size];
                 if (id >= lo && id < hi) {
-                    atomicOr(&lds_bm[(id - origin) >> 5], 1u << ((id - origin) & 31));
+                    atomicOr(&window[(id - origin) >> 5], 1u << ((id - origin) & 31));
                 }
             }
         }
         __syncthreads();
-        bm        = lds_bm;
+        bm_mode   = 1;
         bm_origin = origin;
+    }
+    __device__ __forceinline__ uint32_t bm_word(int w) const
+    {
+        if (BMW > 0) {
+            return fused_lds_bitmap<LDS_WORDS>()[w];
+        }
+        return global_bm[w];
     }
     // whole-row bitmap in global scratch, for the literal replay of rows the gather could not bound
     __device__ __forceinline__ void build_global_bitmap()
     {
-        if (global_bm == nullptr || global_ready) {
-            return;
+        if (BMW > 0 || global_bm == nullptr || global_ready) {
+            return;  // (a workgroup with an LDS window owns the whole row: the window already covers it)
         }
         const int words = (Vp + 31) / 32 + 1;
         for (int i = threadIdx.x; i < words; i += blockDim.x) {
@@ -149,14 +173,14 @@ struct FusedRow {
         }
         __threadfence_block();
         __syncthreads();
-        bm           = global_bm;
+        bm_mode      = 1;
         bm_origin    = 0;
         global_ready = true;
     }
     // history-membership bits of columns first .. first+n-1 (n <= 8)
     __device__ __forceinline__ uint32_t vector_bits(int first, int n) const
     {
-        if (bm == nullptr) {
+        if (bm_mode == 0) {
             return 0u;
         }
         uint32_t bits = 0u;
@@ -164,9 +188,9 @@ struct FusedRow {
             const int rel = first - bm_origin;
             const int w   = rel >> 5;
             const int sh  = rel & 31;
-            bits          = bm[w] >> sh;
+            bits          = bm_word(w) >> sh;
             if (sh + n > 32) {
-                bits |= bm[w + 1] << (32 - sh);  // both bitmaps carry one word of slack
+                bits |= bm_word(w + 1) << (32 - sh);  // both bitmaps carry one word of slack
             }
             bits &= (1u << n) - 1u;
         }
@@ -174,7 +198,7 @@ struct FusedRow {
             for (int j = 0; j < n; ++j) {
                 const int v = first + j;
                 if (v >= bm_origin && v < Vp) {
-                    bits |= ((bm[(v - bm_origin) >> 5] >> ((v - bm_origin) & 31)) & 1u) << j;
+                    bits |= ((bm_word((v - bm_origin) >> 5) >> ((v - bm_origin) & 31)) & 1u) << j;
                 }
             }
         }
@@ -186,7 +210,7 @@ struct FusedRow {
     }
     __device__ __forceinline__ bool has_vector_bits() const
     {
-        return bm != nullptr;
+        return bm_mode != 0;
     }
     // pad columns and the masked end id are -MAX_T whatever the logits hold
     __device__ __forceinline__ bool never_selected(int v) const
@@ -197,6 +221,11 @@ struct FusedRow {
     __device__ __forceinline__ float fast(float x) const
     {
         return temp_active ? round_t<DT>(x * inv) : x;
+    }
+    // the same column when it is in the history
+    __device__ __forceinline__ float flagged(float xf) const
+    {
+        return round_t<DT>(repetition_value(xf, penalty, penalty_type));
     }
     // the value top-k would see for column v: temperature(+bias) -> history penalty -> min-length mask
     // -> pad mask, each rounded to T where the reference stores T
@@ -226,7 +255,7 @@ struct FusedRow {
     }
     __device__ __forceinline__ uint32_t key_at(int v) const
     {
-        const uint32_t bit = bm != nullptr ? (bm[(v - bm_origin) >> 5] >> ((v - bm_origin) & 31)) & 1u : 0u;
+        const uint32_t bit = bm_mode != 0 ? (bm_word((v - bm_origin) >> 5) >> ((v - bm_origin) & 31)) & 1u : 0u;
         return order_key(slow(v, S::ld(rowp[v]), bit));
     }
     // before key_at() may be used over the whole row
@@ -276,53 +305,102 @@ history_bitmap_kernel(uint32_t* __restrict__ bitmaps, int bitmap_words, const in
     }
 }
 
-template<int DT>
-__global__ void __launch_bounds__(TK_THREADS, 4)
-fused_gather_kernel(FusedParams p, int splits, int nvt, int cap, size_t row_entries,
-                    TopkChunkHeader* __restrict__ headers, TopkEntry* __restrict__ entries)
+struct FusedLaunch {
+    int*             ids;
+    int*             sequence_length;
+    bool*            finished;
+    RngState*        rng;
+    const float*     uniforms;
+    int              splits;
+    int              tiles_per_wg;
+    size_t           row_entries;
+    TopkChunkHeader* headers;
+    TopkEntry*       entries;
+};
+
+__device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch& l, int row)
 {
-    const int row   = blockIdx.y;
-    const int chunk = blockIdx.x;
+    if (threadIdx.x == 0) {
+        s.misc[0] = __float_as_int(row_uniform(l.rng, l.uniforms, row));
+    }
+    __syncthreads();
+    return __int_as_float(s.misc[0]);
+}
+
+template<int DT, int BMW>
+__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? 4 : 3)
+fused_row_kernel(FusedParams p, FusedLaunch l)
+{
+    __shared__ TopkShared s;
+    const int             row = blockIdx.x;
+    if (p.skip_decode != nullptr && p.skip_decode[row]) {
+        return;
+    }
+    if (l.finished != nullptr && l.finished[row]) {
+        if (threadIdx.x == 0) {
+            l.ids[row] = p.end_ids[row];  // a finished row emits its end id without looking at the logits
+        }
+        return;
+    }
+    const int    k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    const float  tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
+    const float  u  = fused_row_draw(s, l, row);
+    const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row);
+    FusedRow<DT, BMW> r(p, row);
+    uint32_t     thr = 0u;
+    const int    n   = topk_stream<DT>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
+    topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, l.entries + (size_t)row * l.row_entries, false, u,
+                        p.end_ids, out);
+}
+
+template<int DT, int BMW>
+__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? 4 : 3)
+fused_gather_kernel(FusedParams p, FusedLaunch l)
+{
+    __shared__ TopkShared s;
+    const int             row   = blockIdx.y;
+    const int             chunk = blockIdx.x;
     if (p.skip_decode != nullptr && p.skip_decode[row]) {
         return;
     }
     if (p.finished_in != nullptr && p.finished_in[row]) {
-        return;  // a finished row emits its end id without looking at the logits
+        return;
     }
     const int    k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    FusedRow<DT> r(p, row);
-    topk_gather_chunk<DT>(r, p.Vp, k, chunk, splits, nvt, cap, headers + (size_t)row * splits + chunk,
-                          entries + (size_t)row * row_entries + (size_t)chunk * cap);
+    FusedRow<DT, BMW> r(p, row);
+    const int    tiles = topk_row_tiles<DT>(r.rowp, p.Vp);
+    const int    t0    = min(tiles, chunk * l.tiles_per_wg);
+    const int    t1    = min(tiles, t0 + l.tiles_per_wg);
+    uint32_t     thr   = 0u;
+    const int    n     = topk_stream<DT>(r, s, p.Vp, k, t0, t1, &thr);
+    topk_dump_list(s, n, k, l.splits, thr, l.headers + (size_t)row * l.splits + chunk,
+                   l.entries + (size_t)row * l.row_entries + (size_t)chunk * TK_CCAP);
 }
 
 template<int DT>
-__global__ void __launch_bounds__(TK_THREADS)
-fused_select_kernel(FusedParams p, int* __restrict__ ids, int* __restrict__ sequence_length, bool* __restrict__ finished,
-                    RngState* rng, const float* __restrict__ uniforms, int splits, int cap, size_t row_entries,
-                    const TopkChunkHeader* __restrict__ headers, TopkEntry* __restrict__ entries)
+__global__ void __launch_bounds__(TK_THREADS) fused_select_kernel(FusedParams p, FusedLaunch l)
 {
-    __shared__ TopkSelectShared s;
-    const int                   row = blockIdx.x;
+    constexpr int BMW = 0;  // the literal replay reads whole-row bitmaps from global memory
+    __shared__ TopkShared s;
+    const int             row = blockIdx.x;
     if (p.skip_decode != nullptr && p.skip_decode[row]) {
         return;
     }
-    if (finished != nullptr && finished[row]) {
+    if (l.finished != nullptr && l.finished[row]) {
         if (threadIdx.x == 0) {
-            ids[row] = p.end_ids[row];
+            l.ids[row] = p.end_ids[row];
         }
         return;
     }
-    const int   k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    const float tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
-    if (threadIdx.x == 0) {
-        s.misc[0] = __float_as_int(row_uniform(rng, uniforms, row));
-    }
-    __syncthreads();
-    const float  u = __int_as_float(s.misc[0]);
-    FusedRow<DT> r(p, row);
-    const TopkOutputs  out{ids, sequence_length, finished, nullptr, nullptr};
-    topk_select_row<DT>(r, s, row, p.Vp, k, tp, p.max_top_k, splits, headers + (size_t)row * splits,
-                        entries + (size_t)row * row_entries, cap, false, u, p.end_ids, out);
+    const int    k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    const float  tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
+    const float  u  = fused_row_draw(s, l, row);
+    const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row);
+    FusedRow<DT, BMW> r(p, row);
+    TopkEntry*   row_entries = l.entries + (size_t)row * l.row_entries;
+    uint32_t     thr         = 0u;
+    const int    n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr);
+    topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
 }
 
 }  // namespace ftk
@@ -472,6 +550,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     p.bitmaps            = nullptr;
     p.bitmap_words       = bitmap_words;
     p.bitmaps_ready      = 0;
+    p.lds_window         = 0;
 
     char* ws = (char*)a->workspace;
     if (p.penalties != nullptr && a->step > 0) {
@@ -479,7 +558,16 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             return FTK_ERR_ARGUMENT;
         }
         p.bitmaps = (uint32_t*)ws;
-        if (a->step > FUSED_LOCAL_BITMAP_MAX_STEP) {
+        // columns one workgroup streams (upper bound): does its bitmap window fit in LDS?
+        const int    epv        = 16 / elem;
+        const size_t range_cols = (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
+        const size_t words      = range_cols / 32 + 4;
+        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE
+                           && (plan.splits == 1 || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
+        if (local) {
+            p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
+        }
+        else {
             ScopedKernelTime timer(0, st);
             history_bitmap_kernel<<<rows, HB_THREADS, 0, st>>>(p.bitmaps, bitmap_words, a->output_ids, a->batch_size,
                                                                a->vocab_size_padded, a->input_lengths,
@@ -492,21 +580,54 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     else {
         p.penalties = nullptr;
     }
-    TopkChunkHeader* headers = (TopkChunkHeader*)(ws + bitmap_bytes);
-    TopkEntry*       entries = (TopkEntry*)(headers + (size_t)rows * plan.splits);
-    dim3             grid(plan.splits, rows);
+    FusedLaunch l;
+    l.ids             = a->ids;
+    l.sequence_length = a->sequence_length;
+    l.finished        = a->finished;
+    l.rng             = (RngState*)a->rng_state;
+    l.uniforms        = a->uniform_draws;
+    l.splits          = plan.splits;
+    l.tiles_per_wg    = plan.tiles_per_wg;
+    l.row_entries     = plan.row_entries;
+    l.headers         = (TopkChunkHeader*)(ws + bitmap_bytes);
+    l.entries         = (TopkEntry*)(l.headers + (size_t)rows * plan.splits);
+    if (plan.splits == 1) {
+        ScopedKernelTime timer(1, st);
+        if (p.bitmaps_ready) {
+            FTK_DISPATCH_DTYPE(a->dtype,
+                               fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL><<<rows, TK_THREADS, 0, st>>>(p, l));
+        }
+        else if (p.lds_window == 2) {
+            FTK_DISPATCH_DTYPE(a->dtype,
+                               fused_row_kernel<DT, FUSED_BITMAP_WORDS_LARGE><<<rows, TK_THREADS, 0, st>>>(p, l));
+        }
+        else {
+            FTK_DISPATCH_DTYPE(a->dtype,
+                               fused_row_kernel<DT, FUSED_BITMAP_WORDS_SMALL><<<rows, TK_THREADS, 0, st>>>(p, l));
+        }
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
+    dim3 grid(plan.splits, rows);
     {
         ScopedKernelTime timer(1, st);
-        FTK_DISPATCH_DTYPE(a->dtype, fused_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(
-                                         p, plan.splits, plan.nvt, plan.cap, plan.row_entries, headers, entries));
+        if (p.bitmaps_ready) {
+            FTK_DISPATCH_DTYPE(a->dtype,
+                               fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL><<<grid, TK_THREADS, 0, st>>>(p, l));
+        }
+        else if (p.lds_window == 2) {
+            FTK_DISPATCH_DTYPE(a->dtype,
+                               fused_gather_kernel<DT, FUSED_BITMAP_WORDS_LARGE><<<grid, TK_THREADS, 0, st>>>(p, l));
+        }
+        else {
+            FTK_DISPATCH_DTYPE(a->dtype,
+                               fused_gather_kernel<DT, FUSED_BITMAP_WORDS_SMALL><<<grid, TK_THREADS, 0, st>>>(p, l));
+        }
     }
     FTK_LAUNCH_CHECK();
     {
         ScopedKernelTime timer(2, st);
-        FTK_DISPATCH_DTYPE(a->dtype, fused_select_kernel<DT><<<rows, TK_THREADS, 0, st>>>(
-                                         p, a->ids, a->sequence_length, a->finished, (RngState*)a->rng_state,
-                                         a->uniform_draws, plan.splits, plan.cap, plan.row_entries, headers,
-                                         entries));
+        FTK_DISPATCH_DTYPE(a->dtype, fused_select_kernel<DT><<<rows, TK_THREADS, 0, st>>>(p, l));
     }
     FTK_LAUNCH_CHECK();
     return 0;

@@ -16,61 +16,120 @@ struct PlainRowAt: PlainRow<DT> {
     __device__ __forceinline__ void prepare_whole_row() {}
 };
 
-template<int DT>
-__global__ void __launch_bounds__(TK_THREADS, 4)
-topk_gather_kernel(const typename Storage<DT>::T* __restrict__ log_probs, const bool* __restrict__ finished,
-                   const bool* __restrict__ skip_decode, const int* __restrict__ top_ks, int max_top_k, int vocab,
-                   int splits, int nvt, int cap, size_t row_entries, TopkChunkHeader* __restrict__ headers,
-                   TopkEntry* __restrict__ entries)
-{
-    const int row   = blockIdx.y;
-    const int chunk = blockIdx.x;
-    if (skip_decode != nullptr && skip_decode[row]) {
-        return;
-    }
-    if (finished != nullptr && finished[row]) {
-        return;
-    }
-    const int      k = top_ks != nullptr ? top_ks[row] : max_top_k;
-    PlainRowAt<DT> r;
-    r.rowp = log_probs + (size_t)row * vocab;
-    topk_gather_chunk<DT>(r, vocab, k, chunk, splits, nvt, cap, headers + (size_t)row * splits + chunk,
-                          entries + (size_t)row * row_entries + (size_t)chunk * cap);
-}
+struct TopkKernelArgs {
+    const void*  log_probs;
+    int*         ids;
+    int*         sequence_length;
+    bool*        finished;
+    float*       cum_log_probs;
+    float*       output_log_probs;
+    RngState*    rng;
+    const float* uniforms;
+    const bool*  skip_decode;
+    const int*   top_ks;
+    int          max_top_k;
+    float        top_p;
+    const float* top_ps;
+    int          vocab;
+    const int*   end_ids;
+    int          splits;
+    int          tiles_per_wg;
+    size_t       row_entries;
+    TopkChunkHeader* headers;
+    TopkEntry*       entries;
+};
 
-template<int DT>
-__global__ void __launch_bounds__(TK_THREADS)
-topk_select_kernel(const typename Storage<DT>::T* __restrict__ log_probs, int* __restrict__ ids,
-                   int* __restrict__ sequence_length, bool* __restrict__ finished, float* __restrict__ cum_log_probs,
-                   float* __restrict__ output_log_probs, RngState* rng, const float* __restrict__ uniforms,
-                   const bool* __restrict__ skip_decode, const int* __restrict__ top_ks, int max_top_k, float top_p,
-                   const float* __restrict__ top_ps, int vocab, const int* __restrict__ end_ids, int splits, int cap,
-                   size_t row_entries, const TopkChunkHeader* __restrict__ headers, TopkEntry* __restrict__ entries)
+// one draw per live row, broadcast to the workgroup
+__device__ __forceinline__ float topk_row_draw(TopkShared& s, RngState* rng, const float* uniforms, int row)
 {
-    __shared__ TopkSelectShared s;
-    const int                   row = blockIdx.x;
-    if (skip_decode != nullptr && skip_decode[row]) {
-        return;
-    }
-    if (finished != nullptr && finished[row]) {
-        if (threadIdx.x == 0) {
-            ids[row] = end_ids[row];  // no draw, no length / log-prob update (:249-252)
-        }
-        return;
-    }
-    const int   k = top_ks != nullptr ? top_ks[row] : max_top_k;
-    const float p = top_ps != nullptr ? top_ps[row] : top_p;
     if (threadIdx.x == 0) {
         s.misc[0] = __float_as_int(row_uniform(rng, uniforms, row));
     }
     __syncthreads();
-    const float    u = __int_as_float(s.misc[0]);
+    return __int_as_float(s.misc[0]);
+}
+
+// rows owned by one workgroup: stream and select in a single launch
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS, 4) topk_row_kernel(TopkKernelArgs a)
+{
+    __shared__ TopkShared s;
+    const int             row = blockIdx.x;
+    if (a.skip_decode != nullptr && a.skip_decode[row]) {
+        return;
+    }
+    if (a.finished != nullptr && a.finished[row]) {
+        if (threadIdx.x == 0) {
+            a.ids[row] = a.end_ids[row];  // no draw, no length / log-prob update (:249-252)
+        }
+        return;
+    }
+    const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
+    const float    p = a.top_ps != nullptr ? a.top_ps[row] : a.top_p;
+    const float    u = topk_row_draw(s, a.rng, a.uniforms, row);
+    const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row);
     PlainRowAt<DT> r;
-    r.rowp = log_probs + (size_t)row * vocab;
-    const TopkOutputs out{ids, sequence_length, finished, cum_log_probs, output_log_probs};
-    topk_select_row<DT>(r, s, row, vocab, k, p, max_top_k, splits, headers + (size_t)row * splits,
-                        entries + (size_t)row * row_entries, cap,
-                        cum_log_probs != nullptr || output_log_probs != nullptr, u, end_ids, out);
+    r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
+    uint32_t  thr = 0u;
+    const int n   = topk_stream<DT>(r, s, a.vocab, k, 0, topk_row_tiles<DT>(r.rowp, a.vocab), &thr);
+    topk_select_lds<DT>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, a.entries + (size_t)row * a.row_entries,
+                        a.cum_log_probs != nullptr || a.output_log_probs != nullptr, u, a.end_ids, out);
+}
+
+// rows split over `splits` workgroups: each leaves its candidate list in the workspace
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS, 4) topk_gather_kernel(TopkKernelArgs a)
+{
+    __shared__ TopkShared s;
+    const int             row   = blockIdx.y;
+    const int             chunk = blockIdx.x;
+    FTK_PHASE_BEGIN();
+    if (a.skip_decode != nullptr && a.skip_decode[row]) {
+        return;
+    }
+    if (a.finished != nullptr && a.finished[row]) {
+        return;
+    }
+    const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
+    PlainRowAt<DT> r;
+    r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
+    FTK_PHASE(0);
+    const int tiles = topk_row_tiles<DT>(r.rowp, a.vocab);
+    const int t0    = min(tiles, chunk * a.tiles_per_wg);
+    const int t1    = min(tiles, t0 + a.tiles_per_wg);
+    uint32_t  thr   = 0u;
+    const int n     = topk_stream<DT>(r, s, a.vocab, k, t0, t1, &thr);
+    topk_dump_list(s, n, k, a.splits, thr, a.headers + (size_t)row * a.splits + chunk,
+                   a.entries + (size_t)row * a.row_entries + (size_t)chunk * TK_CCAP);
+}
+
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS) topk_select_kernel(TopkKernelArgs a)
+{
+    __shared__ TopkShared s;
+    const int             row = blockIdx.x;
+    if (a.skip_decode != nullptr && a.skip_decode[row]) {
+        return;
+    }
+    if (a.finished != nullptr && a.finished[row]) {
+        if (threadIdx.x == 0) {
+            a.ids[row] = a.end_ids[row];
+        }
+        return;
+    }
+    FTK_PHASE_BEGIN();
+    const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
+    const float    p = a.top_ps != nullptr ? a.top_ps[row] : a.top_p;
+    const float    u = topk_row_draw(s, a.rng, a.uniforms, row);
+    const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row);
+    PlainRowAt<DT> r;
+    r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
+    FTK_PHASE(6);
+    TopkEntry* row_entries = a.entries + (size_t)row * a.row_entries;
+    uint32_t   thr         = 0u;
+    const int  n = topk_merge_lists<DT>(s, k, a.splits, a.headers + (size_t)row * a.splits, row_entries, &thr);
+    topk_select_lds<DT>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, row_entries,
+                        a.cum_log_probs != nullptr || a.output_log_probs != nullptr, u, a.end_ids, out);
 }
 
 }  // namespace ftk
@@ -78,6 +137,18 @@ topk_select_kernel(const typename Storage<DT>::T* __restrict__ log_probs, int* _
 using namespace ftk;
 
 extern "C" {
+
+#ifdef FTK_PHASE_TIMING
+int ftk_debug_read_phases(unsigned long long* out, int reset)
+{
+    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ftk_phase), sizeof(unsigned long long) * 32);
+    if (e == hipSuccess && reset) {
+        unsigned long long z[32] = {};
+        e = hipMemcpyToSymbol(HIP_SYMBOL(g_ftk_phase), z, sizeof(z));
+    }
+    return (int)e;
+}
+#endif
 
 int ftk_invoke_batch_topk_sampling(int dtype, void* workspace, size_t* workspace_size, const void* log_probs, int* ids,
                                    int* sequence_length, bool* finished, float* cum_log_probs,
@@ -111,20 +182,37 @@ int ftk_invoke_batch_topk_sampling(int dtype, void* workspace, size_t* workspace
         || (rng_state == nullptr && uniform_draws == nullptr)) {
         return FTK_ERR_ARGUMENT;
     }
-    TopkChunkHeader* headers = (TopkChunkHeader*)workspace;
-    TopkEntry*       entries = (TopkEntry*)(headers + (size_t)batch_size * plan.splits);
-    hipStream_t      st      = (hipStream_t)stream;
-    dim3             grid(plan.splits, batch_size);
-    FTK_DISPATCH_DTYPE(dtype, topk_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(
-                                  (const Storage<DT>::T*)log_probs, finished, skip_decode, top_ks, max_top_k,
-                                  vocab_size_padded, plan.splits, plan.nvt, plan.cap, plan.row_entries, headers,
-                                  entries));
+    TopkKernelArgs a;
+    a.log_probs        = log_probs;
+    a.ids              = ids;
+    a.sequence_length  = sequence_length;
+    a.finished         = finished;
+    a.cum_log_probs    = cum_log_probs;
+    a.output_log_probs = output_log_probs;
+    a.rng              = (RngState*)rng_state;
+    a.uniforms         = uniform_draws;
+    a.skip_decode      = skip_decode;
+    a.top_ks           = top_ks;
+    a.max_top_k        = max_top_k;
+    a.top_p            = top_p;
+    a.top_ps           = top_ps;
+    a.vocab            = vocab_size_padded;
+    a.end_ids          = end_ids;
+    a.splits           = plan.splits;
+    a.tiles_per_wg     = plan.tiles_per_wg;
+    a.row_entries      = plan.row_entries;
+    a.headers          = (TopkChunkHeader*)workspace;
+    a.entries          = (TopkEntry*)(a.headers + (size_t)batch_size * plan.splits);
+    hipStream_t st     = (hipStream_t)stream;
+    if (plan.splits == 1) {
+        FTK_DISPATCH_DTYPE(dtype, topk_row_kernel<DT><<<batch_size, TK_THREADS, 0, st>>>(a));
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
+    dim3 grid(plan.splits, batch_size);
+    FTK_DISPATCH_DTYPE(dtype, topk_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(a));
     FTK_LAUNCH_CHECK();
-    FTK_DISPATCH_DTYPE(dtype, topk_select_kernel<DT><<<batch_size, TK_THREADS, 0, st>>>(
-                                  (const Storage<DT>::T*)log_probs, ids, sequence_length, finished, cum_log_probs,
-                                  output_log_probs, (RngState*)rng_state, uniform_draws, skip_decode, top_ks,
-                                  max_top_k, top_p, top_ps, vocab_size_padded, end_ids, plan.splits, plan.cap,
-                                  plan.row_entries, headers, entries));
+    FTK_DISPATCH_DTYPE(dtype, topk_select_kernel<DT><<<batch_size, TK_THREADS, 0, st>>>(a));
     FTK_LAUNCH_CHECK();
     return 0;
 }
