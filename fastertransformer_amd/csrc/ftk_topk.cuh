@@ -24,6 +24,8 @@
 // literal, slow replay of the reference's passes.
 #pragma once
 #include "ftk_device.cuh"
+#include <stdlib.h>
+
 #include "ftk_transform.cuh"
 
 // Optional phase timing for kernel development: FTK_PHASE(i) adds the time since the previous mark of
@@ -47,11 +49,16 @@ static __device__ unsigned long long g_ftk_phase[32];
 
 namespace ftk {
 
-constexpr int TK_THREADS  = 256;
+#ifndef FTK_TK_THREADS
+#define FTK_TK_THREADS 256
+#endif
+constexpr int TK_THREADS  = FTK_TK_THREADS;
+constexpr int TK_WAVES    = TK_THREADS / 64;
+constexpr int TK_MIN_WGS  = 1024 / TK_THREADS;  // workgroups per compute unit the kernels are built for
 constexpr int TK_NVT      = 16;    // 16-byte vectors per thread and tile: 64 KB per workgroup in flight
 constexpr int TK_CCAP     = 2048;  // candidates a workgroup can hold
 constexpr int TK_MAXSPLIT = 64;
-constexpr int TK_FILL_WGS = 1024;  // workgroups wanted in flight (4 per compute unit)
+constexpr int TK_FILL_WGS = 256 * TK_MIN_WGS;  // workgroups wanted in flight: every compute unit full
 
 struct TopkChunkHeader {
     uint32_t count;      // entries written
@@ -97,6 +104,35 @@ inline TopkPlan topk_plan(int vocab_padded, int batch, int max_top_k, int elem_b
     return p;
 }
 
+// Delay step for topk_stagger: the time a quarter of the resident workgroups needs to load one tile
+// (64 KB each) at ~5 TB/s, in units of 2048 clocks (~0.9 us); no stagger for launches that do not fill
+// the device.
+inline int topk_stagger_units(int workgroups)
+{
+    const char* env = getenv("FTK_STAGGER_UNITS");
+    if (env != nullptr) {
+        return atoi(env);
+    }
+    if (workgroups < 512) {
+        return 0;
+    }
+    const int    resident = workgroups < 1024 ? workgroups : 1024;
+    const double us       = (resident / 4) * 65536.0 / 5.0e6;
+    return (int)(us / 0.9 + 0.5);
+}
+
+// Workgroups that start together and share the memory system fairly also finish each tile together, so
+// the whole device alternates between loading and computing. Delaying three quarters of them by one,
+// two and three tile-load times at the start interleaves the phases. `units` is the delay step in
+// multiples of 2048 clocks.
+__device__ __forceinline__ void topk_stagger(int linear_wg, int units)
+{
+    const int g = (linear_wg >> 8) & 3;
+    for (int i = 0; i < g * units; ++i) {
+        __builtin_amdgcn_s_sleep(32);
+    }
+}
+
 // Workgroup barrier for code that only communicates through LDS: global loads issued earlier stay
 // in flight across it.
 __device__ __forceinline__ void lds_barrier()
@@ -116,6 +152,9 @@ __device__ __forceinline__ void lds_barrier()
 //   plain_vector(first, n) - true when no column of the span needs an index-dependent rule
 //   fast(x)                - index-independent transform of an interior column
 //   flagged(xf)            - fast(x) -> value of a flagged interior column
+//   flagged_upper(xf)      - a cheap value that is never below flagged(xf): decides which vectors are
+//                            looked at again, the exact value is computed for those only
+//   tile_bits(...)         - the flags of a whole tile of an aligned row, EPV bits per vector, packed
 //   slow(v, x, bit)        - the full chain for column v
 //   never_selected(v)      - column v is masked to -MAX_T whatever it holds (pad columns)
 // -------------------------------------------------------------------------------------------
@@ -157,6 +196,17 @@ struct PlainRow {
     {
         return xf;
     }
+    __device__ __forceinline__ float flagged_upper(float xf) const
+    {
+        return xf;
+    }
+    template<int EPV, int NVT>
+    __device__ __forceinline__ void tile_bits(int first0, int stride, uint32_t* packed) const
+    {
+        (void)first0;
+        (void)stride;
+        (void)packed;
+    }
     __device__ __forceinline__ float slow(int v, float x, uint32_t bit) const
     {
         (void)v;
@@ -187,7 +237,7 @@ __device__ __forceinline__ int topk_row_tiles(const void* rowp, int vocab)
     return (nvec + TILE_VECS - 1) / TILE_VECS;
 }
 
-constexpr int TK_STAGE = 128;  // vectors a wave can park per tile
+constexpr int TK_STAGE = 512 / TK_WAVES;  // vectors a wave can park per tile
 
 struct TopkShared {
     union {
@@ -361,7 +411,7 @@ __device__ __forceinline__ int topk_tighten(TopkShared& s, int n, int k, uint32_
 // n_before entries, all >= thr, from earlier tiles. Looks for a higher bound that leaves between k and
 // TK_CCAP candidates; returns the new list length (bound in s.thr_new) or -1 when no bound does.
 template<int DT, class Row>
-__device__ __noinline__ int topk_stream_rare(const Row& rowctx, TopkShared& s, int k, int n_before, int lo_col, int hi_col,
+__device__ __noinline__ int topk_stream_rare(Row rowctx, TopkShared& s, int k, int n_before, int lo_col, int hi_col,
                                              uint32_t thr)
 {
     const int t        = threadIdx.x;
@@ -474,6 +524,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         }
     };
 
+    FTK_PHASE_BEGIN();
     if (t == 0) {
         s.n_cand = 0;
     }
@@ -482,18 +533,35 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
     rowctx.prepare(lo_col, hi_col);
     lds_barrier();
     const bool bitsv = rowctx.has_vector_bits();
+    // flags of the tile being examined, EPV bits per vector of this thread, fetched in one go for plain
+    // tiles of rows that start on a 16-byte boundary (no vector straddles a word of the bitmap then)
+    constexpr int PW = NVT * EPV / 32;
+    uint32_t      packed[PW];
+    const bool    packed_ok = bitsv && a == 0;
+    auto          flags_of  = [&](int it, int first) -> uint32_t {
+        if (packed_ok) {
+            return (packed[(it * EPV) >> 5] >> ((it * EPV) & 31)) & ((1u << EPV) - 1u);
+        }
+        return rowctx.vector_bits(first, EPV);
+    };
     FTK_PHASE(1);
 
     // ---- initial bound from the first tile: maxima over the vectors that take the fast transform
     // (leaving the others out only lowers the bound).
     uint32_t thr;
     {
-        const int vec0    = tile_begin * TILE_VECS;
-        auto      vec_max = [&](int it) -> float {
+        const int  vec0        = tile_begin * TILE_VECS;
+        const bool first_plain = tile_plain(tile_begin);
+        if (first_plain && packed_ok) {
+            rowctx.template tile_bits<EPV, NVT>((vec0 + t) * EPV - a, TK_THREADS * EPV, packed);
+        }
+        auto vec_max = [&](int it) -> float {
             const int  vi    = vec0 + it * TK_THREADS + t;
             const int  first = vi * EPV - a;
-            const bool fastv = any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV)
-                               && (!bitsv || rowctx.vector_bits(first, EPV) == 0u);
+            const bool fastv = first_plain ?
+                                   (!bitsv || flags_of(it, first) == 0u) :
+                                   (any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV)
+                                    && (!bitsv || rowctx.vector_bits(first, EPV) == 0u));
             float vmax = NEG_INF;
 #pragma unroll
             for (int j = 0; j < EPV; ++j) {
@@ -507,17 +575,17 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         for (int it = 0; it < NVT; ++it) {
             gm[it / (NVT / 4)] = __builtin_fmaxf(gm[it / (NVT / 4)], vec_max(it));
         }
-        if (k <= 4 * WAVE) {
-            // each wave sorts its 64 thread maxima; the q-th largest of each wave, minimised over the 4
-            // waves, has >= 4q >= k elements of the tile at or above it
+        if (k <= TK_WAVES * WAVE) {
+            // each wave sorts its 64 thread maxima; the q-th largest of each wave, minimised over the
+            // waves, has >= waves * q >= k elements of the tile at or above it
             const float    tmax   = __builtin_fmaxf(__builtin_fmaxf(gm[0], gm[1]), __builtin_fmaxf(gm[2], gm[3]));
             const uint32_t sorted = wave_sort_desc(order_key(tmax));
-            const int      q      = (k + 3) / 4;
+            const int      q      = (k + TK_WAVES - 1) / TK_WAVES;
             thr = block_min<uint32_t>(__shfl(sorted, q - 1, WAVE), s.red32, 0xFFFFFFFFu);
         }
         else {
-            // the same with the group maxima: 16 sorted sequences, >= 16q >= k elements
-            const int q = (k + 15) / 16;
+            // the same with the group maxima: four sorted sequences per wave
+            const int q = (k + 4 * TK_WAVES - 1) / (4 * TK_WAVES);
             uint32_t  m = 0xFFFFFFFFu;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
@@ -621,6 +689,9 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         const int first0   = (vec0 + t) * EPV - a;
         uint32_t  slowmask = 0u;  // bit `it`: vector `it` of this thread takes the per-column path
         if (tile_plain(tile)) {
+            if (packed_ok && tile != tile_begin) {
+                rowctx.template tile_bits<EPV, NVT>(first0, TK_THREADS * EPV, packed);
+            }
 #pragma unroll
             for (int it = 0; it < NVT; ++it) {
                 const int first = first0 + it * TK_THREADS * EPV;
@@ -630,13 +701,11 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
                     x[j] = rowctx.fast(vector_element<DT>(raw[it], j));
                 }
                 if (bitsv) {
-                    const uint32_t bits = rowctx.vector_bits(first, EPV);
+                    const uint32_t bits = flags_of(it, first);
                     if (bits != 0u) {
 #pragma unroll
                         for (int j = 0; j < EPV; ++j) {
-                            if ((bits >> j) & 1u) {
-                                x[j] = rowctx.flagged(x[j]);
-                            }
+                            x[j] = ((bits >> j) & 1u) ? rowctx.flagged_upper(x[j]) : x[j];
                         }
                     }
                 }
@@ -653,13 +722,27 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
             for (int it = 0; it < NVT; ++it) {
                 const int  vi    = vec0 + it * TK_THREADS + t;
                 const int  first = first0 + it * TK_THREADS * EPV;
-                const bool fastv = any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV)
-                                   && (!bitsv || rowctx.vector_bits(first, EPV) == 0u);
+                // vectors inside the row with no index-dependent column stay on the register path
+                const bool fastv = any_full && vi >= vfull_lo && vi < vfull_hi && rowctx.plain_vector(first, EPV);
                 slowmask |= (vi < nvec && !fastv) ? (1u << it) : 0u;
-                float vmax = NEG_INF;
+                float x[EPV];
 #pragma unroll
                 for (int j = 0; j < EPV; ++j) {
-                    vmax = __builtin_fmaxf(vmax, rowctx.fast(vector_element<DT>(raw[it], j)));
+                    x[j] = rowctx.fast(vector_element<DT>(raw[it], j));
+                }
+                if (bitsv && fastv) {
+                    const uint32_t bits = rowctx.vector_bits(first, EPV);
+                    if (bits != 0u) {
+#pragma unroll
+                        for (int j = 0; j < EPV; ++j) {
+                            x[j] = ((bits >> j) & 1u) ? rowctx.flagged_upper(x[j]) : x[j];
+                        }
+                    }
+                }
+                float vmax = x[0];
+#pragma unroll
+                for (int j = 1; j < EPV; ++j) {
+                    vmax = __builtin_fmaxf(vmax, x[j]);
                 }
                 park(fastv && vmax >= thr_f, raw[it], first);
             }
@@ -1056,17 +1139,18 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 n_list = block_sum_i(cnt, (int*)s.red32);
             }
             // resolve the payload (position in the first sort) into the vocabulary index
-            int   my_idx[4];
-            float my_val[4];
+            constexpr int LPT = 1024 / TK_THREADS;  // list entries per thread (k <= 1024)
+            int           my_idx[LPT];
+            float         my_val[LPT];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            for (int r = 0; r < LPT; ++r) {
                 const int i = t + r * TK_THREADS;
                 my_idx[r]   = i < n_list ? s.sel.idx[(int)(s.keys[i] & 0xFFFull)] : 0;
                 my_val[r]   = i < n_list ? key_to_float(~(uint32_t)(s.keys[i] >> 32)) : 0.0f;
             }
             __syncthreads();
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            for (int r = 0; r < LPT; ++r) {
                 const int i = t + r * TK_THREADS;
                 if (i < n_list) {
                     s.sel.idx[i] = my_idx[r];

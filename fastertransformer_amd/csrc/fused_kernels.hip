@@ -73,8 +73,11 @@ struct FusedRow {
     int                   V, Vp;
     bool                  temp_active, keep_pads;
     float                 inv;
+    float                 fast_mul;  // inv, or 1 when no temperature applies
     int                   penalty_type;  // 2 = none
     float                 penalty;
+    float                 up_mul_neg, up_mul_pos, up_add;  // see flagged_upper
+    bool                  up_ok;
     int                   masked_end_id;  // end id when the min-length mask applies, else -1
     // history bitmap
     int             bm_mode;    // 0: no history penalty, otherwise the bitmap is in place
@@ -93,9 +96,22 @@ struct FusedRow {
         temp_active = p.temperatures != nullptr;
         const TemperatureCtx<DT> tc(temp_active ? p.temperatures[row] : 1.0f, V, Vp, false);
         inv           = tc.inv;
+        fast_mul      = temp_active ? tc.inv : 1.0f;
         keep_pads     = tc.keep_pads;
         penalty_type  = p.penalties != nullptr ? p.penalty_type : 2;
         penalty       = p.penalties != nullptr ? p.penalties[row] : 0.0f;
+        if (penalty_type == 0) {  // additive
+            up_mul_neg = 1.0f;
+            up_mul_pos = 1.0f;
+            up_add     = -penalty;
+            up_ok      = true;
+        }
+        else {
+            up_ok      = penalty > 1e-30f && penalty < 1e30f;  // positive, finite, reciprocal not subnormal
+            up_mul_neg = penalty;
+            up_mul_pos = up_ok ? (1.0f / penalty) * 1.00000095367431640625f : 0.0f;
+            up_add     = 0.0f;
+        }
         global_bm     = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
         global_ready  = p.bitmaps_ready != 0;
         bm_mode       = (BMW == 0 && global_bm != nullptr && global_ready) ? 1 : 0;
@@ -132,11 +148,20 @@ struct FusedRow {
             window[i] = 0u;
         }
         __syncthreads();
-        for (int t = threadIdx.x; t < step; t += blockDim.x) {
-            if (history_position_counts(t)) {
-                const int id = history[(size_t)t * batch_size];
-                if (id >= lo && id < hi) {
-                    atomicOr(&window[(id - origin) >> 5], 1u << ((id - origin) & 31));
+        // the history is time-major: every id is a cache line of its own, so the reads are issued eight
+        // deep before the first one is used
+        constexpr int U = 8;
+        for (int t0 = threadIdx.x; t0 < step; t0 += U * blockDim.x) {
+            int ids[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * blockDim.x;
+                ids[u]      = (t < step && history_position_counts(t)) ? history[(size_t)t * batch_size] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (ids[u] >= lo && ids[u] < hi) {
+                    atomicOr(&window[(ids[u] - origin) >> 5], 1u << ((ids[u] - origin) & 31));
                 }
             }
         }
@@ -220,12 +245,38 @@ struct FusedRow {
     // interior column, no bias, not in the history, not the masked end id
     __device__ __forceinline__ float fast(float x) const
     {
-        return temp_active ? round_t<DT>(x * inv) : x;
+        return round_t<DT>(x * fast_mul);  // fast_mul is 1 without a temperature: exact, and x is a T already
     }
     // the same column when it is in the history
     __device__ __forceinline__ float flagged(float xf) const
     {
         return round_t<DT>(repetition_value(xf, penalty, penalty_type));
+    }
+    // Never below flagged(xf), without the division and without branches: for the multiplicative rule
+    // x * RN(1/p) * (1 + 2^-20) >= x / p for x >= 0 and a positive finite p (as real numbers, so also after
+    // the monotone roundings); x < 0 and the additive rule are the exact operation. Rows whose penalty has
+    // no usable reciprocal report +inf, which sends every flagged column to the exact evaluation.
+    __device__ __forceinline__ float flagged_upper(float xf) const
+    {
+        const float y = round_t<DT>(xf * (xf < 0.0f ? up_mul_neg : up_mul_pos) + up_add);
+        return up_ok ? y : __builtin_inff();
+    }
+    // flags of the NVT vectors a thread owns in one tile (first column first0, `stride` columns apart),
+    // EPV bits each; requires (first0 - bm_origin) to be a multiple of EPV
+    template<int EPV, int NVT>
+    __device__ __forceinline__ void tile_bits(int first0, int stride, uint32_t* packed) const
+    {
+        constexpr int PW = NVT * EPV / 32;
+#pragma unroll
+        for (int i = 0; i < PW; ++i) {
+            packed[i] = 0u;
+        }
+#pragma unroll
+        for (int it = 0; it < NVT; ++it) {
+            const int      rel = first0 + it * stride - bm_origin;
+            const uint32_t b   = (bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
+            packed[(it * EPV) >> 5] |= b << ((it * EPV) & 31);
+        }
     }
     // the value top-k would see for column v: temperature(+bias) -> history penalty -> min-length mask
     // -> pad mask, each rounded to T where the reference stores T
@@ -328,7 +379,7 @@ __device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch
 }
 
 template<int DT, int BMW>
-__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? 4 : 3)
+__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
 fused_row_kernel(FusedParams p, FusedLaunch l)
 {
     __shared__ TopkShared s;
@@ -344,9 +395,11 @@ fused_row_kernel(FusedParams p, FusedLaunch l)
     }
     const int    k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
     const float  tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
+    FTK_PHASE_BEGIN();
     const float  u  = fused_row_draw(s, l, row);
     const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row);
     FusedRow<DT, BMW> r(p, row);
+    FTK_PHASE(0);
     uint32_t     thr = 0u;
     const int    n   = topk_stream<DT>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
     topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, l.entries + (size_t)row * l.row_entries, false, u,
@@ -354,7 +407,7 @@ fused_row_kernel(FusedParams p, FusedLaunch l)
 }
 
 template<int DT, int BMW>
-__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? 4 : 3)
+__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
 fused_gather_kernel(FusedParams p, FusedLaunch l)
 {
     __shared__ TopkShared s;
@@ -437,6 +490,18 @@ struct ScopedKernelTime {
     }
 };
 }  // namespace
+
+#ifdef FTK_PHASE_TIMING
+extern "C" int ftk_debug_read_phases_fused(unsigned long long* out, int reset)
+{
+    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ftk_phase), sizeof(unsigned long long) * 32);
+    if (e == hipSuccess && reset) {
+        unsigned long long z[32] = {};
+        e = hipMemcpyToSymbol(HIP_SYMBOL(g_ftk_phase), z, sizeof(z));
+    }
+    return (int)e;
+}
+#endif
 
 extern "C" int ftk_profile_enable(int max_launches)
 {
