@@ -62,6 +62,10 @@ _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_c
              "ftk_test_set_topp_force_deep": None, "ftk_host_philox4x32_10": None}
 
 
+# error codes of include/ftk_sampling.h (positive values are hipError_t)
+FTK_ERR_DTYPE, FTK_ERR_TOPK_DOMAIN, FTK_ERR_ARGUMENT, FTK_ERR_WORKSPACE = -1, -2, -3, -4
+
+
 def exported_symbols():
     """names every entry point include/ftk_sampling.h declares"""
     return sorted(_SIGNATURES)

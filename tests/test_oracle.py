@@ -1,0 +1,600 @@
+"""Pins the CPU oracle (oracle/ft_oracle.cc) without a GPU: against the reference's known-answer sets, against
+closed forms evaluated independently in float64 / numpy / torch, and against a literal thread-by-thread
+simulation of the reference's two-stage top-k written from its source description.
+
+Every function the GPU parity tests lean on has a check here that a plausible mistake (a wrong sign, a
+swapped operand, a dropped term, a different tie rule) would fail.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import ft_oracle as O
+from decode_harness import Case, OracleRunner
+from helpers import DTYPE_NAMES, DTYPES, make_word_list, uniforms
+
+KAT = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "sampling_layer_kat.json")))
+FLT_MAX = np.finfo(np.float32).max
+
+
+# ---- elementary functions and storage conversions ------------------------------------------------
+def test_expf_logf_against_float64():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.uniform(-87, 88, 20000), rng.uniform(-1, 1, 20000), [0.0, -0.0, 1.0, -1.0]])
+    x = x.astype(np.float32)
+    got = O.expf(x)
+    ref = np.exp(x.astype(np.float64))
+    assert np.max(np.abs(got - ref) / ref) < 2.5e-7
+    assert O.expf(np.array([0.0], np.float32))[0] == 1.0
+    assert O.expf(np.array([-np.inf], np.float32))[0] == 0.0
+    assert O.expf(np.array([-200.0], np.float32))[0] == 0.0
+    y = np.concatenate([np.exp(rng.uniform(-80, 80, 20000)), rng.uniform(0.5, 2.0, 20000), [1.0]]).astype(np.float32)
+    got = O.logf(y)
+    ref = np.log(y.astype(np.float64))
+    err = np.abs(got - ref)
+    assert np.max(err / np.maximum(np.abs(ref), 1e-3)) < 3e-7
+    assert O.logf(np.array([1.0], np.float32))[0] == 0.0
+    assert O.logf(np.array([0.0], np.float32))[0] == -np.inf
+
+
+def test_storage_conversions_against_numpy_and_torch():
+    import torch
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(50000) * 10, rng.standard_normal(20000) * 1e-6,
+                        rng.standard_normal(20000) * 6e4, [0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 6e-8, 3e38,
+                                                           -3.4e38, np.inf, -np.inf]]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        ref16 = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(O.to_storage(x, O.F16).view(np.uint16), ref16)
+    refbf = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(O.to_storage(x, O.BF16), refbf)
+    # widening is exact
+    assert np.array_equal(O.to_f32(ref16.view(np.float16), O.F16), ref16.view(np.float16).astype(np.float32))
+    assert np.array_equal(O.to_f32(refbf, O.BF16),
+                          torch.from_numpy(refbf.view(np.int16)).view(torch.bfloat16).float().numpy())
+
+
+# ---- the reference's known-answer sets --------------------------------------------------------------
+def _kat_logits(dt):
+    rows = [[-FLT_MAX if v == "-FLT_MAX" else v for v in row] for row in KAT["logits_per_step"]]
+    return [O.to_storage(np.tile(np.array(r, np.float32), (KAT["batch_size"], 1)), dt) for r in rows]
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("kat", KAT["cases"], ids=lambda c: c["name"])
+@pytest.mark.parametrize("logprobs", [True, False], ids=["logprobs", "plain"])
+def test_known_answer_sets(dt, kat, logprobs):
+    """tests/unittests/test_sampling_layer.cu:318-592: whatever the draw, the sampled id lies in the set."""
+    B, V = KAT["batch_size"], KAT["vocab_size"]
+    logits = _kat_logits(dt)
+    local = B // 3 if kat["use_local_batch"] else B
+    ite = 1 if kat["use_local_batch"] else 0
+    rng = np.random.default_rng(11)
+    for trial in range(30):
+        c = Case(dt, B, V, V, gen_len=3, local_batch=local, runtime_top_k=kat["top_k"], runtime_top_p=kat["top_p"],
+                 end_ids=np.full(B, KAT["end_id"], np.int32), with_finished=False, with_seq_len=False,
+                 with_cum=logprobs, with_out_lp=logprobs)
+        o = OracleRunner(c)
+        for step in range(3):
+            u = uniforms(rng, B)
+            if trial == 0:
+                u[:] = 1.0  # the largest draw curand_uniform can return
+            if trial == 1:
+                u[:] = np.float32(2.0 ** -32)
+            o.step(step, logits[step], u, ite=ite)
+        ids = o.snapshot()["output_ids"]
+        rows = range(ite * local, ite * local + local)
+        for step in range(3):
+            for b in rows:
+                assert int(ids[step, b]) in kat["expected"][step][b], (kat["name"], trial, step, b)
+
+
+# ---- top-k: literal simulation of the two-stage scheme --------------------------------------------------
+def _block_reduce_top1(cands):
+    """cub::BlockReduce over (value, id) pairs with the reference's `a.u > b.u ? a : b`
+    (reduce_kernel_utils.cuh:345-348): 32-lane shuffle-down trees (the lower lane is the left operand,
+    warp_reduce_shfl.cuh:389-401), then warps folded in ascending order
+    (block_reduce_warp_reductions.cuh:113-125)."""
+    def comb(a, b):
+        return a if a[0] > b[0] else b
+    warps = []
+    for w in range(len(cands) // 32):
+        lanes = list(cands[32 * w:32 * w + 32])
+        for off in (1, 2, 4, 8, 16):
+            new = list(lanes)
+            for lane in range(32):
+                if lane + off < 32:
+                    new[lane] = comb(lanes[lane], lanes[lane + off])
+            lanes = new
+        warps.append(lanes[0])
+    agg = warps[0]
+    for w in warps[1:]:
+        agg = comb(agg, w)
+    return agg
+
+
+def _simulate_reference_topk(row, k, max_top_k):
+    """sampling_topk_kernels.cu:130-280 for one fp32 row: returns the ordered candidate list [(id, value)]."""
+    V = len(row)
+    bs1 = 128 if max_top_k <= 16 else 256
+    bs2 = 128 if max_top_k <= 32 else 256
+    tmp = np.array(row, np.float32).copy()
+    neg = np.float32(-FLT_MAX)
+    ids = np.full(8 * k, -1, np.int64)
+    vals = np.full(8 * k, neg, np.float32)
+    for block in range(8):
+        for ite in range(k):
+            cands = []
+            for tid in range(bs1):
+                u, p = neg, -1
+                for e in range(tid + block * bs1, V, bs1 * 8):
+                    if tmp[e] > u:
+                        u, p = tmp[e], e
+                cands.append((u, p))
+            u, p = _block_reduce_top1(cands)
+            ids[block * k + ite] = p
+            vals[block * k + ite] = u
+            if p >= 0:
+                tmp[p] = neg
+    out = []
+    s_val = vals.copy()
+    for ite in range(k):
+        cands = []
+        for tid in range(bs2):
+            u, p = neg, -1
+            for i in range(tid, 8 * k, bs2):
+                if s_val[i] > u:
+                    u, p = s_val[i], i
+            cands.append((u, p))
+        u, p = _block_reduce_top1(cands)
+        if p < 0:
+            break
+        out.append((int(ids[p]), float(u)))
+        s_val[p] = neg
+    return out
+
+
+def _oracle_topk_pick(row, k, max_top_k, u, p=1.0):
+    V = len(row)
+    lp = np.ascontiguousarray(np.asarray(row, np.float32).reshape(1, V))
+    ids = np.zeros(1, np.int32)
+    O.batch_topk_sampling(O.F32, lp, ids, None, None, None, None, np.array([u], np.float32), max_top_k,
+                          np.array([k], np.int32), p, None, V, np.array([V - 1], np.int32), 1, None)
+    return int(ids[0])
+
+
+@pytest.mark.parametrize("case", ["ties", "distinct", "few_valid", "two_values"])
+def test_topk_order_against_thread_level_simulation(case):
+    rng = np.random.default_rng({"ties": 3, "distinct": 4, "few_valid": 5, "two_values": 6}[case])
+    for trial in range(3):
+        V = int(rng.integers(300, 2600))
+        k = int(rng.integers(1, 7))
+        max_top_k = int(rng.choice([k, 16, 17, 32, 33, 64]))
+        max_top_k = max(max_top_k, k)
+        if case == "ties":
+            row = rng.integers(0, 4, V).astype(np.float32)
+        elif case == "two_values":
+            row = np.where(rng.random(V) < 0.02, 5.0, 1.0).astype(np.float32)
+        elif case == "few_valid":
+            row = np.full(V, -FLT_MAX, np.float32)
+            row[rng.choice(V, 3, replace=False)] = rng.standard_normal(3).astype(np.float32)
+            row[rng.integers(0, V)] = -np.inf
+        else:
+            row = rng.standard_normal(V).astype(np.float32)
+        order = _simulate_reference_topk(row, k, max_top_k)
+        assert len(order) >= 1
+        # draws that land in the middle of each position's share of the cumulative weight
+        x0 = order[0][1]
+        w = np.array([np.exp(np.float64(v) - np.float64(x0)) for _, v in order])
+        cum = np.concatenate([[0.0], np.cumsum(w)])
+        for j, (tok, _) in enumerate(order):
+            u = (cum[j] + 0.5 * w[j]) / cum[-1]
+            assert _oracle_topk_pick(row, k, max_top_k, np.float32(u)) == tok, (case, trial, j, order)
+
+
+def test_topk_set_is_the_k_largest_when_values_are_distinct():
+    rng = np.random.default_rng(8)
+    V, k = 5000, 37
+    row = rng.permutation(V).astype(np.float32) / 64.0
+    want = set(np.argsort(-row)[:k].tolist())
+    seen = set()
+    for u in np.linspace(1e-6, 1.0, 400):
+        seen.add(_oracle_topk_pick(row, k, 64, np.float32(u)))
+    assert seen <= want
+    assert _oracle_topk_pick(row, k, 64, np.float32(1e-9)) == int(np.argmax(row))
+    # all k positions are reachable when the weights are equal
+    flat = np.zeros(V, np.float32)
+    flat[rng.choice(V, k, replace=False)] = 1.0
+    got = {_oracle_topk_pick(flat, k, 64, np.float32((j + 0.5) / k)) for j in range(k)}
+    assert got == set(np.nonzero(flat)[0].tolist())
+
+
+def test_topk_inverse_cdf_and_logprobs_closed_form():
+    """sampling_topk_kernels.cu:264-311: r = u*p*S walked down the ordered list; log-prob outputs."""
+    rng = np.random.default_rng(9)
+    B, V, k = 64, 3000, 12
+    logits = (rng.standard_normal((B, V)) * 2).astype(np.float32)
+    top_p = 0.8
+    u = rng.random(B).astype(np.float32) * 0.98 + 0.01
+    # probabilities in, as the layer does when log-probs are requested
+    m = logits.max(axis=1, keepdims=True).astype(np.float64)
+    e = np.exp(logits.astype(np.float64) - m)
+    probs = (e / (e.sum(axis=1, keepdims=True) + 1e-6)).astype(np.float32)
+    ids = np.zeros(B, np.int32)
+    cum = np.zeros(B, np.float32)
+    out = np.zeros(B, np.float32)
+    seq = np.full(B, 5, np.int32)
+    fin = np.zeros(B, np.bool_)
+    end = rng.integers(0, V, B).astype(np.int32)
+    O.batch_topk_sampling(O.F32, probs, ids, seq, fin, cum, out, u, k, np.full(B, k, np.int32), top_p, None, V, end,
+                          B, None)
+    mismatch = 0
+    for b in range(B):
+        order = np.argsort(-probs[b].astype(np.float64), kind="stable")[:k]
+        w = probs[b][order].astype(np.float64)
+        r = np.float64(u[b]) * top_p * w.sum()
+        j = int(np.searchsorted(np.cumsum(w), r, side="left"))
+        j = min(j, k - 1)
+        if ids[b] != order[j]:
+            mismatch += 1  # a draw within rounding of a boundary may fall either way
+            assert abs(int(np.nonzero(order == ids[b])[0][0]) - j) == 1
+            continue
+        np.testing.assert_allclose(cum[b], np.log(w[j]), rtol=2e-6, atol=1e-6)
+        np.testing.assert_allclose(out[b], np.log(w[j]) - np.log(w.sum()), rtol=2e-6, atol=2e-6)
+    assert mismatch <= 1
+    assert np.array_equal(seq, np.full(B, 6, np.int32))
+    assert np.array_equal(fin, ids == end)
+
+
+def test_topk_finished_and_skipped_rows():
+    B, V = 4, 100
+    rng = np.random.default_rng(10)
+    lp = rng.standard_normal((B, V)).astype(np.float32)
+    ids = np.full(B, -7, np.int32)
+    seq = np.full(B, 3, np.int32)
+    fin = np.array([False, True, False, True])
+    skip = np.array([False, False, True, True])
+    end = np.array([9, 8, 7, 6], np.int32)
+    O.batch_topk_sampling(O.F32, lp, ids, seq, fin, None, None, np.full(B, 0.5, np.float32), 1,
+                          np.full(B, 1, np.int32), 1.0, None, V, end, B, skip)
+    assert ids[0] == int(np.argmax(lp[0])) and seq[0] == 4
+    assert ids[1] == 8 and seq[1] == 3 and fin[1]          # finished: end id, nothing else moves
+    assert ids[2] == -7 and ids[3] == -7 and seq[2] == 3   # skipped rows are untouched
+
+
+# ---- penalties ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_temperature_closed_form(dt, with_bias):
+    """sampling_penalty_kernels.cu:134-146 / :171-177, and the reference test's own expectation
+    (tests/unittests/test_penalty_kernels.cu:188-208: (logit + bias) / temperature within tolerance)."""
+    rng = np.random.default_rng(12)
+    B, V, Vp = 6, 50, 56
+    x = O.to_storage((rng.standard_normal((B, Vp)) * 3).astype(np.float32), dt)
+    bias = O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt) if with_bias else None
+    temps = rng.uniform(0.5, 2.0, B).astype(np.float32)
+    got = x.copy()
+    O.batch_apply_temperature_penalty(dt, got, bias, temps, B, V, Vp)
+    gf = O.to_f32(got, dt)
+    xf = O.to_f32(x, dt).astype(np.float64)
+    bf = O.to_f32(bias, dt).astype(np.float64) if with_bias else np.zeros(Vp)
+    want = (xf + bf) / temps[:, None].astype(np.float64)
+    tol = {O.F32: 1e-5, O.F16: 4e-3, O.BF16: 2e-2}[dt]
+    np.testing.assert_allclose(gf[:, :V], want[:, :V], rtol=tol, atol=tol)
+    if dt == O.F16:
+        assert np.array_equal(got[:, V:], x[:, V:])  # the half2 kernel leaves pad columns alone (V, Vp even)
+    else:
+        assert np.all(gf[:, V:] == -O.max_t(dt))
+    if dt == O.F32:
+        # operation by operation in float32: bit-exact
+        inv = (np.float32(1.0) / (temps + np.float32(1e-6))).astype(np.float32)
+        step = O.to_f32(x, dt)[:, :V]
+        if with_bias:
+            step = (step + O.to_f32(bias, dt)[None, :V]).astype(np.float32)
+        step = (step * inv[:, None]).astype(np.float32)
+        assert np.array_equal(gf[:, :V].view(np.uint32), step.view(np.uint32))
+
+
+def _reference_repetition(x, ids_col, penalty, multiplicative, input_length, max_input_length):
+    """the reference test's host expectation (tests/unittests/test_penalty_kernels.cu:58-119), in float64"""
+    y = x.astype(np.float64).copy()
+    seen = set()
+    for t, tok in enumerate(ids_col):
+        if input_length <= t < max_input_length:
+            continue
+        tok = int(tok)
+        if tok in seen:
+            continue
+        seen.add(tok)
+        v = float(x[tok])
+        y[tok] = (v * penalty if v < 0 else v / penalty) if multiplicative else v - penalty
+    return y
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("multiplicative", [True, False])
+def test_repetition_penalty_closed_form(dt, multiplicative):
+    rng = np.random.default_rng(13)
+    B, V, step, max_in = 5, 40, 30, 12
+    x = O.to_storage((rng.standard_normal((B, V)) * 2).astype(np.float32), dt)
+    out_ids = rng.integers(0, V, (step, B)).astype(np.int32)
+    out_ids[3] = out_ids[7]                      # repeated tokens are penalised once
+    input_lengths = rng.integers(4, max_in + 1, B).astype(np.int32)
+    pens = rng.uniform(1.1, 2.0, B).astype(np.float32) if multiplicative else rng.uniform(0.1, 2.0, B).astype(np.float32)
+    got = x.copy()
+    O.batch_apply_repetition_penalty(dt, got, pens, out_ids, B, B, V, input_lengths, max_in, step,
+                                     O.PEN_MULTIPLICATIVE if multiplicative else O.PEN_ADDITIVE)
+    gf = O.to_f32(got, dt)
+    xf = O.to_f32(x, dt)
+    tol = {O.F32: 1e-6, O.F16: 2e-3, O.BF16: 1.6e-2}[dt]
+    for b in range(B):
+        want = _reference_repetition(xf[b], out_ids[:, b], float(pens[b]), multiplicative, int(input_lengths[b]),
+                                     max_in)
+        np.testing.assert_allclose(gf[b], want, rtol=tol, atol=tol)
+        untouched = np.ones(V, bool)
+        hist = [int(t) for i, t in enumerate(out_ids[:, b]) if not (input_lengths[b] <= i < max_in)]
+        untouched[hist] = False
+        assert np.array_equal(got[b][untouched], x[b][untouched])
+
+
+def test_frequency_penalty_reduces_to_presence():
+    """extension (no reference code): with frequency 0 it must equal the additive penalty bit for bit"""
+    rng = np.random.default_rng(14)
+    B, V, step = 4, 64, 40
+    for dt in DTYPES:
+        x = O.to_storage((rng.standard_normal((B, V)) * 2).astype(np.float32), dt)
+        out_ids = rng.integers(0, V, (step, B)).astype(np.int32)
+        pres = rng.uniform(0.1, 1.0, B).astype(np.float32)
+        a, b = x.copy(), x.copy()
+        O.batch_apply_repetition_penalty(dt, a, pres, out_ids, B, B, V, None, 0, step, O.PEN_ADDITIVE)
+        O.batch_apply_frequency_penalty(dt, b, pres, np.zeros(B, np.float32), out_ids, B, B, V, None, 0, step)
+        assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+        # and with a frequency term: x - presence - frequency * count, in float64
+        freq = rng.uniform(0.1, 0.5, B).astype(np.float32)
+        c = x.copy()
+        O.batch_apply_frequency_penalty(dt, c, pres, freq, out_ids, B, B, V, None, 0, step)
+        xf, cf = O.to_f32(x, dt).astype(np.float64), O.to_f32(c, dt)
+        for r in range(B):
+            counts = np.bincount(out_ids[:, r], minlength=V)
+            want = np.where(counts > 0, xf[r] - pres[r] - freq[r] * counts, xf[r])
+            tol = {O.F32: 1e-6, O.F16: 2e-3, O.BF16: 1.6e-2}[dt]
+            np.testing.assert_allclose(cf[r], want, rtol=tol, atol=tol)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_min_length_and_end_mask(dt):
+    rng = np.random.default_rng(15)
+    B, V, Vp, max_in = 6, 30, 32, 4
+    x = O.to_storage(rng.standard_normal((B, Vp)).astype(np.float32), dt)
+    end = rng.integers(0, V, B).astype(np.int32)
+    seq = np.array([3, 4, 5, 6, 7, 8], np.int32)
+    min_len = np.array([3, 3, 3, 3, 3, 3], np.int32)
+    got = x.copy()
+    O.min_length_penalty(dt, got, min_len, end, seq, max_in, B, Vp)
+    gf = O.to_f32(got, dt)
+    for b in range(B):
+        masked = seq[b] + 1 - max_in < min_len[b]   # sampling_penalty_kernels.cu:493-499
+        assert (gf[b, end[b]] == -O.max_t(dt)) == masked
+        keep = np.ones(Vp, bool)
+        keep[end[b]] = False
+        assert np.array_equal(got[b][keep], x[b][keep])
+    fin = np.array([False, True, False, True, False, False])
+    got = x.copy()
+    O.add_bias_end_mask(dt, got, None, end, fin, B, V, Vp)
+    gf = O.to_f32(got, dt)
+    for b in range(B):
+        assert np.all(gf[b, V:] == -O.max_t(dt))
+        if fin[b]:
+            want = np.full(V, -O.max_t(dt), np.float32)
+            want[end[b]] = O.max_t(dt)
+            assert np.array_equal(gf[b, :V], want)
+        else:
+            assert np.array_equal(got[b, :V], x[b, :V])
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_softmax_closed_form(dt):
+    """sampling_topp_kernels.cu:1308-1344 against float64; the reference's own host check
+    (tests/unittests/test_sampling_kernels.cu:51-104) agrees to the same tolerance"""
+    rng = np.random.default_rng(16)
+    B, V, Vp = 5, 700, 704
+    x = O.to_storage((rng.standard_normal((B, Vp)) * 3).astype(np.float32), dt)
+    end = rng.integers(0, V, B).astype(np.int32)
+    fin = np.array([False, False, True, False, False])
+    got = x.copy()
+    O.add_bias_softmax(dt, got, None, end, fin, B, Vp, V)
+    gf = O.to_f32(got, dt).astype(np.float64)
+    xf = O.to_f32(x, dt).astype(np.float64)
+    tol = {O.F32: 2e-6, O.F16: 2e-3, O.BF16: 1.6e-2}[dt]
+    for b in range(B):
+        assert np.all(gf[b, V:] == 0.0)
+        if fin[b]:
+            assert abs(gf[b, end[b]] - 1.0) < 4e-3 and np.count_nonzero(gf[b]) == 1
+            continue
+        e = np.exp(xf[b, :V] - xf[b, :V].max())
+        want = e / (e.sum() + 1e-6)
+        np.testing.assert_allclose(gf[b, :V], want, rtol=tol, atol=1e-7 if dt == O.F32 else 1e-4)
+        assert abs(gf[b].sum() - 1.0) < (1e-4 if dt == O.F32 else 3e-2)
+
+
+# ---- top-p ----------------------------------------------------------------------------------------------
+def _oracle_topp(probs, u, top_p, end=None):
+    B, V = probs.shape
+    ids = np.full(B, -1, np.int32)
+    seq = np.zeros(B, np.int32)
+    fin = np.zeros(B, np.bool_)
+    cum = np.zeros(B, np.float32)
+    out = np.zeros(B, np.float32)
+    end = np.full(B, V - 1, np.int32) if end is None else end
+    O.batch_topp_sampling(O.F32, np.ascontiguousarray(probs, np.float32), ids, seq, fin, cum, out,
+                          np.asarray(u, np.float32), B, V, end, 0.0, np.asarray(top_p, np.float32), None)
+    return ids, seq, fin, cum, out
+
+
+def test_topp_exact_cases():
+    """probabilities that are exact in binary make every comparison of the walk exact
+    (sampling_topp_kernels.cu:958-1003): stable descending order, first i with r <= c_i"""
+    probs = np.array([[0.25, 0.25, 0.25, 0.25],        # ties keep ascending id order
+                      [0.125, 0.5, 0.125, 0.25],
+                      [0.125, 0.5, 0.125, 0.25],
+                      [0.125, 0.5, 0.125, 0.25],
+                      [0.125, 0.5, 0.125, 0.25]], np.float32)
+    p = np.array([1.0, 1.0, 1.0, 1.0, 0.5], np.float32)
+    u = np.array([0.5, 0.5, 0.75, 0.875, 0.99], np.float32)
+    ids, seq, fin, cum, out = _oracle_topp(probs, u, p)
+    # row 0: r = 0.5 -> c = .25, .5 -> second entry of the stable order -> id 1
+    # row 1: order 1,3,0,2 with c = .5,.75,.875,1; r = .5 -> id 1
+    # row 2: r = .75 -> id 3;  row 3: r = .875 -> id 0
+    # row 4: max prob 0.5 >= p = 0.5 -> arg-max shortcut whatever the draw
+    assert ids.tolist() == [1, 1, 3, 0, 1]
+    assert np.allclose(cum, np.log([0.25, 0.5, 0.25, 0.125, 0.5]))
+    assert np.array_equal(cum, out)          # no renormalisation for top-p (:986-990)
+    assert seq.tolist() == [1, 1, 1, 1, 1]
+    assert fin.tolist() == [False, False, True, False, False]
+
+
+def test_topp_nucleus_property_random_rows():
+    rng = np.random.default_rng(17)
+    B, V = 48, 2000
+    x = rng.standard_normal((B, V)) * 2.5
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    probs = (e / e.sum(axis=1, keepdims=True)).astype(np.float32)
+    p = rng.uniform(0.3, 0.99, B).astype(np.float32)
+    u = (rng.random(B) * 0.98 + 0.01).astype(np.float32)
+    ids, _, _, cum, _ = _oracle_topp(probs, u, p)
+    for b in range(B):
+        pr = probs[b].astype(np.float64)
+        order = np.argsort(-pr, kind="stable")
+        if pr[order[0]] >= p[b]:
+            assert ids[b] == order[0]
+            continue
+        c = np.cumsum(pr[order])
+        r = np.float64(u[b]) * np.float64(p[b])
+        j = int(np.searchsorted(c, r, side="left"))
+        pos = int(np.nonzero(order == ids[b])[0][0])
+        assert abs(pos - j) <= 1 and (pos == j or abs(c[min(pos, j)] - r) < 1e-5)
+        np.testing.assert_allclose(cum[b], np.log(pr[ids[b]]), rtol=1e-5, atol=1e-6)
+
+
+def test_topp_decay_closed_form():
+    n = 7
+    initial = np.linspace(0.5, 0.95, n).astype(np.float32)
+    runtime = (initial * 0.8).astype(np.float32)
+    decay = np.full(n, 0.9, np.float32)
+    pmin = np.full(n, 0.45, np.float32)
+    reset = np.array([5, 5, -1, 5, 5, 5, 5], np.int32)
+    ids = np.array([5, 4, 5, 5, 0, 1, 2], np.int32)
+    want = np.where(ids == reset, initial, np.maximum((runtime * decay).astype(np.float32), pmin))
+    O.compute_topp_decay(runtime, initial, ids, decay, pmin, reset, n)
+    assert np.array_equal(runtime, want.astype(np.float32))
+
+
+# ---- word lists and stop criteria -------------------------------------------------------------------------
+def _words(word_list):
+    ids, offs = word_list
+    out, start = [], 0
+    for o in offs:
+        if o < 0:
+            break
+        out.append([int(t) for t in ids[start:o]])
+        start = o
+    return out
+
+
+def test_bad_words_against_brute_force():
+    rng = np.random.default_rng(18)
+    B, V, step = 6, 50, 9
+    history = rng.integers(1, V, (step + 1, B)).astype(np.int32)
+    for shared in (True, False):
+        lists = []
+        for b in range(1 if shared else B):
+            wl, _ = make_word_list(rng, 10, 4, V, L=48, history=history, step=step - 1, row=b)
+            lists.append(wl)
+        bad = np.ascontiguousarray(lists[0] if shared else np.stack(lists))
+        for dt in DTYPES:
+            x = O.to_storage(rng.standard_normal((B, V)).astype(np.float32), dt)
+            got = x.copy()
+            O.ban_bad_words(dt, got, history, B, B, bad, shared, bad.shape[-1], 0, V, step)
+            gf, xf = O.to_f32(got, dt), O.to_f32(x, dt)
+            for b in range(B):
+                banned = set()
+                for w in _words(lists[0] if shared else lists[b]):
+                    n = len(w)
+                    if n == 0:
+                        continue
+                    ok = n == 1 or (step >= n - 1 and all(history[step - (n - 1) + t, b] == w[t] for t in range(n - 1)))
+                    if ok and 0 < w[-1] < V:
+                        banned.add(w[-1])
+                for v in range(V):
+                    if v in banned:
+                        assert gf[b, v] == -np.inf
+                    else:
+                        assert gf[b, v] == xf[b, v]
+
+
+def test_stop_words_and_length_against_brute_force():
+    rng = np.random.default_rng(19)
+    B, V, step = 8, 30, 7
+    history = rng.integers(1, V, (step + 1, B)).astype(np.int32)
+    lists = []
+    for b in range(B):
+        wl, words = make_word_list(rng, 6, 3, V, L=24)
+        lists.append(wl)
+    # plant matches: row 1 ends with its first word, row 4 with its second
+    for b, wi in ((1, 0), (4, 1)):
+        w = _words(lists[b])[wi]
+        history[step - len(w) + 1:step + 1, b] = w
+    stop = np.ascontiguousarray(np.stack(lists))
+    fin = np.zeros(B, np.bool_)
+    O.stop_words_criterion(history, stop, fin, 0, stop.shape[-1], B, B, step)
+    for b in range(B):
+        want = any(step + 1 >= len(w) and len(w) > 0
+                   and all(history[step - (len(w) - 1) + t, b] == w[t] for t in range(len(w)))
+                   for w in _words(lists[b]))
+        assert fin[b] == want
+    assert fin[1] and fin[4]
+    limit = np.array([3, 8, 7, 100, 6, 7, 8, 9], np.uint32)
+    fin2 = np.array([False, False, False, True, False, False, False, False])
+    should = np.zeros(1, np.bool_)
+    O.length_criterion(fin2, should, limit, B, step)
+    assert fin2.tolist() == [True, False, True, True, True, True, False, False] and not should[0]
+    O.length_criterion(fin2, should, np.zeros(B, np.uint32), B, step)
+    assert fin2.all() and should[0]
+
+
+# ---- the layer restatement: routing of (k, p) and the reference's Python known answers ------------------------
+def test_python_known_answers_repetition_and_min_length():
+    """tests/unittests/th_op/test_th_decode_op.py:233-324: with logits 2 / 1.8 / 1.6 on the last three ids and
+    greedy decoding, a repetition penalty of 2 (or presence 0.5 / 1.0) must produce v-1, v-2, v-3, v-1, v-1;
+    with the end id made the most probable token, min_length must hold generation open."""
+    V = 1024
+    for B, kwargs in [(4, dict(repetition_penalty=[2.0])), (256, dict(repetition_penalty=[2.0])),
+                      (4, dict(presence_penalty=[0.5])), (4, dict(presence_penalty=[1.0]))]:
+        H = 4
+        x = np.zeros((B, V), np.float32)
+        x[:, V - 1], x[:, V - 2], x[:, V - 3] = 2.0, 1.8, 1.6
+        c = Case(O.F32, B, V, V, max_input_length=H, gen_len=5, runtime_top_k=[1], runtime_top_p=[0.0],
+                 end_ids=np.zeros(B, np.int32), prompt=np.ones((H, B), np.int32),
+                 input_lengths=np.full(B, H, np.int32), **kwargs)
+        o = OracleRunner(c)
+        for i in range(5):
+            o.step(H + i, x, np.full(B, 0.5, np.float32))
+        ids = o.snapshot()["output_ids"][H:]
+        expect = np.array([V - 1, V - 2, V - 3, V - 1, V - 1], np.int32)
+        assert (ids == expect[:, None]).all(), kwargs
+    rng = np.random.default_rng(0)
+    for method in (dict(runtime_top_k=[1], runtime_top_p=[0.0]), dict(runtime_top_k=[0], runtime_top_p=[0.8])):
+        for B, H, min_len, gen in [(4, 4, 2, 4), (4, 4, 32, 40), (64, 6, 4, 8)]:
+            c = Case(O.F32, B, V, V, max_input_length=H, gen_len=gen, min_length=[min_len],
+                     end_ids=np.zeros(B, np.int32), prompt=rng.integers(1, V, (H, B)).astype(np.int32), **method)
+            o = OracleRunner(c)
+            for i in range(gen):
+                x = rng.standard_normal((B, V)).astype(np.float32)
+                x[:, 0] = x.max(axis=1) + 1  # end id is the most probable token
+                o.step(H + i, x, uniforms(rng, B))
+            snap = o.snapshot()
+            assert ((snap["sequence_length"] + 1) >= H + min_len).all(), (method, B, min_len)
+            if method["runtime_top_k"] == [1]:
+                assert snap["finished"].all()  # greedy: it does stop as soon as it is allowed to
