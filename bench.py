@@ -22,6 +22,9 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel on the headline workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script scaled by a copy kernel of known size (profiles/); None until measured
+TRAFFIC_BYTES_PER_LAUNCH = None
 
 WORKLOADS = {
     # the configuration the metric is quoted on (BASELINE.json "metric" / north-star target)
@@ -102,11 +105,13 @@ def run_gpu(name, w, steps, warmup, nbuf=4):
     alg = algorithmic_bytes(w, mid_step)
     gather_ms = kernel_ms[1]
     achieved = alg / (gather_ms * 1e-3) / 1e9 if gather_ms > 0 else 0.0
+    # batches of at least 1024 rows run the one-launch row kernel; smaller ones stream, then select
+    dominant = "fused_gather_kernel" if kernel_ms[2] > 0 else "fused_row_kernel"
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
         kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2]),
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                      traffic=None, kernel="fused_gather_kernel", algorithmic_bytes_per_launch=alg),
+                      traffic=TRAFFIC_BYTES_PER_LAUNCH, kernel=dominant, algorithmic_bytes_per_launch=alg),
         step_gbs=alg / (gpu_ms / steps * 1e-3) / 1e9,
         sampled_ids_checksum=int(output_ids[H + warmup:H + total].to(torch.int64).sum().item()),
     )
@@ -122,23 +127,27 @@ def run_cpu_baseline(w, budget_s=12.0):
     rng = np.random.default_rng(99)
     layer = O.OracleDynamicDecodeLayer(dt, V, Vp)
     layer.setup(rows, [w["top_k"]], [w["top_p"]], [w["temperature"]], [w["repetition_penalty"]])
-    out_ids = np.zeros((H + 64, rows), np.int32)
+    max_steps = 4096
+    out_ids = np.zeros((H + max_steps + 1, rows), np.int32)
     out_ids[:H] = rng.integers(0, V, (H, rows))
     finished = np.zeros(rows, np.bool_)
     seq = np.full(rows, H - 1, np.int32)
     end = np.full(rows, V - 1, np.int32)
+    # a few logits batches generated up front and reused, so that the loop times the oracle and nothing else
+    batches = [O.to_storage((rng.standard_normal((rows, Vp)) * w["sigma"]).astype(np.float32), dt) for _ in range(4)]
     done, spent, step = 0, 0.0, H
-    while spent < budget_s and step < H + 63:
-        logits = O.to_storage((rng.standard_normal((rows, Vp)) * w["sigma"]).astype(np.float32), dt)
+    while spent < budget_s and step < H + max_steps:
+        logits = batches[(step - H) % len(batches)].copy()
         u = rng.random(rows).astype(np.float32) * 0.999 + 0.001
+        finished[:] = False
         t0 = time.perf_counter()
         layer.forward(logits, end, out_ids, step, H, u, finished=finished, sequence_length=seq)
         spent += time.perf_counter() - t0
         done += rows
         step += 1
     return dict(value=done / spent, unit="tokens/s", cores=1, kind="port",
-                sample="%d rows of the same step (%d decode steps of a %d-row batch), %.1f s of CPU time"
-                       % (done, step - H, rows, spent))
+                sample="%d rows of the same workload (%d decode steps of a %d-row batch, V=%d), %.1f s of CPU time"
+                       % (done, step - H, rows, V, spent))
 
 
 def main():
@@ -147,6 +156,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run five plain device copies of 128 MiB, the known-size kernel that FETCH_SIZE / "
+                         "WRITE_SIZE counter readings are scaled by")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (rows shard across GPUs with no "
@@ -155,6 +167,13 @@ def main():
     name = next(iter(WORKLOADS))
     w = WORKLOADS[name]
     r = run_gpu(name, w, a.steps, a.warmup)
+    if a.copy_calibration:
+        import torch
+        src = torch.empty(128 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     line = {
         "metric": "sampled tokens/s, decode step B=256 V=128256 (full top-k+top-p+penalty DynamicDecodeLayer step)",
         "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

@@ -600,6 +600,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         }
     }
     FTK_PHASE(2);
+    thr         = (uint32_t)__builtin_amdgcn_readfirstlane((int)thr);  // uniform: keep it in a scalar register
     float thr_f = key_to_float(thr);  // x >= thr_f  <=>  order_key(x) >= thr (NaN fails both)
     // The first tile is examined a second time below. Keep the compiler from carrying the converted
     // values of the first pass along in registers: make the tile opaque here (no instructions).

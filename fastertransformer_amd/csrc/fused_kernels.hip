@@ -63,6 +63,11 @@ __device__ __forceinline__ uint32_t* fused_lds_bitmap()
 // BMW > 0: the history bitmap is a window of BMW words in LDS, built by prepare().
 // BMW == 0: whole-row bitmaps in global memory (built by history_bitmap_kernel, or by
 //           prepare_whole_row() for the literal replay).
+__device__ __forceinline__ float uniform_f(float x)
+{
+    return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x)));
+}
+
 template<int DT, int BMW>
 struct FusedRow {
     static constexpr int  LDS_WORDS = BMW > 0 ? BMW : 1;
@@ -121,6 +126,14 @@ struct FusedRow {
         step          = p.step;
         max_input_length = p.max_input_length;
         input_length  = p.input_lengths != nullptr ? p.input_lengths[row] : p.max_input_length;
+        // values that are the same for every lane of the workgroup but come out of floating-point
+        // arithmetic: move them to scalar registers, they stay live for the whole kernel
+        inv        = uniform_f(inv);
+        fast_mul   = uniform_f(fast_mul);
+        penalty    = uniform_f(penalty);
+        up_mul_neg = uniform_f(up_mul_neg);
+        up_mul_pos = uniform_f(up_mul_pos);
+        up_add     = uniform_f(up_add);
         masked_end_id = -1;
         if (p.min_lengths != nullptr
             && min_length_masks(p.sequence_length_in[row], p.max_input_length, p.min_lengths[row])) {
