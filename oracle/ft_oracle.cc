@@ -17,11 +17,21 @@
 //  * bfloat16 storage and the frequency penalty have no reference code ("parity unpinned");
 //    they follow the generic `T` branches with fp32 arithmetic and one rounding per store.
 //
-// Pinning: tests/test_oracle_*.py check this file against the reference tests' known-answer id
-// sets (tests/unittests/test_sampling_layer.cu:318-592), the Python KATs
-// (tests/unittests/th_op/test_th_decode_op.py:233-324), closed forms, numpy brute force on small
-// rows and float64 softmax. ban_bad_words / stop criteria / padding have no reference test and
-// are pinned by brute force only.
+// Pinning (tests/test_oracle.py, runs without a GPU):
+//  * whole layer: the reference tests' known-answer id sets
+//    (tests/unittests/test_sampling_layer.cu:318-592, 20 argument combinations x 3 dtypes) and the
+//    Python known answers (tests/unittests/th_op/test_th_decode_op.py:233-324);
+//  * top-k order and tie rule: a thread-by-thread Python simulation of topk_stage1 /
+//    topk_stage2_sampling and of the cub reduction trees, written from the reference sources;
+//    top-k set against numpy on distinct values; inverse CDF and log-probs against float64;
+//  * temperature, repetition / presence, min-length, end mask, softmax, top-p walk and decay:
+//    closed forms in float64 / exact binary cases; storage conversions against numpy and torch;
+//    det_expf / det_logf against float64;
+//  * ban_bad_words, stop words, length criterion: no reference test exists, pinned by brute force
+//    written from the source description only.
+//  PARITY UNPINNED (no reference code or no way to run it here): bfloat16 storage, the frequency
+//  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), and the last-ulp
+//  behaviour of __expf / logf (tolerance 1e-5 relative instead).
 //
 // Build: oracle/Makefile (g++ -O2 -ffp-contract=off).
 
