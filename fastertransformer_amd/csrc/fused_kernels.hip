@@ -12,6 +12,8 @@
 //                           are split over several workgroups
 //   history_bitmap_kernel - very large vocabularies only: turns the time-major token history into a
 //                           bitmap over the vocabulary (who gets the repetition / presence penalty)
+#include <hip/hip_ext.h>
+
 #include <vector>
 
 #include "ftk_sampling.h"
@@ -482,26 +484,20 @@ struct KernelTimer {
 KernelTimer g_timers[3];
 bool        g_profile = false;
 
-struct ScopedKernelTime {
-    KernelTimer* t  = nullptr;
-    hipStream_t  st = nullptr;
-    int          i  = -1;
-    ScopedKernelTime(int which, hipStream_t stream)
-    {
-        if (g_profile && g_timers[which].used < (int)g_timers[which].start.size()) {
-            t  = &g_timers[which];
-            st = stream;
-            i  = t->used++;
-            (void)hipEventRecord(t->start[i], st);
-        }
+// Launches `kernel`; when timing is on, the launch itself carries a start and a stop event, so the
+// pair brackets the kernel's execution and nothing else.
+template<typename K, typename... Args>
+void launch_timed(int which, K kernel, dim3 grid, dim3 block, hipStream_t st, Args... args)
+{
+    KernelTimer& t = g_timers[which];
+    if (g_profile && t.used < (int)t.start.size()) {
+        const int i = t.used++;
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, st, t.start[i], t.stop[i], 0, args...);
     }
-    ~ScopedKernelTime()
-    {
-        if (t != nullptr) {
-            (void)hipEventRecord(t->stop[i], st);
-        }
+    else {
+        hipLaunchKernelGGL(kernel, grid, block, 0, st, args...);
     }
-};
+}
 }  // namespace
 
 #ifdef FTK_PHASE_TIMING
@@ -646,8 +642,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
         }
         else {
-            ScopedKernelTime timer(0, st);
-            history_bitmap_kernel<<<rows, HB_THREADS, 0, st>>>(p.bitmaps, bitmap_words, a->output_ids, a->batch_size,
+            launch_timed(0, history_bitmap_kernel, dim3(rows), dim3(HB_THREADS), st, p.bitmaps, bitmap_words, a->output_ids, a->batch_size,
                                                                a->vocab_size_padded, a->input_lengths,
                                                                a->max_input_length, a->step, a->skip_decode,
                                                                a->finished);
@@ -670,42 +665,42 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     l.headers         = (TopkChunkHeader*)(ws + bitmap_bytes);
     l.entries         = (TopkEntry*)(l.headers + (size_t)rows * plan.splits);
     if (plan.splits == 1) {
-        ScopedKernelTime timer(1, st);
+        const dim3 grid1(rows), block(TK_THREADS);
         if (p.bitmaps_ready) {
-            FTK_DISPATCH_DTYPE(a->dtype,
-                               fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL><<<rows, TK_THREADS, 0, st>>>(p, l));
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>, grid1, block,
+                                                      st, p, l));
         }
         else if (p.lds_window == 2) {
-            FTK_DISPATCH_DTYPE(a->dtype,
-                               fused_row_kernel<DT, FUSED_BITMAP_WORDS_LARGE><<<rows, TK_THREADS, 0, st>>>(p, l));
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_LARGE>, grid1, block,
+                                                      st, p, l));
         }
         else {
-            FTK_DISPATCH_DTYPE(a->dtype,
-                               fused_row_kernel<DT, FUSED_BITMAP_WORDS_SMALL><<<rows, TK_THREADS, 0, st>>>(p, l));
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_SMALL>, grid1, block,
+                                                      st, p, l));
         }
         FTK_LAUNCH_CHECK();
         return 0;
     }
     dim3 grid(plan.splits, rows);
     {
-        ScopedKernelTime timer(1, st);
+        const dim3 block(TK_THREADS);
         if (p.bitmaps_ready) {
-            FTK_DISPATCH_DTYPE(a->dtype,
-                               fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL><<<grid, TK_THREADS, 0, st>>>(p, l));
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>, grid, block,
+                                                      st, p, l));
         }
         else if (p.lds_window == 2) {
-            FTK_DISPATCH_DTYPE(a->dtype,
-                               fused_gather_kernel<DT, FUSED_BITMAP_WORDS_LARGE><<<grid, TK_THREADS, 0, st>>>(p, l));
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_LARGE>, grid, block,
+                                                      st, p, l));
         }
         else {
-            FTK_DISPATCH_DTYPE(a->dtype,
-                               fused_gather_kernel<DT, FUSED_BITMAP_WORDS_SMALL><<<grid, TK_THREADS, 0, st>>>(p, l));
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_SMALL>, grid, block,
+                                                      st, p, l));
         }
     }
     FTK_LAUNCH_CHECK();
     {
-        ScopedKernelTime timer(2, st);
-        FTK_DISPATCH_DTYPE(a->dtype, fused_select_kernel<DT><<<rows, TK_THREADS, 0, st>>>(p, l));
+        FTK_DISPATCH_DTYPE(a->dtype,
+                           launch_timed(2, fused_select_kernel<DT>, dim3(rows), dim3(TK_THREADS), st, p, l));
     }
     FTK_LAUNCH_CHECK();
     return 0;

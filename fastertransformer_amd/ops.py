@@ -214,6 +214,28 @@ def _pack(tensors):
     return names, descs, keep
 
 
+class _PackedMap:
+    """Named tensors marshalled for the handle API, reused from call to call: a decode loop passes the same
+    objects every step (only the logits buffer or a draw array may differ), so only entries whose object
+    changed are described again. Objects are compared by identity; a torch tensor that was resized in place
+    must be passed as a new object."""
+
+    def __init__(self):
+        self.keys = None
+
+    def update(self, tensors):
+        keys = tuple(tensors)
+        if keys != self.keys:
+            self.names, self.descs, self.objs = _pack(tensors)
+            self.keys = keys
+            return
+        objs, descs = self.objs, self.descs
+        for i, v in enumerate(tensors.values()):
+            if v is not objs[i]:
+                descs[i] = _describe(v)
+                objs[i] = v
+
+
 class DynamicDecodeLayer:
     """fastertransformer::DynamicDecodeLayer<T>: setup(batch, beam, named tensors), forward(outputs, inputs).
 
@@ -230,6 +252,7 @@ class DynamicDecodeLayer:
                                                      int(is_free_buffer_after_forward))
         if not self._h:
             raise FtkError("ft_dynamic_decode_create: " + self._lib.ft_decode_last_error().decode())
+        self._packed_in, self._packed_out = _PackedMap(), _PackedMap()
 
     def close(self):
         if getattr(self, "_h", None):
@@ -252,9 +275,10 @@ class DynamicDecodeLayer:
             self._raise(rc, "setup")
 
     def forward(self, output_tensors, input_tensors):
-        in_names, in_descs, keep_in = _pack(input_tensors)
-        out_names, out_descs, keep_out = _pack(output_tensors)
-        rc = self._lib.ft_dynamic_decode_forward(self._h, len(keep_in), in_names, in_descs, len(keep_out), out_names,
-                                                 out_descs)
+        pin, pout = self._packed_in, self._packed_out
+        pin.update(input_tensors)
+        pout.update(output_tensors)
+        rc = self._lib.ft_dynamic_decode_forward(self._h, len(pin.objs), pin.names, pin.descs, len(pout.objs),
+                                                 pout.names, pout.descs)
         if rc != 0:
             self._raise(rc, "forward")
