@@ -20,7 +20,7 @@ INCLUDE = os.path.join(ROOT, "include")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 KERNEL_SOURCES = ["penalty_kernels.hip", "criteria_kernels.hip", "topp_kernels.hip", "topk_kernels.hip",
-                  "fused_kernels.hip"]
+                  "fused_kernels.hip", "decode_step_kernels.hip"]
 
 # -ffp-contract=off: results must match a plain IEEE evaluation operation by operation.
 # packed-fp32 instructions are disabled on purpose (hardware notes).

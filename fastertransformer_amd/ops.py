@@ -48,6 +48,10 @@ _SIGNATURES = {
     "ftk_invoke_stop_words_criterion_rows": [_vp, _vp, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _vp],
     "ftk_invoke_length_criterion": [_vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_fused_topk_step": [_vp, _vp],
+    "ftk_invoke_log_prob_from_logits": [_i, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _b],
+    "ftk_invoke_decoding_initialize": [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "ftk_invoke_plus_scalar": [_vp, _i, _i, _vp],
+    "ftk_invoke_transpose_axis01": [_vp, _vp, _vp, _i, _i, _vp],
     "ftk_host_expf": [_f],
     "ftk_host_logf": [_f],
     "ftk_test_device_math": [_i, _vp, _vp, _sz, _vp],

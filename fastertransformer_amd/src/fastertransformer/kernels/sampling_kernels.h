@@ -235,4 +235,36 @@ inline void invokeLengthCriterion(bool* finished, bool* should_stop, int* h_pinn
                                           batch_size, beam_width, step, stream));
 }
 
+// ---- logprob_kernels.h, decoding_kernels.h, gpt_kernels.h (the steps either side of the sampling path) ----
+template<typename T>
+void invokeLogProbFromLogits(float* cum_log_probs, const T* logits, const int* input_ids, const int* input_lengths,
+                             const size_t max_input_length, const size_t batch_size, const size_t vocab_size,
+                             const size_t vocab_size_padded, void* workspace, const size_t workspace_size,
+                             hipStream_t stream, const bool batch_first = false)
+{
+    check_ftk(ftk_invoke_log_prob_from_logits(FtkDType<T>::value, cum_log_probs, logits, input_ids, input_lengths,
+                                              max_input_length, batch_size, vocab_size, vocab_size_padded, workspace,
+                                              workspace_size, stream, batch_first));
+}
+
+template<typename T>
+void invokeDecodingInitialize(bool* finished, int* sequence_length, int* word_ids, T* cum_log_probs,
+                              const int* sentence_ids, const int batch_size, const int beam_width,
+                              const int max_input_length, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_decoding_initialize(FtkDType<T>::value, finished, sequence_length, word_ids, cum_log_probs,
+                                             sentence_ids, batch_size, beam_width, max_input_length, stream));
+}
+
+inline void invokePlusScalar(int* buf, const int val, const int size, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_plus_scalar(buf, val, size, stream));
+}
+
+inline void invokeTransposeAxis01(int* out, int* in, const int* in_skipping_dim1, const int dim0, const int dim1,
+                                  hipStream_t stream)
+{
+    check_ftk(ftk_invoke_transpose_axis01(out, in, in_skipping_dim1, dim0, dim1, stream));
+}
+
 }  // namespace fastertransformer

@@ -210,6 +210,33 @@ typedef struct ftk_fused_topk_args {
 /* workspace == NULL in args: writes the required size into args->workspace_size, launches nothing. */
 int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
 
+/* ---- the steps either side of the sampling path -------------------------------------------- */
+/* kernels/logprob_kernels.cu:137-183 invokeLogProbFromLogits<T>: cum_log_probs[b] = sum over step < lengths[b]-1 of
+ * log softmax(logits[step, b, :vocab_size])[input_ids[step+1, b]]. logits [max_input_length, batch, Vp] or, with
+ * batch_first, [batch, max_input_length, Vp]; input_ids laid out the same way; workspace >= 4 * max_input_length *
+ * batch bytes (FTK_ERR_WORKSPACE otherwise; the reference asserts). Results agree with the reference within
+ * rounding (1e-5 relative), not bit for bit. */
+int ftk_invoke_log_prob_from_logits(int dtype, float* cum_log_probs, const void* logits, const int* input_ids,
+                                    const int* input_lengths, size_t max_input_length, size_t batch_size,
+                                    size_t vocab_size, size_t vocab_size_padded, void* workspace,
+                                    size_t workspace_size, ftk_stream_t stream, bool batch_first);
+
+/* kernels/decoding_kernels.cu:49-65 invokeDecodingInitialize<T>: finished = false, sequence_length =
+ * max_input_length, word_ids = sentence_ids[batch] (when word_ids != NULL), cum_log_probs = 0 for the first beam of a
+ * batch entry and -MAX_T_VAL (65504 for half, 1e20 otherwise) for the others; cum_log_probs is a T array. */
+int ftk_invoke_decoding_initialize(int dtype, bool* finished, int* sequence_length, int* word_ids, void* cum_log_probs,
+                                   const int* sentence_ids, int batch_size, int beam_width, int max_input_length,
+                                   ftk_stream_t stream);
+
+/* kernels/decoding_kernels.cu:688-696 invokePlusScalar<int>: buf[i] += val */
+int ftk_invoke_plus_scalar(int* buf, int val, int size, ftk_stream_t stream);
+
+/* kernels/gpt_kernels.cu:347-357 invokeTransposeAxis01<int>(out, in, in_skipping_dim1, dim0, dim1): out [dim1, dim0],
+ * in [dim0, dim1]; with in_skipping_dim1 != NULL column i1 is read at an extra offset in_skipping_dim1[i1] * dim1.
+ * This is how the time-major output ids [max_seq, batch] become [batch, max_seq]. out must not alias in. */
+int ftk_invoke_transpose_axis01(int* out, const int* in, const int* in_skipping_dim1, int dim0, int dim1,
+                                ftk_stream_t stream);
+
 /* ---- per-kernel timing of the fused step (the reference's counterpart is its CudaTimer / NVTX ranges,
  * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
  * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on

@@ -788,6 +788,43 @@ struct Layer {
     SamplingState topk, topp;
 };
 
+// ------------------------------------------------------------------------------------------
+// Steps either side of the sampling path.
+//   kernels/logprob_kernels.cu:35-135   log_probs_kernel + accumulate_log_probs (beam folded into batch)
+// ------------------------------------------------------------------------------------------
+template<int DT>
+void log_prob_from_logits(float* cum_log_probs, float* log_probs, const void* logits_v, const int* ids,
+                          const int* lengths, size_t max_len, size_t batch, size_t V, size_t Vp, bool batch_first)
+{
+    typedef St<DT>       S;
+    const typename S::T* logits = (const typename S::T*)logits_v;
+    for (size_t b = 0; b < batch; ++b) {
+        float accum = 0.0f;
+        for (size_t step = 0; step + 1 < max_len; ++step) {
+            if ((int)step >= lengths[b] - 1) {
+                continue;
+            }
+            const size_t         off = batch_first ? (b * max_len + step) * Vp : (step * batch + b) * Vp;
+            const typename S::T* row = logits + off;
+            float                mx  = -S::max_t();
+            for (size_t v = 0; v < V; ++v) {
+                mx = fmaxf(mx, S::ld(row[v]));
+            }
+            float sum = 0.0f;
+            for (size_t v = 0; v < V; ++v) {
+                sum += det_expf(S::ld(row[v]) - mx);
+            }
+            const size_t tok = batch_first ? b * max_len + step + 1 : (step + 1) * batch + b;
+            const float  lp  = S::ld(row[ids[tok]]) - mx - det_logf(sum + 1e-9f);
+            if (log_probs != nullptr) {
+                log_probs[batch_first ? b * (max_len - 1) + step : step * batch + b] = lp;
+            }
+            accum += lp;
+        }
+        cum_log_probs[b] = accum;
+    }
+}
+
 }  // namespace oracle
 
 using namespace oracle;
@@ -1224,6 +1261,59 @@ int oracle_layer_forward(void* h, const OracleForwardArgs* a)
         length_criterion(a->finished, a->should_stop, a->sequence_limit_length, a->batch_size, a->step);
     }
     return 0;
+}
+
+// kernels/logprob_kernels.cu:137-183
+void oracle_log_prob_from_logits(int dtype, float* cum_log_probs, float* log_probs, const void* logits, const int* ids,
+                                 const int* lengths, size_t max_len, size_t batch, size_t V, size_t Vp, int batch_first)
+{
+    const bool bf = batch_first != 0;
+    switch (dtype) {
+        case DT_F32:
+            log_prob_from_logits<DT_F32>(cum_log_probs, log_probs, logits, ids, lengths, max_len, batch, V, Vp, bf);
+            break;
+        case DT_F16:
+            log_prob_from_logits<DT_F16>(cum_log_probs, log_probs, logits, ids, lengths, max_len, batch, V, Vp, bf);
+            break;
+        default:
+            log_prob_from_logits<DT_BF16>(cum_log_probs, log_probs, logits, ids, lengths, max_len, batch, V, Vp, bf);
+            break;
+    }
+}
+
+// kernels/decoding_kernels.cu:26-47; cum_log_probs as fp32 images of T: 0 for the first beam,
+// -MAX_T_VAL otherwise (65504 for half, 1e20 for float / bfloat16)
+void oracle_decoding_initialize(int dtype, bool* finished, int* sequence_length, int* word_ids, float* cum_log_probs,
+                                const int* sentence_ids, int batch, int beam, int max_input_length)
+{
+    const float max_t = dtype == DT_F16 ? 65504.0f : 1e20f;
+    for (int i = 0; i < batch * beam; ++i) {
+        finished[i]        = false;
+        sequence_length[i] = max_input_length;
+        if (word_ids != nullptr) {
+            word_ids[i] = sentence_ids[i / beam];
+        }
+        cum_log_probs[i] = (i % beam == 0) ? 0.0f : -max_t;
+    }
+}
+
+// kernels/decoding_kernels.cu:680-694
+void oracle_plus_scalar(int* buf, int val, int size)
+{
+    for (int i = 0; i < size; ++i) {
+        buf[i] += val;
+    }
+}
+
+// kernels/gpt_kernels.cu:329-345 (out [dim1, dim0], in [dim0, dim1], optional per-column source offsets)
+void oracle_transpose_axis01(int* out, const int* in, const int* in_skipping_dim1, int dim0, int dim1)
+{
+    for (int i0 = 0; i0 < dim0; ++i0) {
+        for (int i1 = 0; i1 < dim1; ++i1) {
+            const int off       = in_skipping_dim1 == nullptr ? 0 : in_skipping_dim1[i1] * dim1;
+            out[i1 * dim0 + i0] = in[off + i0 * dim1 + i1];
+        }
+    }
 }
 
 }  // extern "C"

@@ -266,3 +266,35 @@ class OracleDynamicDecodeLayer:
         rc = lib().oracle_layer_forward(self.h, C.byref(a))
         if rc != 0:
             raise RuntimeError("oracle_layer_forward rc=%d" % rc)
+
+# ---- the steps either side of the path --------------------------------------------------------------
+def log_prob_from_logits(dt, logits, ids, lengths, max_len, batch, V, Vp, batch_first=False):
+    """returns (cum_log_probs[batch], log_probs[(max_len-1) * batch])"""
+    cum = np.zeros(batch, np.float32)
+    lp = np.zeros(max(max_len - 1, 1) * batch, np.float32)
+    f = lib().oracle_log_prob_from_logits
+    f.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                  C.c_size_t, C.c_size_t, C.c_int]
+    f(dt, _p(cum), _p(lp), _p(logits), _p(ids), _p(lengths), max_len, batch, V, Vp, int(batch_first))
+    return cum, lp
+
+
+def decoding_initialize(dt, sentence_ids, batch, beam, max_input_length, with_word_ids=True):
+    n = batch * beam
+    finished = np.ones(n, np.bool_)
+    seq = np.zeros(n, np.int32)
+    word_ids = np.zeros(n, np.int32) if with_word_ids else None
+    cum = np.zeros(n, np.float32)
+    lib().oracle_decoding_initialize(dt, _p(finished), _p(seq), _p(word_ids), _p(cum), _p(sentence_ids), batch, beam,
+                                     max_input_length)
+    return finished, seq, word_ids, cum
+
+
+def plus_scalar(buf, val):
+    lib().oracle_plus_scalar(_p(buf), int(val), buf.size)
+
+
+def transpose_axis01(inp, skipping, dim0, dim1):
+    out = np.zeros(dim0 * dim1, np.int32)
+    lib().oracle_transpose_axis01(_p(out), _p(inp), _p(skipping), dim0, dim1)
+    return out.reshape(dim1, dim0)

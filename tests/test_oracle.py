@@ -598,3 +598,56 @@ def test_python_known_answers_repetition_and_min_length():
             assert ((snap["sequence_length"] + 1) >= H + min_len).all(), (method, B, min_len)
             if method["runtime_top_k"] == [1]:
                 assert snap["finished"].all()  # greedy: it does stop as soon as it is allowed to
+
+
+# ---- the steps either side of the path -------------------------------------------------------------------
+@pytest.mark.parametrize("batch_first", [False, True])
+@pytest.mark.parametrize("shape", [(1, 32, 16), (33, 4, 1000), (9, 3, 5001)])
+def test_log_prob_from_logits_closed_form(batch_first, shape):
+    """kernels/logprob_kernels.cu:35-135 against the reference test's host expectation
+    (tests/unittests/test_logprob_kernels.cu:39-75) evaluated in float64"""
+    max_len, batch, V = shape
+    Vp = (V + 7) // 8 * 8
+    rng = np.random.default_rng(21)
+    for dt in DTYPES:
+        shp = (batch, max_len, Vp) if batch_first else (max_len, batch, Vp)
+        logits = O.to_storage((rng.standard_normal(shp) * 3).astype(np.float32), dt)
+        ids = rng.integers(0, V, (batch, max_len) if batch_first else (max_len, batch)).astype(np.int32)
+        lengths = rng.integers(1, max_len + 1, batch).astype(np.int32)
+        cum, lp = O.log_prob_from_logits(dt, logits, ids, lengths, max_len, batch, V, Vp, batch_first)
+        x = O.to_f32(logits, dt).astype(np.float64)
+        want = np.zeros(batch)
+        for b in range(batch):
+            for step in range(1, max_len):
+                if step < lengths[b]:
+                    vec = (x[b, step - 1] if batch_first else x[step - 1, b])[:V]
+                    tok = ids[b, step] if batch_first else ids[step, b]
+                    v = vec[tok] - vec.max() - np.log(np.exp(vec - vec.max()).sum())
+                    want[b] += v
+                    got = lp[b * (max_len - 1) + step - 1] if batch_first else lp[(step - 1) * batch + b]
+                    assert abs(got - v) < 1e-5 * max(1.0, abs(v))
+        np.testing.assert_allclose(cum, want, rtol=2e-6 * max_len, atol=1e-5)
+
+
+def test_decode_state_helpers():
+    """kernels/decoding_kernels.cu:26-47, :680-694 and kernels/gpt_kernels.cu:329-345"""
+    rng = np.random.default_rng(22)
+    sent = rng.integers(0, 100, 5).astype(np.int32)
+    for dt in DTYPES:
+        fin, seq, ids, cum = O.decoding_initialize(dt, sent, 5, 3, 17)
+        assert not fin.any() and (seq == 17).all()
+        assert np.array_equal(ids, np.repeat(sent, 3))
+        big = 65504.0 if dt == O.F16 else 1e20
+        assert np.array_equal(cum.reshape(5, 3), np.tile(np.array([0.0, -big, -big], np.float32), (5, 1)))
+    buf = rng.integers(0, 50, 77).astype(np.int32)
+    want = buf + 9
+    O.plus_scalar(buf, 9)
+    assert np.array_equal(buf, want)
+    a = rng.integers(0, 1000, (37, 53)).astype(np.int32)
+    assert np.array_equal(O.transpose_axis01(a, None, 37, 53), a.T)
+    # with per-column offsets the source of column i1 starts skipping[i1] rows further down
+    big_in = rng.integers(0, 1000, (37 + 4, 53)).astype(np.int32)
+    skip = rng.integers(0, 5, 53).astype(np.int32)
+    got = O.transpose_axis01(big_in, skip, 37, 53)
+    want = np.stack([big_in[skip[i1]:skip[i1] + 37, i1] for i1 in range(53)])
+    assert np.array_equal(got, want)
