@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_BYTES_PER_LAUNCH = 149911116
 
 WORKLOADS = {
-    # the configuration the metric is quoted on (BASELINE.json "metric" / north-star target)
+    # the configuration the headline metric is quoted on
     "decode_step_b256_v128256_f32_topk64_topp0.9_temp0.8_rep1.1": dict(
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=64, sigma=2.5),
@@ -173,7 +173,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (rows shard across GPUs with no "
-              "exchange, see DESIGN.md); run with --gpus 1", file=sys.stderr)
+              "exchange); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     name = next(iter(WORKLOADS))
     w = WORKLOADS[name]

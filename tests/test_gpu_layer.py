@@ -83,7 +83,7 @@ def _run_case(c, rng, steps, logits_fn, check_logits, ite=0):
 
 @pytest.mark.parametrize("logprobs", [True, False], ids=["logprobs", "fused"])
 def test_config1_cpu_reference_step(logprobs):
-    """BASELINE config 1: batch 8, vocab 50257 fp32 N(0,2), repetition penalty 1.2 over 64 prior ids,
+    """Benchmark configuration 1: batch 8, vocab 50257 fp32 N(0,2), repetition penalty 1.2 over 64 prior ids,
     top_k 40, end_id 50256, log-probs on."""
     rng = np.random.default_rng(1)
     B, V = 8, 50257
@@ -95,7 +95,7 @@ def test_config1_cpu_reference_step(logprobs):
 
 @pytest.mark.parametrize("logprobs", [False, True], ids=["fused", "logprobs"])
 def test_config2_batched_topk_fp16_padded(logprobs):
-    """BASELINE config 2 (rows cut to 48): vocab 50257 padded to 51200 fp16, N(0,3) + spikes, per-row
+    """Benchmark configuration 2 (rows cut to 48): vocab 50257 padded to 51200 fp16, N(0,3) + spikes, per-row
     k in {1,4,16,40,64,1024}, per-row temperature U[0.5,1.5]."""
     rng = np.random.default_rng(2)
     B, V, Vp = 48, 50257, 51200
@@ -115,7 +115,7 @@ def _zipf_logits(rng, dt, B, V):
 
 
 def test_config3_batched_topp_decay():
-    """BASELINE config 3 (rows cut to 24, 6 steps): vocab 128256 fp32 Zipf(1.1) log-softmax + N(0,0.5),
+    """Benchmark configuration 3 (rows cut to 24, 6 steps): vocab 128256 fp32 Zipf(1.1) log-softmax + N(0,0.5),
     top_k 0, per-row top_p U[0.5,0.99], decay 0.9, min 0.3, reset id 13."""
     rng = np.random.default_rng(3)
     B, V = 24, 128256
@@ -127,7 +127,7 @@ def test_config3_batched_topp_decay():
 
 @pytest.mark.parametrize("freq", [None, 0.3], ids=["presence", "presence+frequency"])
 def test_config4_penalty_mask_heavy(freq):
-    """BASELINE config 4 (rows cut to 32, history 512): vocab 32000 bf16, Zipf(1.2) history, min_length beyond
+    """Benchmark configuration 4 (rows cut to 32, history 512): vocab 32000 bf16, Zipf(1.2) history, min_length beyond
     the current step (end id masked), presence (+frequency) penalty, bad words len 1-4, stop words len 1-3,
     top_k 50."""
     rng = np.random.default_rng(4)
@@ -177,7 +177,7 @@ def test_config4_stop_words_fire_and_shared_bad_words():
 
 @pytest.mark.parametrize("dt", [O.F16, O.F32], ids=lambda d: DTYPE_NAMES[d])
 def test_config5_full_loop(dt):
-    """BASELINE config 5 (rows cut to 40, vocab 152064, 12 steps): k=64 then p=0.9, temperature 0.8,
+    """Benchmark configuration 5 (rows cut to 40, vocab 152064, 12 steps): k=64 then p=0.9, temperature 0.8,
     repetition penalty 1.1, log-probs, finished / sequence_length / length-limit updates."""
     rng = np.random.default_rng(5)
     B, V, H = 40, 152064, 4
