@@ -8,8 +8,8 @@
 //   stage 1, inside a slice : value desc, (i mod BS1) desc, i asc
 //   stage 2, over positions : value desc, (pos mod BS2) desc, pos asc,  pos = slice*k + rank
 // The reference reads the row k+2 times. Here the row is read once, as a stream:
-//   stream  - a 256-thread workgroup walks its share of the row tile by tile (16 KB per thread
-//             group of loads in flight, the next tile requested before the current one is examined).
+//   stream  - a 256-thread workgroup walks its share of the row tile by tile (16 vectors of 16 bytes per
+//             thread, 64 KB per tile, the next tile requested before the bookkeeping of the current one).
 //             It keeps a lower bound of the row's k-th largest value and an LDS list of everything
 //             at or above it. The bound starts from the order statistics of per-thread maxima of
 //             the first tile and is tightened to the exact k-th largest of the list whenever the
@@ -17,15 +17,13 @@
 //             maximum and a fraction of a compare.
 //   select  - replays both tie orders on the candidates (ranking by counting for <= 256
 //             candidates, two LDS bitonic sorts of 64-bit composite keys otherwise) and samples.
-// When the batch has at least as many rows as the chip has compute units, one workgroup owns a whole
-// row and runs both phases (no scratch traffic, one launch). Smaller batches split each row over
-// several workgroups that leave their lists in the workspace, and a second launch merges them.
+// When the batch has at least four rows per compute unit, one workgroup owns a whole row and runs both
+// phases (no workspace traffic, one launch). Smaller batches split each row over several workgroups
+// that leave their lists in the workspace, and a second launch merges them.
 // Rows whose candidates cannot be bounded (thousands of identical values around the k-th) take a
 // literal, slow replay of the reference's passes.
 #pragma once
 #include "ftk_device.cuh"
-#include <stdlib.h>
-
 #include "ftk_transform.cuh"
 
 // Optional phase timing for kernel development: FTK_PHASE(i) adds the time since the previous mark of
@@ -102,35 +100,6 @@ inline TopkPlan topk_plan(int vocab_padded, int batch, int max_top_k, int elem_b
     p.row_entries = entries;
     p.bytes       = (size_t)batch * (p.splits * sizeof(TopkChunkHeader) + entries * sizeof(TopkEntry));
     return p;
-}
-
-// Delay step for topk_stagger: the time a quarter of the resident workgroups needs to load one tile
-// (64 KB each) at ~5 TB/s, in units of 2048 clocks (~0.9 us); no stagger for launches that do not fill
-// the device.
-inline int topk_stagger_units(int workgroups)
-{
-    const char* env = getenv("FTK_STAGGER_UNITS");
-    if (env != nullptr) {
-        return atoi(env);
-    }
-    if (workgroups < 512) {
-        return 0;
-    }
-    const int    resident = workgroups < 1024 ? workgroups : 1024;
-    const double us       = (resident / 4) * 65536.0 / 5.0e6;
-    return (int)(us / 0.9 + 0.5);
-}
-
-// Workgroups that start together and share the memory system fairly also finish each tile together, so
-// the whole device alternates between loading and computing. Delaying three quarters of them by one,
-// two and three tile-load times at the start interleaves the phases. `units` is the delay step in
-// multiples of 2048 clocks.
-__device__ __forceinline__ void topk_stagger(int linear_wg, int units)
-{
-    const int g = (linear_wg >> 8) & 3;
-    for (int i = 0; i < g * units; ++i) {
-        __builtin_amdgcn_s_sleep(32);
-    }
 }
 
 // Workgroup barrier for code that only communicates through LDS: global loads issued earlier stay

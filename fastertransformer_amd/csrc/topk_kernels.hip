@@ -34,7 +34,6 @@ struct TopkKernelArgs {
     const int*   end_ids;
     int          splits;
     int          tiles_per_wg;
-    int          stagger_units;
     size_t       row_entries;
     TopkChunkHeader* headers;
     TopkEntry*       entries;
@@ -94,7 +93,6 @@ __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_gather_kernel(Top
     const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
-    topk_stagger(row * a.splits + chunk, a.stagger_units);
     FTK_PHASE(0);
     const int tiles = topk_row_tiles<DT>(r.rowp, a.vocab);
     const int t0    = min(tiles, chunk * a.tiles_per_wg);
@@ -202,7 +200,6 @@ int ftk_invoke_batch_topk_sampling(int dtype, void* workspace, size_t* workspace
     a.end_ids          = end_ids;
     a.splits           = plan.splits;
     a.tiles_per_wg     = plan.tiles_per_wg;
-    a.stagger_units    = topk_stagger_units(plan.splits * batch_size);
     a.row_entries      = plan.row_entries;
     a.headers          = (TopkChunkHeader*)workspace;
     a.entries          = (TopkEntry*)(a.headers + (size_t)batch_size * plan.splits);
