@@ -141,12 +141,13 @@ __device__ __forceinline__ uint32_t wave_sort_desc(uint32_t v)
     return v;
 }
 
-// In-LDS bitonic sort (ascending) of n 64-bit keys, n a power of two, by all threads of the block.
+// In-LDS bitonic sort (ascending) of n 64-bit keys, n a power of two, by the THREADS threads of the block.
+template<int THREADS>
 __device__ __forceinline__ void block_bitonic_sort_u64(unsigned long long* keys, int n)
 {
     for (int k = 2; k <= n; k <<= 1) {
         for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = (int)threadIdx.x; i < (n >> 1); i += (int)blockDim.x) {
+            for (int i = (int)threadIdx.x; i < (n >> 1); i += THREADS) {
                 // i-th compare-exchange pair of this stage
                 const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
                 const int hi = lo | j;
@@ -170,6 +171,50 @@ __device__ __forceinline__ int next_pow2(int n)
         p <<= 1;
     }
     return p;
+}
+
+// In-LDS ascending sort of any number n of 64-bit keys by all threads of the block. The network is the
+// bitonic sorter in its form with comparators of one direction only (each merge starts by comparing
+// mirrored positions); with every comparator putting the smaller key first, the positions from n up
+// to the next power of two behave as if they held the largest key and never take part, so they are
+// neither stored nor visited. THREADS is the size of the block (a constant here: reading blockDim
+// costs a trip to memory in every stage).
+template<int THREADS>
+__device__ __forceinline__ void block_sort_u64(unsigned long long* keys, int n)
+{
+    const int half = next_pow2(n) >> 1;
+    for (int k = 2; (k >> 1) <= half && k > 0; k <<= 1) {
+        const int hk = k >> 1;
+        for (int i = (int)threadIdx.x; i < half; i += THREADS) {
+            const int pos = i & (hk - 1);
+            const int lo  = ((i - pos) << 1) | pos;
+            const int hi  = ((i - pos) << 1) | (k - 1 - pos);
+            if (hi < n) {
+                const unsigned long long a = keys[lo];
+                const unsigned long long b = keys[hi];
+                if (a > b) {
+                    keys[lo] = b;
+                    keys[hi] = a;
+                }
+            }
+        }
+        __syncthreads();
+        for (int j = hk >> 1; j > 0; j >>= 1) {
+            for (int i = (int)threadIdx.x; i < half; i += THREADS) {
+                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
+                const int hi = lo | j;
+                if (hi < n) {
+                    const unsigned long long a = keys[lo];
+                    const unsigned long long b = keys[hi];
+                    if (a > b) {
+                        keys[lo] = b;
+                        keys[hi] = a;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+    }
 }
 
 // ---- Philox-4x32-10 (counter-based generator; replaces cuRAND's XORWOW) ---------------------

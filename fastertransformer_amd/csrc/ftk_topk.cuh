@@ -1089,7 +1089,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 s.keys[i] = ~0ull;
             }
             __syncthreads();
-            block_bitonic_sort_u64(s.keys, np2);
+            block_bitonic_sort_u64<TK_THREADS>(s.keys, np2);
             for (int qi = t; qi < np2; qi += TK_THREADS) {
                 unsigned long long nk = ~0ull;
                 if (qi < n) {
@@ -1100,7 +1100,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 s.keys[qi] = nk;
             }
             __syncthreads();
-            block_bitonic_sort_u64(s.keys, np2);
+            block_bitonic_sort_u64<TK_THREADS>(s.keys, np2);
             {
                 int cnt = 0;
                 for (int i = t; i < min(k, n); i += TK_THREADS) {

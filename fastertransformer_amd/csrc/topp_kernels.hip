@@ -7,20 +7,105 @@
 //   :877-1004  topp_sampling           - inclusive prefix sum over 256-wide tiles, first crossing
 //   :1381-1412 computeToppDecay
 //
-// The replacement never sorts a whole row unless it has to. One 1024-thread workgroup per row:
-//   1. one pass: arg-max (ties to the lowest id), number of positive entries, per-thread maxima;
-//   2. a lower bound t0 on the ~500th largest value from the order statistics of the thread maxima;
-//      one pass gathers every entry >= t0 (<= 4096) into LDS; bitonic sort by (prob desc, id asc);
-//   3. the reference's tile scan is replayed on the sorted prefix with its exact rounding order
-//      (32 raking lanes x 8 items, Kogge-Stone over the 32 partials, sequential carry over tiles).
-//   If the draw is not crossed inside the sorted prefix (deep draws on flat distributions) the row
-//   falls back to a stable LSD radix sort of all positive entries in the caller's workspace and
-//   replays the scan from the start.
+// The replacement orders only the part of a row in front of the draw (see the top-p section).
 #include "ftk_device.cuh"
 #include "ftk_sampling.h"
 #include "ftk_transform.cuh"
 
 namespace ftk {
+
+// Calls visit(column, value) for the columns [lo, hi) of a row, 16-byte loads where the address
+// allows, four of them in flight per thread. A thread sees its columns in ascending order.
+template<int DT, int THREADS, typename F>
+__device__ __forceinline__ void stream_columns(const typename Storage<DT>::T* __restrict__ rowp, int lo, int hi,
+                                               F&& visit)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         EPV = (int)(16 / sizeof(T));
+    const int             t   = threadIdx.x;
+    if (hi <= lo) {
+        return;
+    }
+    const int a     = (int)(((16u - ((uintptr_t)(rowp + lo) & 15u)) & 15u) / sizeof(T));
+    const int head  = min(a, hi - lo);
+    const int nvec  = (hi - lo - head) / EPV;
+    const int body0 = lo + head;
+    const int tail0 = body0 + nvec * EPV;
+    if (t < head) {
+        visit(lo + t, S::ld(rowp[lo + t]));
+    }
+    const uint4*  vec = reinterpret_cast<const uint4*>(rowp + body0);
+    constexpr int U   = 4;
+    for (int i0 = t; i0 < nvec; i0 += U * THREADS) {
+        uint4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * THREADS;
+            raw[u]      = i < nvec ? vec[i] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * THREADS;
+            if (i < nvec) {
+                const T* e = reinterpret_cast<const T*>(&raw[u]);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    visit(body0 + i * EPV + j, S::ld(e[j]));
+                }
+            }
+        }
+    }
+    if (tail0 + t < hi) {
+        visit(tail0 + t, S::ld(rowp[tail0 + t]));
+    }
+}
+
+// In-place variant: every column of [lo, hi) is replaced by f(column, value).
+template<int DT, int THREADS, typename F>
+__device__ __forceinline__ void transform_columns(typename Storage<DT>::T* __restrict__ rowp, int lo, int hi, F&& f)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         EPV = (int)(16 / sizeof(T));
+    const int             t   = threadIdx.x;
+    if (hi <= lo) {
+        return;
+    }
+    const int a     = (int)(((16u - ((uintptr_t)(rowp + lo) & 15u)) & 15u) / sizeof(T));
+    const int head  = min(a, hi - lo);
+    const int nvec  = (hi - lo - head) / EPV;
+    const int body0 = lo + head;
+    const int tail0 = body0 + nvec * EPV;
+    if (t < head) {
+        rowp[lo + t] = S::st(f(lo + t, S::ld(rowp[lo + t])));
+    }
+    uint4*        vec = reinterpret_cast<uint4*>(rowp + body0);
+    constexpr int U   = 4;
+    for (int i0 = t; i0 < nvec; i0 += U * THREADS) {
+        uint4 raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * THREADS;
+            raw[u]      = i < nvec ? vec[i] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * THREADS;
+            if (i < nvec) {
+                T* e = reinterpret_cast<T*>(&raw[u]);
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    e[j] = S::st(f(body0 + i * EPV + j, S::ld(e[j])));
+                }
+                vec[i] = raw[u];
+            }
+        }
+    }
+    if (tail0 + t < hi) {
+        rowp[tail0 + t] = S::st(f(tail0 + t, S::ld(rowp[tail0 + t])));
+    }
+}
 
 // =============================================================================================
 // softmax
@@ -57,6 +142,69 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
         const float b = bias != nullptr ? S::ld(bias[v]) : 0.0f;
         return round_t<DT>(S::ld(rowp[v]) + b);
     };
+
+    if (!fin && bias == nullptr) {
+        // Ordinary rows. The maximum and the final division do not depend on the order of the columns
+        // and go through 16-byte accesses; the sum keeps the reference's order (thread t adds its
+        // columns t, t + BLK, ... one after the other), eight loads in flight.
+        float mx = -3.402823466e+38f;
+        stream_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) { mx = __builtin_fmaxf(mx, x + 0.0f); });
+        if (n_padded > n) {
+            mx = __builtin_fmaxf(mx, -MAXT);
+        }
+        mx = block_max<float>(mx, sh, -3.402823466e+38f);
+        if (BLK < 1024) {
+            mx = __builtin_fmaxf(mx, -1e20f);
+        }
+        const float pad_e = round_t<DT>(det_expf(-MAXT - mx));
+        float       sum   = 0.0f;
+        if (active) {
+            constexpr int U = 8;
+            int           v = t;
+            for (; v + (U - 1) * BLK < n; v += U * BLK) {
+                float x[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    x[u] = S::ld(rowp[v + u * BLK]);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    sum += round_t<DT>(det_expf((x[u] + 0.0f) - mx));
+                }
+            }
+            for (; v < n; v += BLK) {
+                sum += round_t<DT>(det_expf((S::ld(rowp[v]) + 0.0f) - mx));
+            }
+            for (; v < n_padded; v += BLK) {
+                sum += pad_e;
+            }
+        }
+#pragma unroll
+        for (int m = 16; m > 0; m >>= 1) {
+            sum += __shfl_xor(sum, m, 32);
+        }
+        if ((t & 31) == 0) {
+            sh[t >> 5] = sum;
+        }
+        __syncthreads();
+        if (t < 32) {
+            float v = ((float)t < (float)BLK / 32.0f) ? sh[t] : 0.0f;
+#pragma unroll
+            for (int m = 16; m > 0; m >>= 1) {
+                v += __shfl_xor(v, m, 32);
+            }
+            if (t == 0) {
+                sh_bcast = v;
+            }
+        }
+        __syncthreads();
+        const float denom = sh_bcast + 1e-6f;
+        transform_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) {
+            return round_t<DT>(det_expf((x + 0.0f) - mx)) / denom;
+        });
+        transform_columns<DT, SM_THREADS>(rowp, n, n_padded, [&](int, float) { return pad_e / denom; });
+        return;
+    }
 
     float mx = -3.402823466e+38f;
     if (active) {
@@ -106,105 +254,886 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
 // =============================================================================================
 // top-p
 // =============================================================================================
+//
+// The reference sorts every row completely and then scans it. Only the part of the sorted order in
+// front of the draw matters, so the rows are cut first and only the part above the cut is ordered:
+//   histogram  - (chunks x rows) workgroups stream the probabilities once: entries per bucket (six
+//                mantissa bits under the exponent, 32 octaves below 1.0), a fixed-point lower bound
+//                of the mass per bucket, and the arg-max;
+//   cut        - one workgroup per row: the lowest bucket whose suffix of mass certainly covers the
+//                draw, where every bucket and every chunk writes inside the ordered prefix, and the
+//                prefix divided into segments of whole buckets;
+//   gather     - second stream: entries at or above the cut go to their bucket's range as
+//                (~key, id) pairs;
+//   sort       - segments are sorted independently (bitonic in LDS, a radix sort in memory for a
+//                segment that one bucket alone makes too long);
+//   pick       - one workgroup per row replays the reference's scan on the ordered prefix with its
+//                exact rounding order (32 raking lanes x 8 items, Kogge-Stone over the 32 partials,
+//                sequential carry over tiles) and emits the token.
+// A row whose draw is not crossed inside its prefix (it cannot be unless the bound above fails)
+// falls back to a stable radix sort of all its positive entries.
 constexpr int      TP_THREADS = 1024;
-constexpr int      TP_BUF     = 4096;         // sorted-prefix capacity (LDS)
 constexpr int      TP_TILE    = 256;          // the reference's scan tile
-constexpr int      TP_MAXT    = TP_BUF / TP_TILE;
+constexpr int      TP_ROUND   = 1024;         // tiles whose totals are held in LDS at a time
 constexpr uint32_t ZERO_KEY   = 0x80000000u;  // order_key(+0.0f); entries at or below never join the scan
 
-struct TopPShared {
-    unsigned long long buf[TP_BUF];
-    unsigned long long red64[16];
-    uint32_t           red32[16];
-    float              agg[TP_MAXT];
-    float              carry[TP_MAXT + 1];
-    uint32_t           tilemask[TP_MAXT][8];
-    int                wtot[256];
-    int                counter;
-    int                misc[8];
-    float              fmisc[4];
+constexpr int TPH_THREADS = 256;
+constexpr int TPB_SHIFT   = 17;                        // key bits below a bucket (6 mantissa bits stay)
+constexpr int TPB_ONE     = 0x3F800000 >> TPB_SHIFT;   // bucket of 1.0 before the shift of origin
+constexpr int TPB_SPAN    = 32 * 64;                   // 32 octaves below 1.0 are resolved
+constexpr int TPB_NB      = TPB_SPAN + 2;              // [0]: everything smaller, [NB-1]: above 1 + 1/64
+constexpr int TPS_SEG     = 2048;                      // segment boundaries follow multiples of this
+constexpr int TPS_CAP     = 5632;                      // longest segment sorted in LDS
+
+constexpr int TOPP_SKIP     = 1;
+constexpr int TOPP_SHORTCUT = 2;
+
+struct ToppRowMeta {
+    unsigned long long best;   // (key << 32) | ~id of the arg-max (lowest id among equals)
+    int                cut;    // lowest gathered bucket
+    int                n;      // entries at or above the cut
+    int                n_pos;  // positive entries of the row
+    int                nseg;
+    int                flags;
+    int                pad;
 };
+
+// Workspace sections (all offsets multiples of 256 bytes). `sorted` keeps the reference's shape of
+// two 64-bit arrays per row; the second one is only touched by the radix sorts.
+struct ToppPlan {
+    int    splits;  // chunks per row of the two streaming kernels
+    int    chunk;   // columns per chunk
+    int    sorters; // workgroups of the sort kernel
+    size_t off_pcnt, off_pmass, off_pbest, off_start, off_seg, off_meta, bytes;
+};
+
+static inline size_t align256(size_t x)
+{
+    return (x + 255) & ~(size_t)255;
+}
+
+static ToppPlan topp_plan(int batch, size_t vocab)
+{
+    ToppPlan p;
+    const int rows = batch > 0 ? batch : 1;
+    int       s    = (1024 + rows - 1) / rows;
+    const int cap  = (int)(vocab / 8192) > 0 ? (int)(vocab / 8192) : 1;
+    s              = s < cap ? s : cap;
+    s              = s < 64 ? s : 64;
+    p.splits       = s;
+    p.chunk        = (int)(((vocab + s - 1) / s + 7) / 8 * 8);
+    p.sorters      = 512;
+    size_t off     = align256((size_t)rows * vocab * 2 * sizeof(unsigned long long));
+    p.off_pcnt     = off;
+    off += align256((size_t)rows * s * TPB_NB * sizeof(uint32_t));
+    p.off_pmass = off;
+    off += align256((size_t)rows * s * TPB_NB * sizeof(uint32_t));
+    p.off_pbest = off;
+    off += align256((size_t)rows * s * sizeof(unsigned long long));
+    p.off_start = off;
+    off += align256((size_t)rows * s * TPB_NB * sizeof(uint32_t));
+    p.off_seg = off;
+    off += align256((size_t)rows * TPB_NB * sizeof(uint32_t));
+    p.off_meta = off;
+    off += align256((size_t)rows * sizeof(ToppRowMeta));
+    p.bytes = off;
+    return p;
+}
+
+__device__ __forceinline__ int topp_bucket(uint32_t key)
+{
+    const int raw = (int)((key & 0x7FFFFFFFu) >> TPB_SHIFT) - (TPB_ONE - TPB_SPAN);
+    return min(max(raw, 0), TPB_NB - 1);
+}
 
 __device__ __forceinline__ float key64_prob(unsigned long long k)
 {
     return key_to_float(~(uint32_t)(k >> 32));
 }
 
-// Replays the reference scan over `nt` tiles held in s.buf (entries >= n_in_buf count as 0).
-// Returns the sorted position (relative to the buffer start) the reference would pick, or -1;
-// s.carry[nt] is the running total afterwards. All threads must call; result is block-uniform.
-__device__ int eval_tiles(TopPShared& s, int n_in_buf, int nt, float carry_in, float rand_num)
+template<int DT>
+__global__ void __launch_bounds__(TPH_THREADS)
+topp_histogram_kernel(const typename Storage<DT>::T* __restrict__ probs, int vocab, int chunk,
+                      const bool* __restrict__ skip_decode, uint32_t* __restrict__ part_cnt,
+                      uint32_t* __restrict__ part_mass, unsigned long long* __restrict__ part_best)
+{
+    __shared__ uint32_t           cnt[TPB_NB];
+    __shared__ uint32_t           mass[TPB_NB];
+    __shared__ unsigned long long red[16];
+    const int                     row = blockIdx.y;
+    const int                     j   = blockIdx.x;
+    const int                     S   = gridDim.x;
+    const int                     t   = threadIdx.x;
+    if (skip_decode != nullptr && skip_decode[row]) {
+        return;
+    }
+    for (int b = t; b < TPB_NB; b += TPH_THREADS) {
+        cnt[b]  = 0u;
+        mass[b] = 0u;
+    }
+    __syncthreads();
+    const int lo   = (int)min((long long)vocab, (long long)j * chunk);
+    const int hi   = (int)min((long long)vocab, (long long)lo + chunk);
+    uint32_t  tmax = 0;
+    int       tidx = 0x7FFFFFFF;
+    stream_columns<DT, TPH_THREADS>(probs + (size_t)row * vocab, lo, hi, [&](int v, float x) {
+        const uint32_t k = order_key(x);
+        if (k > tmax) {
+            tmax = k;
+            tidx = v;
+        }
+        if (k > ZERO_KEY) {
+            const int b = topp_bucket(k);
+            atomicAdd(&cnt[b], 1u);
+            // truncation keeps the sum a lower bound of the mass
+            atomicAdd(&mass[b], (uint32_t)(__builtin_fminf(x, 1.0f) * 2147483648.0f));
+        }
+    });
+    __syncthreads();
+    const size_t base = ((size_t)row * S + j) * TPB_NB;
+    for (int b = t; b < TPB_NB; b += TPH_THREADS) {
+        part_cnt[base + b]  = cnt[b];
+        part_mass[base + b] = mass[b];
+    }
+    unsigned long long best = ((unsigned long long)tmax << 32) | (uint32_t)(~(uint32_t)tidx);
+    best                    = block_max<unsigned long long>(best, red, 0ull);
+    if (t == 0) {
+        part_best[(size_t)row * S + j] = best;
+    }
+}
+
+// The draw of row `b` without consuming it (the pick kernel consumes it).
+__device__ __forceinline__ float row_uniform_peek(const RngState* rng, const float* injected, int b)
+{
+    if (injected != nullptr) {
+        return injected[b];
+    }
+    RngState copy = rng[b];
+    return rng_next_uniform(&copy);
+}
+
+__global__ void __launch_bounds__(TPH_THREADS)
+topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __restrict__ part_mass,
+                const unsigned long long* __restrict__ part_best, uint32_t* __restrict__ start,
+                uint32_t* __restrict__ seg_ends, ToppRowMeta* __restrict__ meta, const RngState* rng,
+                const float* __restrict__ uniforms, float top_p, const float* __restrict__ top_ps,
+                const bool* __restrict__ skip_decode)
+{
+    __shared__ uint32_t           cnt[TPB_NB];
+    __shared__ uint32_t           off[TPB_NB];
+    __shared__ unsigned long long mass[TPB_NB];
+    __shared__ unsigned long long red64[16];
+    __shared__ uint32_t           wcnt[TPH_THREADS / WAVE];
+    __shared__ unsigned long long wmass[TPH_THREADS / WAVE];
+    __shared__ uint32_t           red32[16];
+    const int                     row = blockIdx.x;
+    const int                     t   = threadIdx.x;
+    ToppRowMeta                   m;
+    m.best = 0ull;
+    m.cut = TPB_NB;
+    m.n = m.n_pos = m.nseg = 0;
+    m.flags = 0;
+    m.pad   = 0;
+    if (skip_decode != nullptr && skip_decode[row]) {
+        if (t == 0) {
+            m.flags   = TOPP_SKIP;
+            meta[row] = m;
+        }
+        return;
+    }
+    const size_t base = (size_t)row * S * TPB_NB;
+    for (int b = t; b < TPB_NB; b += TPH_THREADS) {
+        uint32_t           c  = 0;
+        unsigned long long ms = 0;
+        for (int j = 0; j < S; ++j) {
+            c += part_cnt[base + (size_t)j * TPB_NB + b];
+            ms += part_mass[base + (size_t)j * TPB_NB + b];
+        }
+        cnt[b]  = c;
+        mass[b] = ms;
+    }
+    unsigned long long best = 0ull;
+    for (int j = t; j < S; j += TPH_THREADS) {
+        const unsigned long long v = part_best[(size_t)row * S + j];
+        best                       = v > best ? v : best;
+    }
+    best = block_max<unsigned long long>(best, red64, 0ull);  // (also orders the LDS writes above)
+    m.best = best;
+
+    const float p         = top_ps != nullptr ? top_ps[row] : top_p;
+    const float best_prob = (uint32_t)(best >> 32) == 0u ? __builtin_nanf("") : key_to_float((uint32_t)(best >> 32));
+    if (best_prob >= p) {
+        // arg-max shortcut of the reference (:842-849): nothing else of the row is needed
+        if (t == 0) {
+            m.flags   = TOPP_SHORTCUT;
+            meta[row] = m;
+        }
+        return;
+    }
+    const float              rand_num = row_uniform_peek(rng, uniforms, row) * p;
+    // smallest fixed-point mass that certainly covers the draw under the scan's own rounding
+    const unsigned long long target = (unsigned long long)((double)rand_num * (1.0 + 1.0 / 1024.0) * 2147483648.0) + 64ull;
+
+    // descending scan over buckets: thread t owns the descending positions [K*t, K*t + K)
+    constexpr int      K  = (TPB_NB + TPH_THREADS - 1) / TPH_THREADS;
+    uint32_t           lc = 0;
+    unsigned long long lm = 0;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const int d = K * t + i;
+        if (d < TPB_NB) {
+            lc += cnt[TPB_NB - 1 - d];
+            lm += mass[TPB_NB - 1 - d];
+        }
+    }
+    uint32_t           ic = lc;
+    unsigned long long im = lm;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const uint32_t           uc = __shfl_up(ic, o, WAVE);
+        const unsigned long long um = __shfl_up(im, o, WAVE);
+        if (lane_id() >= o) {
+            ic += uc;
+            im += um;
+        }
+    }
+    if (lane_id() == WAVE - 1) {
+        wcnt[wave_id()]  = ic;
+        wmass[wave_id()] = im;
+    }
+    __syncthreads();
+    uint32_t           ec = ic - lc;
+    unsigned long long em = im - lm;
+    uint32_t           total = 0;
+    for (int w = 0; w < TPH_THREADS / WAVE; ++w) {
+        if (w < wave_id()) {
+            ec += wcnt[w];
+            em += wmass[w];
+        }
+        total += wcnt[w];
+    }
+    uint32_t first = 0xFFFFFFFFu;  // first descending position where the suffix covers the target
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const int d = K * t + i;
+        if (d < TPB_NB) {
+            const int b = TPB_NB - 1 - d;
+            off[b]      = ec;
+            ec += cnt[b];
+            em += mass[b];
+            if (em >= target && first == 0xFFFFFFFFu) {
+                first = (uint32_t)d;
+            }
+        }
+    }
+    first = block_min<uint32_t>(first, red32, 0xFFFFFFFFu);
+    const int cut = first == 0xFFFFFFFFu ? 0 : TPB_NB - 1 - (int)first;
+    m.cut         = cut;
+    m.n_pos       = (int)total;
+    m.n           = (int)(off[cut] + cnt[cut]);
+
+    // where chunk j continues inside bucket b
+    for (int b = cut + t; b < TPB_NB; b += TPH_THREADS) {
+        uint32_t at = off[b];
+        for (int j = 0; j < S; ++j) {
+            start[base + (size_t)j * TPB_NB + b] = at;
+            at += part_cnt[base + (size_t)j * TPB_NB + b];
+        }
+    }
+    // Segments of whole buckets, in descending order: a bucket closes a segment when a multiple of
+    // TPS_SEG lies inside it or at its end, and the last gathered bucket closes the last one. A segment
+    // is therefore shorter than TPS_SEG plus its closing bucket. Segment i is [ends[i-1], ends[i]).
+    const uint32_t n_gathered = (uint32_t)m.n;
+    uint32_t       closes[K];
+    uint32_t       lclose = 0;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const int d = K * t + i;
+        closes[i]   = 0u;
+        if (d < TPB_NB && TPB_NB - 1 - d >= cut) {
+            const int      b = TPB_NB - 1 - d;
+            const uint32_t o = off[b];
+            const uint32_t e = o + cnt[b];
+            if (cnt[b] != 0u && (e / TPS_SEG != o / TPS_SEG || e == n_gathered)) {
+                closes[i] = e;
+                lclose++;
+            }
+        }
+    }
+    uint32_t iclose = lclose;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const uint32_t up = __shfl_up(iclose, o, WAVE);
+        if (lane_id() >= o) {
+            iclose += up;
+        }
+    }
+    __syncthreads();
+    if (lane_id() == WAVE - 1) {
+        wcnt[wave_id()] = iclose;
+    }
+    __syncthreads();
+    uint32_t at   = iclose - lclose;
+    uint32_t nseg = 0;
+    for (int w = 0; w < TPH_THREADS / WAVE; ++w) {
+        at += w < wave_id() ? wcnt[w] : 0u;
+        nseg += wcnt[w];
+    }
+    uint32_t* ends = seg_ends + (size_t)row * TPB_NB;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        if (closes[i] != 0u) {
+            ends[at++] = closes[i];
+        }
+    }
+    if (t == 0) {
+        m.nseg    = (int)nseg;
+        meta[row] = m;
+    }
+}
+
+template<int DT>
+__global__ void __launch_bounds__(TPH_THREADS)
+topp_gather_kernel(const typename Storage<DT>::T* __restrict__ probs, int vocab, int chunk,
+                   const ToppRowMeta* __restrict__ meta, const uint32_t* __restrict__ start,
+                   unsigned long long* __restrict__ sorted)
+{
+    __shared__ uint32_t cur[TPB_NB];
+    const int           row = blockIdx.y;
+    const int           j   = blockIdx.x;
+    const int           S   = gridDim.x;
+    const int           t   = threadIdx.x;
+    const ToppRowMeta   m   = meta[row];
+    if (m.flags != 0 || m.n == 0) {
+        return;
+    }
+    const size_t base = ((size_t)row * S + j) * TPB_NB;
+    for (int b = m.cut + t; b < TPB_NB; b += TPH_THREADS) {
+        cur[b] = start[base + b];
+    }
+    __syncthreads();
+    const int           lo  = (int)min((long long)vocab, (long long)j * chunk);
+    const int           hi  = (int)min((long long)vocab, (long long)lo + chunk);
+    const int           cut = m.cut;
+    unsigned long long* A   = sorted + (size_t)row * 2 * vocab;
+    stream_columns<DT, TPH_THREADS>(probs + (size_t)row * vocab, lo, hi, [&](int v, float x) {
+        const uint32_t k = order_key(x);
+        if (k > ZERO_KEY) {
+            const int b = topp_bucket(k);
+            if (b >= cut) {
+                const uint32_t slot = atomicAdd(&cur[b], 1u);
+                A[slot]             = ((unsigned long long)(~k) << 32) | (uint32_t)v;
+            }
+        }
+    });
+}
+
+// Scratch of the radix sort below.
+struct RadixScratch {
+    unsigned short*     cnt16;  // [16][TP_THREADS]
+    int*                wtot;   // [256]
+    unsigned long long* red64;  // [16]
+};
+
+// Stable LSD radix sort (4-bit digits over bits [lowbit, 64)) of n 64-bit entries in memory by a
+// TP_THREADS workgroup; digits that are constant over the range are skipped. Thread t owns the
+// contiguous slice [t*chunk, (t+1)*chunk), n <= 65535 * TP_THREADS. Returns where the result is
+// (a or b).
+__device__ unsigned long long* radix_sort_range(unsigned long long* a, unsigned long long* b, int n, int lowbit,
+                                                RadixScratch rs)
 {
     const int t     = threadIdx.x;
-    const int group = t >> 5;   // one 32-lane group per tile
-    const int l     = t & 31;   // raking lane: items 8l .. 8l+7 of the tile
-    float     x[8];
-    float     incl = 0.0f;
-    if (group < nt) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int i = group * TP_TILE + l * 8 + j;
-            x[j]        = i < n_in_buf ? key64_prob(s.buf[i]) : 0.0f;
+    const int chunk = (n + TP_THREADS - 1) / TP_THREADS;
+    const int lo    = min(n, t * chunk);
+    const int hi    = min(n, lo + chunk);
+    unsigned long long vor = 0ull, vand = ~0ull;
+    for (int i = lo; i < hi; ++i) {
+        vor |= a[i];
+        vand &= a[i];
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        vor |= __shfl_xor(vor, o, WAVE);
+        vand &= __shfl_xor(vand, o, WAVE);
+    }
+    __syncthreads();
+    if (lane_id() == 0) {
+        rs.red64[wave_id()] = vor;
+    }
+    __syncthreads();
+    unsigned long long all_or = 0ull;
+    for (int w = 0; w < TP_THREADS / WAVE; ++w) {
+        all_or |= rs.red64[w];
+    }
+    __syncthreads();
+    if (lane_id() == 0) {
+        rs.red64[wave_id()] = vand;
+    }
+    __syncthreads();
+    unsigned long long all_and = ~0ull;
+    for (int w = 0; w < TP_THREADS / WAVE; ++w) {
+        all_and &= rs.red64[w];
+    }
+    __syncthreads();
+    const unsigned long long diff = all_or ^ all_and;
+
+    unsigned long long* src = a;
+    unsigned long long* dst = b;
+    for (int shift = lowbit; shift < 64; shift += 4) {
+        if (((diff >> shift) & 0xFull) == 0ull) {
+            continue;
         }
-        float seg = x[0];
-#pragma unroll
-        for (int j = 1; j < 8; ++j) {
-            seg = seg + x[j];
+        // 1. private digit counts
+        for (int d = 0; d < 16; ++d) {
+            rs.cnt16[d * TP_THREADS + t] = 0;
         }
-        incl = seg;
+        for (int i = lo; i < hi; ++i) {
+            const int d = (int)((src[i] >> shift) & 0xFull);
+            rs.cnt16[d * TP_THREADS + t]++;
+        }
+        // 2. exclusive prefix over (digit major, thread minor)
+        int base_off[16];
 #pragma unroll
-        for (int d = 1; d < 32; d <<= 1) {
-            const float up = __shfl_up(incl, d, 32);
-            if (l >= d) {
-                incl = up + incl;
+        for (int d = 0; d < 16; ++d) {
+            const int val = rs.cnt16[d * TP_THREADS + t];
+            int       inc = val;
+#pragma unroll
+            for (int o = 1; o < WAVE; o <<= 1) {
+                const int up = __shfl_up(inc, o, WAVE);
+                if (lane_id() >= o) {
+                    inc += up;
+                }
+            }
+            base_off[d] = inc - val;
+            if (lane_id() == WAVE - 1) {
+                rs.wtot[d * 16 + wave_id()] = inc;
             }
         }
-        if (l == 31) {
-            s.agg[group] = incl;
-        }
-    }
-    __syncthreads();
-    if (t == 0) {
-        float c    = carry_in;
-        s.carry[0] = c;
-        for (int g = 0; g < nt; ++g) {
-            c              = c + s.agg[g];
-            s.carry[g + 1] = c;
-        }
-    }
-    __syncthreads();
-    if (group < nt) {
-        const float excl   = __shfl_up(incl, 1, 32);
-        const float prefix = s.carry[group];
-        float       a      = l == 0 ? prefix : prefix + excl;
-        uint32_t    m8     = 0;
+        __syncthreads();
+        {
+            int digit_base = 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            a = a + x[j];
-            if (rand_num <= a) {
-                m8 |= 1u << j;
+            for (int d = 0; d < 16; ++d) {
+                int pre = 0, tot = 0;
+                for (int w = 0; w < TP_THREADS / WAVE; ++w) {
+                    const int x = rs.wtot[d * 16 + w];
+                    pre += w < wave_id() ? x : 0;
+                    tot += x;
+                }
+                base_off[d] += digit_base + pre;
+                digit_base += tot;
             }
         }
-        reinterpret_cast<unsigned char*>(&s.tilemask[group][0])[l] = (unsigned char)m8;
+        __syncthreads();
+        // 3. stable scatter
+        for (int i = lo; i < hi; ++i) {
+            const unsigned long long e = src[i];
+            const int                d = (int)((e >> shift) & 0xFull);
+            int                      pos = 0;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                if (q == d) {
+                    pos = base_off[q]++;
+                }
+            }
+            dst[pos] = e;
+        }
+        __threadfence_block();
+        __syncthreads();
+        unsigned long long* tmp = src;
+        src                     = dst;
+        dst                     = tmp;
     }
-    __syncthreads();
-    if (t == 0) {
-        int found = -1;
-        for (int g = 0; g < nt && found < 0; ++g) {
-            for (int w = 0; w < 8; ++w) {
-                const uint32_t m = s.tilemask[g][w];
-                if (m != 0u) {
-                    found = g * TP_TILE + w * 32 + (32 - __popc(m));
-                    break;
+    return src;
+}
+
+// Ascending bitonic sort of 64 * R 64-bit keys held R per lane by one wave; key r of lane l has the
+// position r * 64 + l. Exchanges inside a register go through lane shuffles, the others stay in the
+// lane.
+template<int R>
+__device__ __forceinline__ void wave_sort_u64(unsigned long long (&v)[R])
+{
+    const int lane = lane_id();
+#pragma unroll
+    for (int k = 2; k <= 64 * R; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            if (j < 64) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int                idx   = r * 64 + lane;
+                    const unsigned long long other = __shfl_xor(v[r], j, WAVE);
+                    const bool               up    = (idx & k) == 0;
+                    const bool               lower = (idx & j) == 0;
+                    const bool               less  = other < v[r];
+                    // the lower position keeps the smaller key in ascending runs
+                    v[r] = ((lower == up) == less) ? other : v[r];
+                }
+            }
+            else {
+                const int jj = j >> 6;
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    if ((r & jj) == 0) {
+                        const bool               up = ((r * 64) & k) == 0;
+                        const unsigned long long a  = v[r];
+                        const unsigned long long b  = v[r | jj];
+                        const bool               sw = (a > b) == up;
+                        v[r]                        = sw ? b : a;
+                        v[r | jj]                   = sw ? a : b;
+                    }
                 }
             }
         }
-        s.misc[0] = found;
+    }
+}
+
+// One wave sorts buf[s0, s0 + len), len <= 64 * R, and writes the result to out[s0, ...).
+template<int R>
+__device__ __forceinline__ void wave_sort_group(const unsigned long long* buf, unsigned long long* out, int s0, int len)
+{
+    const int          lane = lane_id();
+    unsigned long long v[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int i = r * 64 + lane;
+        v[r]        = i < len ? buf[s0 + i] : ~0ull;
+    }
+    wave_sort_u64<R>(v);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int i = r * 64 + lane;
+        if (i < len) {
+            out[s0 + i] = v[r];
+        }
+    }
+}
+
+constexpr int TPS_DIGITS = 1024;  // bins of the partition inside a segment
+constexpr int TPS_GROUP  = 48;    // group boundaries follow multiples of this
+constexpr int TPS_EPT    = (TPS_CAP + TP_THREADS - 1) / TP_THREADS;
+
+// The radix path needs 32 KB of digit counters; its small arrays live behind them in the same buffer.
+struct ToppSortShared {
+    unsigned long long buf[TPS_CAP];
+    uint32_t           hist[TPS_DIGITS];  // entries per bin, then the write cursors
+    uint32_t           base[TPS_DIGITS];  // first position of a bin
+    uint32_t           gend[TPS_DIGITS];  // end of every group of bins
+    uint32_t           psum[TP_THREADS];  // running number of segments over a tile of rows
+    uint32_t           wtot[TP_THREADS / WAVE];
+    uint32_t           red32[16];
+    int                big[64];           // groups left to the whole workgroup
+    int                nbig;
+};
+static_assert(sizeof(ToppSortShared) <= 65536, "static LDS");
+
+// Inclusive scan of one value per thread over the TP_THREADS threads; `total` gets the sum. Two barriers.
+__device__ __forceinline__ uint32_t block_scan_incl(uint32_t v, uint32_t* wtot, uint32_t& total)
+{
+    uint32_t inc = v;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+        const uint32_t up = __shfl_up(inc, o, WAVE);
+        if (lane_id() >= o) {
+            inc += up;
+        }
     }
     __syncthreads();
-    const int found = s.misc[0];
+    if (lane_id() == WAVE - 1) {
+        wtot[wave_id()] = inc;
+    }
     __syncthreads();
-    return found;
+    total = 0;
+    for (int w = 0; w < TP_THREADS / WAVE; ++w) {
+        const uint32_t x = wtot[w];
+        inc += w < wave_id() ? x : 0u;
+        total += x;
+    }
+    return inc;
+}
+
+// Sorts seg[0, n) ascending (descending probability, ascending id among equals), n <= TPS_CAP: the keys
+// are spread over TPS_DIGITS bins of equal width between the smallest and the largest, neighbouring
+// bins are joined into groups of about TPS_GROUP entries, and every group is sorted by one wave in
+// registers. A group too long for that (equal keys land in one bin) is left to the whole workgroup.
+__device__ void sort_segment(ToppSortShared& s, unsigned long long* __restrict__ seg, int n)
+{
+    const int          t = threadIdx.x;
+    unsigned long long e[TPS_EPT];
+    uint32_t           kmin = 0xFFFFFFFFu, kmax = 0u;
+#pragma unroll
+    for (int r = 0; r < TPS_EPT; ++r) {
+        const int i = t + r * TP_THREADS;
+        if (i < n) {
+            e[r]             = seg[i];
+            const uint32_t h = (uint32_t)(e[r] >> 32);
+            kmin             = min(kmin, h);
+            kmax             = max(kmax, h);
+        }
+    }
+    s.hist[t] = 0u;  // TPS_DIGITS == TP_THREADS
+    if (t == 0) {
+        s.nbig = 0;
+    }
+    kmin = block_min<uint32_t>(kmin, s.red32, 0xFFFFFFFFu);
+    kmax = block_max<uint32_t>(kmax, s.red32, 0u);
+    const uint32_t range = kmax - kmin;
+    const int      nbits = range == 0u ? 0 : 32 - __clz(range);
+    const int      shift = nbits > 10 ? nbits - 10 : 0;
+#pragma unroll
+    for (int r = 0; r < TPS_EPT; ++r) {
+        if (t + r * TP_THREADS < n) {
+            atomicAdd(&s.hist[((uint32_t)(e[r] >> 32) - kmin) >> shift], 1u);
+        }
+    }
+    __syncthreads();
+    const uint32_t cnt = s.hist[t];
+    uint32_t       total;
+    const uint32_t en = block_scan_incl(cnt, s.wtot, total);
+    const uint32_t o  = en - cnt;
+    s.base[t]         = o;
+    s.hist[t]         = 0u;
+    const bool     closes = cnt != 0u && (en / TPS_GROUP != o / TPS_GROUP || en == (uint32_t)n);
+    uint32_t       ngroups;
+    const uint32_t gi = block_scan_incl(closes ? 1u : 0u, s.wtot, ngroups);
+    if (closes) {
+        s.gend[gi - 1] = en;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < TPS_EPT; ++r) {
+        if (t + r * TP_THREADS < n) {
+            const uint32_t d   = ((uint32_t)(e[r] >> 32) - kmin) >> shift;
+            const uint32_t pos = s.base[d] + atomicAdd(&s.hist[d], 1u);
+            s.buf[pos]         = e[r];
+        }
+    }
+    __syncthreads();
+    for (int g = wave_id(); g < (int)ngroups; g += TP_THREADS / WAVE) {
+        const int s0  = g > 0 ? (int)s.gend[g - 1] : 0;
+        const int len = (int)s.gend[g] - s0;
+        if (len <= 64) {
+            wave_sort_group<1>(s.buf, seg, s0, len);
+        }
+        else if (len <= 128) {
+            wave_sort_group<2>(s.buf, seg, s0, len);
+        }
+        else if (len <= 256) {
+            wave_sort_group<4>(s.buf, seg, s0, len);
+        }
+        else if (lane_id() == 0) {
+            const int slot = atomicAdd(&s.nbig, 1);
+            if (slot < 64) {
+                s.big[slot] = g;
+            }
+        }
+    }
+    __syncthreads();
+    const int nbig = s.nbig;
+    if (nbig > 64) {
+        // cannot happen with more than 256 entries per long group and n <= TPS_CAP; sort everything
+        block_sort_u64<TP_THREADS>(s.buf, n);
+        for (int i = t; i < n; i += TP_THREADS) {
+            seg[i] = s.buf[i];
+        }
+    }
+    else {
+        for (int q = 0; q < nbig; ++q) {
+            const int g   = s.big[q];
+            const int s0  = g > 0 ? (int)s.gend[g - 1] : 0;
+            const int len = (int)s.gend[g] - s0;
+            block_sort_u64<TP_THREADS>(s.buf + s0, len);
+            for (int i = t; i < len; i += TP_THREADS) {
+                seg[s0 + i] = s.buf[s0 + i];
+            }
+        }
+    }
+    __syncthreads();
+}
+
+// Every workgroup takes the segments whose running number over all rows is its own modulo the grid.
+__global__ void __launch_bounds__(TP_THREADS)
+topp_sort_kernel(unsigned long long* __restrict__ sorted, const uint32_t* __restrict__ seg_ends,
+                 const ToppRowMeta* __restrict__ meta, int vocab, int rows)
+{
+    __shared__ ToppSortShared s;
+    const int                 t     = threadIdx.x;
+    const uint32_t            G     = gridDim.x;
+    uint32_t                  first = 0;  // running number of the first segment of the tile
+    for (int rb = 0; rb < rows; rb += TP_THREADS) {
+        const int row = rb + t;
+        uint32_t  my  = 0;
+        if (row < rows && meta[row].flags == 0) {
+            my = (uint32_t)meta[row].nseg;
+        }
+        uint32_t       tile_total;
+        const uint32_t incl = block_scan_incl(my, s.wtot, tile_total);
+        s.psum[t]           = incl;
+        __syncthreads();
+        uint32_t w = first + (blockIdx.x + G - first % G) % G;
+        for (; w < first + tile_total; w += G) {
+            const uint32_t local = w - first;
+            int            lo = 0, hi = TP_THREADS - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (s.psum[mid] > local) {
+                    hi = mid;
+                }
+                else {
+                    lo = mid + 1;
+                }
+            }
+            const int       r    = rb + lo;
+            const int       i    = (int)(local - (lo > 0 ? s.psum[lo - 1] : 0u));
+            const uint32_t* ends = seg_ends + (size_t)r * TPB_NB;
+            const uint32_t  s0   = i > 0 ? ends[i - 1] : 0u;
+            const int       n    = (int)(ends[i] - s0);
+            unsigned long long* A   = sorted + (size_t)r * 2 * vocab;
+            unsigned long long* seg = A + s0;
+            if (n < 2) {
+                continue;
+            }
+            if (n <= TPS_CAP) {
+                sort_segment(s, seg, n);
+            }
+            else {
+                RadixScratch        rs{reinterpret_cast<unsigned short*>(s.buf), reinterpret_cast<int*>(s.buf + 4096),
+                                reinterpret_cast<unsigned long long*>(s.buf + 4096 + 128)};
+                unsigned long long* res = radix_sort_range(seg, A + vocab + s0, n, 0, rs);
+                if (res != seg) {
+                    for (int q = t; q < n; q += TP_THREADS) {
+                        seg[q] = res[q];
+                    }
+                }
+                __threadfence_block();
+                __syncthreads();
+            }
+        }
+        first += tile_total;
+        __syncthreads();
+    }
+}
+
+struct TopPShared {
+    unsigned long long buf[4096];  // digit counters of the fallback sort
+    unsigned long long red64[16];
+    uint32_t           red32[16];
+    float              agg[TP_ROUND];
+    float              carry[TP_ROUND + 1];
+    uint32_t           tilemask[32][8];
+    int                wtot[256];
+    int                misc[8];
+    float              fmisc[4];
+};
+
+// One 32-lane group loads the eight items of each of its lanes from tile `tile` of the ordered
+// array (entries at or beyond n count as 0) and returns the inclusive raking scan of the lane totals.
+__device__ __forceinline__ float tile_partials(const unsigned long long* __restrict__ src, int n, int tile, int l,
+                                               float x[8])
+{
+    const int i0 = tile * TP_TILE + l * 8;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        x[j] = i0 + j < n ? key64_prob(src[i0 + j]) : 0.0f;
+    }
+    float seg = x[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) {
+        seg = seg + x[j];
+    }
+    float incl = seg;
+#pragma unroll
+    for (int d = 1; d < 32; d <<= 1) {
+        const float up = __shfl_up(incl, d, 32);
+        if (l >= d) {
+            incl = up + incl;
+        }
+    }
+    return incl;
+}
+
+// Replays the reference scan over the ordered array `src[0, n)`. Returns the position the
+// reference would pick (it can lie in the zero padding of the last tile, >= n) or -1 when the draw
+// is never reached. All threads must call; the result is block-uniform.
+__device__ int scan_sorted(TopPShared& s, const unsigned long long* __restrict__ src, int n, float rand_num)
+{
+    const int t     = threadIdx.x;
+    const int group = t >> 5;
+    const int l     = t & 31;
+    const int nt    = (n + TP_TILE - 1) / TP_TILE;
+    // a tile whose running total stays below this cannot hold the crossing: the prefixes inside a
+    // tile and the tile's total differ by rounding only
+    const float near = rand_num * (1.0f - 1.0f / 4096.0f);
+    float       carry_in = 0.0f;
+    for (int base = 0; base < nt; base += TP_ROUND) {
+        const int ntr = min(TP_ROUND, nt - base);
+        for (int g = group; g < ntr; g += TP_THREADS / 32) {
+            float       x[8];
+            const float incl = tile_partials(src, n, base + g, l, x);
+            if (l == 31) {
+                s.agg[g] = incl;
+            }
+        }
+        __syncthreads();
+        if (t == 0) {
+            float c  = carry_in;
+            int   g0 = -1;
+            for (int g = 0; g < ntr; ++g) {
+                s.carry[g] = c;
+                c          = c + s.agg[g];
+                if (g0 < 0 && c >= near) {
+                    g0 = g;
+                }
+            }
+            s.carry[ntr] = c;
+            s.misc[1]    = g0;
+        }
+        __syncthreads();
+        const int g0 = s.misc[1];
+        if (g0 >= 0) {
+            for (int gs = g0; gs < ntr; gs += TP_THREADS / 32) {
+                const int g  = gs + group;
+                uint32_t  m8 = 0;
+                if (g < ntr) {
+                    float       x[8];
+                    const float incl   = tile_partials(src, n, base + g, l, x);
+                    const float excl   = __shfl_up(incl, 1, 32);
+                    const float prefix = s.carry[g];
+                    float       a      = l == 0 ? prefix : prefix + excl;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        a = a + x[j];
+                        if (rand_num <= a) {
+                            m8 |= 1u << j;
+                        }
+                    }
+                }
+                reinterpret_cast<unsigned char*>(&s.tilemask[group][0])[l] = (unsigned char)m8;
+                __syncthreads();
+                if (t == 0) {
+                    int found = -1;
+                    for (int q = 0; q < TP_THREADS / 32 && found < 0; ++q) {
+                        for (int w = 0; w < 8; ++w) {
+                            const uint32_t mk = s.tilemask[q][w];
+                            if (mk != 0u) {
+                                found = (base + gs + q) * TP_TILE + w * 32 + (32 - __popc(mk));
+                                break;
+                            }
+                        }
+                    }
+                    s.misc[0] = found;
+                }
+                __syncthreads();
+                const int found = s.misc[0];
+                __syncthreads();
+                if (found >= 0) {
+                    return found;
+                }
+            }
+        }
+        carry_in = s.carry[ntr];
+        __syncthreads();
+    }
+    return -1;
 }
 
 // id of the `nth` (0-based) entry with probability exactly zero, in ascending id order: what a
@@ -228,40 +1157,25 @@ __device__ int nth_zero_entry(const typename Storage<DT>::T* __restrict__ rowp, 
 
 template<int DT>
 __global__ void __launch_bounds__(TP_THREADS)
-topp_kernel(const typename Storage<DT>::T* __restrict__ probs, int* __restrict__ ids,
-            int* __restrict__ sequence_length, bool* __restrict__ finished, float* __restrict__ cum_log_probs,
-            float* __restrict__ output_log_probs, RngState* rng, const float* __restrict__ uniforms, int vocab,
-            const int* __restrict__ end_ids, float top_p, const float* __restrict__ top_ps,
-            const bool* __restrict__ skip_decode, unsigned long long* __restrict__ workspace, int force_deep)
+topp_pick_kernel(const typename Storage<DT>::T* __restrict__ probs, int* __restrict__ ids,
+                 int* __restrict__ sequence_length, bool* __restrict__ finished, float* __restrict__ cum_log_probs,
+                 float* __restrict__ output_log_probs, RngState* rng, const float* __restrict__ uniforms, int vocab,
+                 const int* __restrict__ end_ids, float top_p, const float* __restrict__ top_ps,
+                 const bool* __restrict__ skip_decode, unsigned long long* __restrict__ sorted,
+                 const ToppRowMeta* __restrict__ meta, int force_deep)
 {
-    typedef Storage<DT>            S;
-    __shared__ TopPShared          s;
-    const int                      row = blockIdx.x;
-    const int                      t   = threadIdx.x;
+    typedef Storage<DT>   S;
+    __shared__ TopPShared s;
+    const int             row = blockIdx.x;
+    const int             t   = threadIdx.x;
     if (skip_decode != nullptr && skip_decode[row]) {
         return;
     }
     const typename S::T* rowp = probs + (size_t)row * vocab;
     const float          p    = top_ps != nullptr ? top_ps[row] : top_p;
-
-    // ---- pass 1: arg-max (lowest id on ties), positive count, thread maximum
-    uint32_t tmax = 0;
-    int      tidx = 0x7FFFFFFF;
-    int      npos = 0;
-    for (int v = t; v < vocab; v += TP_THREADS) {
-        const uint32_t k = order_key(S::ld(rowp[v]));
-        if (k > tmax) {
-            tmax = k;
-            tidx = v;
-        }
-        npos += k > ZERO_KEY ? 1 : 0;
-    }
-    // (key, ~id) packs "largest key, then lowest id" into one max-reduction
-    unsigned long long best = ((unsigned long long)tmax << 32) | (uint32_t)(~(uint32_t)tidx);
-    best                    = block_max<unsigned long long>(best, s.red64, 0ull);
-    const int n_pos         = block_sum_i(npos, (int*)s.red32);
-    int       best_id       = (int)(~(uint32_t)best);
-    if ((uint32_t)(best >> 32) == 0u) {
+    const ToppRowMeta    m    = meta[row];
+    int                  best_id = (int)(~(uint32_t)m.best);
+    if ((uint32_t)(m.best >> 32) == 0u) {
         best_id = 0;  // nothing comparable in the row (all NaN): the reference keeps index 0
     }
     const float best_prob = S::ld(rowp[best_id]);
@@ -302,89 +1216,45 @@ topp_kernel(const typename Storage<DT>::T* __restrict__ probs, int* __restrict__
         ids[row] = best_id;  // kept when no prefix sum ever reaches the draw (:954)
     }
 
-    bool done = false;
-    if (!force_deep) {
-        // ---- threshold from the order statistics of the 1024 thread maxima: every wave sorts its
-        // 64 maxima; the q-th largest of each wave, minimised over the 16 waves, has at least 16q
-        // entries above it. Four candidates, tightest first.
-        const uint32_t sorted = wave_sort_desc(tmax);
-        const int      qs[4]  = {30, 16, 6, 1};
-        for (int a = 0; a < 4 && !done; ++a) {
-            uint32_t cand = __shfl(sorted, qs[a] - 1, WAVE);
-            uint32_t t0   = block_min<uint32_t>(cand, s.red32, 0xFFFFFFFFu);
-            if (t0 <= ZERO_KEY) {
-                t0 = ZERO_KEY + 1;
-            }
+    unsigned long long* A = sorted + (size_t)row * 2 * vocab;
+    unsigned long long* B = A + vocab;
+    if (!force_deep && m.flags == 0) {
+        const bool all   = m.n == m.n_pos;
+        const int  found = m.n > 0 ? scan_sorted(s, A, m.n, rand_num) : -1;
+        if (found >= 0 && (found < m.n || all)) {
             if (t == 0) {
-                s.counter = 0;
-            }
-            __syncthreads();
-            for (int v = t; v < vocab; v += TP_THREADS) {
-                const uint32_t k = order_key(S::ld(rowp[v]));
-                if (k >= t0) {
-                    const int slot = atomicAdd(&s.counter, 1);
-                    if (slot < TP_BUF) {
-                        s.buf[slot] = ((unsigned long long)(~k) << 32) | (uint32_t)v;
-                    }
+                if (found < m.n) {
+                    const unsigned long long e = A[found];
+                    emit((int)(uint32_t)e, key64_prob(e));
+                }
+                else {
+                    const int id = nth_zero_entry<DT>(rowp, vocab, found - m.n);
+                    emit(id, S::ld(rowp[id]));
                 }
             }
-            __syncthreads();
-            const int n = s.counter;
-            __syncthreads();
-            if (n > TP_BUF) {
-                continue;  // too many ties / too flat at this quantile: try a tighter threshold
-            }
-            const int np2 = max(2, next_pow2(n));
-            for (int i = n + t; i < np2; i += TP_THREADS) {
-                s.buf[i] = ~0ull;
-            }
-            __syncthreads();
-            block_bitonic_sort_u64(s.buf, np2);
-            const bool all = n == n_pos;
-            const int  nt  = all ? (n + TP_TILE - 1) / TP_TILE : n / TP_TILE;
-            if (nt > 0) {
-                const int found = eval_tiles(s, n, nt, 0.0f, rand_num);
-                if (found >= 0) {
-                    if (t == 0) {
-                        if (found < n) {
-                            const unsigned long long e = s.buf[found];
-                            emit((int)(uint32_t)e, key64_prob(e));
-                        }
-                        else {
-                            const int id = nth_zero_entry<DT>(rowp, vocab, found - n);
-                            emit(id, S::ld(rowp[id]));
-                        }
-                    }
-                    return;
-                }
-            }
-            if (all) {
-                return;  // every positive entry scanned, never crossed: ids keeps the arg-max
-            }
-            break;  // sorted prefix exhausted without crossing: deep path
+            return;
+        }
+        if (all) {
+            return;  // every positive entry scanned, never crossed: ids keeps the arg-max
         }
     }
 
-    // ---- deep path: stable LSD radix sort (4-bit digits) of all positive entries in `workspace`
-    // (2 * vocab 64-bit slots per row), then the same scan over the whole sorted row.
-    unsigned long long* A = workspace + (size_t)row * 2 * vocab;
-    unsigned long long* B = A + vocab;
-    // stable compaction in id order, 1024 consecutive ids per round
+    // ---- fallback: every positive entry, compacted in id order, stable radix sort on the key bits
     if (t == 0) {
-        s.misc[1] = 0;
+        s.misc[2] = 0;
     }
     __syncthreads();
     for (int base = 0; base < vocab; base += TP_THREADS) {
-        const int      v    = base + t;
-        const uint32_t k    = v < vocab ? order_key(S::ld(rowp[v])) : 0u;
-        const bool     keep = k > ZERO_KEY;
-        const unsigned long long bal = __ballot(keep);
-        const int      below = __popcll(bal & ((1ull << lane_id()) - 1ull));
+        const int                v    = base + t;
+        const uint32_t           k    = v < vocab ? order_key(S::ld(rowp[v])) : 0u;
+        const bool               keep = k > ZERO_KEY;
+        const unsigned long long bal  = __ballot(keep);
+        const int                below = __popcll(bal & ((1ull << lane_id()) - 1ull));
         if (lane_id() == 0) {
             s.red32[wave_id()] = (uint32_t)__popcll(bal);
         }
         __syncthreads();
-        int off = s.misc[1];
+        int off = s.misc[2];
         for (int w = 0; w < wave_id(); ++w) {
             off += (int)s.red32[w];
         }
@@ -397,141 +1267,24 @@ topp_kernel(const typename Storage<DT>::T* __restrict__ probs, int* __restrict__
             for (int w = 0; w < TP_THREADS / WAVE; ++w) {
                 tot += (int)s.red32[w];
             }
-            s.misc[1] += tot;
+            s.misc[2] += tot;
         }
         __syncthreads();
     }
-    const int n = s.misc[1];  // == n_pos
-    // digit passes over bits 32..63; thread t owns the contiguous slice [t*chunk, (t+1)*chunk)
-    {
-        // [16][1024] 16-bit counters alias the (idle) sort buffer; a slice holds <= 65535 entries
-        unsigned short* cnt16 = reinterpret_cast<unsigned short*>(s.buf);
-        const int       chunk = (n + TP_THREADS - 1) / TP_THREADS;
-        const int       lo    = min(n, t * chunk);
-        const int       hi    = min(n, lo + chunk);
-        // digits that are constant over the whole row need no pass
-        unsigned long long vor = 0ull, vand = ~0ull;
-        for (int i = lo; i < hi; ++i) {
-            vor |= A[i];
-            vand &= A[i];
+    const int n = s.misc[2];
+    __threadfence_block();
+    __syncthreads();
+    RadixScratch              rs{reinterpret_cast<unsigned short*>(s.buf), s.wtot, s.red64};
+    const unsigned long long* src   = radix_sort_range(A, B, n, 32, rs);
+    const int                 found = n > 0 ? scan_sorted(s, src, n, rand_num) : -1;
+    if (found >= 0 && t == 0) {
+        if (found < n) {
+            const unsigned long long e = src[found];
+            emit((int)(uint32_t)e, key64_prob(e));
         }
-        for (int o = 32; o > 0; o >>= 1) {
-            vor |= __shfl_xor(vor, o, WAVE);
-            vand &= __shfl_xor(vand, o, WAVE);
-        }
-        if (lane_id() == 0) {
-            s.red64[wave_id()] = vor;
-        }
-        __syncthreads();
-        unsigned long long all_or = 0ull;
-        for (int w = 0; w < TP_THREADS / WAVE; ++w) {
-            all_or |= s.red64[w];
-        }
-        __syncthreads();
-        if (lane_id() == 0) {
-            s.red64[wave_id()] = vand;
-        }
-        __syncthreads();
-        unsigned long long all_and = ~0ull;
-        for (int w = 0; w < TP_THREADS / WAVE; ++w) {
-            all_and &= s.red64[w];
-        }
-        __syncthreads();
-        const unsigned long long diff = all_or ^ all_and;
-
-        unsigned long long* src = A;
-        unsigned long long* dst = B;
-        for (int shift = 32; shift < 64; shift += 4) {
-            if (((diff >> shift) & 0xFull) == 0ull) {
-                continue;
-            }
-            // 1. private digit counts
-            for (int d = 0; d < 16; ++d) {
-                cnt16[d * TP_THREADS + t] = 0;
-            }
-            for (int i = lo; i < hi; ++i) {
-                const int d = (int)((src[i] >> shift) & 0xFull);
-                cnt16[d * TP_THREADS + t]++;
-            }
-            // 2. exclusive prefix over (digit major, thread minor)
-            int base_off[16];
-#pragma unroll
-            for (int d = 0; d < 16; ++d) {
-                const int val = cnt16[d * TP_THREADS + t];
-                int       inc = val;
-#pragma unroll
-                for (int o = 1; o < WAVE; o <<= 1) {
-                    const int up = __shfl_up(inc, o, WAVE);
-                    if (lane_id() >= o) {
-                        inc += up;
-                    }
-                }
-                base_off[d] = inc - val;
-                if (lane_id() == WAVE - 1) {
-                    s.wtot[d * 16 + wave_id()] = inc;
-                }
-            }
-            __syncthreads();
-            {
-                int digit_base = 0;
-#pragma unroll
-                for (int d = 0; d < 16; ++d) {
-                    int pre = 0, tot = 0;
-                    for (int w = 0; w < TP_THREADS / WAVE; ++w) {
-                        const int x = s.wtot[d * 16 + w];
-                        pre += w < wave_id() ? x : 0;
-                        tot += x;
-                    }
-                    base_off[d] += digit_base + pre;
-                    digit_base += tot;
-                }
-            }
-            __syncthreads();
-            // 3. stable scatter
-            for (int i = lo; i < hi; ++i) {
-                const unsigned long long e = src[i];
-                const int                d = (int)((e >> shift) & 0xFull);
-                int                      pos = 0;
-#pragma unroll
-                for (int q = 0; q < 16; ++q) {
-                    if (q == d) {
-                        pos = base_off[q]++;
-                    }
-                }
-                dst[pos] = e;
-            }
-            __threadfence_block();
-            __syncthreads();
-            unsigned long long* tmp = src;
-            src                     = dst;
-            dst                     = tmp;
-        }
-        // sorted data is in `src`
-        float carry_in = 0.0f;
-        for (int base = 0; base < n; base += TP_BUF) {
-            const int m = min(TP_BUF, n - base);
-            for (int i = t; i < m; i += TP_THREADS) {
-                s.buf[i] = src[base + i];
-            }
-            __syncthreads();
-            const bool last = base + m == n;
-            const int  nt   = last ? (m + TP_TILE - 1) / TP_TILE : m / TP_TILE;  // m == TP_BUF unless last
-            const int  found = eval_tiles(s, m, nt, carry_in, rand_num);
-            if (found >= 0) {
-                if (t == 0) {
-                    if (found < m) {
-                        const unsigned long long e = s.buf[found];
-                        emit((int)(uint32_t)e, key64_prob(e));
-                    }
-                    else {
-                        const int id = nth_zero_entry<DT>(rowp, vocab, base + found - n);
-                        emit(id, S::ld(rowp[id]));
-                    }
-                }
-                return;
-            }
-            carry_in = s.carry[nt];
-            __syncthreads();
+        else {
+            const int id = nth_zero_entry<DT>(rowp, vocab, found - n);
+            emit(id, S::ld(rowp[id]));
         }
     }
 }
@@ -621,8 +1374,11 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     if (dtype < 0 || dtype > 2) {
         return FTK_ERR_DTYPE;
     }
-    // fallback sort: two 64-bit (key, id) arrays per row
-    const size_t need = (size_t)batch_size * vocab_size_padded * 2 * sizeof(unsigned long long);
+    if (batch_size < 0 || batch_size > 65535) {
+        return FTK_ERR_ARGUMENT;
+    }
+    const ToppPlan plan = topp_plan(batch_size, vocab_size_padded);
+    const size_t   need = plan.bytes;
     if (workspace == nullptr) {
         if (workspace_size == nullptr) {
             return FTK_ERR_ARGUMENT;
@@ -645,11 +1401,35 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     if (vocab_size_padded > (size_t)65535 * TP_THREADS) {
         return FTK_ERR_ARGUMENT;
     }
-    FTK_DISPATCH_DTYPE(dtype, topp_kernel<DT><<<batch_size, TP_THREADS, 0, (hipStream_t)stream>>>(
+    char*               ws      = (char*)workspace;
+    unsigned long long* sorted  = (unsigned long long*)ws;
+    uint32_t*           pcnt    = (uint32_t*)(ws + plan.off_pcnt);
+    uint32_t*           pmass   = (uint32_t*)(ws + plan.off_pmass);
+    unsigned long long* pbest   = (unsigned long long*)(ws + plan.off_pbest);
+    uint32_t*           start   = (uint32_t*)(ws + plan.off_start);
+    uint32_t*           segs    = (uint32_t*)(ws + plan.off_seg);
+    ToppRowMeta*        meta    = (ToppRowMeta*)(ws + plan.off_meta);
+    const int           vocab   = (int)vocab_size_padded;
+    hipStream_t         st      = (hipStream_t)stream;
+    const dim3          chunks(plan.splits, batch_size);
+    FTK_DISPATCH_DTYPE(dtype, topp_histogram_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
+                                  (const Storage<DT>::T*)log_probs, vocab, plan.chunk, skip_decode, pcnt, pmass, pbest));
+    FTK_LAUNCH_CHECK();
+    topp_cut_kernel<<<batch_size, TPH_THREADS, 0, st>>>(plan.splits, pcnt, pmass, pbest, start, segs, meta,
+                                                        (const RngState*)rng_state, uniform_draws, max_top_p, top_ps,
+                                                        skip_decode);
+    FTK_LAUNCH_CHECK();
+    if (!g_topp_force_deep) {
+        FTK_DISPATCH_DTYPE(dtype, topp_gather_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
+                                      (const Storage<DT>::T*)log_probs, vocab, plan.chunk, meta, start, sorted));
+        FTK_LAUNCH_CHECK();
+        topp_sort_kernel<<<plan.sorters, TP_THREADS, 0, st>>>(sorted, segs, meta, vocab, batch_size);
+        FTK_LAUNCH_CHECK();
+    }
+    FTK_DISPATCH_DTYPE(dtype, topp_pick_kernel<DT><<<batch_size, TP_THREADS, 0, st>>>(
                                   (const Storage<DT>::T*)log_probs, output_ids, sequence_length, finished,
-                                  cum_log_probs, output_log_probs, (RngState*)rng_state, uniform_draws,
-                                  (int)vocab_size_padded, end_ids, max_top_p, top_ps, skip_decode,
-                                  (unsigned long long*)workspace, g_topp_force_deep));
+                                  cum_log_probs, output_log_probs, (RngState*)rng_state, uniform_draws, vocab,
+                                  end_ids, max_top_p, top_ps, skip_decode, sorted, meta, g_topp_force_deep));
     FTK_LAUNCH_CHECK();
     return 0;
 }
