@@ -74,9 +74,10 @@ __device__ __forceinline__ int wave_sum_i(int v)
     return v;
 }
 
-// Block-wide reductions over blockDim.x threads (multiple of 64, <= 1024). `smem` holds >= 16
-// elements of V. The result is returned to every thread. Two barriers.
-template<typename V>
+// Block-wide reductions over the threads of the block (multiple of 64, <= 1024). `smem` holds >= 16
+// elements of V. The result is returned to every thread. Two barriers. NW is the number of waves of
+// the block when the caller knows it (0: read from the launch, which costs a trip to memory).
+template<typename V, int NW = 0>
 __device__ __forceinline__ V block_max(V v, V* smem, V identity)
 {
     v = wave_max(v);
@@ -84,13 +85,13 @@ __device__ __forceinline__ V block_max(V v, V* smem, V identity)
         smem[wave_id()] = v;
     }
     __syncthreads();
-    const int nw = (int)(blockDim.x >> 6);
+    const int nw = NW > 0 ? NW : (int)(blockDim.x >> 6);
     V         r  = (lane_id() < nw) ? smem[lane_id()] : identity;
     r            = wave_max(r);
     __syncthreads();
     return r;
 }
-template<typename V>
+template<typename V, int NW = 0>
 __device__ __forceinline__ V block_min(V v, V* smem, V identity)
 {
     v = wave_min(v);
@@ -98,12 +99,13 @@ __device__ __forceinline__ V block_min(V v, V* smem, V identity)
         smem[wave_id()] = v;
     }
     __syncthreads();
-    const int nw = (int)(blockDim.x >> 6);
+    const int nw = NW > 0 ? NW : (int)(blockDim.x >> 6);
     V         r  = (lane_id() < nw) ? smem[lane_id()] : identity;
     r            = wave_min(r);
     __syncthreads();
     return r;
 }
+template<int NW = 0>
 __device__ __forceinline__ int block_sum_i(int v, int* smem)
 {
     v = wave_sum_i(v);
@@ -111,7 +113,7 @@ __device__ __forceinline__ int block_sum_i(int v, int* smem)
         smem[wave_id()] = v;
     }
     __syncthreads();
-    const int nw = (int)(blockDim.x >> 6);
+    const int nw = NW > 0 ? NW : (int)(blockDim.x >> 6);
     int       r  = (lane_id() < nw) ? smem[lane_id()] : 0;
     r            = wave_sum_i(r);
     __syncthreads();

@@ -393,7 +393,7 @@ __device__ __noinline__ int topk_stream_rare(Row rowctx, TopkShared& s, int k, i
         for (int v = lo_col + t; v < hi_col; v += TK_THREADS) {
             c += topk_value_at<DT>(rowctx, v) >= f ? 1 : 0;
         }
-        return block_sum_i(c, (int*)s.red32);
+        return block_sum_i<TK_WAVES>(c, (int*)s.red32);
     };
     uint32_t lo = thr, hi = 0xFFFFFFFFu;  // count(lo) > TK_CCAP, count(hi) == 0
     bool     ok = count_ge(thr) <= TK_CCAP;  // (a wave ran out of parking space, the list itself fits)
@@ -550,7 +550,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
             const float    tmax   = __builtin_fmaxf(__builtin_fmaxf(gm[0], gm[1]), __builtin_fmaxf(gm[2], gm[3]));
             const uint32_t sorted = wave_sort_desc(order_key(tmax));
             const int      q      = (k + TK_WAVES - 1) / TK_WAVES;
-            thr = block_min<uint32_t>(__shfl(sorted, q - 1, WAVE), s.red32, 0xFFFFFFFFu);
+            thr = block_min<uint32_t, TK_WAVES>(__shfl(sorted, q - 1, WAVE), s.red32, 0xFFFFFFFFu);
         }
         else {
             // the same with the group maxima: four sorted sequences per wave
@@ -562,7 +562,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
                 const uint32_t qth    = __shfl(sorted, q - 1, WAVE);
                 m                     = qth < m ? qth : m;
             }
-            thr = block_min<uint32_t>(m, s.red32, 0xFFFFFFFFu);
+            thr = block_min<uint32_t, TK_WAVES>(m, s.red32, 0xFFFFFFFFu);
         }
         if (thr < KMIN) {
             thr = KMIN;  // fewer than k usable maxima: take every selectable element
@@ -907,7 +907,7 @@ __device__ void topk_literal(Row& rowctx, TopkShared& s, int vocab, int k, int B
                     }
                 }
             }
-            best = ~block_max<unsigned long long>(~best, s.red64, 0ull);
+            best = ~block_max<unsigned long long, TK_WAVES>(~best, s.red64, 0ull);
             if (t == 0) {
                 TopkEntry e{0u, 0xFFFFFFFFu};
                 if (best != ~0ull) {
@@ -949,7 +949,7 @@ __device__ void topk_literal(Row& rowctx, TopkShared& s, int vocab, int k, int B
                 }
             }
         }
-        best = ~block_max<unsigned long long>(~best, s.red64, 0ull);
+        best = ~block_max<unsigned long long, TK_WAVES>(~best, s.red64, 0ull);
         if (best == ~0ull) {
             break;
         }
@@ -1074,7 +1074,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
             lds_barrier();
             const int q2 = rank(k2);
             const bool kept = k2 != ~0ull;
-            n_list          = block_sum_i(kept ? 1 : 0, (int*)s.red32);
+            n_list          = block_sum_i<TK_WAVES>(kept ? 1 : 0, (int*)s.red32);
             n_list          = n_list < k ? n_list : k;
             if (kept && q2 < n_list) {
                 s.sel.w[q2]   = key_to_float(~(uint32_t)(k2 >> 32));
@@ -1106,7 +1106,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 for (int i = t; i < min(k, n); i += TK_THREADS) {
                     cnt += s.keys[i] != ~0ull ? 1 : 0;
                 }
-                n_list = block_sum_i(cnt, (int*)s.red32);
+                n_list = block_sum_i<TK_WAVES>(cnt, (int*)s.red32);
             }
             // resolve the payload (position in the first sort) into the vocabulary index
             constexpr int LPT = 1024 / TK_THREADS;  // list entries per thread (k <= 1024)
@@ -1231,7 +1231,7 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
                     c += e[i].key >= thr ? 1 : 0;
                 }
             }
-            return block_sum_i(c, (int*)s.red32);
+            return block_sum_i<TK_WAVES>(c, (int*)s.red32);
         };
         uint32_t lo = T0, hi = 0xFFFFFFFFu;  // count(lo) >= k always holds
         while (hi - lo > 1u) {

@@ -152,7 +152,7 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
         if (n_padded > n) {
             mx = __builtin_fmaxf(mx, -MAXT);
         }
-        mx = block_max<float>(mx, sh, -3.402823466e+38f);
+        mx = block_max<float, SM_THREADS / WAVE>(mx, sh, -3.402823466e+38f);
         if (BLK < 1024) {
             mx = __builtin_fmaxf(mx, -1e20f);
         }
@@ -212,7 +212,7 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
             mx = __builtin_fmaxf(mx, masked(v));
         }
     }
-    mx = block_max<float>(mx, sh, -3.402823466e+38f);
+    mx = block_max<float, SM_THREADS / WAVE>(mx, sh, -3.402823466e+38f);
     if (BLK < 1024) {
         mx = __builtin_fmaxf(mx, -1e20f);  // blockReduceMax pads its second stage with -1e20f
     }
@@ -278,6 +278,7 @@ constexpr int      TP_ROUND   = 1024;         // tiles whose totals are held in 
 constexpr uint32_t ZERO_KEY   = 0x80000000u;  // order_key(+0.0f); entries at or below never join the scan
 
 constexpr int TPH_THREADS = 256;
+constexpr int TPC_THREADS = 1024;  // the cut kernel
 constexpr int TPB_SHIFT   = 17;                        // key bits below a bucket (6 mantissa bits stay)
 constexpr int TPB_ONE     = 0x3F800000 >> TPB_SHIFT;   // bucket of 1.0 before the shift of origin
 constexpr int TPB_SPAN    = 32 * 64;                   // 32 octaves below 1.0 are resolved
@@ -304,7 +305,7 @@ struct ToppPlan {
     int    splits;  // chunks per row of the two streaming kernels
     int    chunk;   // columns per chunk
     int    sorters; // workgroups of the sort kernel
-    size_t off_pcnt, off_pmass, off_pbest, off_start, off_seg, off_meta, bytes;
+    size_t off_pcnt, off_pmass, off_pbest, off_start, off_boff, off_seg, off_meta, bytes;
 };
 
 static inline size_t align256(size_t x)
@@ -332,6 +333,8 @@ static ToppPlan topp_plan(int batch, size_t vocab)
     off += align256((size_t)rows * s * sizeof(unsigned long long));
     p.off_start = off;
     off += align256((size_t)rows * s * TPB_NB * sizeof(uint32_t));
+    p.off_boff = off;
+    off += align256((size_t)rows * TPB_NB * sizeof(uint32_t));
     p.off_seg = off;
     off += align256((size_t)rows * TPB_NB * sizeof(uint32_t));
     p.off_meta = off;
@@ -396,7 +399,7 @@ topp_histogram_kernel(const typename Storage<DT>::T* __restrict__ probs, int voc
         part_mass[base + b] = mass[b];
     }
     unsigned long long best = ((unsigned long long)tmax << 32) | (uint32_t)(~(uint32_t)tidx);
-    best                    = block_max<unsigned long long>(best, red, 0ull);
+    best                    = block_max<unsigned long long, TPH_THREADS / WAVE>(best, red, 0ull);
     if (t == 0) {
         part_best[(size_t)row * S + j] = best;
     }
@@ -412,10 +415,11 @@ __device__ __forceinline__ float row_uniform_peek(const RngState* rng, const flo
     return rng_next_uniform(&copy);
 }
 
-__global__ void __launch_bounds__(TPH_THREADS)
+__global__ void __launch_bounds__(TPC_THREADS)
 topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __restrict__ part_mass,
                 const unsigned long long* __restrict__ part_best, uint32_t* __restrict__ start,
-                uint32_t* __restrict__ seg_ends, ToppRowMeta* __restrict__ meta, const RngState* rng,
+                uint32_t* __restrict__ bucket_off, uint32_t* __restrict__ seg_ends, ToppRowMeta* __restrict__ meta,
+                const RngState* rng,
                 const float* __restrict__ uniforms, float top_p, const float* __restrict__ top_ps,
                 const bool* __restrict__ skip_decode)
 {
@@ -423,8 +427,8 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
     __shared__ uint32_t           off[TPB_NB];
     __shared__ unsigned long long mass[TPB_NB];
     __shared__ unsigned long long red64[16];
-    __shared__ uint32_t           wcnt[TPH_THREADS / WAVE];
-    __shared__ unsigned long long wmass[TPH_THREADS / WAVE];
+    __shared__ uint32_t           wcnt[TPC_THREADS / WAVE];
+    __shared__ unsigned long long wmass[TPC_THREADS / WAVE];
     __shared__ uint32_t           red32[16];
     const int                     row = blockIdx.x;
     const int                     t   = threadIdx.x;
@@ -441,23 +445,57 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
         }
         return;
     }
-    const size_t base = (size_t)row * S * TPB_NB;
-    for (int b = t; b < TPB_NB; b += TPH_THREADS) {
-        uint32_t           c  = 0;
-        unsigned long long ms = 0;
-        for (int j = 0; j < S; ++j) {
-            c += part_cnt[base + (size_t)j * TPB_NB + b];
-            ms += part_mass[base + (size_t)j * TPB_NB + b];
+    // sums over the chunks; what the chunks before chunk j hold of a bucket goes to `start` on the way.
+    // All loads of one chunk are issued together: the chunks follow each other, not the buckets.
+    constexpr int      K    = (TPB_NB + TPC_THREADS - 1) / TPC_THREADS;
+    const size_t       base = (size_t)row * S * TPB_NB;
+    uint32_t           c[K];
+    unsigned long long ms[K];
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        c[i]  = 0u;
+        ms[i] = 0ull;
+    }
+    constexpr int J = 8;  // chunks whose loads are in flight together
+    for (int j0 = 0; j0 < S; j0 += J) {
+        uint32_t pc[J][K], pm[J][K];
+#pragma unroll
+        for (int jj = 0; jj < J; ++jj) {
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                const int  b  = t + i * TPC_THREADS;
+                const bool ok = j0 + jj < S && b < TPB_NB;
+                pc[jj][i]     = ok ? part_cnt[base + (size_t)(j0 + jj) * TPB_NB + b] : 0u;
+                pm[jj][i]     = ok ? part_mass[base + (size_t)(j0 + jj) * TPB_NB + b] : 0u;
+            }
         }
-        cnt[b]  = c;
-        mass[b] = ms;
+#pragma unroll
+        for (int jj = 0; jj < J; ++jj) {
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                const int b = t + i * TPC_THREADS;
+                if (j0 + jj < S && b < TPB_NB) {
+                    start[base + (size_t)(j0 + jj) * TPB_NB + b] = c[i];
+                }
+                c[i] += pc[jj][i];
+                ms[i] += pm[jj][i];
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+        const int b = t + i * TPC_THREADS;
+        if (b < TPB_NB) {
+            cnt[b]  = c[i];
+            mass[b] = ms[i];
+        }
     }
     unsigned long long best = 0ull;
-    for (int j = t; j < S; j += TPH_THREADS) {
+    for (int j = t; j < S; j += TPC_THREADS) {
         const unsigned long long v = part_best[(size_t)row * S + j];
         best                       = v > best ? v : best;
     }
-    best = block_max<unsigned long long>(best, red64, 0ull);  // (also orders the LDS writes above)
+    best = block_max<unsigned long long, TPC_THREADS / WAVE>(best, red64, 0ull);  // (also orders the LDS writes above)
     m.best = best;
 
     const float p         = top_ps != nullptr ? top_ps[row] : top_p;
@@ -475,7 +513,6 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
     const unsigned long long target = (unsigned long long)((double)rand_num * (1.0 + 1.0 / 1024.0) * 2147483648.0) + 64ull;
 
     // descending scan over buckets: thread t owns the descending positions [K*t, K*t + K)
-    constexpr int      K  = (TPB_NB + TPH_THREADS - 1) / TPH_THREADS;
     uint32_t           lc = 0;
     unsigned long long lm = 0;
 #pragma unroll
@@ -505,7 +542,7 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
     uint32_t           ec = ic - lc;
     unsigned long long em = im - lm;
     uint32_t           total = 0;
-    for (int w = 0; w < TPH_THREADS / WAVE; ++w) {
+    for (int w = 0; w < TPC_THREADS / WAVE; ++w) {
         if (w < wave_id()) {
             ec += wcnt[w];
             em += wmass[w];
@@ -526,19 +563,15 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
             }
         }
     }
-    first = block_min<uint32_t>(first, red32, 0xFFFFFFFFu);
+    first = block_min<uint32_t, TPC_THREADS / WAVE>(first, red32, 0xFFFFFFFFu);
     const int cut = first == 0xFFFFFFFFu ? 0 : TPB_NB - 1 - (int)first;
     m.cut         = cut;
     m.n_pos       = (int)total;
     m.n           = (int)(off[cut] + cnt[cut]);
 
-    // where chunk j continues inside bucket b
-    for (int b = cut + t; b < TPB_NB; b += TPH_THREADS) {
-        uint32_t at = off[b];
-        for (int j = 0; j < S; ++j) {
-            start[base + (size_t)j * TPB_NB + b] = at;
-            at += part_cnt[base + (size_t)j * TPB_NB + b];
-        }
+    // where the bucket starts in the ordered prefix (the gather adds what earlier chunks hold)
+    for (int b = cut + t; b < TPB_NB; b += TPC_THREADS) {
+        bucket_off[(size_t)row * TPB_NB + b] = off[b];
     }
     // Segments of whole buckets, in descending order: a bucket closes a segment when a multiple of
     // TPS_SEG lies inside it or at its end, and the last gathered bucket closes the last one. A segment
@@ -575,7 +608,7 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
     __syncthreads();
     uint32_t at   = iclose - lclose;
     uint32_t nseg = 0;
-    for (int w = 0; w < TPH_THREADS / WAVE; ++w) {
+    for (int w = 0; w < TPC_THREADS / WAVE; ++w) {
         at += w < wave_id() ? wcnt[w] : 0u;
         nseg += wcnt[w];
     }
@@ -596,7 +629,7 @@ template<int DT>
 __global__ void __launch_bounds__(TPH_THREADS)
 topp_gather_kernel(const typename Storage<DT>::T* __restrict__ probs, int vocab, int chunk,
                    const ToppRowMeta* __restrict__ meta, const uint32_t* __restrict__ start,
-                   unsigned long long* __restrict__ sorted)
+                   const uint32_t* __restrict__ bucket_off, unsigned long long* __restrict__ sorted)
 {
     __shared__ uint32_t cur[TPB_NB];
     const int           row = blockIdx.y;
@@ -609,7 +642,7 @@ topp_gather_kernel(const typename Storage<DT>::T* __restrict__ probs, int vocab,
     }
     const size_t base = ((size_t)row * S + j) * TPB_NB;
     for (int b = m.cut + t; b < TPB_NB; b += TPH_THREADS) {
-        cur[b] = start[base + b];
+        cur[b] = bucket_off[(size_t)row * TPB_NB + b] + start[base + b];
     }
     __syncthreads();
     const int           lo  = (int)min((long long)vocab, (long long)j * chunk);
@@ -874,8 +907,8 @@ __device__ void sort_segment(ToppSortShared& s, unsigned long long* __restrict__
     if (t == 0) {
         s.nbig = 0;
     }
-    kmin = block_min<uint32_t>(kmin, s.red32, 0xFFFFFFFFu);
-    kmax = block_max<uint32_t>(kmax, s.red32, 0u);
+    kmin = block_min<uint32_t, TP_THREADS / WAVE>(kmin, s.red32, 0xFFFFFFFFu);
+    kmax = block_max<uint32_t, TP_THREADS / WAVE>(kmax, s.red32, 0u);
     const uint32_t range = kmax - kmin;
     const int      nbits = range == 0u ? 0 : 32 - __clz(range);
     const int      shift = nbits > 10 ? nbits - 10 : 0;
@@ -992,7 +1025,18 @@ topp_sort_kernel(unsigned long long* __restrict__ sorted, const uint32_t* __rest
             if (n < 2) {
                 continue;
             }
-            if (n <= TPS_CAP) {
+            if (n <= 256) {
+                // one wave, straight from memory (most rows only order a few dozen entries)
+                if (wave_id() == 0) {
+                    if (n <= 64) {
+                        wave_sort_group<1>(seg, seg, 0, n);
+                    }
+                    else {
+                        wave_sort_group<4>(seg, seg, 0, n);
+                    }
+                }
+            }
+            else if (n <= TPS_CAP) {
                 sort_segment(s, seg, n);
             }
             else {
@@ -1026,15 +1070,30 @@ struct TopPShared {
 };
 
 // One 32-lane group loads the eight items of each of its lanes from tile `tile` of the ordered
-// array (entries at or beyond n count as 0) and returns the inclusive raking scan of the lane totals.
-__device__ __forceinline__ float tile_partials(const unsigned long long* __restrict__ src, int n, int tile, int l,
-                                               float x[8])
+// array (entries at or beyond n count as 0).
+__device__ __forceinline__ void tile_load(const unsigned long long* __restrict__ src, int n, int tile, int l, float x[8])
 {
     const int i0 = tile * TP_TILE + l * 8;
+    if (i0 + 8 <= n && ((uintptr_t)src & 15u) == 0u) {
+        const ulonglong2* v = reinterpret_cast<const ulonglong2*>(src + i0);  // i0 is a multiple of 8
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        x[j] = i0 + j < n ? key64_prob(src[i0 + j]) : 0.0f;
+        for (int j = 0; j < 4; ++j) {
+            const ulonglong2 p = v[j];
+            x[2 * j]           = key64_prob(p.x);
+            x[2 * j + 1]       = key64_prob(p.y);
+        }
     }
+    else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            x[j] = i0 + j < n ? key64_prob(src[i0 + j]) : 0.0f;
+        }
+    }
+}
+
+// Inclusive raking scan of the lane totals of a tile.
+__device__ __forceinline__ float tile_scan(const float x[8], int l)
+{
     float seg = x[0];
 #pragma unroll
     for (int j = 1; j < 8; ++j) {
@@ -1066,22 +1125,46 @@ __device__ int scan_sorted(TopPShared& s, const unsigned long long* __restrict__
     float       carry_in = 0.0f;
     for (int base = 0; base < nt; base += TP_ROUND) {
         const int ntr = min(TP_ROUND, nt - base);
-        for (int g = group; g < ntr; g += TP_THREADS / 32) {
-            float       x[8];
-            const float incl = tile_partials(src, n, base + g, l, x);
-            if (l == 31) {
-                s.agg[g] = incl;
+        constexpr int NG = TP_THREADS / 32;
+        constexpr int Q  = 8;  // tiles in flight per lane group
+        for (int g = group; g < ntr; g += Q * NG) {
+            float x[Q][8];
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                if (g + q * NG < ntr) {
+                    tile_load(src, n, base + g + q * NG, l, x[q]);
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                if (g + q * NG < ntr) {
+                    const float incl = tile_scan(x[q], l);
+                    if (l == 31) {
+                        s.agg[g + q * NG] = incl;
+                    }
+                }
             }
         }
         __syncthreads();
         if (t == 0) {
+            // the additions depend on each other, the loads do not: eight totals are fetched at a time
             float c  = carry_in;
             int   g0 = -1;
-            for (int g = 0; g < ntr; ++g) {
-                s.carry[g] = c;
-                c          = c + s.agg[g];
-                if (g0 < 0 && c >= near) {
-                    g0 = g;
+            for (int g = 0; g < ntr; g += 8) {
+                float a[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    a[j] = s.agg[g + j];  // TP_ROUND is a multiple of 8; entries from ntr on are not used
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (g + j < ntr) {
+                        s.carry[g + j] = c;
+                        c              = c + a[j];
+                        if (g0 < 0 && c >= near) {
+                            g0 = g + j;
+                        }
+                    }
                 }
             }
             s.carry[ntr] = c;
@@ -1094,8 +1177,9 @@ __device__ int scan_sorted(TopPShared& s, const unsigned long long* __restrict__
                 const int g  = gs + group;
                 uint32_t  m8 = 0;
                 if (g < ntr) {
-                    float       x[8];
-                    const float incl   = tile_partials(src, n, base + g, l, x);
+                    float x[8];
+                    tile_load(src, n, base + g, l, x);
+                    const float incl   = tile_scan(x, l);
                     const float excl   = __shfl_up(incl, 1, 32);
                     const float prefix = s.carry[g];
                     float       a      = l == 0 ? prefix : prefix + excl;
@@ -1407,6 +1491,7 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     uint32_t*           pmass   = (uint32_t*)(ws + plan.off_pmass);
     unsigned long long* pbest   = (unsigned long long*)(ws + plan.off_pbest);
     uint32_t*           start   = (uint32_t*)(ws + plan.off_start);
+    uint32_t*           boff    = (uint32_t*)(ws + plan.off_boff);
     uint32_t*           segs    = (uint32_t*)(ws + plan.off_seg);
     ToppRowMeta*        meta    = (ToppRowMeta*)(ws + plan.off_meta);
     const int           vocab   = (int)vocab_size_padded;
@@ -1415,13 +1500,13 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     FTK_DISPATCH_DTYPE(dtype, topp_histogram_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
                                   (const Storage<DT>::T*)log_probs, vocab, plan.chunk, skip_decode, pcnt, pmass, pbest));
     FTK_LAUNCH_CHECK();
-    topp_cut_kernel<<<batch_size, TPH_THREADS, 0, st>>>(plan.splits, pcnt, pmass, pbest, start, segs, meta,
+    topp_cut_kernel<<<batch_size, TPC_THREADS, 0, st>>>(plan.splits, pcnt, pmass, pbest, start, boff, segs, meta,
                                                         (const RngState*)rng_state, uniform_draws, max_top_p, top_ps,
                                                         skip_decode);
     FTK_LAUNCH_CHECK();
     if (!g_topp_force_deep) {
         FTK_DISPATCH_DTYPE(dtype, topp_gather_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
-                                      (const Storage<DT>::T*)log_probs, vocab, plan.chunk, meta, start, sorted));
+                                      (const Storage<DT>::T*)log_probs, vocab, plan.chunk, meta, start, boff, sorted));
         FTK_LAUNCH_CHECK();
         topp_sort_kernel<<<plan.sorters, TP_THREADS, 0, st>>>(sorted, segs, meta, vocab, batch_size);
         FTK_LAUNCH_CHECK();

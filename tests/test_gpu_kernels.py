@@ -565,3 +565,71 @@ def test_rng_determinism_and_range(env):
     # known answer: first draw of seed 0 is Philox4x32-10(ctr=0,key=0)[0] = 0x6627e8d5
     expect = np.float32(np.float32(0x6627e8d5) * np.float32(2.3283064365386963e-10) + np.float32(1.16415321826934814453125e-10))
     assert b[0, 0] == expect
+
+
+def _softmax_rows(dt, x):
+    logits = O.to_storage(x, dt)
+    probs = logits.copy()
+    batch, V = x.shape
+    O.add_bias_softmax(dt, probs, None, np.zeros(batch, np.int32), None, batch, V, V)
+    return probs
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_topp_sampling_sort_paths(env, dt):
+    """Rows built to reach every way a segment of the ordered prefix is sorted: a few dozen entries (one
+    wave), bins joined into groups, one long group of equal keys (whole workgroup), a bucket longer than the
+    in-LDS limit (radix sort in memory), and draws at the far end so that everything is ordered."""
+    rng = np.random.default_rng(77 + dt)
+    V = 12000
+    x = np.full((8, V), -30.0, np.float32)
+    x[0, :40] = rng.normal(0, 1, 40)                       # 40 candidates, the rest negligible
+    x[1, :3000] = 0.0                                      # 3000 equal keys: one long group
+    x[2, :7000] = 0.0                                      # 7000 equal keys: longer than the LDS limit
+    x[3] = rng.normal(0, 0.02, V)                          # one or two crowded buckets, distinct keys
+    x[4] = rng.normal(0, 3.0, V)                           # wide: many buckets
+    x[5, :300] = np.repeat(rng.normal(0, 1, 3), 100)       # three groups of 100 equal keys
+    x[6] = np.round(rng.normal(0, 1.0, V) * 4) / 4         # heavy ties over a wide range
+    x[7, :5000] = rng.normal(0, 0.001, 5000)               # 5000 nearly equal, distinct keys
+    probs = _softmax_rows(dt, x)
+    end_ids = np.zeros(8, np.int32)
+    for u_val in (0.05, 0.5, 0.93, 0.9999):
+        p_arr = np.full(8, 1.0, np.float32)
+        u = np.full(8, u_val, np.float32)
+        args = (dt, probs, p_arr, end_ids, u, None, None, None, True)
+        _compare_topk(_run_topp(env, *args), _oracle_topp(*args), dt)
+
+
+def test_topp_sampling_unnormalised_input(env):
+    """The entry point takes any numbers: values above 1, denormals, zeros, negatives. (NaN is left out: the
+    reference's order of a row with NaN is that of cub's radix sort on the bit patterns, which the oracle's
+    comparison sort does not define.)"""
+    rng = np.random.default_rng(5)
+    V = 9000
+    probs = rng.random((5, V)).astype(np.float32)
+    probs[0] *= 3.0                                         # mass far above 1
+    probs[1] *= 1e-12                                       # everything in the lowest bucket
+    probs[2, ::2] = 0.0
+    probs[3, ::3] = -1.0
+    probs[4] = np.float32(1e-40)                            # denormal, all equal
+    end_ids = np.zeros(5, np.int32)
+    for u_val in (0.2, 0.999):
+        p_arr = np.full(5, 0.9, np.float32)
+        u = np.full(5, u_val, np.float32)
+        args = (O.F32, probs, p_arr, end_ids, u)
+        _compare_topk(_run_topp(env, *args), _oracle_topp(*args), O.F32)
+
+
+def test_topp_sampling_many_rows(env):
+    """More rows than one tile of the segment scheduler (1024), a third of them deep."""
+    rng = np.random.default_rng(9)
+    batch, V = 2500, 700
+    x = rng.normal(0, 1.5, (batch, V)).astype(np.float32)
+    probs = _softmax_rows(O.F32, x)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    p_arr = rng.uniform(0.3, 1.0, batch).astype(np.float32)
+    u = uniforms(rng, batch)
+    u[::3] = 0.999
+    skip = rng.random(batch) < 0.1
+    args = (O.F32, probs, p_arr, end_ids, u, None, None, skip, True)
+    _compare_topk(_run_topp(env, *args), _oracle_topp(*args), O.F32)
