@@ -31,6 +31,11 @@ WORKLOADS = {
     "decode_step_b256_v128256_f32_topk64_topp0.9_temp0.8_rep1.1": dict(
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=64, sigma=2.5),
+    # secondary line (only with --workload): the top-p layer on Zipf-distributed rows, per-row top_p in
+    # [0.5, 0.99] with decay; the logits buffer is restored outside the timed events (softmax is in place)
+    "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9": dict(
+        dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=0, top_p=(0.5, 0.99), top_p_decay=0.9,
+        top_p_min=0.3, top_p_reset_id=13, zipf_s=1.1, noise=0.5, prompt=0),
 }
 
 
@@ -128,6 +133,62 @@ def run_gpu(name, w, steps, warmup, nbuf=4):
     )
 
 
+def run_gpu_topp(name, w, steps, warmup, nbuf=3):
+    """Top-p layer steps; every step is bracketed by its own pair of events so that restoring the logits (the
+    layer turns them into probabilities in place) stays outside the measured time."""
+    import torch
+    import fastertransformer_amd as fa
+
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    B, V = w["batch"], w["vocab"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4321)
+    base = -w["zipf_s"] * torch.log(torch.arange(1, V + 1, device=dev, dtype=torch.float64))
+    base = base - torch.logsumexp(base, 0)
+    bufs = []
+    for _ in range(nbuf):
+        x = torch.empty((B, V), device=dev, dtype=torch.float32)
+        for b in range(B):
+            perm = torch.randperm(V, device=dev, generator=gen)
+            x[b] = (base[perm] + torch.randn(V, device=dev, generator=gen, dtype=torch.float64) * w["noise"]).float()
+        bufs.append(x.reshape(B, 1, V))
+    work = torch.empty_like(bufs[0])
+    total = steps + warmup
+    lo, hi = w["top_p"]
+    top_ps = (torch.rand(B, generator=gen, device=dev) * (hi - lo) + lo).cpu().numpy().astype(np.float32)
+    layer = fa.DynamicDecodeLayer(fa.F32, V, V)
+    layer.setup(B, 1, {"runtime_top_k": np.array([0], np.uint32), "runtime_top_p": top_ps,
+                       "top_p_decay": torch.full((B,), w["top_p_decay"], device=dev),
+                       "top_p_min": torch.full((B,), w["top_p_min"], device=dev),
+                       "top_p_reset_ids": torch.full((B,), w["top_p_reset_id"], dtype=torch.int32, device=dev),
+                       "random_seed": np.array([1], np.uint64)})
+    output_ids = torch.zeros((total + 1, B), dtype=torch.int32, device=dev)
+    finished = torch.zeros(B, dtype=torch.bool, device=dev)
+    seq_len = torch.zeros(B, dtype=torch.int32, device=dev)
+    end_id = torch.full((B,), V - 1, dtype=torch.int32, device=dev)
+    outs = {"output_ids": output_ids, "finished": finished, "sequence_length": seq_len}
+    step_arr = np.zeros(1, np.int32)
+    fixed = {"step": step_arr, "max_input_length": np.array([0], np.int32), "ite": np.array([0], np.uint32),
+             "local_batch_size": np.array([B], np.int32), "end_id": end_id}
+    events = []
+    for i in range(total):
+        step_arr[0] = i
+        finished.zero_()
+        work.copy_(bufs[i % nbuf])
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        layer.forward(outs, dict(fixed, logits=work))
+        e1.record()
+        if i >= warmup:
+            events.append((e0, e1))
+    torch.cuda.synchronize()
+    ms = [a.elapsed_time(b) for a, b in events]
+    gpu_ms = sum(ms) / len(ms)
+    return dict(tokens_per_s=B / (gpu_ms * 1e-3), ms_per_step=gpu_ms, p50_ms=float(np.median(ms)), max_ms=max(ms),
+                sampled_ids_checksum=int(output_ids[warmup:total].to(torch.int64).sum().item()))
+
+
 def run_cpu_baseline(w, budget_s=12.0):
     """the oracle (a scalar, single-threaded restatement of the reference algorithm) on rows of the same
     workload, until `budget_s` seconds of CPU work have been spent"""
@@ -170,13 +231,25 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run five plain device copies of 128 MiB, the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE counter readings are scaled by")
+    ap.add_argument("--workload", default=next(iter(WORKLOADS)), choices=list(WORKLOADS),
+                    help="default: the headline decode step; the others print a secondary line of their own")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (rows shard across GPUs with no "
               "exchange); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
-    name = next(iter(WORKLOADS))
+    name = a.workload
     w = WORKLOADS[name]
+    if name.startswith("topp_step"):
+        r = run_gpu_topp(name, w, a.steps, a.warmup)
+        print(json.dumps({
+            "metric": "sampled tokens/s, top-p decode step B=256 V=128256 (softmax + nucleus sampling + decay)",
+            "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": r["ms_per_step"], "p50_ms": r["p50_ms"], "max_ms": r["max_ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"]},
+            "sampled_ids_checksum": r["sampled_ids_checksum"]}))
+        return
     r = run_gpu(name, w, a.steps, a.warmup)
     if a.copy_calibration:
         import torch

@@ -3,6 +3,8 @@
   fastertransformer_amd/lib/libftk_sampling.so  HIP kernels + C ABI (include/ftk_sampling.h), gfx950
   fastertransformer_amd/lib/libft_decode.so     host C++ layers (DynamicDecodeLayer, TopK/TopPSamplingLayer)
                                                 + the handle API used by bindings
+  fastertransformer_amd/lib/libth_transformer.so  torch.classes.FasterTransformer.DynamicDecodeOp (PyTorch-ROCm
+                                                custom class over libft_decode.so; skipped with --no-torch)
 
 Run `python -m fastertransformer_amd.build`. hipcc cross-compiles for gfx950 without a GPU.
 """
@@ -44,7 +46,7 @@ def _newer(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force=True, verbose=True):
+def build(force=True, verbose=True, with_torch=True):
     os.makedirs(LIB, exist_ok=True)
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".cuh"))]
     headers.append(os.path.join(INCLUDE, "ftk_sampling.h"))
@@ -60,9 +62,10 @@ def build(force=True, verbose=True):
     kernels_so = os.path.join(LIB, "libftk_sampling.so")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", kernels_so] + objs)
 
-    host_sources = []
+    host_sources, th_sources = [], []
     for d, _, files in os.walk(SRC):
-        host_sources += [os.path.join(d, f) for f in files if f.endswith(".cc")]
+        into = th_sources if os.sep + "th_op" in d else host_sources
+        into += [os.path.join(d, f) for f in files if f.endswith(".cc")]
     if host_sources:
         decode_so = os.path.join(LIB, "libft_decode.so")
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
@@ -70,8 +73,29 @@ def build(force=True, verbose=True):
              + sorted(host_sources)
              + ["-L", LIB, "-lftk_sampling", "-L", "/opt/rocm/lib", "-lamdhip64",
                 "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"])
+    if th_sources and with_torch:
+        build_th_op(sorted(th_sources))
     return LIB
 
 
+def build_th_op(sources):
+    """The PyTorch custom class: plain g++ against the headers and libraries of the installed torch."""
+    import torch
+    from torch.utils import cpp_extension as ce
+    th_so = os.path.join(LIB, "libth_transformer.so")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function", "-Wno-sign-compare",
+           "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I", PKG, "-I", INCLUDE, "-I", "/opt/rocm/include"]
+    for inc in ce.include_paths():
+        cmd += ["-isystem", inc]
+    cmd += ["-o", th_so] + sources + ["-L", LIB, "-lft_decode", "-lftk_sampling"]
+    for lp in ce.library_paths():
+        cmd += ["-L", lp, "-Wl,-rpath," + lp]
+    cmd += ["-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip", "-L", "/opt/rocm/lib", "-lamdhip64",
+            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath,/opt/rocm/lib"]
+    _run(cmd)
+    return th_so
+
+
 if __name__ == "__main__":
-    build(force="--incremental" not in sys.argv)
+    build(force="--incremental" not in sys.argv, with_torch="--no-torch" not in sys.argv)
