@@ -1165,9 +1165,27 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
 // Rows split over several workgroups: merge their lists from the workspace into s.cand.
 // Returns the candidate count, or -1 for the literal replay; *thr_out is a valid bound when the result
 // is >= k.
+// What a select workgroup asks for before it knows anything about its row: wave w takes the header of
+// chunk list w and its first 2 * 64 entries (most lists are shorter). Issued at the top of the kernel, the
+// loads are in flight while the row's arguments arrive; topk_merge_lists consumes them.
+struct TopkListPrefetch {
+    TopkEntry first[2];
+};
+
+__device__ __forceinline__ TopkListPrefetch topk_prefetch_lists(int splits, const TopkEntry* entries)
+{
+    TopkListPrefetch pf;
+    const int        ch = wave_id();
+    const TopkEntry* e  = entries + (size_t)(ch < splits ? ch : 0) * TK_CCAP;  // always inside the row's slots
+    pf.first[0]         = e[lane_id()];
+    pf.first[1]         = e[WAVE + lane_id()];
+    return pf;
+}
+
 template<int DT>
 __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits, const TopkChunkHeader* headers,
-                                                const TopkEntry* entries, uint32_t* thr_out)
+                                                const TopkEntry* entries, uint32_t* thr_out,
+                                                const TopkListPrefetch& pf)
 {
     const int t = threadIdx.x;
     FTK_PHASE_BEGIN();
@@ -1203,7 +1221,8 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
             const int        cnt = (int)headers[ch].count;
             const TopkEntry* e   = entries + (size_t)ch * TK_CCAP;
             for (int i = lane_id(); i < cnt; i += WAVE) {
-                const TopkEntry en = e[i];
+                // the first two rounds of a wave's first list were requested at the top of the kernel
+                const TopkEntry en = (ch == wave_id() && i < 2 * WAVE) ? pf.first[i >> 6] : e[i];
                 if (en.key >= thr) {
                     const int slot = atomicAdd(&s.n_cand, 1);
                     if (slot < TK_CCAP) {

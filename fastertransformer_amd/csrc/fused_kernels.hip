@@ -451,23 +451,28 @@ __global__ void __launch_bounds__(TK_THREADS) fused_select_kernel(FusedParams p,
     constexpr int BMW = 0;  // the literal replay reads whole-row bitmaps from global memory
     __shared__ TopkShared s;
     const int             row = blockIdx.x;
-    if (p.skip_decode != nullptr && p.skip_decode[row]) {
+    // everything the row needs is requested before the first decision: the arguments (scalar loads), the
+    // chunk lists (vector loads), the draw
+    TopkEntry*             row_entries = l.entries + (size_t)row * l.row_entries;
+    const TopkListPrefetch pf          = topk_prefetch_lists(l.splits, row_entries);
+    const bool   skip = p.skip_decode != nullptr && p.skip_decode[row];
+    const bool   fin  = l.finished != nullptr && l.finished[row];
+    const int    k    = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    const float  tp   = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
+    FusedRow<DT, BMW> r(p, row);
+    if (skip) {
         return;
     }
-    if (l.finished != nullptr && l.finished[row]) {
+    if (fin) {
         if (threadIdx.x == 0) {
             l.ids[row] = p.end_ids[row];
         }
         return;
     }
-    const int    k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    const float  tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
     const float  u  = fused_row_draw(s, l, row);
     const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row);
-    FusedRow<DT, BMW> r(p, row);
-    TopkEntry*   row_entries = l.entries + (size_t)row * l.row_entries;
     uint32_t     thr         = 0u;
-    const int    n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr);
+    const int    n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr, pf);
     topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
 }
 

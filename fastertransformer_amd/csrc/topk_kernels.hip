@@ -108,26 +108,30 @@ __global__ void __launch_bounds__(TK_THREADS) topk_select_kernel(TopkKernelArgs 
 {
     __shared__ TopkShared s;
     const int             row = blockIdx.x;
-    if (a.skip_decode != nullptr && a.skip_decode[row]) {
+    // the chunk lists and the row's arguments are requested before the first decision
+    TopkEntry*             row_entries = a.entries + (size_t)row * a.row_entries;
+    const TopkListPrefetch pf          = topk_prefetch_lists(a.splits, row_entries);
+    const bool     skip = a.skip_decode != nullptr && a.skip_decode[row];
+    const bool     fin  = a.finished != nullptr && a.finished[row];
+    const int      k    = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
+    const float    p    = a.top_ps != nullptr ? a.top_ps[row] : a.top_p;
+    if (skip) {
         return;
     }
-    if (a.finished != nullptr && a.finished[row]) {
+    if (fin) {
         if (threadIdx.x == 0) {
             a.ids[row] = a.end_ids[row];
         }
         return;
     }
     FTK_PHASE_BEGIN();
-    const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
-    const float    p = a.top_ps != nullptr ? a.top_ps[row] : a.top_p;
     const float    u = topk_row_draw(s, a.rng, a.uniforms, row);
     const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row);
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
     FTK_PHASE(6);
-    TopkEntry* row_entries = a.entries + (size_t)row * a.row_entries;
-    uint32_t   thr         = 0u;
-    const int  n = topk_merge_lists<DT>(s, k, a.splits, a.headers + (size_t)row * a.splits, row_entries, &thr);
+    uint32_t   thr = 0u;
+    const int  n   = topk_merge_lists<DT>(s, k, a.splits, a.headers + (size_t)row * a.splits, row_entries, &thr, pf);
     topk_select_lds<DT>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, row_entries,
                         a.cum_log_probs != nullptr || a.output_log_probs != nullptr, u, a.end_ids, out);
 }

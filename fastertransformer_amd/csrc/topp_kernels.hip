@@ -146,7 +146,7 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
     if (!fin && bias == nullptr) {
         // Ordinary rows. The maximum and the final division do not depend on the order of the columns
         // and go through 16-byte accesses; the sum keeps the reference's order (thread t adds its
-        // columns t, t + BLK, ... one after the other), eight loads in flight.
+        // columns t, t + BLK, ... one after the other), eight or sixteen loads in flight.
         float mx = -3.402823466e+38f;
         stream_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) { mx = __builtin_fmaxf(mx, x + 0.0f); });
         if (n_padded > n) {
@@ -159,7 +159,7 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
         const float pad_e = round_t<DT>(det_expf(-MAXT - mx));
         float       sum   = 0.0f;
         if (active) {
-            constexpr int U = 8;
+            constexpr int U = DT == DT_F32 ? 8 : 16;  // 2-byte loads move half as much per instruction
             int           v = t;
             for (; v + (U - 1) * BLK < n; v += U * BLK) {
                 float x[U];
