@@ -36,6 +36,12 @@ WORKLOADS = {
     "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9": dict(
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=0, top_p=(0.5, 0.99), top_p_decay=0.9,
         top_p_min=0.3, top_p_reset_id=13, zipf_s=1.1, noise=0.5, prompt=0),
+    # secondary line (only with --workload): the full decode loop of BASELINE config 5, per-step latency with
+    # cum_log_probs / output_log_probs and the length criterion on (the kernel-by-kernel path: log-probs need the
+    # probabilities of the whole row)
+    "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs": dict(
+        dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
+        repetition_penalty=1.1, prompt=8, sigma=2.5),
 }
 
 
@@ -189,6 +195,58 @@ def run_gpu_topp(name, w, steps, warmup, nbuf=3):
                 sampled_ids_checksum=int(output_ids[warmup:total].to(torch.int64).sum().item()))
 
 
+def run_gpu_loop(name, w, steps, warmup, nbuf=2):
+    """Decode loop with log-probs and stop criteria; per-step events, logits restored outside them (this path
+    works in place, like the reference)."""
+    import torch
+    import fastertransformer_amd as fa
+
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    dt = {"f32": fa.F32, "f16": fa.F16, "bf16": fa.BF16}[w["dtype"]]
+    B, V, Vp, H = w["batch"], w["vocab"], w["vocab_padded"], w["prompt"]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(55)
+    bufs = [(torch.randn((B, 1, Vp), generator=gen, device=dev, dtype=torch.float32) * w["sigma"]).to(fa.torch_dtype(dt))
+            for _ in range(nbuf)]
+    work = torch.empty_like(bufs[0])
+    total = steps + warmup
+    layer = fa.DynamicDecodeLayer(dt, V, Vp)
+    layer.setup(B, 1, {"runtime_top_k": np.array([w["top_k"]], np.uint32),
+                       "runtime_top_p": np.array([w["top_p"]], np.float32),
+                       "temperature": np.array([w["temperature"]], np.float32),
+                       "repetition_penalty": np.array([w["repetition_penalty"]], np.float32),
+                       "random_seed": np.array([1], np.uint64)})
+    output_ids = torch.zeros((H + total + 1, B), dtype=torch.int32, device=dev)
+    output_ids[:H] = torch.randint(0, V, (H, B), generator=gen, device=dev, dtype=torch.int32)
+    finished = torch.zeros(B, dtype=torch.bool, device=dev)
+    seq_len = torch.full((B,), H - 1, dtype=torch.int32, device=dev)
+    cum = torch.zeros(B, device=dev)
+    out_lp = torch.zeros((total + 1, B), device=dev)
+    end_id = torch.full((B,), V - 1, dtype=torch.int32, device=dev)
+    limit = torch.full((B,), H + total + 8, dtype=torch.int32, device=dev)
+    outs = {"output_ids": output_ids, "finished": finished, "sequence_length": seq_len, "cum_log_probs": cum,
+            "output_log_probs": out_lp, "should_stop": np.zeros(1, np.bool_)}
+    step_arr = np.zeros(1, np.int32)
+    fixed = {"step": step_arr, "max_input_length": np.array([H], np.int32), "ite": np.array([0], np.uint32),
+             "local_batch_size": np.array([B], np.int32), "end_id": end_id, "sequence_limit_length": limit}
+    ms = []
+    for i in range(total):
+        step_arr[0] = H + i
+        work.copy_(bufs[i % nbuf])
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        layer.forward(outs, dict(fixed, logits=work))   # returns with should_stop valid
+        e1.record()
+        torch.cuda.synchronize()
+        if i >= warmup:
+            ms.append(e0.elapsed_time(e1))
+    ms = np.array(ms)
+    return dict(tokens_per_s=B / (ms.mean() * 1e-3), ms_per_step=float(ms.mean()), p50_ms=float(np.percentile(ms, 50)),
+                p99_ms=float(np.percentile(ms, 99)), max_ms=float(ms.max()),
+                sampled_ids_checksum=int(output_ids[H + warmup:H + total].to(torch.int64).sum().item()))
+
+
 def run_cpu_baseline(w, budget_s=12.0):
     """the oracle (a scalar, single-threaded restatement of the reference algorithm) on rows of the same
     workload, until `budget_s` seconds of CPU work have been spent"""
@@ -248,6 +306,18 @@ def main():
             "ms_per_step": r["ms_per_step"], "p50_ms": r["p50_ms"], "max_ms": r["max_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"]},
+            "sampled_ids_checksum": r["sampled_ids_checksum"]}))
+        return
+    if name.startswith("decode_loop"):
+        r = run_gpu_loop(name, w, a.steps, a.warmup)
+        print(json.dumps({
+            "metric": "per-step latency, decode loop B=1024 V=152064 f16 (top-k + top-p + penalties, log-probs, "
+                      "stop criteria)",
+            "value": r["p50_ms"], "unit": "ms (p50)", "p99_ms": r["p99_ms"], "max_ms": r["max_ms"], "n_gpus": 1,
+            "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"], "tokens_per_s": r["tokens_per_s"],
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"], "top_k": w["top_k"],
+                       "top_p": w["top_p"]},
             "sampled_ids_checksum": r["sampled_ids_checksum"]}))
         return
     r = run_gpu(name, w, a.steps, a.warmup)

@@ -1162,11 +1162,8 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
     FTK_PHASE(13);
 }
 
-// Rows split over several workgroups: merge their lists from the workspace into s.cand.
-// Returns the candidate count, or -1 for the literal replay; *thr_out is a valid bound when the result
-// is >= k.
-// What a select workgroup asks for before it knows anything about its row: wave w takes the header of
-// chunk list w and its first 2 * 64 entries (most lists are shorter). Issued at the top of the kernel, the
+// What a select workgroup asks for before it knows anything about its row: wave w takes the first
+// 2 * 64 entries of chunk list w (most lists are shorter). Issued at the top of the kernel, the
 // loads are in flight while the row's arguments arrive; topk_merge_lists consumes them.
 struct TopkListPrefetch {
     TopkEntry first[2];
@@ -1182,6 +1179,9 @@ __device__ __forceinline__ TopkListPrefetch topk_prefetch_lists(int splits, cons
     return pf;
 }
 
+// Rows split over several workgroups: merge their lists from the workspace into s.cand.
+// Returns the candidate count, or -1 for the literal replay; *thr_out is a valid bound when the result
+// is >= k.
 template<int DT>
 __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits, const TopkChunkHeader* headers,
                                                 const TopkEntry* entries, uint32_t* thr_out,

@@ -633,3 +633,51 @@ def test_topp_sampling_many_rows(env):
     skip = rng.random(batch) < 0.1
     args = (O.F32, probs, p_arr, end_ids, u, None, None, skip, True)
     _compare_topk(_run_topp(env, *args), _oracle_topp(*args), O.F32)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_softmax_and_topp_random_shapes(env, dt, seed):
+    """Seeded random vocabulary sizes (odd ones included: rows that do not start on a 16-byte boundary, heads
+    and tails of the vector loops), pad columns, batch sizes, shapes of distribution and draws; the softmax is
+    compared bit for bit, top-p by ids, flags, lengths and log-probs."""
+    torch, lib, ops = env
+    rng = np.random.default_rng(1000 * dt + seed)
+    for case in range(4):
+        V = int(rng.choice([rng.integers(9, 300), rng.integers(300, 9000), rng.integers(9000, 70000)]))
+        Vp = V + int(rng.choice([0, 0, 1, 7, 64]))
+        batch = int(rng.integers(1, 10))
+        kind = int(rng.integers(0, 4))
+        if kind == 0:
+            x = rng.standard_normal((batch, Vp)) * rng.uniform(0.1, 4.0)
+        elif kind == 1:
+            ranks = np.arange(1, Vp + 1, dtype=np.float64)
+            x = np.stack([(-rng.uniform(0.8, 1.5) * np.log(ranks))[rng.permutation(Vp)] for _ in range(batch)])
+            x = x + rng.standard_normal((batch, Vp)) * 0.3
+        elif kind == 2:
+            x = rng.integers(0, 4, (batch, Vp)).astype(np.float64) * rng.uniform(0.2, 2.0)   # few distinct values
+        else:
+            x = np.where(rng.random((batch, Vp)) < 0.7, -np.inf, rng.standard_normal((batch, Vp)))
+            x[:, 0] = 0.0
+        logits = O.to_storage(x.astype(np.float32), dt)
+        end_ids = rng.integers(0, V, batch).astype(np.int32)
+        finished = rng.random(batch) < 0.15
+        want = logits.copy()
+        O.add_bias_softmax(dt, want, None, end_ids, finished, batch, Vp, V)
+        d_probs = to_torch(logits, dt)
+        d_end, d_fin = to_torch(end_ids), to_torch(finished)
+        ops.check(lib.ftk_invoke_add_bias_softmax(dt, d_probs.data_ptr(), None, d_end.data_ptr(), d_fin.data_ptr(),
+                                                  batch, Vp, V, ops.current_stream()))
+        _sync(torch)
+        got = to_numpy(d_probs)
+        assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8)), (V, Vp, batch, kind)
+        for trial in range(2):
+            p_arr = rng.uniform(0.1, 1.0, batch).astype(np.float32)
+            u = uniforms(rng, batch)
+            if trial == 1:
+                u[:] = rng.choice([1e-6, 0.5, 0.999, 1.0], batch).astype(np.float32)
+                p_arr[::2] = 1.0
+            seq = rng.integers(1, 9, batch).astype(np.int32)
+            skip = rng.random(batch) < 0.2
+            args = (dt, want, p_arr, end_ids, u, finished.copy(), seq, skip, True)
+            _compare_topk(_run_topp(env, *args), _oracle_topp(*args), dt)
