@@ -57,6 +57,7 @@ constexpr int TK_NVT      = 16;    // 16-byte vectors per thread and tile: 64 KB
 constexpr int TK_CCAP     = 2048;  // candidates a workgroup can hold
 constexpr int TK_MAXSPLIT = 64;
 constexpr int TK_FILL_WGS = 256 * TK_MIN_WGS;  // workgroups wanted in flight: every compute unit full
+constexpr int TK_STAGE    = 512 / TK_WAVES;    // vectors a wave can park per tile
 
 struct TopkChunkHeader {
     uint32_t count;      // entries written
@@ -71,6 +72,12 @@ struct TopkEntry {
     uint32_t key;
     uint32_t idx;
 };
+
+// which variant of the streaming kernels a launch takes (see topk_stream)
+inline int topk_many_level(int max_top_k)
+{
+    return max_top_k > TK_CCAP / 4 ? 2 : (max_top_k > TK_STAGE ? 1 : 0);
+}
 
 struct TopkPlan {
     int    splits;         // workgroups per row
@@ -206,8 +213,6 @@ __device__ __forceinline__ int topk_row_tiles(const void* rowp, int vocab)
     return (nvec + TILE_VECS - 1) / TILE_VECS;
 }
 
-constexpr int TK_STAGE = 512 / TK_WAVES;  // vectors a wave can park per tile
-
 struct TopkShared {
     union {
         struct {
@@ -287,77 +292,125 @@ __device__ __forceinline__ int topk_prune(TopkShared& s, int n, uint32_t thr)
     return m;
 }
 
-// The exact k-th largest key of the list (n >= k, every entry >= lower).
+// The exact k-th largest key of the list (n >= k, every entry >= lower). Uses the staging area of the
+// stream (idle between tiles) as scratch.
+template<bool DEEP = false>
 __device__ __forceinline__ uint32_t topk_kth_key(TopkShared& s, int n, int k, uint32_t lower)
 {
     const int t = threadIdx.x;
     uint32_t  nt;
     if (n <= TK_THREADS) {
-        // rank by counting; ties are ordered by position so exactly one entry has rank k-1
-        const uint32_t k0 = t < n ? s.cand.key[t] : 0u;
-        int            r0 = 0;
-        // entry j precedes entry i when key_j > key_i, or the keys are equal and j < i:
+        // Rank by counting; ties are ordered by position so exactly one entry has rank k-1.
+        // Entry j precedes entry i when key_j > key_i, or the keys are equal and j < i:
         //   key_j >= key_i for j < i,  key_j > key_i for j > i   <=>   key_j + (j < i) > key_i
-        // (keys stay below 0xFFFFFFFF, so the increment cannot wrap)
-        const int n4 = (n + 3) & ~3;  // the list is read four entries at a time; the tail is masked
+        // (keys stay below 0xFFFFFFFF, so the increment cannot wrap).
+        // The work is cut the other way round from "one entry per thread": every wave compares a
+        // quarter of the list (read four entries at a time) against all entries, four per lane, so a
+        // thread waits for a quarter of the LDS reads and does sixteen compares per read; the partial
+        // ranks meet in LDS.
+        static_assert(TK_WAVES * WAVE == TK_THREADS && TK_STAGE * sizeof(uint4) >= TK_THREADS * sizeof(int),
+                      "partial ranks live in the idle staging area");
+        int (*part)[TK_THREADS] = reinterpret_cast<int(*)[TK_THREADS]>(&s.stage.raw[0][0]);
+        const int l = lane_id(), w = wave_id();
+        uint32_t  mk[TK_WAVES];
+        int       mr[TK_WAVES];
+#pragma unroll
+        for (int q = 0; q < TK_WAVES; ++q) {
+            const int i = l + q * WAVE;
+            mk[q]       = i < n ? s.cand.key[i] : 0xFFFFFFFFu;
+            mr[q]       = 0;
+        }
+        const int n4  = (n + 3) & ~3;
+        const int per = ((n4 / 4 + TK_WAVES - 1) / TK_WAVES) * 4;  // entries per wave, a multiple of four
+        const int jlo = w * per;
+        const int jhi = min(n4, jlo + per);
 #pragma unroll 2
-        for (int j = 0; j < n4; j += 4) {
+        for (int j = jlo; j < jhi; j += 4) {
             const uint4    kk    = *reinterpret_cast<const uint4*>(&s.cand.key[j]);
             const uint32_t kj[4] = {kk.x, kk.y, kk.z, kk.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int      jj = j + e;
                 const uint32_t kv = jj < n ? kj[e] : 0u;
-                r0 += (kv + (jj < t ? 1u : 0u)) > k0 ? 1 : 0;
+#pragma unroll
+                for (int q = 0; q < TK_WAVES; ++q) {
+                    mr[q] += (kv + (jj < l + q * WAVE ? 1u : 0u)) > mk[q] ? 1 : 0;
+                }
             }
         }
-        if (t < n && r0 == k - 1) {
-            s.thr_new = k0;
+#pragma unroll
+        for (int q = 0; q < TK_WAVES; ++q) {
+            part[w][l + q * WAVE] = mr[q];
+        }
+        lds_barrier();
+        if (t < n) {
+            int r0 = 0;
+#pragma unroll
+            for (int q = 0; q < TK_WAVES; ++q) {
+                r0 += part[q][t];
+            }
+            if (r0 == k - 1) {
+                s.thr_new = s.cand.key[t];
+            }
         }
         lds_barrier();
         nt = s.thr_new;
     }
     else {
-        // bisection on the key; per step one ballot per held entry, one LDS atomic per wave, one barrier
-        constexpr int PER = TK_CCAP / TK_THREADS;
+        // Radix select on the key, most significant byte first: a 256-bin histogram of the entries that
+        // still match the bytes found so far, a suffix sum over the bins (one bin per thread), and the
+        // bin that holds the k-th largest gives the next byte. Four rounds of four barriers.
+        static_assert(TK_THREADS == 256, "one histogram bin per thread");
+        constexpr int PER  = TK_CCAP / TK_THREADS;
+        int*          hist = reinterpret_cast<int*>(&s.stage.raw[0][0]);
         uint32_t      ck[PER];
 #pragma unroll
         for (int r = 0; r < PER; ++r) {
             const int i = t + r * TK_THREADS;
             ck[r]       = i < n ? s.cand.key[i] : 0u;
         }
-        if (t < 3) {
-            s.misc[1 + t] = 0;
-        }
-        lds_barrier();
-        uint32_t lo = lower, hi = 0xFFFFFFFFu;  // count(lo) >= k; no key reaches hi
-        int      it = 0;                        // three counters in rotation: add, read, clear
-        while (hi - lo > 1u) {
-            const uint32_t mid = lo + (hi - lo) / 2u;
-            int            c   = 0;
+        (void)lower;
+        uint32_t prefix = 0u, mask = 0u;
+        int      kk     = k;  // rank wanted among the entries that match `prefix` on `mask`
+#pragma unroll 1
+        for (int shift = 24; shift >= 0; shift -= 8) {
+            hist[t] = 0;
+            lds_barrier();
 #pragma unroll
             for (int r = 0; r < PER; ++r) {
-                if (r * TK_THREADS < n) {
-                    c += __builtin_popcountll(__ballot(ck[r] >= mid));
+                if (r * TK_THREADS < n && t + r * TK_THREADS < n && (ck[r] & mask) == prefix) {
+                    atomicAdd(&hist[(ck[r] >> shift) & 255u], 1);
                 }
             }
-            int* counter = &s.misc[1 + it % 3];
+            lds_barrier();
+            // entries in bins >= t: suffix sum inside the wave, then the totals of the higher waves
+            const int mine = hist[t];
+            int       suf  = mine;
+#pragma unroll
+            for (int o = 1; o < WAVE; o <<= 1) {
+                const int dn = __shfl_down(suf, o, WAVE);
+                if (lane_id() + o < WAVE) {
+                    suf += dn;
+                }
+            }
             if (lane_id() == 0) {
-                atomicAdd(counter, c);
+                s.red32[wave_id()] = (uint32_t)suf;
             }
             lds_barrier();
-            c = *counter;
-            if (t == 0) {
-                s.misc[1 + (it + 2) % 3] = 0;  // last read before this step's barrier, next used after the next one
+#pragma unroll
+            for (int w = 0; w < TK_WAVES; ++w) {
+                suf += w > wave_id() ? (int)s.red32[w] : 0;
             }
-            ++it;
-            if (c >= k) {
-                lo = mid;
+            if (suf >= kk && suf - mine < kk) {  // exactly one bin
+                s.misc[1] = t;
+                s.misc[2] = kk - (suf - mine);
             }
-            else {
-                hi = mid;
-            }
+            lds_barrier();
+            prefix |= (uint32_t)s.misc[1] << shift;
+            mask |= 255u << shift;
+            kk = s.misc[2];
         }
+        const uint32_t lo = prefix;
         nt = lo;
     }
     lds_barrier();  // s.thr_new and the counters may be reused right away
@@ -366,9 +419,10 @@ __device__ __forceinline__ uint32_t topk_kth_key(TopkShared& s, int n, int k, ui
 
 // Raise the bound to the exact k-th largest key of the list (n >= k, every entry >= *thr) and drop
 // what falls below it: k entries plus ties with the k-th remain.
+template<bool DEEP = false>
 __device__ __forceinline__ int topk_tighten(TopkShared& s, int n, int k, uint32_t* thr)
 {
-    *thr = topk_kth_key(s, n, k, *thr);
+    *thr = topk_kth_key<DEEP>(s, n, k, *thr);
     return topk_prune(s, n, *thr);
 }
 
@@ -436,7 +490,11 @@ __device__ __noinline__ int topk_stream_rare(Row rowctx, TopkShared& s, int k, i
 // Returns the number of candidates left in s.cand (all elements of the tiles with key >= *thr_out), or
 // -1 when the range could not be bounded. When the result is >= k, *thr_out bounds the k-th largest key
 // of the range from below; otherwise the list holds every selectable element of the range.
-template<int DT, class Row>
+// MANY > 0: the variant for launches whose largest k exceeds what a wave can park per tile (TK_STAGE): the
+// bound of the first tile is refined on the registers that hold it, and every tile takes the general loop,
+// which then drains every second vector. MANY == 2 (largest k beyond a quarter of the list's capacity)
+// also cuts the list back in the middle of a tile. Rows of such a launch with a small k run the same code.
+template<int DT, class Row, int MANY = 0>
 __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab, int k, int tile_begin, int tile_end,
                                            uint32_t* thr_out)
 {
@@ -567,6 +625,51 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         if (thr < KMIN) {
             thr = KMIN;  // fewer than k usable maxima: take every selectable element
         }
+        if constexpr (MANY > 0) {
+            // The maxima bound is loose for a large k (for k = 1024 a third of the tile lies above it).
+            // Raise it by bisection on the key, counting the tile's elements in the registers that hold
+            // them (vectors on the fast transform only: leaving the others out keeps the count a lower
+            // bound), until between k and 1.25 k of them remain.
+            if (k > TK_STAGE) {
+                uint32_t fastmask = 0u;
+#pragma unroll
+                for (int it = 0; it < NVT; ++it) {
+                    fastmask |= vec_max(it) > NEG_INF ? (1u << it) : 0u;
+                }
+                float tmax = NEG_INF;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    tmax = __builtin_fmaxf(tmax, gm[g]);
+                }
+                uint32_t lo = thr;
+                uint32_t hi = block_max<uint32_t, TK_WAVES>(order_key(tmax), s.red32, 0u) + 1u;  // no element reaches it
+                for (int round = 0; round < 24 && hi - lo > 1u; ++round) {
+                    const uint32_t mid  = lo + (hi - lo) / 2u;
+                    const float    midf = key_to_float(mid);
+                    int            c    = 0;
+#pragma unroll
+                    for (int it = 0; it < NVT; ++it) {
+                        if ((fastmask >> it) & 1u) {
+#pragma unroll
+                            for (int j = 0; j < EPV; ++j) {
+                                c += rowctx.fast(vector_element<DT>(raw[it], j)) >= midf ? 1 : 0;
+                            }
+                        }
+                    }
+                    c = block_sum_i<TK_WAVES>(c, (int*)s.red32);
+                    if (c >= k) {
+                        lo = mid;
+                        if (c <= k + k / 4) {
+                            break;
+                        }
+                    }
+                    else {
+                        hi = mid;
+                    }
+                }
+                thr = lo;
+            }
+        }
     }
     FTK_PHASE(2);
     thr         = (uint32_t)__builtin_amdgcn_readfirstlane((int)thr);  // uniform: keep it in a scalar register
@@ -651,14 +754,23 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         }
         wcount = 0;
     };
-    const int tighten_at = min(max(256, 2 * k), 3 * TK_CCAP / 4);
+    // the list is cut back to its k largest between tiles when it has grown past this; with a large k
+    // after every tile (another tile's worth at the old bound would not fit)
+    const int tighten_at = MANY > 0 ? k : min(max(256, 2 * k), 3 * TK_CCAP / 4);
     int       n          = 0;
+    // With a large k a tile holds more candidates than a wave can park between two drains of a whole
+    // tile (k alone can exceed it): such launches take the general tile loop, which then drains every
+    // second vector.
+    static_assert(2 * WAVE <= TK_STAGE, "two vectors per lane fit the parking space");
+    constexpr bool many    = MANY > 0;
+    constexpr bool cut_mid = MANY > 1;
 
     for (int tile = tile_begin; tile < tile_end; ++tile) {
-        const int vec0     = tile * TILE_VECS;
+        bool      cut_early = false;  // large k: the list was cut back in the middle of this tile
+        const int vec0      = tile * TILE_VECS;
         const int first0   = (vec0 + t) * EPV - a;
         uint32_t  slowmask = 0u;  // bit `it`: vector `it` of this thread takes the per-column path
-        if (tile_plain(tile)) {
+        if (tile_plain(tile) && !many) {
             if (packed_ok && tile != tile_begin) {
                 rowctx.template tile_bits<EPV, NVT>(first0, TK_THREADS * EPV, packed);
             }
@@ -715,6 +827,21 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
                     vmax = __builtin_fmaxf(vmax, x[j]);
                 }
                 park(fastv && vmax >= thr_f, raw[it], first);
+                if (many && (it & 1)) {
+                    drain();  // two vectors per lane never overfill the wave's parking space
+                    if (cut_mid && it == NVT / 2 - 1 && k > TK_CCAP / 4) {
+                        // Half a tile at the bound of the tiles before it can add more than half of k: with
+                        // k beyond a quarter of the list's capacity the list is cut back in mid-tile too.
+                        lds_barrier();
+                        const int n_mid = s.n_cand;
+                        lds_barrier();
+                        if (n_mid > k && n_mid <= TK_CCAP) {
+                            n         = topk_tighten(s, n_mid, k, &thr);
+                            thr_f     = key_to_float(thr);
+                            cut_early = true;
+                        }
+                    }
+                }
             }
             for (; slowmask != 0u; slowmask &= slowmask - 1u) {
                 const int first = first0 + __builtin_ctz(slowmask) * TK_THREADS * EPV;
@@ -738,6 +865,9 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         lds_barrier();
         const int n_now = s.n_cand;
         lds_barrier();
+        if (n_now > TK_CCAP && cut_early) {
+            return -1;  // the list already holds part of this tile: the recovery path cannot redo the tile
+        }
         if (n_now > TK_CCAP) {
             const int tlo = max(0, vec0 * EPV - a);
             const int thi = max(tlo, min(vocab, (vec0 + TILE_VECS) * EPV - a));
@@ -769,19 +899,26 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
     return n;
 }
 
-// a workgroup's list -> workspace, for rows that are split over several workgroups
+// A workgroup's list -> workspace, for rows that are split over several workgroups. A short list goes
+// out as it is, with the bound it was gathered under: cutting it to its k largest here would keep every
+// workgroup of the launch busy for several microseconds at the end of its stream, while the merging
+// kernel cuts the union once per row. A long list is cut to the chunk's k largest first, and the chunk
+// also reports its ceil(k/splits)-th largest key (`share`), which gives the merge a bound that keeps the
+// union inside its list.
+constexpr int TK_RAW_DUMP = 448;
+
 __device__ __forceinline__ void topk_dump_list(TopkShared& s, int n, int k, int splits, uint32_t thr,
                                                TopkChunkHeader* header, TopkEntry* entries)
 {
     const int t = threadIdx.x;
     FTK_PHASE_BEGIN();
-    if (n > k) {
-        n = topk_tighten(s, n, k, &thr);  // exact k-th largest of the chunk: keeps the merge short
-    }
-    const int kshare = (k + splits - 1) / splits;
-    uint32_t  share  = 0u;
-    if (n >= kshare && n > 0) {
-        share = topk_kth_key(s, n, kshare, thr);
+    uint32_t share = 0u;
+    if (n > k && (n > TK_RAW_DUMP || n * splits > TK_CCAP)) {  // the union of raw lists fits the merge's list
+        n                = topk_tighten(s, n, k, &thr);
+        const int kshare = (k + splits - 1) / splits;
+        if (n >= kshare) {
+            share = topk_kth_key(s, n, kshare, thr);
+        }
     }
     for (int i = t; i < n; i += TK_THREADS) {
         entries[i] = TopkEntry{s.cand.key[i], s.cand.idx[i]};
@@ -842,17 +979,31 @@ __device__ __forceinline__ int topk_sample_walk(const float* w, int n, float u, 
         s_sum          = s_sum + v.z;
         s_sum          = s_sum + v.w;
     }
+    // the subtractions depend on each other, the loads do not: sixteen weights are fetched at a time
+    // (reading a few entries past n is harmless, they are not used)
     float rand_num = u * p * s_sum;
-    int   pick     = n - 1;
-    for (int i = 0; i < n; ++i) {
-        rand_num = rand_num - w[i];
-        if (rand_num <= 0.0f || i == n - 1) {
-            pick = i;
-            break;
+    int   pick     = -1;
+    for (int i0 = 0; i0 < n && pick < 0; i0 += 16) {
+        float4 v[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            v[b] = w4[(i0 >> 2) + b];
+        }
+        const float x[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
+                             v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int i = i0 + j;
+            if (pick < 0 && i < n) {
+                rand_num = rand_num - x[j];
+                if (rand_num <= 0.0f || i == n - 1) {
+                    pick = i;
+                }
+            }
         }
     }
     *s_sum_out = s_sum;
-    return pick;
+    return pick < 0 ? n - 1 : pick;
 }
 
 __device__ __forceinline__ void topk_emit(const TopkOutputs& o, int row, int id, bool probs_in, float w, float s_sum,
@@ -970,7 +1121,8 @@ __device__ void topk_literal(Row& rowctx, TopkShared& s, int vocab, int k, int B
 // select: replay the reference's two tie orders on the candidates in s.cand, sample, emit.
 // `n` < 0 asks for the literal replay.
 // -------------------------------------------------------------------------------------------
-template<int DT, class Row>
+// DEEP: see topk_kth_key.
+template<int DT, class Row, bool DEEP = false>
 __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int n, uint32_t thr, int row, int vocab,
                                                 int k, float p, int max_top_k, TopkEntry* picks, bool probs_in,
                                                 float u, const int* end_ids, const TopkOutputs& out)
@@ -984,7 +1136,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
 
     if (n >= 0) {
         if (n > TK_THREADS && n > k) {
-            n = topk_tighten(s, n, k, &thr);
+            n = topk_tighten<DEEP>(s, n, k, &thr);
         }
         FTK_PHASE(9);
         // candidates -> stage-1 composite keys, in place
@@ -1051,19 +1203,36 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
             // Composite keys are unique, so "number of smaller keys" is the sorted position.
             // (keys are read two at a time; an odd list is padded with a key that never counts)
             const unsigned long long mine = t < n ? s.keys[t] : ~0ull;
-            const int                n2   = (n + 1) & ~1;
-            auto                     rank = [&](unsigned long long key) -> int {
+            // sixteen keys per round; DEEP: all eight loads in flight before the first compare
+            const int n16 = (n + 15) & ~15;
+            auto      rank = [&](unsigned long long key) -> int {
                 int q = 0;
+                if constexpr (DEEP) {
+                    for (int j0 = 0; j0 < n16; j0 += 16) {
+                        ulonglong2 kk[8];
+#pragma unroll
+                        for (int b = 0; b < 8; ++b) {
+                            kk[b] = *reinterpret_cast<const ulonglong2*>(&s.keys[j0 + 2 * b]);
+                        }
+#pragma unroll
+                        for (int b = 0; b < 8; ++b) {
+                            q += kk[b].x < key ? 1 : 0;
+                            q += kk[b].y < key ? 1 : 0;
+                        }
+                    }
+                }
+                else {
 #pragma unroll 4
-                for (int j = 0; j < n2; j += 2) {
-                    const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&s.keys[j]);
-                    q += kk.x < key ? 1 : 0;
-                    q += kk.y < key ? 1 : 0;
+                    for (int j = 0; j < n16; j += 2) {
+                        const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&s.keys[j]);
+                        q += kk.x < key ? 1 : 0;
+                        q += kk.y < key ? 1 : 0;
+                    }
                 }
                 return q;
             };
-            if (t == 0 && n2 != n) {
-                s.keys[n] = ~0ull;
+            if (t >= n && t < n16) {
+                s.keys[t] = ~0ull;  // padding that never counts
             }
             lds_barrier();
             const int                q      = rank(mine);
@@ -1220,11 +1389,23 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
         for (int ch = wave_id(); ch < splits; ch += TK_THREADS / WAVE) {
             const int        cnt = (int)headers[ch].count;
             const TopkEntry* e   = entries + (size_t)ch * TK_CCAP;
-            for (int i = lane_id(); i < cnt; i += WAVE) {
+            for (int i0 = 0; i0 < cnt; i0 += WAVE) {
+                const int i = i0 + lane_id();
                 // the first two rounds of a wave's first list were requested at the top of the kernel
-                const TopkEntry en = (ch == wave_id() && i < 2 * WAVE) ? pf.first[i >> 6] : e[i];
-                if (en.key >= thr) {
-                    const int slot = atomicAdd(&s.n_cand, 1);
+                TopkEntry en = TopkEntry{0u, 0u};
+                if (i < cnt) {
+                    en = (ch == wave_id() && i < 2 * WAVE) ? pf.first[i >> 6] : e[i];
+                }
+                // one slot reservation per wave and round
+                const bool               keep = i < cnt && en.key >= thr;
+                const unsigned long long m    = __ballot(keep);
+                int                      base = 0;
+                if (lane_id() == 0 && m != 0ull) {
+                    base = atomicAdd(&s.n_cand, (int)__builtin_popcountll(m));
+                }
+                base = __shfl(base, 0, WAVE);
+                if (keep) {
+                    const int slot = base + (int)__builtin_popcountll(m & ((1ull << lane_id()) - 1ull));
                     if (slot < TK_CCAP) {
                         s.cand.key[slot] = en.key;
                         s.cand.idx[slot] = en.idx;

@@ -393,7 +393,7 @@ __device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch
     return __int_as_float(s.misc[0]);
 }
 
-template<int DT, int BMW>
+template<int DT, int BMW, int MANY = 0>
 __global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
 fused_row_kernel(FusedParams p, FusedLaunch l)
 {
@@ -416,12 +416,12 @@ fused_row_kernel(FusedParams p, FusedLaunch l)
     FusedRow<DT, BMW> r(p, row);
     FTK_PHASE(0);
     uint32_t     thr = 0u;
-    const int    n   = topk_stream<DT>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
+    const int    n   = topk_stream<DT, FusedRow<DT, BMW>, MANY>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
     topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, l.entries + (size_t)row * l.row_entries, false, u,
                         p.end_ids, out);
 }
 
-template<int DT, int BMW>
+template<int DT, int BMW, int MANY = 0>
 __global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
 fused_gather_kernel(FusedParams p, FusedLaunch l)
 {
@@ -440,7 +440,7 @@ fused_gather_kernel(FusedParams p, FusedLaunch l)
     const int    t0    = min(tiles, chunk * l.tiles_per_wg);
     const int    t1    = min(tiles, t0 + l.tiles_per_wg);
     uint32_t     thr   = 0u;
-    const int    n     = topk_stream<DT>(r, s, p.Vp, k, t0, t1, &thr);
+    const int    n     = topk_stream<DT, FusedRow<DT, BMW>, MANY>(r, s, p.Vp, k, t0, t1, &thr);
     topk_dump_list(s, n, k, l.splits, thr, l.headers + (size_t)row * l.splits + chunk,
                    l.entries + (size_t)row * l.row_entries + (size_t)chunk * TK_CCAP);
 }
@@ -473,7 +473,7 @@ __global__ void __launch_bounds__(TK_THREADS) fused_select_kernel(FusedParams p,
     const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row);
     uint32_t     thr         = 0u;
     const int    n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr, pf);
-    topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
+    topk_select_lds<DT, FusedRow<DT, BMW>, true>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
 }
 
 }  // namespace ftk
@@ -586,6 +586,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const int      elem         = a->dtype == FTK_DTYPE_F32 ? 4 : 2;
     const int      rows         = a->local_batch_size;
     const TopkPlan plan         = topk_plan(a->vocab_size_padded, rows, a->max_top_k, elem);
+    const int      many         = topk_many_level(a->max_top_k);  // > 0: the large-k kernels (whole-row bitmaps only)
     const int      bitmap_words = (a->vocab_size_padded + 31) / 32 + 1;  // +1: vector_bits may peek one word ahead
     const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
     const size_t   need         = bitmap_bytes + plan.bytes;
@@ -641,7 +642,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         const int    epv        = 16 / elem;
         const size_t range_cols = (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
         const size_t words      = range_cols / 32 + 4;
-        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE
+        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && many == 0
                            && (plan.splits == 1 || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
         if (local) {
             p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
@@ -671,7 +672,15 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     l.entries         = (TopkEntry*)(l.headers + (size_t)rows * plan.splits);
     if (plan.splits == 1) {
         const dim3 grid1(rows), block(TK_THREADS);
-        if (p.bitmaps_ready) {
+        if (many == 2) {
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 2>, grid1,
+                                                      block, st, p, l));
+        }
+        else if (many == 1) {
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 1>, grid1,
+                                                      block, st, p, l));
+        }
+        else if (p.bitmaps_ready) {
             FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>, grid1, block,
                                                       st, p, l));
         }
@@ -689,7 +698,15 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     dim3 grid(plan.splits, rows);
     {
         const dim3 block(TK_THREADS);
-        if (p.bitmaps_ready) {
+        if (many == 2) {
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 2>, grid,
+                                                      block, st, p, l));
+        }
+        else if (many == 1) {
+            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 1>, grid,
+                                                      block, st, p, l));
+        }
+        else if (p.bitmaps_ready) {
             FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>, grid, block,
                                                       st, p, l));
         }

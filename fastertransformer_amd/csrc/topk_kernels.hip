@@ -50,7 +50,7 @@ __device__ __forceinline__ float topk_row_draw(TopkShared& s, RngState* rng, con
 }
 
 // rows owned by one workgroup: stream and select in a single launch
-template<int DT>
+template<int DT, int MANY = 0>
 __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_row_kernel(TopkKernelArgs a)
 {
     __shared__ TopkShared s;
@@ -71,13 +71,13 @@ __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_row_kernel(TopkKe
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
     uint32_t  thr = 0u;
-    const int n   = topk_stream<DT>(r, s, a.vocab, k, 0, topk_row_tiles<DT>(r.rowp, a.vocab), &thr);
+    const int n   = topk_stream<DT, PlainRowAt<DT>, MANY>(r, s, a.vocab, k, 0, topk_row_tiles<DT>(r.rowp, a.vocab), &thr);
     topk_select_lds<DT>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, a.entries + (size_t)row * a.row_entries,
                         a.cum_log_probs != nullptr || a.output_log_probs != nullptr, u, a.end_ids, out);
 }
 
 // rows split over `splits` workgroups: each leaves its candidate list in the workspace
-template<int DT>
+template<int DT, int MANY = 0>
 __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_gather_kernel(TopkKernelArgs a)
 {
     __shared__ TopkShared s;
@@ -98,7 +98,7 @@ __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_gather_kernel(Top
     const int t0    = min(tiles, chunk * a.tiles_per_wg);
     const int t1    = min(tiles, t0 + a.tiles_per_wg);
     uint32_t  thr   = 0u;
-    const int n     = topk_stream<DT>(r, s, a.vocab, k, t0, t1, &thr);
+    const int n     = topk_stream<DT, PlainRowAt<DT>, MANY>(r, s, a.vocab, k, t0, t1, &thr);
     topk_dump_list(s, n, k, a.splits, thr, a.headers + (size_t)row * a.splits + chunk,
                    a.entries + (size_t)row * a.row_entries + (size_t)chunk * TK_CCAP);
 }
@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(TK_THREADS) topk_select_kernel(TopkKernelArgs 
     FTK_PHASE(6);
     uint32_t   thr = 0u;
     const int  n   = topk_merge_lists<DT>(s, k, a.splits, a.headers + (size_t)row * a.splits, row_entries, &thr, pf);
-    topk_select_lds<DT>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, row_entries,
+    topk_select_lds<DT, PlainRowAt<DT>, true>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, row_entries,
                         a.cum_log_probs != nullptr || a.output_log_probs != nullptr, u, a.end_ids, out);
 }
 
@@ -208,13 +208,30 @@ int ftk_invoke_batch_topk_sampling(int dtype, void* workspace, size_t* workspace
     a.headers          = (TopkChunkHeader*)workspace;
     a.entries          = (TopkEntry*)(a.headers + (size_t)batch_size * plan.splits);
     hipStream_t st     = (hipStream_t)stream;
+    const int many = topk_many_level(max_top_k);  // > 0: the large-k variants of the streaming kernels
     if (plan.splits == 1) {
-        FTK_DISPATCH_DTYPE(dtype, topk_row_kernel<DT><<<batch_size, TK_THREADS, 0, st>>>(a));
+        if (many == 2) {
+            FTK_DISPATCH_DTYPE(dtype, topk_row_kernel<DT, 2><<<batch_size, TK_THREADS, 0, st>>>(a));
+        }
+        else if (many == 1) {
+            FTK_DISPATCH_DTYPE(dtype, topk_row_kernel<DT, 1><<<batch_size, TK_THREADS, 0, st>>>(a));
+        }
+        else {
+            FTK_DISPATCH_DTYPE(dtype, topk_row_kernel<DT><<<batch_size, TK_THREADS, 0, st>>>(a));
+        }
         FTK_LAUNCH_CHECK();
         return 0;
     }
     dim3 grid(plan.splits, batch_size);
-    FTK_DISPATCH_DTYPE(dtype, topk_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(a));
+    if (many == 2) {
+        FTK_DISPATCH_DTYPE(dtype, topk_gather_kernel<DT, 2><<<grid, TK_THREADS, 0, st>>>(a));
+    }
+    else if (many == 1) {
+        FTK_DISPATCH_DTYPE(dtype, topk_gather_kernel<DT, 1><<<grid, TK_THREADS, 0, st>>>(a));
+    }
+    else {
+        FTK_DISPATCH_DTYPE(dtype, topk_gather_kernel<DT><<<grid, TK_THREADS, 0, st>>>(a));
+    }
     FTK_LAUNCH_CHECK();
     FTK_DISPATCH_DTYPE(dtype, topk_select_kernel<DT><<<batch_size, TK_THREADS, 0, st>>>(a));
     FTK_LAUNCH_CHECK();
