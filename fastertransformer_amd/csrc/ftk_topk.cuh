@@ -947,10 +947,12 @@ struct TopkOutputs {
     // memory again; rows that are already finished never get here
     int   sequence_length_in;
     float cum_log_prob_in;
+    int   end_id_in;  // -1 when the caller passed no end ids to topk_outputs
 };
 
 __device__ __forceinline__ TopkOutputs topk_outputs(int* ids, int* sequence_length, bool* finished,
-                                                    float* cum_log_probs, float* output_log_probs, int row)
+                                                    float* cum_log_probs, float* output_log_probs, int row,
+                                                    const int* end_ids = nullptr)
 {
     TopkOutputs o;
     o.ids                = ids;
@@ -960,6 +962,7 @@ __device__ __forceinline__ TopkOutputs topk_outputs(int* ids, int* sequence_leng
     o.output_log_probs   = output_log_probs;
     o.sequence_length_in = sequence_length != nullptr ? sequence_length[row] : 0;
     o.cum_log_prob_in    = cum_log_probs != nullptr ? cum_log_probs[row] : 0.0f;
+    o.end_id_in          = end_ids != nullptr ? end_ids[row] : -1;
     return o;
 }
 
@@ -1021,7 +1024,7 @@ __device__ __forceinline__ void topk_emit(const TopkOutputs& o, int row, int id,
     }
     if (o.sequence_length != nullptr && o.finished != nullptr) {
         o.sequence_length[row] = o.sequence_length_in + 1;  // the row was not finished (:317-320)
-        o.finished[row]        = id == end_ids[row];
+        o.finished[row]        = id == (o.end_id_in >= 0 ? o.end_id_in : end_ids[row]);
     }
 }
 
@@ -1332,10 +1335,11 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
 }
 
 // What a select workgroup asks for before it knows anything about its row: wave w takes the first
-// 2 * 64 entries of chunk list w (most lists are shorter). Issued at the top of the kernel, the
+// 4 * 64 entries of chunk list w (most lists are shorter). Issued at the top of the kernel, the
 // loads are in flight while the row's arguments arrive; topk_merge_lists consumes them.
+constexpr int TK_PREFETCH = 4;
 struct TopkListPrefetch {
-    TopkEntry first[2];
+    TopkEntry first[TK_PREFETCH];
 };
 
 __device__ __forceinline__ TopkListPrefetch topk_prefetch_lists(int splits, const TopkEntry* entries)
@@ -1343,8 +1347,10 @@ __device__ __forceinline__ TopkListPrefetch topk_prefetch_lists(int splits, cons
     TopkListPrefetch pf;
     const int        ch = wave_id();
     const TopkEntry* e  = entries + (size_t)(ch < splits ? ch : 0) * TK_CCAP;  // always inside the row's slots
-    pf.first[0]         = e[lane_id()];
-    pf.first[1]         = e[WAVE + lane_id()];
+#pragma unroll
+    for (int r = 0; r < TK_PREFETCH; ++r) {
+        pf.first[r] = e[r * WAVE + lane_id()];
+    }
     return pf;
 }
 
@@ -1391,10 +1397,19 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
             const TopkEntry* e   = entries + (size_t)ch * TK_CCAP;
             for (int i0 = 0; i0 < cnt; i0 += WAVE) {
                 const int i = i0 + lane_id();
-                // the first two rounds of a wave's first list were requested at the top of the kernel
+                // the first rounds of a wave's first list were requested at the top of the kernel
                 TopkEntry en = TopkEntry{0u, 0u};
                 if (i < cnt) {
-                    en = (ch == wave_id() && i < 2 * WAVE) ? pf.first[i >> 6] : e[i];
+                    if (ch == wave_id() && i0 < TK_PREFETCH * WAVE) {
+                        en = pf.first[0];
+#pragma unroll
+                        for (int r = 1; r < TK_PREFETCH; ++r) {
+                            en = i0 == r * WAVE ? pf.first[r] : en;
+                        }
+                    }
+                    else {
+                        en = e[i];
+                    }
                 }
                 // one slot reservation per wave and round
                 const bool               keep = i < cnt && en.key >= thr;

@@ -67,7 +67,7 @@ __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_row_kernel(TopkKe
     const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
     const float    p = a.top_ps != nullptr ? a.top_ps[row] : a.top_p;
     const float    u = topk_row_draw(s, a.rng, a.uniforms, row);
-    const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row);
+    const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row, a.end_ids);
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
     uint32_t  thr = 0u;
@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(TK_THREADS) topk_select_kernel(TopkKernelArgs 
     }
     FTK_PHASE_BEGIN();
     const float    u = topk_row_draw(s, a.rng, a.uniforms, row);
-    const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row);
+    const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row, a.end_ids);
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
     FTK_PHASE(6);
