@@ -24,7 +24,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel on the headline workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by a copy kernel of known size (summary under profiles/)
-TRAFFIC_BYTES_PER_LAUNCH = 149911116
+TRAFFIC_BYTES_PER_LAUNCH = 152029196
 
 WORKLOADS = {
     # the configuration the headline metric is quoted on
