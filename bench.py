@@ -36,7 +36,7 @@ WORKLOADS = {
     "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9": dict(
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=0, top_p=(0.5, 0.99), top_p_decay=0.9,
         top_p_min=0.3, top_p_reset_id=13, zipf_s=1.1, noise=0.5, prompt=0),
-    # secondary line (only with --workload): the full decode loop of BASELINE config 5, per-step latency with
+    # secondary line (only with --workload): the full decode loop at batch 1024 (fp16, vocabulary 152064), per-step latency with
     # cum_log_probs / output_log_probs and the length criterion on (the kernel-by-kernel path: log-probs need the
     # probabilities of the whole row)
     "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs": dict(
