@@ -681,3 +681,45 @@ def test_softmax_and_topp_random_shapes(env, dt, seed):
             skip = rng.random(batch) < 0.2
             args = (dt, want, p_arr, end_ids, u, finished.copy(), seq, skip, True)
             _compare_topk(_run_topp(env, *args), _oracle_topp(*args), dt)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("max_k", [129, 512, 513, 1024])
+def test_topk_sampling_large_k_variants(env, dt, max_k):
+    """Launches whose largest k exceeds 128 (and 512) take their own streaming variants: rows of several tiles,
+    odd vocabulary (rows off the 16-byte grid), small k next to large k in one launch, smooth and heavily tied
+    distributions, a row that is constant from some column on (cutting the list back in mid-tile cannot bound
+    it: literal replay)."""
+    rng = np.random.default_rng(max_k + dt)
+    V = 70001
+    batch = 6
+    x = (rng.standard_normal((batch, V)) * 2.0).astype(np.float32)
+    x[1] = rng.integers(0, 6, V).astype(np.float32) * 0.5        # six distinct values
+    x[2, 20000:] = 3.0                                           # constant tail above most of the head
+    x[3] = np.round(x[3] * 8) / 8                                # many small tie groups
+    x[4, ::3] = -np.inf
+    logits = O.to_storage(x, dt)
+    k_arr = np.array([max_k, max_k, max_k, max(1, max_k // 2), max_k - 1, 5], np.int32)
+    end_ids = np.zeros(batch, np.int32)
+    for trial in range(2):
+        p_arr = np.ones(batch, np.float32) if trial == 0 else rng.uniform(0.3, 1.0, batch).astype(np.float32)
+        u = uniforms(rng, batch)
+        args = (dt, logits, k_arr, p_arr, max_k, end_ids, u)
+        _compare_topk(_run_topk(env, *args), _oracle_topk(*args), dt)
+
+
+@pytest.mark.parametrize("max_k", [200, 700, 1024])
+def test_topk_sampling_large_k_many_tiles_per_workgroup(env, max_k):
+    """A vocabulary of more tiles than a row can be split into, so that every workgroup streams two tiles:
+    the large-k variants then cut their list back between tiles (and in mid-tile beyond k = 512)."""
+    rng = np.random.default_rng(max_k)
+    V, batch = 1100003, 2
+    x = (rng.standard_normal((batch, V)) * 2.0).astype(np.float32)
+    x[1] = np.round(x[1] * 16) / 16   # tie groups of a few thousand columns
+    logits = O.to_storage(x, O.F32)
+    k_arr = np.array([max_k, max(1, max_k - 3)], np.int32)
+    end_ids = np.zeros(batch, np.int32)
+    p_arr = np.array([1.0, 0.7], np.float32)
+    u = uniforms(rng, batch)
+    args = (O.F32, logits, k_arr, p_arr, max_k, end_ids, u)
+    _compare_topk(_run_topk(env, *args), _oracle_topk(*args), O.F32)
