@@ -228,15 +228,20 @@ void TopKSamplingLayer<T>::runSampling(TensorMap* output_tensors, TensorMap* inp
 
     const int* end_ids  = input_tensors->at("end_id").template getPtr<const int>();
     bool*      finished = output_tensors->at("finished", Tensor()).template getPtr<bool>();
-    invokeAddBiasEndMask(logits, (T*)nullptr, end_ids, finished, local_batch_size, (int)vocab_size_,
-                         (int)vocab_size_padded_, stream_);
-    sync_check_hip_error();
-
     float* cum_log_probs    = output_tensors->at("cum_log_probs", Tensor()).template getPtr<float>();
     float* output_log_probs = output_tensors->at("output_log_probs", Tensor()).template getPtr<float>();
     if (cum_log_probs != nullptr || output_log_probs != nullptr) {
+        // The reference masks pads and finished rows (invokeAddBiasEndMask) and then takes the softmax of the
+        // result (TopKSamplingLayer.cu:220-245). The softmax applies the very same mask to what it reads
+        // (pad columns -> -MAX_T, finished rows -> +-MAX_T by end id), so the first pass over the logits
+        // changes nothing in its result and is left out.
         invokeAddBiasSoftMax(logits, (T*)nullptr, end_ids, finished, local_batch_size, (int)vocab_size_padded_,
                              (int)vocab_size_, stream_);
+        sync_check_hip_error();
+    }
+    else {
+        invokeAddBiasEndMask(logits, (T*)nullptr, end_ids, finished, local_batch_size, (int)vocab_size_,
+                             (int)vocab_size_padded_, stream_);
         sync_check_hip_error();
     }
     ensureWorkspace(local_batch_size);
