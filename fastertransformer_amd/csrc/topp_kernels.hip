@@ -265,8 +265,11 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
 //                prefix divided into segments of whole buckets;
 //   gather     - second stream: entries at or above the cut go to their bucket's range as
 //                (~key, id) pairs;
-//   sort       - segments are sorted independently (bitonic in LDS, a radix sort in memory for a
-//                segment that one bucket alone makes too long);
+//   sort       - segments are sorted independently, dealt out over the workgroups of one launch: the
+//                keys of a segment are spread over bins, neighbouring bins joined into groups of a few
+//                dozen entries, and every group sorted by one wave in registers (a long group of equal
+//                keys by the whole workgroup in LDS, a segment that one bucket alone makes too long
+//                by a radix sort in memory);
 //   pick       - one workgroup per row replays the reference's scan on the ordered prefix with its
 //                exact rounding order (32 raking lanes x 8 items, Kogge-Stone over the 32 partials,
 //                sequential carry over tiles) and emits the token.
