@@ -723,3 +723,41 @@ def test_topk_sampling_large_k_many_tiles_per_workgroup(env, max_k):
     u = uniforms(rng, batch)
     args = (O.F32, logits, k_arr, p_arr, max_k, end_ids, u)
     _compare_topk(_run_topk(env, *args), _oracle_topk(*args), O.F32)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_topk_sampling_random_shapes(env, dt, seed):
+    """Seeded random vocabulary sizes (odd ones included), batch sizes (hence different numbers of chunk lists
+    per row), per-row k from 1 to the launch maximum, per-row top-p, smooth / tied / mostly masked rows,
+    finished and skipped rows, log-probs on probabilities for half of the cases."""
+    rng = np.random.default_rng(500 * dt + seed)
+    for case in range(5):
+        V = int(rng.choice([rng.integers(9, 400), rng.integers(400, 20000), rng.integers(20000, 140000)]))
+        batch = int(rng.choice([1, 2, 5, 9, 17, 40]))
+        max_k = int(rng.choice([1, 7, 64, 100, 200, 600, 1024]))
+        max_k = max(1, min(max_k, 1024))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            x = rng.standard_normal((batch, V)) * rng.uniform(0.3, 4.0)
+        elif kind == 1:
+            x = rng.integers(0, 5, (batch, V)).astype(np.float64) * rng.uniform(0.2, 1.5)
+        else:
+            x = np.where(rng.random((batch, V)) < 0.9, -np.inf, rng.standard_normal((batch, V)) * 2.0)
+            x[:, 0] = 0.5
+        logits = O.to_storage(x.astype(np.float32), dt)
+        end_ids = rng.integers(0, V, batch).astype(np.int32)
+        k_arr = rng.integers(1, max_k + 1, batch).astype(np.int32)
+        k_arr[0] = max_k
+        p_arr = np.where(rng.random(batch) < 0.5, 1.0, rng.uniform(0.1, 1.0, batch)).astype(np.float32)
+        finished = rng.random(batch) < 0.1
+        seq = rng.integers(1, 9, batch).astype(np.int32)
+        skip = rng.random(batch) < 0.1
+        u = uniforms(rng, batch)
+        logprobs = bool(case & 1)
+        src = logits
+        if logprobs:
+            src = logits.copy()
+            O.add_bias_softmax(dt, src, None, end_ids, None, batch, V, V)
+        args = (dt, src, k_arr, p_arr, max_k, end_ids, u, finished.copy(), seq, skip, logprobs)
+        _compare_topk(_run_topk(env, *args), _oracle_topk(*args), dt)

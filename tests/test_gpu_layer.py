@@ -323,3 +323,37 @@ def test_error_behaviour():
     layer.setup(2, 1, {"runtime_top_k": np.array([5000], np.uint32)})
     layer.forward({"output_ids": out_ids}, base)
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_fused_step_random_scenarios(dt, seed):
+    """Seeded random decode scenarios through the fused top-k step (no log-probs): batch sizes that split a row
+    over different numbers of workgroups, odd and padded vocabularies, per-row k up to several hundred with
+    and without top-p, temperature, repetition or presence penalty over short and long histories with short
+    prompts, min length; three steps each, ids / flags / lengths bit-exact against the oracle."""
+    rng = np.random.default_rng(900 + 10 * dt + seed)
+    for case in range(3):
+        B = int(rng.choice([1, 3, 7, 20, 48]))
+        V = int(rng.choice([rng.integers(600, 3000), rng.integers(3000, 40000), rng.integers(40000, 131000)]))
+        Vp = V + int(rng.choice([0, 0, 3, 61]))
+        H = int(rng.choice([4, 40, 300]))
+        max_k = int(rng.choice([1, 8, 64, 150, 400]))
+        ks = rng.integers(1, max_k + 1, B).astype(np.uint32)
+        ks[0] = max_k
+        ps = np.where(rng.random(B) < 0.5, 1.0, rng.uniform(0.2, 0.99, B)).astype(np.float32)
+        kw = {}
+        if rng.random() < 0.7:
+            kw["temperature"] = rng.uniform(0.5, 1.6, B)
+        pen = int(rng.integers(0, 3))
+        if pen == 1:
+            kw["repetition_penalty"] = rng.uniform(1.0, 1.6, B)
+        elif pen == 2:
+            kw["presence_penalty"] = rng.uniform(0.0, 1.5, B)
+        if rng.random() < 0.5:
+            kw["min_length"] = rng.integers(0, 4, B)
+        c = Case(dt, B, V, Vp, max_input_length=H, gen_len=3, runtime_top_k=ks, runtime_top_p=ps,
+                 prompt=_history(rng, H, B, V, zipf=1.3 if rng.random() < 0.5 else None),
+                 input_lengths=rng.integers(1, H + 1, B), end_ids=rng.integers(0, V, B).astype(np.int32), **kw)
+        scale = float(rng.uniform(0.5, 4.0))
+        _run_case(c, rng, 3, lambda i: make_logits(rng, dt, B, V, Vp, scale), check_logits=False)
