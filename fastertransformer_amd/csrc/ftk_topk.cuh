@@ -756,13 +756,13 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
     };
     // the list is cut back to its k largest between tiles when it has grown past this; with a large k
     // after every tile (another tile's worth at the old bound would not fit)
-    const int tighten_at = MANY > 0 ? k : min(max(256, 2 * k), 3 * TK_CCAP / 4);
+    const int tighten_at = (MANY > 0 && k > TK_STAGE) ? k : min(max(256, 2 * k), 3 * TK_CCAP / 4);
     int       n          = 0;
     // With a large k a tile holds more candidates than a wave can park between two drains of a whole
     // tile (k alone can exceed it): such launches take the general tile loop, which then drains every
     // second vector.
     static_assert(2 * WAVE <= TK_STAGE, "two vectors per lane fit the parking space");
-    constexpr bool many    = MANY > 0;
+    const bool     many    = MANY > 0 && k > TK_STAGE;  // rows with a small k of such a launch keep the fast loop
     constexpr bool cut_mid = MANY > 1;
 
     for (int tile = tile_begin; tile < tile_end; ++tile) {
