@@ -143,29 +143,6 @@ __device__ __forceinline__ uint32_t wave_sort_desc(uint32_t v)
     return v;
 }
 
-// In-LDS bitonic sort (ascending) of n 64-bit keys, n a power of two, by the THREADS threads of the block.
-template<int THREADS>
-__device__ __forceinline__ void block_bitonic_sort_u64(unsigned long long* keys, int n)
-{
-    for (int k = 2; k <= n; k <<= 1) {
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int i = (int)threadIdx.x; i < (n >> 1); i += THREADS) {
-                // i-th compare-exchange pair of this stage
-                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
-                const int hi = lo | j;
-                const bool up = (lo & k) == 0;
-                const unsigned long long a = keys[lo];
-                const unsigned long long b = keys[hi];
-                if ((a > b) == up) {
-                    keys[lo] = b;
-                    keys[hi] = a;
-                }
-            }
-            __syncthreads();
-        }
-    }
-}
-
 __device__ __forceinline__ int next_pow2(int n)
 {
     int p = 1;

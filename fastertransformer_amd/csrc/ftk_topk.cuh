@@ -53,6 +53,9 @@ namespace ftk {
 constexpr int TK_THREADS  = FTK_TK_THREADS;
 constexpr int TK_WAVES    = TK_THREADS / 64;
 constexpr int TK_MIN_WGS  = 1024 / TK_THREADS;  // workgroups per compute unit the kernels are built for
+// The variants for a large k hold a whole tile and two transformed copies of a vector in registers beside the
+// bookkeeping of the general tile loop: they are built for half as many workgroups, with twice the registers.
+constexpr int TK_MIN_WGS_MANY = TK_MIN_WGS / 2;
 constexpr int TK_NVT      = 16;    // 16-byte vectors per thread and tile: 64 KB per workgroup in flight
 constexpr int TK_CCAP     = 2048;  // candidates a workgroup can hold
 constexpr int TK_MAXSPLIT = 64;
@@ -492,8 +495,9 @@ __device__ __noinline__ int topk_stream_rare(Row rowctx, TopkShared& s, int k, i
 // of the range from below; otherwise the list holds every selectable element of the range.
 // MANY > 0: the variant for launches whose largest k exceeds what a wave can park per tile (TK_STAGE): the
 // bound of the first tile is refined on the registers that hold it, and every tile takes the general loop,
-// which then drains every second vector. MANY == 2 (largest k beyond a quarter of the list's capacity)
-// also cuts the list back in the middle of a tile. Rows of such a launch with a small k run the same code.
+// which then writes its candidates to the list directly. MANY == 2 (largest k beyond a quarter of the
+// list's capacity) also cuts the list back in the middle of a tile. Rows of such a launch with a small k
+// keep the parking loop.
 template<int DT, class Row, int MANY = 0>
 __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab, int k, int tile_begin, int tile_end,
                                            uint32_t* thr_out)
@@ -758,10 +762,9 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
     // after every tile (another tile's worth at the old bound would not fit)
     const int tighten_at = (MANY > 0 && k > TK_STAGE) ? k : min(max(256, 2 * k), 3 * TK_CCAP / 4);
     int       n          = 0;
-    // With a large k a tile holds more candidates than a wave can park between two drains of a whole
-    // tile (k alone can exceed it): such launches take the general tile loop, which then drains every
-    // second vector.
-    static_assert(2 * WAVE <= TK_STAGE, "two vectors per lane fit the parking space");
+    // With a large k a tile holds more candidates than a wave can park before the tile's drain (k alone
+    // can exceed the space): such rows take the general tile loop, which then writes its candidates to the
+    // list directly.
     const bool     many    = MANY > 0 && k > TK_STAGE;  // rows with a small k of such a launch keep the fast loop
     constexpr bool cut_mid = MANY > 1;
 
@@ -800,8 +803,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
             }
         }
         else {
-#pragma unroll
-            for (int it = 0; it < NVT; ++it) {
+            auto general_vector = [&](int it) {
                 const int  vi    = vec0 + it * TK_THREADS + t;
                 const int  first = first0 + it * TK_THREADS * EPV;
                 // vectors inside the row with no index-dependent column stay on the register path
@@ -812,36 +814,77 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
                 for (int j = 0; j < EPV; ++j) {
                     x[j] = rowctx.fast(vector_element<DT>(raw[it], j));
                 }
-                if (bitsv && fastv) {
-                    const uint32_t bits = rowctx.vector_bits(first, EPV);
+                if constexpr (MANY == 0) {
+                    if (bitsv && fastv) {
+                        const uint32_t bits = rowctx.vector_bits(first, EPV);
+                        if (bits != 0u) {
+#pragma unroll
+                            for (int j = 0; j < EPV; ++j) {
+                                x[j] = ((bits >> j) & 1u) ? rowctx.flagged_upper(x[j]) : x[j];
+                            }
+                        }
+                    }
+                    float vmax = x[0];
+#pragma unroll
+                    for (int j = 1; j < EPV; ++j) {
+                        vmax = __builtin_fmaxf(vmax, x[j]);
+                    }
+                    park(fastv && vmax >= thr_f, raw[it], first);
+                    return;
+                }
+                float xu[EPV];  // the same with upper bounds in the history's columns
+#pragma unroll
+                for (int j = 0; j < EPV; ++j) {
+                    xu[j] = x[j];
+                }
+                const uint32_t bits = (bitsv && fastv) ? rowctx.vector_bits(first, EPV) : 0u;
+                if (bits != 0u) {
+#pragma unroll
+                    for (int j = 0; j < EPV; ++j) {
+                        xu[j] = ((bits >> j) & 1u) ? rowctx.flagged_upper(x[j]) : x[j];
+                    }
+                }
+                float vmax = xu[0];
+#pragma unroll
+                for (int j = 1; j < EPV; ++j) {
+                    vmax = __builtin_fmaxf(vmax, xu[j]);
+                }
+                if (!many) {
+                    park(fastv && vmax >= thr_f, raw[it], first);
+                }
+                else if (fastv && vmax >= thr_f) {
+                    // With a large k a quarter or more of the vectors hold a candidate: they go to the list
+                    // directly, with the exact values of the history's columns.
                     if (bits != 0u) {
 #pragma unroll
                         for (int j = 0; j < EPV; ++j) {
-                            x[j] = ((bits >> j) & 1u) ? rowctx.flagged_upper(x[j]) : x[j];
+                            if ((bits >> j) & 1u) {
+                                x[j] = rowctx.flagged(x[j]);
+                            }
                         }
                     }
+                    push_vector(first, x);
                 }
-                float vmax = x[0];
+            };
 #pragma unroll
-                for (int j = 1; j < EPV; ++j) {
-                    vmax = __builtin_fmaxf(vmax, x[j]);
+            for (int it = 0; it < (MANY > 0 ? NVT / 2 : NVT); ++it) {
+                general_vector(it);
+            }
+            if (cut_mid && many && k > TK_CCAP / 4) {
+                // Half a tile at the bound of the tiles before it can add more than half of k: with
+                // k beyond a quarter of the list's capacity the list is cut back in mid-tile too.
+                lds_barrier();
+                const int n_mid = s.n_cand;
+                lds_barrier();
+                if (n_mid > k && n_mid <= TK_CCAP) {
+                    n         = topk_tighten(s, n_mid, k, &thr);
+                    thr_f     = key_to_float(thr);
+                    cut_early = true;
                 }
-                park(fastv && vmax >= thr_f, raw[it], first);
-                if (many && (it & 1)) {
-                    drain();  // two vectors per lane never overfill the wave's parking space
-                    if (cut_mid && it == NVT / 2 - 1 && k > TK_CCAP / 4) {
-                        // Half a tile at the bound of the tiles before it can add more than half of k: with
-                        // k beyond a quarter of the list's capacity the list is cut back in mid-tile too.
-                        lds_barrier();
-                        const int n_mid = s.n_cand;
-                        lds_barrier();
-                        if (n_mid > k && n_mid <= TK_CCAP) {
-                            n         = topk_tighten(s, n_mid, k, &thr);
-                            thr_f     = key_to_float(thr);
-                            cut_early = true;
-                        }
-                    }
-                }
+            }
+#pragma unroll
+            for (int it = (MANY > 0 ? NVT / 2 : NVT); it < NVT; ++it) {
+                general_vector(it);
             }
             for (; slowmask != 0u; slowmask &= slowmask - 1u) {
                 const int first = first0 + __builtin_ctz(slowmask) * TK_THREADS * EPV;
@@ -1255,24 +1298,16 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
             __syncthreads();
         }
         else {
-            // ---- large candidate sets: two bitonic sorts
-            const int np2 = max(2, next_pow2(n));
-            for (int i = n + t; i < np2; i += TK_THREADS) {
-                s.keys[i] = ~0ull;
+            // ---- large candidate sets: two bitonic sorts (of exactly n keys: no padding to a power of two)
+            block_sort_u64<TK_THREADS>(s.keys, n);
+            for (int qi = t; qi < n; qi += TK_THREADS) {
+                int                      idx;
+                const unsigned long long nk = stage2_key(s.keys[qi], qi, qi, &idx);
+                s.sel.idx[qi]               = idx;
+                s.keys[qi]                  = nk;
             }
             __syncthreads();
-            block_bitonic_sort_u64<TK_THREADS>(s.keys, np2);
-            for (int qi = t; qi < np2; qi += TK_THREADS) {
-                unsigned long long nk = ~0ull;
-                if (qi < n) {
-                    int idx;
-                    nk        = stage2_key(s.keys[qi], qi, qi, &idx);
-                    s.sel.idx[qi] = idx;
-                }
-                s.keys[qi] = nk;
-            }
-            __syncthreads();
-            block_bitonic_sort_u64<TK_THREADS>(s.keys, np2);
+            block_sort_u64<TK_THREADS>(s.keys, n);
             {
                 int cnt = 0;
                 for (int i = t; i < min(k, n); i += TK_THREADS) {

@@ -394,7 +394,7 @@ __device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch
 }
 
 template<int DT, int BMW, int MANY = 0>
-__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
+__global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
 fused_row_kernel(FusedParams p, FusedLaunch l)
 {
     __shared__ TopkShared s;
@@ -422,7 +422,7 @@ fused_row_kernel(FusedParams p, FusedLaunch l)
 }
 
 template<int DT, int BMW, int MANY = 0>
-__global__ void __launch_bounds__(TK_THREADS, BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
+__global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
 fused_gather_kernel(FusedParams p, FusedLaunch l)
 {
     __shared__ TopkShared s;

@@ -51,7 +51,7 @@ __device__ __forceinline__ float topk_row_draw(TopkShared& s, RngState* rng, con
 
 // rows owned by one workgroup: stream and select in a single launch
 template<int DT, int MANY = 0>
-__global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_row_kernel(TopkKernelArgs a)
+__global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : TK_MIN_WGS) topk_row_kernel(TopkKernelArgs a)
 {
     __shared__ TopkShared s;
     const int             row = blockIdx.x;
@@ -78,7 +78,7 @@ __global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_row_kernel(TopkKe
 
 // rows split over `splits` workgroups: each leaves its candidate list in the workspace
 template<int DT, int MANY = 0>
-__global__ void __launch_bounds__(TK_THREADS, TK_MIN_WGS) topk_gather_kernel(TopkKernelArgs a)
+__global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : TK_MIN_WGS) topk_gather_kernel(TopkKernelArgs a)
 {
     __shared__ TopkShared s;
     const int             row   = blockIdx.y;
