@@ -96,7 +96,9 @@ inline TopkPlan topk_plan(int vocab_padded, int batch, int max_top_k, int elem_b
     const int tile_vecs = TK_THREADS * TK_NVT;
     const int nvec      = vocab_padded / epv + 2;  // worst case over row misalignments
     const int tiles     = (nvec + tile_vecs - 1) / tile_vecs;
-    int       s         = (TK_FILL_WGS + batch - 1) / (batch > 0 ? batch : 1);
+    // as many workgroups as the chip holds at once (the large-k variants are built for fewer per compute unit)
+    const int fill      = topk_many_level(max_top_k) > 0 ? 256 * TK_MIN_WGS_MANY : TK_FILL_WGS;
+    int       s         = (fill + batch - 1) / (batch > 0 ? batch : 1);
     s                   = s > tiles ? tiles : s;
     s                   = s > TK_MAXSPLIT ? TK_MAXSPLIT : s;
     s                   = s < 1 ? 1 : s;
@@ -803,6 +805,11 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
             }
         }
         else {
+            // a plain tile of a row with a large k: the flags of all its vectors are requested in one go
+            const bool flags_packed = MANY > 0 && packed_ok && tile_plain(tile);
+            if (flags_packed && tile != tile_begin) {
+                rowctx.template tile_bits<EPV, NVT>(first0, TK_THREADS * EPV, packed);
+            }
             auto general_vector = [&](int it) {
                 const int  vi    = vec0 + it * TK_THREADS + t;
                 const int  first = first0 + it * TK_THREADS * EPV;
@@ -837,7 +844,8 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
                 for (int j = 0; j < EPV; ++j) {
                     xu[j] = x[j];
                 }
-                const uint32_t bits = (bitsv && fastv) ? rowctx.vector_bits(first, EPV) : 0u;
+                const uint32_t bits =
+                    (bitsv && fastv) ? (flags_packed ? flags_of(it, first) : rowctx.vector_bits(first, EPV)) : 0u;
                 if (bits != 0u) {
 #pragma unroll
                     for (int j = 0; j < EPV; ++j) {
