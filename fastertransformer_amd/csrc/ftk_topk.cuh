@@ -97,20 +97,28 @@ inline TopkPlan topk_plan(int vocab_padded, int batch, int max_top_k, int elem_b
     const int nvec      = vocab_padded / epv + 2;  // worst case over row misalignments
     const int tiles     = (nvec + tile_vecs - 1) / tile_vecs;
     // as many workgroups as the chip holds at once (the large-k variants are built for fewer per compute unit)
-    const int fill      = topk_many_level(max_top_k) > 0 ? 256 * TK_MIN_WGS_MANY : TK_FILL_WGS;
-    int       s         = (fill + batch - 1) / (batch > 0 ? batch : 1);
-    s                   = s > tiles ? tiles : s;
-    s                   = s > TK_MAXSPLIT ? TK_MAXSPLIT : s;
-    s                   = s < 1 ? 1 : s;
-    p.tiles_per_wg      = (tiles + s - 1) / s;
-    p.splits            = (tiles + p.tiles_per_wg - 1) / p.tiles_per_wg;
-    size_t entries      = p.splits > 1 ? (size_t)p.splits * TK_CCAP : 0;
-    const size_t lit    = (size_t)8 * (max_top_k > 0 ? max_top_k : 1);  // the literal replay keeps 8k picks
+    auto split = [&](int fill, int* tiles_per_wg) -> int {
+        int s         = (fill + batch - 1) / (batch > 0 ? batch : 1);
+        s             = s > tiles ? tiles : s;
+        s             = s > TK_MAXSPLIT ? TK_MAXSPLIT : s;
+        s             = s < 1 ? 1 : s;
+        *tiles_per_wg = (tiles + s - 1) / s;
+        return (tiles + *tiles_per_wg - 1) / *tiles_per_wg;
+    };
+    int       unused;
+    const int splits_most = split(TK_FILL_WGS, &unused);
+    p.splits = split(topk_many_level(max_top_k) > 0 ? 256 * TK_MIN_WGS_MANY : TK_FILL_WGS, &p.tiles_per_wg);
+    size_t entries   = p.splits > 1 ? (size_t)p.splits * TK_CCAP : 0;
+    const size_t lit = (size_t)8 * (max_top_k > 0 ? max_top_k : 1);  // the literal replay keeps 8k picks
     if (entries < lit) {
         entries = lit;
     }
     p.row_entries = entries;
-    p.bytes       = (size_t)batch * (p.splits * sizeof(TopkChunkHeader) + entries * sizeof(TopkEntry));
+    // the size asked for never shrinks with a larger k: it covers the split of the small-k variants too
+    const size_t entries_most = splits_most > 1 ? (size_t)splits_most * TK_CCAP : 0;
+    p.bytes = (size_t)batch
+              * ((size_t)(splits_most > p.splits ? splits_most : p.splits) * sizeof(TopkChunkHeader)
+                 + (entries_most > entries ? entries_most : entries) * sizeof(TopkEntry));
     return p;
 }
 
