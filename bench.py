@@ -39,6 +39,11 @@ WORKLOADS = {
     # secondary line (only with --workload): the full decode loop at batch 1024 (fp16, vocabulary 152064), per-step latency with
     # cum_log_probs / output_log_probs and the length criterion on (the kernel-by-kernel path: log-probs need the
     # probabilities of the whole row)
+    # secondary line (only with --workload): the fused step with a per-row k drawn from {1, 4, 16, 40, 64, 1024}
+    # (fp16, vocabulary 51200): the rows with k = 1024 set the pace of the launch
+    "decode_step_b256_v51200_f16_topk1-1024_topp0.9_temp0.8_rep1.1": dict(
+        dtype="f16", batch=256, vocab=51200, vocab_padded=51200, top_k=(1, 4, 16, 40, 64, 1024), top_p=0.9,
+        temperature=0.8, repetition_penalty=1.1, prompt=64, sigma=2.5),
     "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs": dict(
         dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=8, sigma=2.5),
@@ -74,7 +79,11 @@ def run_gpu(name, w, steps, warmup, nbuf=4):
     draws = [torch.rand(B, generator=gen, device=dev).clamp_(min=1e-7) for _ in range(nbuf)]
 
     layer = fa.DynamicDecodeLayer(dt, V, Vp)
-    args = {"runtime_top_k": np.array([w["top_k"]], np.uint32), "runtime_top_p": np.array([w["top_p"]], np.float32),
+    if isinstance(w["top_k"], tuple):  # one k per row, drawn from the choices
+        top_ks = np.random.default_rng(0).choice(np.array(w["top_k"], np.uint32), B).astype(np.uint32)
+    else:
+        top_ks = np.array([w["top_k"]], np.uint32)
+    args = {"runtime_top_k": top_ks, "runtime_top_p": np.array([w["top_p"]], np.float32),
             "temperature": np.array([w["temperature"]], np.float32),
             "repetition_penalty": np.array([w["repetition_penalty"]], np.float32),
             "random_seed": np.array([7], np.uint64)}
@@ -321,6 +330,20 @@ def main():
             "sampled_ids_checksum": r["sampled_ids_checksum"]}))
         return
     r = run_gpu(name, w, a.steps, a.warmup)
+    if name != next(iter(WORKLOADS)):
+        r["roofline"]["traffic"] = None  # the counter runs cover the headline workload only
+        print(json.dumps({
+            "metric": "sampled tokens/s, decode step B=%d V=%d (full top-k+top-p+penalty DynamicDecodeLayer step)"
+                      % (w["batch"], w["vocab"]),
+            "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": w["dtype"], "data": "synthetic",
+            "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"], "top_k": list(w["top_k"]),
+                       "top_p": w["top_p"], "temperature": w["temperature"],
+                       "repetition_penalty": w["repetition_penalty"], "history": w["prompt"]},
+            "roofline": r["roofline"], "gpu_ms_per_step": r["gpu_ms_per_step"], "kernel_ms": r["kernel_ms"],
+            "sampled_ids_checksum": r["sampled_ids_checksum"]}))
+        return
     if a.copy_calibration:
         import torch
         src = torch.empty(128 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
