@@ -357,3 +357,30 @@ def test_fused_step_random_scenarios(dt, seed):
                  input_lengths=rng.integers(1, H + 1, B), end_ids=rng.integers(0, V, B).astype(np.int32), **kw)
         scale = float(rng.uniform(0.5, 4.0))
         _run_case(c, rng, 3, lambda i: make_logits(rng, dt, B, V, Vp, scale), check_logits=False)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("max_k", [200, 700, 1024])
+def test_fused_step_large_k_with_bias_and_history(dt, max_k):
+    """The large-k variants of the fused step (largest k above 128, above 512): rows with small and large k in one
+    launch, an unaligned and padded vocabulary, embedding bias (no tile takes the fast transform), long histories
+    with repeated tokens under a repetition penalty, temperature, min length; a second scenario without bias so
+    that plain tiles fetch their history flags in one go. Three steps each, bit-exact against the oracle."""
+    rng = np.random.default_rng(4100 + 7 * dt + max_k)
+    for with_bias in (True, False):
+        B = 9
+        V = int(rng.integers(36000, 70000)) | 1
+        Vp = V + 5
+        H = 200
+        ks = rng.integers(1, max_k + 1, B).astype(np.uint32)
+        ks[0], ks[1] = max_k, 3
+        kw = {"temperature": rng.uniform(0.6, 1.4, B), "repetition_penalty": rng.uniform(1.05, 1.5, B),
+              "min_length": rng.integers(0, 3, B)}
+        if with_bias:
+            kw["embedding_bias"] = O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt)
+        c = Case(dt, B, V, Vp, max_input_length=H, gen_len=3, runtime_top_k=ks,
+                 runtime_top_p=rng.uniform(0.5, 1.0, B).astype(np.float32),
+                 prompt=_history(rng, H, B, V, zipf=1.3), input_lengths=rng.integers(H // 2, H + 1, B),
+                 end_ids=rng.integers(0, V, B).astype(np.int32), **kw)
+        _run_case(c, rng, 3, lambda i: make_logits(rng, dt, B, V, Vp, 2.0), check_logits=False)
