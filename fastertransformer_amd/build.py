@@ -21,8 +21,19 @@ INCLUDE = os.path.join(ROOT, "include")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-KERNEL_SOURCES = ["penalty_kernels.hip", "criteria_kernels.hip", "topp_kernels.hip", "topk_kernels.hip",
-                  "fused_kernels.hip", "decode_step_kernels.hip"]
+# (source, object, extra flags): lean_kernels.hip is built once per element type so the three sets of kernels
+# compile side by side
+KERNEL_UNITS = [
+    ("fused_kernels.hip", "fused_kernels.o", []),
+    ("topp_kernels.hip", "topp_kernels.o", []),
+    ("topk_kernels.hip", "topk_kernels.o", []),
+    ("lean_kernels.hip", "lean_kernels_f32.o", ["-DFTK_LEAN_DT=0"]),
+    ("lean_kernels.hip", "lean_kernels_f16.o", ["-DFTK_LEAN_DT=1"]),
+    ("lean_kernels.hip", "lean_kernels_bf16.o", ["-DFTK_LEAN_DT=2"]),
+    ("penalty_kernels.hip", "penalty_kernels.o", []),
+    ("criteria_kernels.hip", "criteria_kernels.o", []),
+    ("decode_step_kernels.hip", "decode_step_kernels.o", []),
+]
 
 # -ffp-contract=off: results must match a plain IEEE evaluation operation by operation.
 # Packed fp32 instructions are disabled on purpose: the compiler forms them from ordinary float code, and some of
@@ -50,15 +61,17 @@ def build(force=True, verbose=True, with_torch=True):
     os.makedirs(LIB, exist_ok=True)
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".cuh"))]
     headers.append(os.path.join(INCLUDE, "ftk_sampling.h"))
-    objs = []
-    for src in KERNEL_SOURCES:
+    objs, jobs = [], []
+    for src, obj_name, extra in KERNEL_UNITS:
         path = os.path.join(CSRC, src)
-        if not os.path.exists(path):
-            continue
-        obj = os.path.join(LIB, src.replace(".hip", ".o"))
+        obj = os.path.join(LIB, obj_name)
         if force or _newer(obj, [path] + headers):
-            _run([HIPCC] + HIP_FLAGS + ["-c", path, "-o", obj])
+            jobs.append([HIPCC] + HIP_FLAGS + extra + ["-c", path, "-o", obj])
         objs.append(obj)
+    # the translation units are independent: compile them side by side (at most 8 at a time)
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        list(pool.map(_run, jobs))
     kernels_so = os.path.join(LIB, "libftk_sampling.so")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", kernels_so] + objs)
 

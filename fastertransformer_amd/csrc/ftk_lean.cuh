@@ -1,0 +1,452 @@
+// Streaming candidate gather of the fused decode step for launches whose largest k is at most 128.
+//
+// Same contract as the stream of ftk_topk.cuh (reference behaviour: topk_stage1 of
+// src/fastertransformer/kernels/sampling_topk_kernels.cu:130-202 after the penalty kernels of
+// src/fastertransformer/kernels/sampling_penalty_kernels.cu): a workgroup walks its share of a row once and
+// leaves, in the workspace, every element at or above a lower bound of the row's k-th largest value. What
+// differs is how the walk is organised, so that the memory system never waits for the arithmetic:
+//   - a thread keeps a ring of R sub-tiles (4 vectors of 16 bytes each) in registers; the loads of all R are
+//     issued before anything else happens, from kernel arguments alone (the per-row arguments arrive while
+//     they are in flight), and a slot is refilled as soon as it has been examined;
+//   - the inner loop is a maximum, a multiply and a compare per vector, without barriers and without looking
+//     at the history bitmap: a vector is parked when its largest element, taken as if no history penalty
+//     applied, reaches a threshold that no penalised or rounded value can get past; parked vectors are
+//     evaluated exactly, by the wave that parked them, when its parking list fills up;
+//   - the bound is the k-th largest of 256 values of distinct elements - first the thread maxima over the
+//     first two sub-tiles, later the largest candidate each lane has evaluated - found by every wave on its
+//     own with 24 rounds of ballots (one workgroup barrier per bound, no sort);
+//   - candidates go straight to the workgroup's list in the workspace.
+// A workgroup that cannot keep its list inside the workspace slot says so in the header; the merging kernel
+// then walks that row again with the general stream.
+#pragma once
+#include <hip/hip_ext.h>
+
+#include "ftk_fused.cuh"
+
+namespace ftk {
+
+constexpr int LG_THREADS  = 256;
+constexpr int LG_WAVES    = LG_THREADS / WAVE;
+constexpr int LG_NV       = 4;                   // 16-byte vectors per thread and sub-tile
+constexpr int LG_SUB_VECS = LG_THREADS * LG_NV;  // a sub-tile: 16 KB
+constexpr int LG_STAGE    = 128;                 // vectors a wave can park between two evaluations
+constexpr int LG_MAX_K    = TK_STAGE;            // the launches that take the general stream start above this
+
+struct LeanShared {
+    uint4    stage_raw[LG_WAVES][LG_STAGE];
+    int      stage_first[LG_WAVES][LG_STAGE];
+    uint32_t slot_key[2][LG_THREADS];
+    int      n_out;
+};
+
+struct LeanPlan {
+    int splits;       // workgroups per row
+    int subs_per_wg;  // sub-tiles each of them streams
+};
+
+// `fill`: workgroups the chip holds at once
+inline LeanPlan lean_plan(int vocab, int rows, int elem_bytes, int fill)
+{
+    const int epv  = 16 / elem_bytes;
+    const int nvec = vocab / epv + 1;
+    const int nsub = (nvec + LG_SUB_VECS - 1) / LG_SUB_VECS;
+    int       s    = (fill + rows - 1) / (rows > 0 ? rows : 1);
+    const int most = nsub / 2 > 1 ? nsub / 2 : 1;  // a workgroup takes its first bound from two sub-tiles
+    s              = s > most ? most : s;
+    s              = s > TK_MAXSPLIT ? TK_MAXSPLIT : s;
+    s              = s < 1 ? 1 : s;
+    LeanPlan p;
+    p.subs_per_wg = (nsub + s - 1) / s;
+    p.splits      = (nsub + p.subs_per_wg - 1) / p.subs_per_wg;
+    return p;
+}
+
+// The largest value P, to within its low eight bits, such that at least k of the 256 keys are >= P
+// (0 when fewer than k keys are non-zero). Every wave calls it on the same keys and gets the same answer.
+__device__ __forceinline__ uint32_t lean_kth_of_slots(const uint32_t* keys, int k)
+{
+    uint32_t kk[LG_WAVES];
+#pragma unroll
+    for (int g = 0; g < LG_WAVES; ++g) {
+        kk[g] = keys[lane_id() + g * WAVE];
+    }
+    uint32_t P = 0u;
+#pragma unroll
+    for (int bit = 31; bit >= 8; --bit) {
+        const uint32_t cand = P | (1u << bit);
+        int            c    = 0;
+#pragma unroll
+        for (int g = 0; g < LG_WAVES; ++g) {
+            c += (int)__builtin_popcountll(__ballot(kk[g] >= cand));
+        }
+        P = c >= k ? cand : P;
+    }
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)P);
+}
+
+// largest element of a 16-byte vector as stored (no transform); NaN elements are ignored
+template<int DT>
+__device__ __forceinline__ float lean_raw_max(const uint4& v)
+{
+    if constexpr (DT == DT_F32) {
+        return __builtin_fmaxf(__builtin_fmaxf(__uint_as_float(v.x), __uint_as_float(v.y)),
+                               __builtin_fmaxf(__uint_as_float(v.z), __uint_as_float(v.w)));
+    }
+    else if constexpr (DT == DT_F16) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2         a = __builtin_bit_cast(h2, v.x), b = __builtin_bit_cast(h2, v.y);
+        const h2         c = __builtin_bit_cast(h2, v.z), d = __builtin_bit_cast(h2, v.w);
+        const h2 m = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+        return __builtin_fmaxf((float)m.x, (float)m.y);
+    }
+    else {
+        auto pair_max = [](uint32_t w) -> float {
+            return __builtin_fmaxf(__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u));
+        };
+        return __builtin_fmaxf(__builtin_fmaxf(pair_max(v.x), pair_max(v.y)),
+                               __builtin_fmaxf(pair_max(v.z), pair_max(v.w)));
+    }
+}
+
+// A value that an unrounded product must reach before its rounding to T can reach `x`.
+template<int DT>
+__device__ __forceinline__ float lean_below_rounding(float x)
+{
+    if constexpr (DT == DT_F32) {
+        return x;
+    }
+    else {
+        const float rel  = DT == DT_F16 ? 0.0009765625f : 0.0078125f;             // one unit in the last place of T
+        const float tiny = DT == DT_F16 ? 5.9604644775390625e-08f : 1.0e-38f;  // ... of T's subnormals
+        return x - __builtin_fmaxf(__builtin_fabsf(x) * rel, tiny);
+    }
+}
+
+// a 16-byte load that is read once: it does not displace what the caches hold for others
+__device__ __forceinline__ uint4 lean_stream_load(const uint4* p)
+{
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const u4             v = __builtin_nontemporal_load(reinterpret_cast<const u4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+constexpr int LG_HIST_U = 8;  // history ids a thread requests before the logits (2048 positions per workgroup)
+
+template<int DT, int BMW, int OCC, int R>
+__global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParams p, FusedLaunch l)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         EPV = (int)(16 / sizeof(T));
+    static_assert(R >= 2, "the first bound reads two sub-tiles");
+    __shared__ LeanShared s;
+    const int             t     = threadIdx.x;
+    const int             row   = blockIdx.y;
+    const int             chunk = blockIdx.x;
+    const int             lane  = lane_id();
+    const int             wv    = wave_id();
+
+    // ---- geometry, from kernel arguments alone: the first loads leave before anything is read from memory
+    const T*     rowp     = (const T*)p.logits + (size_t)row * p.Vp;
+    const int    a        = (int)(((uintptr_t)rowp & 15u) / sizeof(T));
+    const uint4* base     = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(rowp) - a * sizeof(T));
+    const int    vfull_lo = (a + EPV - 1) / EPV;  // vectors [vfull_lo, vfull_hi) lie inside columns [0, V)
+    const int    vfull_hi = max(vfull_lo, (a + p.V) / EPV);
+    const int    vb       = min(vfull_hi, vfull_lo + chunk * l.subs_per_wg * LG_SUB_VECS);
+    const int    ve       = min(vfull_hi, vb + l.subs_per_wg * LG_SUB_VECS);
+    const int    nvec     = ve - vb;
+    const int    nsub     = (nvec + LG_SUB_VECS - 1) / LG_SUB_VECS;
+
+    // The token history comes first (it is time-major: every id is a cache line of its own), so that the
+    // bitmap of penalised columns is built while the logits are still on their way.
+    const bool hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
+    int        hist_ids[LG_HIST_U];
+    if (hist) {
+#pragma unroll
+        for (int u = 0; u < LG_HIST_U; ++u) {
+            const int pos = t + u * LG_THREADS;
+            hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
+        }
+    }
+    uint4 raw[R][LG_NV];
+    auto  load = [&](int slot, int q) {
+#pragma unroll
+        for (int j = 0; j < LG_NV; ++j) {
+            const int vi = min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1);  // past the end: a harmless vector
+            raw[slot][j] = lean_stream_load(base + vi);
+        }
+    };
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (r < nsub) {
+            load(r, r);
+        }
+    }
+
+    // ---- per-row arguments
+    if (p.skip_decode != nullptr && p.skip_decode[row]) {
+        return;
+    }
+    if (p.finished_in != nullptr && p.finished_in[row]) {
+        return;
+    }
+    const int         k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    FusedRow<DT, BMW> rowctx(p, row);
+    if (t == 0) {
+        s.n_out = 0;
+    }
+    // columns this workgroup looks at: its vectors, plus the few columns in front of the first whole vector
+    // (first workgroup of the row) and behind the last one (last workgroup)
+    const bool first_wg = chunk == 0;
+    const bool last_wg  = chunk == (int)gridDim.x - 1;
+    const int  lo_col   = first_wg ? 0 : vb * EPV - a;
+    const int  hi_col   = last_wg ? p.V : ve * EPV - a;
+    if (hist) {
+        // the window of the history bitmap that covers [lo_col, hi_col), in LDS
+        uint32_t* window = fused_lds_bitmap<FusedRow<DT, BMW>::LDS_WORDS>();
+        const int origin = lo_col & ~31;
+        const int words  = min(FusedRow<DT, BMW>::LDS_WORDS, (hi_col - origin + 31) / 32 + 1);
+        for (int i = t; i < words; i += LG_THREADS) {
+            window[i] = 0u;
+        }
+        lds_barrier();
+        auto mark = [&](int pos, int id) {
+            if (id >= lo_col && id < hi_col && rowctx.history_position_counts(pos)) {
+                atomicOr(&window[(id - origin) >> 5], 1u << ((id - origin) & 31));
+            }
+        };
+#pragma unroll
+        for (int u = 0; u < LG_HIST_U; ++u) {
+            mark(t + u * LG_THREADS, hist_ids[u]);
+        }
+        for (int pos = t + LG_HIST_U * LG_THREADS; pos < p.step; pos += LG_THREADS) {
+            mark(pos, p.output_ids[(size_t)pos * p.batch_size + row]);
+        }
+        rowctx.bm_mode   = 1;
+        rowctx.bm_origin = origin;
+    }
+    lds_barrier();
+    const bool     bitsv = rowctx.has_vector_bits();
+    const uint32_t KMIN  = min_valid_key<DT>();
+    const float    NEG_INF = -__builtin_inff();
+    const float    mul   = rowctx.fast_mul;
+    // a multiplier that is not positive and finite does not keep the order: every vector is evaluated exactly
+    const bool all_hit = !(mul > 0.0f && mul < __builtin_inff());
+
+    uint32_t thr   = KMIN;   // candidates are the elements with key >= thr
+    bool     valid = false;  // at least k elements of this workgroup's columns have key >= thr
+    float    thr_f = key_to_float(thr);
+    float    thr_hot;
+    auto     set_threshold = [&](uint32_t key) {
+        thr        = key;
+        thr_f      = key_to_float(key);
+        // What the unrounded, unpenalised product of an element must reach for its final value to reach thr_f:
+        // rounding to T can lift a product by half a unit of T, and a history penalty that raises values
+        // (a multiplicative one below 1, a negative additive one) can lift it further.
+        float h = lean_below_rounding<DT>(thr_f);
+        if (bitsv) {
+            const float pen = rowctx.penalty;
+            float       g   = h;
+            bool        raises;
+            if (rowctx.penalty_type == 0) {
+                raises = !(pen >= 0.0f);
+                g      = h + pen;
+            }
+            else {
+                raises = !(pen >= 1.0f);
+                g      = (pen > 0.0f && pen < 1.0f) ? (h > 0.0f ? h * pen : h / pen) : NEG_INF;
+            }
+            if (raises) {
+                g = g - (__builtin_fabsf(g) * 9.5367431640625e-07f + 1.0e-37f);
+                g = lean_below_rounding<DT>(g);
+                h = __builtin_fminf(h, g);
+            }
+        }
+        if (!(h == h) || !(__builtin_fabsf(thr_f) < __builtin_inff())) {
+            h = NEG_INF;
+        }
+        thr_hot = uniform_f(h);
+    };
+    set_threshold(KMIN);
+
+    // ---- first bound: the k-th largest of the thread maxima over the first two sub-tiles. Only vectors whose
+    // elements all take the plain transform count (no history column, not the masked end id), so every
+    // maximum is the final value of an element.
+    if (nsub > 0) {
+        float tmax = NEG_INF;
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb) {
+            if (sb < nsub) {
+#pragma unroll
+                for (int j = 0; j < LG_NV; ++j) {
+                    const int  rel   = sb * LG_SUB_VECS + j * LG_THREADS + t;
+                    const int  first = (vb + rel) * EPV - a;
+                    const bool clean = rel < nvec && rowctx.plain_vector(first, EPV)
+                                       && (!bitsv || rowctx.vector_bits(first, EPV) == 0u);
+                    float vm = NEG_INF;
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) {
+                        vm = __builtin_fmaxf(vm, rowctx.fast(vector_element<DT>(raw[sb][j], e)));
+                    }
+                    tmax = __builtin_fmaxf(tmax, clean ? vm : NEG_INF);
+                }
+            }
+        }
+        s.slot_key[0][t] = order_key(tmax);
+        lds_barrier();
+        const uint32_t P = lean_kth_of_slots(s.slot_key[0], k);
+        if (P >= KMIN) {
+            set_threshold(P);
+            valid = true;
+        }
+    }
+    int par = 1;  // which half of slot_key the next bound uses
+
+    // ---- parking and exact evaluation
+    TopkEntry* out    = l.entries + (size_t)row * l.row_entries + (size_t)chunk * TK_CCAP;
+    int        wcount = 0;  // vectors parked by this wave (wave-uniform)
+    int        rot    = 0;  // spreads the evaluated vectors over the lanes from one evaluation to the next
+    uint32_t   dmax   = 0u; // largest key this lane has put on the list
+    auto       emit   = [&](uint32_t mask, int first, const float* x) {
+        int slot = atomicAdd(&s.n_out, __builtin_popcount(mask));
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+            if ((mask >> e) & 1u) {
+                const uint32_t key = order_key(x[e]);
+                if (slot < TK_CCAP) {
+                    out[slot] = TopkEntry{key, (uint32_t)(first + e)};
+                }
+                dmax = key > dmax ? key : dmax;
+                ++slot;
+            }
+        }
+    };
+    auto drain = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        const int staged = wcount;
+        for (int e0 = 0; e0 < staged; e0 += WAVE) {
+            const int e = e0 + ((lane - rot) & (WAVE - 1));
+            if (e < staged) {
+                const uint4 v     = s.stage_raw[wv][e];
+                const int   first = s.stage_first[wv][e];
+                const uint32_t bits = bitsv ? rowctx.vector_bits(first, EPV) : 0u;
+                float    x[EPV];
+                uint32_t mask = 0u;
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    x[c] = rowctx.fast(vector_element<DT>(v, c));
+                    if ((bits >> c) & 1u) {
+                        x[c] = rowctx.flagged(x[c]);
+                    }
+                    mask |= (x[c] >= thr_f && first + c != rowctx.masked_end_id) ? (1u << c) : 0u;
+                }
+                if (mask != 0u) {
+                    emit(mask, first, x);
+                }
+            }
+        }
+        rot    = (rot + staged) & (WAVE - 1);
+        wcount = 0;
+    };
+    auto park = [&](bool hit, const uint4& v, int first) {
+        const unsigned long long m = __ballot(hit);
+        if (m != 0ull) {
+            if (wcount > LG_STAGE - WAVE) {
+                drain();
+            }
+            if (hit) {
+                const int slot = wcount
+                                 + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                                  __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                s.stage_raw[wv][slot]   = v;
+                s.stage_first[wv][slot] = first;
+            }
+            wcount += (int)__builtin_popcountll(m);
+        }
+    };
+
+    // ---- the stream. The bound is raised again after 4, 8, 16, ... sub-tiles: the k-th largest of the lanes'
+    // largest candidates bounds the k-th largest of everything seen so far.
+    int next_tighten = 4;
+    for (int q0 = 0; q0 < nsub; q0 += R) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int q = q0 + r;
+            if (q < nsub) {
+#pragma unroll
+                for (int j = 0; j < LG_NV; ++j) {
+                    const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
+                    const float m   = lean_raw_max<DT>(raw[r][j]) * mul;
+                    park((all_hit || m >= thr_hot) && rel < nvec, raw[r][j], (vb + rel) * EPV - a);
+                }
+                if (q + R < nsub) {
+                    load(r, q + R);
+                }
+                if (q + 1 == next_tighten && q + 1 < nsub) {
+                    next_tighten *= 2;
+                    drain();
+                    s.slot_key[par][t] = dmax;
+                    lds_barrier();
+                    const uint32_t P = lean_kth_of_slots(s.slot_key[par], k);
+                    par ^= 1;
+                    if (P > thr) {
+                        set_threshold(P);
+                        valid = true;
+                    }
+                }
+            }
+        }
+    }
+    drain();
+
+    // ---- the columns outside whole vectors, one by one
+    auto edge = [&](int v0, int v1) {
+        for (int v = v0 + t; v < v1; v += LG_THREADS) {
+            if (!rowctx.never_selected(v)) {
+                const float xv = topk_value_at<DT>(rowctx, v);
+                if (xv >= thr_f) {
+                    const int slot = atomicAdd(&s.n_out, 1);
+                    if (slot < TK_CCAP) {
+                        out[slot] = TopkEntry{order_key(xv), (uint32_t)v};
+                    }
+                }
+            }
+        }
+    };
+    if (first_wg) {
+        edge(0, min(p.V, vfull_lo * EPV - a));
+    }
+    if (last_wg) {
+        edge(max(vfull_hi * EPV - a, first_wg ? min(p.V, vfull_lo * EPV - a) : 0), p.V);
+    }
+    lds_barrier();
+    if (t == 0) {
+        const int       n = s.n_out;
+        TopkChunkHeader h;
+        h.count     = n > TK_CCAP ? 0u : (uint32_t)n;
+        h.threshold = thr;
+        h.flags     = n > TK_CCAP ? 2u : (valid ? 1u : 0u);
+        h.share     = 0u;
+        l.headers[(size_t)row * l.splits + chunk] = h;
+    }
+}
+
+// Launchers, one translation unit per element type (lean_kernels.hip built with FTK_LEAN_DT = 0, 1, 2).
+// window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large; variant: see lean_occupancy.
+// start / stop: optional events carried by the launch.
+int lean_gather_launch_f32(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
+                           const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
+int lean_gather_launch_f16(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
+                           const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
+int lean_gather_launch_bf16(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
+                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
+
+// workgroups per compute unit a variant of the lean gather is built for
+inline int lean_occupancy(int variant)
+{
+    return variant == 2 ? 8 : 4;
+}
+
+}  // namespace ftk

@@ -77,7 +77,7 @@ struct TopkEntry {
 };
 
 // which variant of the streaming kernels a launch takes (see topk_stream)
-inline int topk_many_level(int max_top_k)
+__host__ __device__ inline int topk_many_level(int max_top_k)
 {
     return max_top_k > TK_CCAP / 4 ? 2 : (max_top_k > TK_STAGE ? 1 : 0);
 }

@@ -14,322 +14,14 @@
 //                           bitmap over the vocabulary (who gets the repetition / presence penalty)
 #include <hip/hip_ext.h>
 
+#include <cstdlib>
 #include <vector>
 
 #include "ftk_sampling.h"
-#include "ftk_topk.cuh"
+#include "ftk_fused.cuh"
+#include "ftk_lean.cuh"
 
 namespace ftk {
-
-struct FusedParams {
-    const void*  logits;
-    const void*  bias;
-    int          V, Vp, batch_size, step, max_input_length;
-    const float* temperatures;
-    const float* penalties;
-    int          penalty_type;
-    const int*   min_lengths;
-    const int*   end_ids;
-    const int*   input_lengths;
-    const int*   output_ids;
-    const int*   sequence_length_in;
-    const int*   top_ks;
-    const float* top_ps;
-    int          max_top_k;
-    const bool*  skip_decode;
-    const bool*  finished_in;
-    uint32_t*    bitmaps;        // [rows][bitmap_words] scratch, or null when no history penalty applies
-    int          bitmap_words;
-    int          bitmaps_ready;  // history_bitmap_kernel filled `bitmaps`
-    int          lds_window;        // 0: none, 1: small LDS bitmap window, 2: large
-};
-
-// History bitmaps: bit v set <=> token v occurs in the row's (non-padding) history, i.e. column v gets
-// the repetition / presence penalty. A streaming workgroup builds the window of the bitmap that covers
-// its own columns in LDS (strided 4-byte reads of the history that overlap the logits loads already in
-// flight). When the window does not fit, or many workgroups per row would each scan a long history,
-// history_bitmap_kernel builds whole-row bitmaps in the workspace first.
-constexpr int FUSED_BITMAP_WORDS_SMALL     = 2048 + 4;  // LDS window of 64 Ki columns: four workgroups per compute unit
-constexpr int FUSED_BITMAP_WORDS_LARGE     = 5120 + 4;  // 160 Ki columns: three
-constexpr int FUSED_BITMAP_WORDS_GLOBAL    = 0;         // no window: bitmaps in global memory
-constexpr int FUSED_SPLIT_BITMAP_MAX_STEP  = 8192;
-
-// the LDS window of the history bitmap (one per workgroup)
-template<int BMW>
-__device__ __forceinline__ uint32_t* fused_lds_bitmap()
-{
-    __shared__ uint32_t words[BMW];
-    return words;
-}
-
-// BMW > 0: the history bitmap is a window of BMW words in LDS, built by prepare().
-// BMW == 0: whole-row bitmaps in global memory (built by history_bitmap_kernel, or by
-//           prepare_whole_row() for the literal replay).
-__device__ __forceinline__ float uniform_f(float x)
-{
-    return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x)));
-}
-
-template<int DT, int BMW>
-struct FusedRow {
-    static constexpr int  LDS_WORDS = BMW > 0 ? BMW : 1;
-    typedef Storage<DT>   S;
-    typedef typename S::T T;
-    const T*              rowp;
-    const T*              bias;
-    int                   V, Vp;
-    bool                  temp_active, keep_pads;
-    float                 inv;
-    float                 fast_mul;  // inv, or 1 when no temperature applies
-    int                   penalty_type;  // 2 = none
-    float                 penalty;
-    float                 up_mul_neg, up_mul_pos, up_add;  // see flagged_upper
-    bool                  up_ok;
-    int                   masked_end_id;  // end id when the min-length mask applies, else -1
-    // history bitmap
-    int             bm_mode;    // 0: no history penalty, otherwise the bitmap is in place
-    int             bm_origin;  // column of bit 0 of word 0
-    uint32_t*       global_bm;  // this row's slice of the scratch bitmaps
-    bool            global_ready;
-    const int*      history;  // output_ids + row, stride batch_size
-    int             batch_size, step, input_length, max_input_length;
-
-    __device__ __forceinline__ FusedRow(const FusedParams& p, int row)
-    {
-        rowp        = (const T*)p.logits + (size_t)row * p.Vp;
-        bias        = (const T*)p.bias;
-        V           = p.V;
-        Vp          = p.Vp;
-        temp_active = p.temperatures != nullptr;
-        const TemperatureCtx<DT> tc(temp_active ? p.temperatures[row] : 1.0f, V, Vp, false);
-        inv           = tc.inv;
-        fast_mul      = temp_active ? tc.inv : 1.0f;
-        keep_pads     = tc.keep_pads;
-        penalty_type  = p.penalties != nullptr ? p.penalty_type : 2;
-        penalty       = p.penalties != nullptr ? p.penalties[row] : 0.0f;
-        if (penalty_type == 0) {  // additive
-            up_mul_neg = 1.0f;
-            up_mul_pos = 1.0f;
-            up_add     = -penalty;
-            up_ok      = true;
-        }
-        else {
-            up_ok      = penalty > 1e-30f && penalty < 1e30f;  // positive, finite, reciprocal not subnormal
-            up_mul_neg = penalty;
-            up_mul_pos = up_ok ? (1.0f / penalty) * 1.00000095367431640625f : 0.0f;
-            up_add     = 0.0f;
-        }
-        global_bm     = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
-        global_ready  = p.bitmaps_ready != 0;
-        bm_mode       = (BMW == 0 && global_bm != nullptr && global_ready) ? 1 : 0;
-        bm_origin     = 0;
-        history       = p.output_ids != nullptr ? p.output_ids + row : nullptr;
-        batch_size    = p.batch_size;
-        step          = p.step;
-        max_input_length = p.max_input_length;
-        input_length  = p.input_lengths != nullptr ? p.input_lengths[row] : p.max_input_length;
-        // values that are the same for every lane of the workgroup but come out of floating-point
-        // arithmetic: move them to scalar registers, they stay live for the whole kernel
-        inv        = uniform_f(inv);
-        fast_mul   = uniform_f(fast_mul);
-        penalty    = uniform_f(penalty);
-        up_mul_neg = uniform_f(up_mul_neg);
-        up_mul_pos = uniform_f(up_mul_pos);
-        up_add     = uniform_f(up_add);
-        masked_end_id = -1;
-        if (p.min_lengths != nullptr
-            && min_length_masks(p.sequence_length_in[row], p.max_input_length, p.min_lengths[row])) {
-            masked_end_id = p.end_ids[row];
-        }
-    }
-    __device__ __forceinline__ const T* data() const
-    {
-        return rowp;
-    }
-    __device__ __forceinline__ bool history_position_counts(int t) const
-    {
-        return !(t >= input_length && t < max_input_length);  // skip the padding of short prompts
-    }
-    // called by every thread of the gather workgroup before it touches columns [lo, hi)
-    __device__ __forceinline__ void prepare(int lo, int hi)
-    {
-        if (BMW == 0 || global_bm == nullptr) {
-            return;
-        }
-        uint32_t* window = fused_lds_bitmap<LDS_WORDS>();
-        const int origin = lo & ~31;
-        const int words  = min(LDS_WORDS, (hi - origin + 31) / 32 + 1);
-        for (int i = threadIdx.x; i < words; i += blockDim.x) {
-            window[i] = 0u;
-        }
-        __syncthreads();
-        // the history is time-major: every id is a cache line of its own, so the reads are issued eight
-        // deep before the first one is used
-        constexpr int U = 8;
-        for (int t0 = threadIdx.x; t0 < step; t0 += U * blockDim.x) {
-            int ids[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int t = t0 + u * blockDim.x;
-                ids[u]      = (t < step && history_position_counts(t)) ? history[(size_t)t * batch_size] : -1;
-            }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (ids[u] >= lo && ids[u] < hi) {
-                    atomicOr(&window[(ids[u] - origin) >> 5], 1u << ((ids[u] - origin) & 31));
-                }
-            }
-        }
-        __syncthreads();
-        bm_mode   = 1;
-        bm_origin = origin;
-    }
-    __device__ __forceinline__ uint32_t bm_word(int w) const
-    {
-        if (BMW > 0) {
-            return fused_lds_bitmap<LDS_WORDS>()[w];
-        }
-        return global_bm[w];
-    }
-    // whole-row bitmap in global scratch, for the literal replay of rows the gather could not bound
-    __device__ __forceinline__ void build_global_bitmap()
-    {
-        if (BMW > 0 || global_bm == nullptr || global_ready) {
-            return;  // (a workgroup with an LDS window owns the whole row: the window already covers it)
-        }
-        const int words = (Vp + 31) / 32 + 1;
-        for (int i = threadIdx.x; i < words; i += blockDim.x) {
-            global_bm[i] = 0u;
-        }
-        __threadfence_block();
-        __syncthreads();
-        for (int t = threadIdx.x; t < step; t += blockDim.x) {
-            if (history_position_counts(t)) {
-                const int id = history[(size_t)t * batch_size];
-                if (id >= 0 && id < Vp) {
-                    atomicOr(&global_bm[id >> 5], 1u << (id & 31));
-                }
-            }
-        }
-        __threadfence_block();
-        __syncthreads();
-        bm_mode      = 1;
-        bm_origin    = 0;
-        global_ready = true;
-    }
-    // history-membership bits of columns first .. first+n-1 (n <= 8)
-    __device__ __forceinline__ uint32_t vector_bits(int first, int n) const
-    {
-        if (bm_mode == 0) {
-            return 0u;
-        }
-        uint32_t bits = 0u;
-        if (first >= bm_origin) {
-            const int rel = first - bm_origin;
-            const int w   = rel >> 5;
-            const int sh  = rel & 31;
-            bits          = bm_word(w) >> sh;
-            if (sh + n > 32) {
-                bits |= bm_word(w + 1) << (32 - sh);  // both bitmaps carry one word of slack
-            }
-            bits &= (1u << n) - 1u;
-        }
-        else {
-            for (int j = 0; j < n; ++j) {
-                const int v = first + j;
-                if (v >= bm_origin && v < Vp) {
-                    bits |= ((bm_word((v - bm_origin) >> 5) >> ((v - bm_origin) & 31)) & 1u) << j;
-                }
-            }
-        }
-        return bits;
-    }
-    __device__ __forceinline__ bool plain_vector(int first, int n) const
-    {
-        return bias == nullptr && first + n <= V && !(masked_end_id >= first && masked_end_id < first + n);
-    }
-    __device__ __forceinline__ bool has_vector_bits() const
-    {
-        return bm_mode != 0;
-    }
-    // pad columns and the masked end id are -MAX_T whatever the logits hold
-    __device__ __forceinline__ bool never_selected(int v) const
-    {
-        return v >= V || v == masked_end_id;
-    }
-    // interior column, no bias, not in the history, not the masked end id
-    __device__ __forceinline__ float fast(float x) const
-    {
-        return round_t<DT>(x * fast_mul);  // fast_mul is 1 without a temperature: exact, and x is a T already
-    }
-    // the same column when it is in the history
-    __device__ __forceinline__ float flagged(float xf) const
-    {
-        return round_t<DT>(repetition_value(xf, penalty, penalty_type));
-    }
-    // Never below flagged(xf), without the division and without branches: for the multiplicative rule
-    // x * RN(1/p) * (1 + 2^-20) >= x / p for x >= 0 and a positive finite p (as real numbers, so also after
-    // the monotone roundings); x < 0 and the additive rule are the exact operation. Rows whose penalty has
-    // no usable reciprocal report +inf, which sends every flagged column to the exact evaluation.
-    __device__ __forceinline__ float flagged_upper(float xf) const
-    {
-        const float y = round_t<DT>(xf * (xf < 0.0f ? up_mul_neg : up_mul_pos) + up_add);
-        return up_ok ? y : __builtin_inff();
-    }
-    // flags of the NVT vectors a thread owns in one tile (first column first0, `stride` columns apart),
-    // EPV bits each; requires (first0 - bm_origin) to be a multiple of EPV
-    template<int EPV, int NVT>
-    __device__ __forceinline__ void tile_bits(int first0, int stride, uint32_t* packed) const
-    {
-        constexpr int PW = NVT * EPV / 32;
-#pragma unroll
-        for (int i = 0; i < PW; ++i) {
-            packed[i] = 0u;
-        }
-#pragma unroll
-        for (int it = 0; it < NVT; ++it) {
-            const int      rel = first0 + it * stride - bm_origin;
-            const uint32_t b   = (bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
-            packed[(it * EPV) >> 5] |= b << ((it * EPV) & 31);
-        }
-    }
-    // the value top-k would see for column v: temperature(+bias) -> history penalty -> min-length mask
-    // -> pad mask, each rounded to T where the reference stores T
-    __device__ __forceinline__ float slow(int v, float x, uint32_t in_history) const
-    {
-        if (temp_active) {
-            if (v < V) {
-                if (bias != nullptr) {
-                    x = round_t<DT>(x + S::ld(bias[v]));
-                }
-                x = round_t<DT>(x * inv);
-            }
-            else if (!keep_pads) {
-                x = -S::max_t();
-            }
-        }
-        if (in_history) {
-            x = round_t<DT>(repetition_value(x, penalty, penalty_type));
-        }
-        if (v == masked_end_id) {
-            x = -S::max_t();
-        }
-        if (v >= V) {
-            x = -S::max_t();  // addBiasEndMask: pad columns
-        }
-        return x;
-    }
-    __device__ __forceinline__ uint32_t key_at(int v) const
-    {
-        const uint32_t bit = bm_mode != 0 ? (bm_word((v - bm_origin) >> 5) >> ((v - bm_origin) & 31)) & 1u : 0u;
-        return order_key(slow(v, S::ld(rowp[v]), bit));
-    }
-    // before key_at() may be used over the whole row
-    __device__ __forceinline__ void prepare_whole_row()
-    {
-        build_global_bitmap();
-    }
-};
 
 // Row -> bitmap of the token ids in its history window (skipping prompt padding), built in LDS and
 // written out coalesced. Ids outside [0, Vp) are ignored.
@@ -369,28 +61,6 @@ history_bitmap_kernel(uint32_t* __restrict__ bitmaps, int bitmap_words, const in
         }
         __syncthreads();
     }
-}
-
-struct FusedLaunch {
-    int*             ids;
-    int*             sequence_length;
-    bool*            finished;
-    RngState*        rng;
-    const float*     uniforms;
-    int              splits;
-    int              tiles_per_wg;
-    size_t           row_entries;
-    TopkChunkHeader* headers;
-    TopkEntry*       entries;
-};
-
-__device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch& l, int row)
-{
-    if (threadIdx.x == 0) {
-        s.misc[0] = __float_as_int(row_uniform(l.rng, l.uniforms, row));
-    }
-    __syncthreads();
-    return __int_as_float(s.misc[0]);
 }
 
 template<int DT, int BMW, int MANY = 0>
@@ -472,7 +142,14 @@ __global__ void __launch_bounds__(TK_THREADS) fused_select_kernel(FusedParams p,
     const float  u  = fused_row_draw(s, l, row);
     const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row, p.end_ids);
     uint32_t     thr         = 0u;
-    const int    n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr, pf);
+    int          n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr, pf);
+    if (n < 0 && topk_many_level(p.max_top_k) == 0) {
+        // A workgroup of the gather could not hold its candidates. Walk the whole row again, here, with the
+        // stream that recovers from overfull tiles; only rows it cannot bound either take the literal replay.
+        r.prepare_whole_row();
+        __syncthreads();
+        n = topk_stream<DT, FusedRow<DT, BMW>, 0>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
+    }
     topk_select_lds<DT, FusedRow<DT, BMW>, true>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
 }
 
@@ -572,6 +249,17 @@ extern "C" int ftk_profile_read(int kernel, double* total_ms, int* launches)
     return 0;
 }
 
+// Which build of the lean gather a launch takes: 0 switches it off (every launch takes the general stream),
+// 1 = four workgroups per compute unit with four sub-tiles in flight per thread, 2 = eight with two.
+// Read once from FTK_LEAN.
+static int lean_variant()
+{
+    static const int v = []() {
+        const char* e = std::getenv("FTK_LEAN");
+        return e != nullptr ? std::atoi(e) : 1;
+    }();
+    return v;
+}
 extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
 {
     if (a == nullptr) {
@@ -589,7 +277,12 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const int      many         = topk_many_level(a->max_top_k);  // > 0: the large-k kernels (whole-row bitmaps only)
     const int      bitmap_words = (a->vocab_size_padded + 31) / 32 + 1;  // +1: vector_bits may peek one word ahead
     const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
-    const size_t   need         = bitmap_bytes + plan.bytes;
+    // Launches with a small k and no bias take the lean gather, which cuts a row differently.
+    const int      lean_mode = many == 0 && a->embedding_bias == nullptr ? lean_variant() : 0;
+    const LeanPlan lplan     = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * lean_occupancy(lean_mode));
+    const size_t   lean_bytes =
+        (size_t)(rows > 0 ? rows : 0) * lplan.splits * (sizeof(TopkChunkHeader) + (size_t)TK_CCAP * sizeof(TopkEntry));
+    const size_t   need = bitmap_bytes + (lean_mode != 0 && lean_bytes > plan.bytes ? lean_bytes : plan.bytes);
     if (a->workspace == nullptr) {
         a->workspace_size = need;
         return 0;
@@ -640,10 +333,12 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         p.bitmaps = (uint32_t*)ws;
         // columns one workgroup streams (upper bound): does its bitmap window fit in LDS?
         const int    epv        = 16 / elem;
-        const size_t range_cols = (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
+        const size_t range_cols = lean_mode != 0 ? (size_t)lplan.subs_per_wg * LG_SUB_VECS * epv + 2 * epv :
+                                                   (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
         const size_t words      = range_cols / 32 + 4;
         const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && many == 0
-                           && (plan.splits == 1 || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
+                           && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1
+                               || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
         if (local) {
             p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
         }
@@ -668,8 +363,44 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     l.splits          = plan.splits;
     l.tiles_per_wg    = plan.tiles_per_wg;
     l.row_entries     = plan.row_entries;
+    l.subs_per_wg     = 0;
     l.headers         = (TopkChunkHeader*)(ws + bitmap_bytes);
     l.entries         = (TopkEntry*)(l.headers + (size_t)rows * plan.splits);
+    if (lean_mode != 0) {
+        l.splits       = lplan.splits;
+        l.subs_per_wg  = lplan.subs_per_wg;
+        l.row_entries  = (size_t)lplan.splits * TK_CCAP;
+        l.entries      = (TopkEntry*)(l.headers + (size_t)rows * lplan.splits);
+        const dim3 lgrid(lplan.splits, rows);
+        const int  window = p.bitmaps_ready ? 0 : (p.lds_window == 2 ? 2 : 1);
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        {
+            KernelTimer& tm = g_timers[1];
+            if (g_profile && tm.used < (int)tm.start.size()) {
+                e0 = tm.start[tm.used];
+                e1 = tm.stop[tm.used];
+                tm.used++;
+            }
+        }
+        int rc;
+        if (a->dtype == FTK_DTYPE_F32) {
+            rc = lean_gather_launch_f32(window, lean_mode, lgrid, st, p, l, e0, e1);
+        }
+        else if (a->dtype == FTK_DTYPE_F16) {
+            rc = lean_gather_launch_f16(window, lean_mode, lgrid, st, p, l, e0, e1);
+        }
+        else {
+            rc = lean_gather_launch_bf16(window, lean_mode, lgrid, st, p, l, e0, e1);
+        }
+        if (rc != 0) {
+            return rc;
+        }
+        FTK_LAUNCH_CHECK();
+        FTK_DISPATCH_DTYPE(a->dtype,
+                           launch_timed(2, fused_select_kernel<DT>, dim3(rows), dim3(TK_THREADS), st, p, l));
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
     if (plan.splits == 1) {
         const dim3 grid1(rows), block(TK_THREADS);
         if (many == 2) {

@@ -1,0 +1,54 @@
+// Instances of the lean gather (ftk_lean.cuh) for one element type: this file is compiled once per type with
+// -DFTK_LEAN_DT=0 (f32), 1 (f16), 2 (bf16), so that the three sets of kernels build side by side.
+#include "ftk_lean.cuh"
+
+#ifndef FTK_LEAN_DT
+#error "build with -DFTK_LEAN_DT=0|1|2"
+#endif
+
+namespace ftk {
+
+template<int BMW, int OCC, int R>
+static int lean_launch_one(dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+                           hipEvent_t stop)
+{
+    if (start != nullptr) {
+        hipExtLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R>), grid, dim3(LG_THREADS), 0, st, start,
+                              stop, 0, p, l);
+    }
+    else {
+        hipLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R>), grid, dim3(LG_THREADS), 0, st, p, l);
+    }
+    return (int)hipGetLastError();
+}
+
+template<int OCC, int R>
+static int lean_launch_window(int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                              hipEvent_t start, hipEvent_t stop)
+{
+    if (window == 0) {
+        return lean_launch_one<FUSED_BITMAP_WORDS_GLOBAL, OCC, R>(grid, st, p, l, start, stop);
+    }
+    if (window == 2) {
+        return lean_launch_one<FUSED_BITMAP_WORDS_LARGE, OCC, R>(grid, st, p, l, start, stop);
+    }
+    return lean_launch_one<FUSED_BITMAP_WORDS_SMALL, OCC, R>(grid, st, p, l, start, stop);
+}
+
+#if FTK_LEAN_DT == 0
+int lean_gather_launch_f32
+#elif FTK_LEAN_DT == 1
+int lean_gather_launch_f16
+#else
+int lean_gather_launch_bf16
+#endif
+    (int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+     hipEvent_t stop)
+{
+    if (variant == 2) {
+        return lean_launch_window<8, 2>(window, grid, st, p, l, start, stop);
+    }
+    return lean_launch_window<4, 4>(window, grid, st, p, l, start, stop);
+}
+
+}  // namespace ftk
