@@ -15,6 +15,7 @@
 #include <hip/hip_ext.h>
 
 #include <cstdlib>
+#include <mutex>
 #include <vector>
 
 #include "ftk_sampling.h"
@@ -457,4 +458,62 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     }
     FTK_LAUNCH_CHECK();
     return 0;
+}
+
+// ---- the fused step for callers that cannot allocate ------------------------------------------------
+// Same step, with the workspace taken from a fixed array in device memory instead of the caller. Every GPU
+// the library runs on holds its own copy of the array from the moment the code object is loaded until the
+// process ends; its address on a device is looked up once, with that device current.
+static __device__ __align__(256) unsigned char scratch[FTK_FUSED_STATIC_WORKSPACE_BYTES];
+
+namespace {
+constexpr int FTK_MAX_DEVICES = 64;
+std::mutex    g_scratch_mutex;
+void*         g_scratch_ptr[FTK_MAX_DEVICES] = {};
+}  // namespace
+
+extern "C" int ftk_fused_topk_step_static(ftk_fused_topk_args* a, ftk_stream_t stream)
+{
+    if (a == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    int        device = -1;
+    hipError_t e      = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        return (int)e;
+    }
+    if (device < 0 || device >= FTK_MAX_DEVICES) {
+        return FTK_ERR_ARGUMENT;
+    }
+    void* ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_ptr[device] == nullptr) {
+            void* found = nullptr;
+            e           = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) {
+                return (int)e;
+            }
+            g_scratch_ptr[device] = found;
+        }
+        ptr = g_scratch_ptr[device];
+    }
+    // size the step exactly as the caller-workspace entry point would, and refuse what the array cannot hold
+    ftk_fused_topk_args q = *a;
+    q.workspace           = nullptr;
+    q.workspace_size      = 0;
+    const int rc          = ftk_fused_topk_step(&q, stream);
+    if (rc != 0) {
+        return rc;
+    }
+    a->workspace_size = q.workspace_size;  // reported back, so that the caller sees what was needed
+    if (q.workspace_size > (size_t)FTK_FUSED_STATIC_WORKSPACE_BYTES) {
+        return FTK_ERR_STATIC_WORKSPACE;
+    }
+    // Nothing in the workspace has to start at zero: list headers are written by every streaming workgroup
+    // before the merging kernel reads them, lists are read up to the count in their header, and the history
+    // bitmaps are cleared by the kernel that fills them.
+    q.workspace      = ptr;
+    q.workspace_size = (size_t)FTK_FUSED_STATIC_WORKSPACE_BYTES;
+    return ftk_fused_topk_step(&q, stream);
 }

@@ -48,6 +48,7 @@ _SIGNATURES = {
     "ftk_invoke_stop_words_criterion_rows": [_vp, _vp, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _vp],
     "ftk_invoke_length_criterion": [_vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_fused_topk_step": [_vp, _vp],
+    "ftk_fused_topk_step_static": [_vp, _vp],
     "ftk_invoke_log_prob_from_logits": [_i, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _b],
     "ftk_invoke_decoding_initialize": [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_invoke_plus_scalar": [_vp, _i, _i, _vp],
@@ -67,7 +68,8 @@ _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_c
 
 
 # error codes of include/ftk_sampling.h (positive values are hipError_t)
-FTK_ERR_DTYPE, FTK_ERR_TOPK_DOMAIN, FTK_ERR_ARGUMENT, FTK_ERR_WORKSPACE = -1, -2, -3, -4
+FTK_ERR_DTYPE, FTK_ERR_TOPK_DOMAIN, FTK_ERR_ARGUMENT, FTK_ERR_WORKSPACE, FTK_ERR_STATIC_WORKSPACE = -1, -2, -3, -4, -5
+FUSED_STATIC_WORKSPACE_BYTES = 32 << 20
 
 
 def exported_symbols():

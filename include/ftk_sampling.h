@@ -36,7 +36,8 @@ enum {
     FTK_ERR_DTYPE       = -1, /* unknown dtype */
     FTK_ERR_TOPK_DOMAIN = -2, /* top-k outside [1, 1024]: std::domain_error in sampling_topk_kernels.cu:393-394 */
     FTK_ERR_ARGUMENT    = -3, /* null / inconsistent argument */
-    FTK_ERR_WORKSPACE   = -4  /* workspace smaller than the queried size */
+    FTK_ERR_WORKSPACE   = -4, /* workspace smaller than the queried size */
+    FTK_ERR_STATIC_WORKSPACE = -5 /* ftk_fused_topk_step_static: the step needs more than the library's fixed array */
 };
 
 /* Per-row generator state; replaces curandState_t (48 bytes) in every signature. Row b draws
@@ -209,6 +210,18 @@ typedef struct ftk_fused_topk_args {
 
 /* workspace == NULL in args: writes the required size into args->workspace_size, launches nothing. */
 int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
+
+/* The fused step for callers that cannot allocate device memory (code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arguments and results as
+ * ftk_fused_topk_step, except that args->workspace is ignored: the workspace is a fixed array of
+ * FTK_FUSED_STATIC_WORKSPACE_BYTES inside the library's device code, one copy per GPU, held until the process
+ * ends. The call allocates and frees nothing. On return args->workspace_size holds the size the step needed;
+ * a step that needs more than the array returns FTK_ERR_STATIC_WORKSPACE and launches nothing (the headline
+ * step, 256 rows x 128256 fp32 with a history penalty, needs about 21 MB). All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (different streams or threads) race; calls on one stream
+ * are safe back to back. */
+#define FTK_FUSED_STATIC_WORKSPACE_BYTES (32u << 20)
+int ftk_fused_topk_step_static(ftk_fused_topk_args* args, ftk_stream_t stream);
 
 /* ---- the steps either side of the sampling path -------------------------------------------- */
 /* kernels/logprob_kernels.cu:137-183 invokeLogProbFromLogits<T>: cum_log_probs[b] = sum over step < lengths[b]-1 of
