@@ -24,6 +24,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # (source, object, extra flags): lean_kernels.hip is built once per element type so the three sets of kernels
 # compile side by side
 KERNEL_UNITS = [
+    ("fused_dtype_kernels.hip", "fused_kernels_f16.o", ["-DFTK_FUSED_DT=1"]),
+    ("fused_dtype_kernels.hip", "fused_kernels_bf16.o", ["-DFTK_FUSED_DT=2"]),
+    ("fused_dtype_kernels.hip", "fused_kernels_f32.o", ["-DFTK_FUSED_DT=0"]),
     ("fused_kernels.hip", "fused_kernels.o", []),
     ("topp_kernels.hip", "topp_kernels.o", []),
     ("topk_kernels.hip", "topk_kernels.o", []),
@@ -57,15 +60,28 @@ def _newer(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+def _includes(path, seen=None):
+    """the files a source includes with #include "..." (searched in csrc/ and include/), transitively"""
+    seen = set() if seen is None else seen
+    for line in open(path):
+        line = line.strip()
+        if line.startswith('#include "'):
+            name = line.split('"')[1]
+            for d in (CSRC, INCLUDE):
+                dep = os.path.join(d, name)
+                if os.path.exists(dep) and dep not in seen:
+                    seen.add(dep)
+                    _includes(dep, seen)
+    return seen
+
+
 def build(force=True, verbose=True, with_torch=True):
     os.makedirs(LIB, exist_ok=True)
-    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".h", ".cuh"))]
-    headers.append(os.path.join(INCLUDE, "ftk_sampling.h"))
     objs, jobs = [], []
     for src, obj_name, extra in KERNEL_UNITS:
         path = os.path.join(CSRC, src)
         obj = os.path.join(LIB, obj_name)
-        if force or _newer(obj, [path] + headers):
+        if force or _newer(obj, [path] + sorted(_includes(path))):
             jobs.append([HIPCC] + HIP_FLAGS + extra + ["-c", path, "-o", obj])
         objs.append(obj)
     # the translation units are independent: compile them side by side (at most 8 at a time)

@@ -50,6 +50,36 @@ __device__ __forceinline__ uint32_t* fused_lds_bitmap()
 // BMW > 0: the history bitmap is a window of BMW words in LDS, built by prepare().
 // BMW == 0: whole-row bitmaps in global memory (built by history_bitmap_kernel, or by
 //           prepare_whole_row() for the literal replay).
+// One flag of a bool array at an index that is the same for the whole workgroup, read through the aligned
+// 32-bit word that holds it: a scalar load, which does not queue behind the vector loads in flight (a byte
+// load would, and its consumer would wait for all of them).
+__device__ __forceinline__ bool uniform_flag(const bool* flags, int index)
+{
+    const bool*    flag = flags + index;
+    const uint32_t mis  = (uint32_t)(reinterpret_cast<uintptr_t>(flag) & 3u);
+    const uint32_t word = *reinterpret_cast<const uint32_t*>(flag - mis);  // stays inside the flag's own word
+    return ((word >> (8u * mis)) & 0xFFu) != 0u;
+}
+
+// Per-row arguments are optional arrays. Reading them behind their null checks makes a chain of loads that
+// each wait for the one before; these helpers always load - from the array when it exists, from `safe` (any
+// valid 4-byte aligned address, the row's end id) when it does not - so that all of a row's arguments are
+// requested together and cost one trip to memory.
+template<typename V>
+__device__ __forceinline__ V row_arg_or(const V* array, int row, const void* safe, V otherwise)
+{
+    static_assert(sizeof(V) == 4, "32-bit arguments");
+    const V* from = array != nullptr ? array + row : reinterpret_cast<const V*>(safe);
+    const V  v    = *from;
+    return array != nullptr ? v : otherwise;
+}
+__device__ __forceinline__ bool row_flag_or(const bool* flags, int row, const void* safe, bool otherwise)
+{
+    const bool* from = flags != nullptr ? flags + row : reinterpret_cast<const bool*>(safe);
+    const bool  v    = uniform_flag(from, 0);
+    return flags != nullptr ? v : otherwise;
+}
+
 __device__ __forceinline__ float uniform_f(float x)
 {
     return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x)));
@@ -86,12 +116,13 @@ struct FusedRow {
         V           = p.V;
         Vp          = p.Vp;
         temp_active = p.temperatures != nullptr;
-        const TemperatureCtx<DT> tc(temp_active ? p.temperatures[row] : 1.0f, V, Vp, false);
+        const void*              safe = p.end_ids + row;
+        const TemperatureCtx<DT> tc(row_arg_or(p.temperatures, row, safe, 1.0f), V, Vp, false);
         inv           = tc.inv;
         fast_mul      = temp_active ? tc.inv : 1.0f;
         keep_pads     = tc.keep_pads;
         penalty_type  = p.penalties != nullptr ? p.penalty_type : 2;
-        penalty       = p.penalties != nullptr ? p.penalties[row] : 0.0f;
+        penalty       = row_arg_or(p.penalties, row, safe, 0.0f);
         if (penalty_type == 0) {  // additive
             up_mul_neg = 1.0f;
             up_mul_pos = 1.0f;
@@ -112,7 +143,7 @@ struct FusedRow {
         batch_size    = p.batch_size;
         step          = p.step;
         max_input_length = p.max_input_length;
-        input_length  = p.input_lengths != nullptr ? p.input_lengths[row] : p.max_input_length;
+        input_length  = row_arg_or(p.input_lengths, row, safe, p.max_input_length);
         // values that are the same for every lane of the workgroup but come out of floating-point
         // arithmetic: move them to scalar registers, they stay live for the whole kernel
         inv        = uniform_f(inv);
@@ -121,11 +152,11 @@ struct FusedRow {
         up_mul_neg = uniform_f(up_mul_neg);
         up_mul_pos = uniform_f(up_mul_pos);
         up_add     = uniform_f(up_add);
-        masked_end_id = -1;
-        if (p.min_lengths != nullptr
-            && min_length_masks(p.sequence_length_in[row], p.max_input_length, p.min_lengths[row])) {
-            masked_end_id = p.end_ids[row];
-        }
+        const int min_length = row_arg_or(p.min_lengths, row, safe, 0);
+        const int seq_length = row_arg_or(p.min_lengths != nullptr ? p.sequence_length_in : nullptr, row, safe, 0);
+        const int end_id     = p.end_ids[row];
+        masked_end_id =
+            (p.min_lengths != nullptr && min_length_masks(seq_length, p.max_input_length, min_length)) ? end_id : -1;
     }
     __device__ __forceinline__ const T* data() const
     {
@@ -338,5 +369,16 @@ __device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch
     __syncthreads();
     return __int_as_float(s.misc[0]);
 }
+
+// Launchers of the general-stream kernels, one translation unit per element type (fused_dtype_kernels.hip).
+// kind: which kernel; window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large;
+// many: the large-k level of the launch (topk_many_level); start / stop: optional events carried by the launch.
+enum { FUSED_KIND_ROW = 0, FUSED_KIND_GATHER = 1, FUSED_KIND_SELECT = 2 };
+int fused_launch_f32(int kind, int window, int many, dim3 grid, hipStream_t st, const FusedParams& p,
+                     const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
+int fused_launch_f16(int kind, int window, int many, dim3 grid, hipStream_t st, const FusedParams& p,
+                     const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
+int fused_launch_bf16(int kind, int window, int many, dim3 grid, hipStream_t st, const FusedParams& p,
+                      const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 
 }  // namespace ftk

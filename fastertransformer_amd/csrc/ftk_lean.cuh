@@ -29,7 +29,8 @@ constexpr int LG_THREADS  = 256;
 constexpr int LG_WAVES    = LG_THREADS / WAVE;
 constexpr int LG_NV       = 4;                   // 16-byte vectors per thread and sub-tile
 constexpr int LG_SUB_VECS = LG_THREADS * LG_NV;  // a sub-tile: 16 KB
-constexpr int LG_STAGE    = 128;                 // vectors a wave can park between two evaluations
+constexpr int LG_DRAIN_AT = 64;                  // parked vectors at which a wave evaluates them (checked once per sub-tile)
+constexpr int LG_STAGE    = LG_DRAIN_AT + LG_NV * WAVE;  // vectors a wave can park between two evaluations
 constexpr int LG_MAX_K    = TK_STAGE;            // the launches that take the general stream start above this
 
 struct LeanShared {
@@ -132,7 +133,7 @@ __device__ __forceinline__ uint4 lean_stream_load(const uint4* p)
 
 constexpr int LG_HIST_U = 8;  // history ids a thread requests before the logits (2048 positions per workgroup)
 
-template<int DT, int BMW, int OCC, int R>
+template<int DT, int BMW, int OCC, int R, int EXP = 0>
 __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParams p, FusedLaunch l)
 {
     typedef Storage<DT>   S;
@@ -159,7 +160,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 
     // The token history comes first (it is time-major: every id is a cache line of its own), so that the
     // bitmap of penalised columns is built while the logits are still on their way.
-    const bool hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
+    const bool hist = !(EXP & 1) && BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
     int        hist_ids[LG_HIST_U];
     if (hist) {
 #pragma unroll
@@ -184,14 +185,14 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     }
 
     // ---- per-row arguments
-    if (p.skip_decode != nullptr && p.skip_decode[row]) {
-        return;
-    }
-    if (p.finished_in != nullptr && p.finished_in[row]) {
-        return;
-    }
-    const int         k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
+    // (all requested together; a row that does not take part leaves once they are here)
+    const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
+    const bool        fin  = row_flag_or(p.finished_in, row, p.end_ids + row, false);
+    const int         k    = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
     FusedRow<DT, BMW> rowctx(p, row);
+    if (skip || fin) {
+        return;
+    }
     if (t == 0) {
         s.n_out = 0;
     }
@@ -227,6 +228,8 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     }
     lds_barrier();
     const bool     bitsv = rowctx.has_vector_bits();
+    // Rows that start on a 16-byte boundary: the flags of a vector never straddle a word of the bitmap.
+    const bool     aligned_bits = bitsv && a == 0 && BMW > 0;
     const uint32_t KMIN  = min_valid_key<DT>();
     const float    NEG_INF = -__builtin_inff();
     const float    mul   = rowctx.fast_mul;
@@ -272,7 +275,11 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     // ---- first bound: the k-th largest of the thread maxima over the first two sub-tiles. Only vectors whose
     // elements all take the plain transform count (no history column, not the masked end id), so every
     // maximum is the final value of an element.
-    if (nsub > 0) {
+    if (EXP & 2) {
+        set_threshold(order_key((EXP & 32) ? 10.0f : 7.4f));
+        valid = true;
+    }
+    else if (nsub > 0) {
         float tmax = NEG_INF;
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
@@ -281,8 +288,15 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 for (int j = 0; j < LG_NV; ++j) {
                     const int  rel   = sb * LG_SUB_VECS + j * LG_THREADS + t;
                     const int  first = (vb + rel) * EPV - a;
-                    const bool clean = rel < nvec && rowctx.plain_vector(first, EPV)
-                                       && (!bitsv || rowctx.vector_bits(first, EPV) == 0u);
+                    uint32_t   bits  = 0u;
+                    if (aligned_bits) {
+                        const int brel = max(first - rowctx.bm_origin, 0);
+                        bits           = (rowctx.bm_word(brel >> 5) >> (brel & 31)) & ((1u << EPV) - 1u);
+                    }
+                    else if (bitsv) {
+                        bits = rowctx.vector_bits(first, EPV);
+                    }
+                    const bool clean = rel < nvec && rowctx.plain_vector(first, EPV) && bits == 0u;
                     float vm = NEG_INF;
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) {
@@ -304,58 +318,90 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 
     // ---- parking and exact evaluation
     TopkEntry* out    = l.entries + (size_t)row * l.row_entries + (size_t)chunk * TK_CCAP;
-    int        wcount = 0;  // vectors parked by this wave (wave-uniform)
-    int        rot    = 0;  // spreads the evaluated vectors over the lanes from one evaluation to the next
-    uint32_t   dmax   = 0u; // largest key this lane has put on the list
-    auto       emit   = [&](uint32_t mask, int first, const float* x) {
-        int slot = atomicAdd(&s.n_out, __builtin_popcount(mask));
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-            if ((mask >> e) & 1u) {
-                const uint32_t key = order_key(x[e]);
-                if (slot < TK_CCAP) {
-                    out[slot] = TopkEntry{key, (uint32_t)(first + e)};
-                }
-                dmax = key > dmax ? key : dmax;
-                ++slot;
-            }
-        }
-    };
+    int        wcount = 0;   // vectors parked by this wave (wave-uniform)
+    int        rot    = 0;   // spreads the evaluated vectors over the lanes from one evaluation to the next
+    uint32_t   dmax   = 0u;  // largest key this lane has put on the list
+    // Evaluate what the wave has parked: one vector per lane and round. The elements that reach the bound get
+    // their slots on the workgroup's list with one LDS atomic per round (prefix sums of the per-lane counts,
+    // which are at most EPV, from one ballot per bit of the count).
     auto drain = [&]() {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-        const int staged = wcount;
+        const int staged = (EXP & 16) ? 0 : wcount;
         for (int e0 = 0; e0 < staged; e0 += WAVE) {
-            const int e = e0 + ((lane - rot) & (WAVE - 1));
-            if (e < staged) {
-                const uint4 v     = s.stage_raw[wv][e];
-                const int   first = s.stage_first[wv][e];
-                const uint32_t bits = bitsv ? rowctx.vector_bits(first, EPV) : 0u;
-                float    x[EPV];
-                uint32_t mask = 0u;
+            const int  e    = e0 + ((lane - rot) & (WAVE - 1));
+            const bool have = e < staged;
+            float      x[EPV];
+            uint32_t   mask  = 0u;
+            int        first = 0;
+            if (have) {
+                const uint4 v = s.stage_raw[wv][e];
+                first         = s.stage_first[wv][e];
+                uint32_t bits = 0u;
+                if (aligned_bits) {
+                    const int rel = first - rowctx.bm_origin;
+                    bits          = (rowctx.bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
+                }
+                else if (bitsv) {
+                    bits = rowctx.vector_bits(first, EPV);
+                }
 #pragma unroll
                 for (int c = 0; c < EPV; ++c) {
                     x[c] = rowctx.fast(vector_element<DT>(v, c));
-                    if ((bits >> c) & 1u) {
-                        x[c] = rowctx.flagged(x[c]);
-                    }
-                    mask |= (x[c] >= thr_f && first + c != rowctx.masked_end_id) ? (1u << c) : 0u;
                 }
-                if (mask != 0u) {
-                    emit(mask, first, x);
+                if (bits != 0u) {  // rare: a column of the history
+#pragma unroll
+                    for (int c = 0; c < EPV; ++c) {
+                        if ((bits >> c) & 1u) {
+                            x[c] = rowctx.flagged(x[c]);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    mask |= x[c] >= thr_f ? (1u << c) : 0u;
+                }
+                const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - first);  // the masked end id is no candidate
+                mask &= rel_end < (uint32_t)EPV ? ~(1u << rel_end) : ~0u;
+            }
+            const int cnt = __builtin_popcount(mask);
+            int       pre = 0, total = 0;
+#pragma unroll
+            for (int bit = 0; (1 << bit) <= EPV; ++bit) {
+                const unsigned long long bm = __ballot((cnt >> bit) & 1);
+                pre += (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bm, 0u))
+                       << bit;
+                total += (int)__builtin_popcountll(bm) << bit;
+            }
+            if (total > 0) {
+                int base_slot = 0;
+                if (lane == 0) {
+                    base_slot = atomicAdd(&s.n_out, total);
+                }
+                int slot = __builtin_amdgcn_readfirstlane(base_slot) + pre;
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    if ((mask >> c) & 1u) {
+                        const uint32_t key = order_key(x[c]);
+                        if (slot < TK_CCAP) {
+                            out[slot] = TopkEntry{key, (uint32_t)(first + c)};
+                        }
+                        dmax = key > dmax ? key : dmax;
+                        ++slot;
+                    }
                 }
             }
         }
         rot    = (rot + staged) & (WAVE - 1);
         wcount = 0;
     };
+    // The parking list holds what is left from before a sub-tile (fewer than LG_DRAIN_AT vectors) plus every
+    // vector of a sub-tile: it cannot overflow.
+    static_assert(LG_STAGE >= LG_DRAIN_AT - 1 + LG_NV * WAVE, "a sub-tile always fits the parking list");
     auto park = [&](bool hit, const uint4& v, int first) {
         const unsigned long long m = __ballot(hit);
         if (m != 0ull) {
-            if (wcount > LG_STAGE - WAVE) {
-                drain();
-            }
             if (hit) {
                 const int slot = wcount
                                  + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
@@ -384,9 +430,12 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 if (q + R < nsub) {
                     load(r, q + R);
                 }
-                if (q + 1 == next_tighten && q + 1 < nsub) {
-                    next_tighten *= 2;
+                const bool tighten = !(EXP & 8) && q + 1 == next_tighten && q + 1 < nsub;
+                if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
                     drain();
+                }
+                if (tighten) {
+                    next_tighten *= 2;
                     s.slot_key[par][t] = dmax;
                     lds_barrier();
                     const uint32_t P = lean_kth_of_slots(s.slot_key[par], k);
@@ -399,7 +448,6 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
             }
         }
     }
-    drain();
 
     // ---- the columns outside whole vectors, one by one
     auto edge = [&](int v0, int v1) {
@@ -433,11 +481,229 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     }
 }
 
+// -------------------------------------------------------------------------------------------
+// merge + select for the lists of the lean gather
+// -------------------------------------------------------------------------------------------
+constexpr int LS_PF_LISTS  = 2;  // lists a wave requests up front (wave w: lists w and w + 4)
+constexpr int LS_PF_ROUNDS = 4;  // 64 entries each: the first 256 entries of a list
+
+struct LeanListPrefetch {
+    TopkEntry e[LS_PF_LISTS][LS_PF_ROUNDS];
+};
+
+// Requested at the top of the kernel, before anything is known about the row: the loads are in flight while
+// the row's arguments and the list headers arrive. Reads stay inside the row's slots of the workspace.
+__device__ __forceinline__ LeanListPrefetch lean_prefetch_lists(int splits, const TopkEntry* entries)
+{
+    LeanListPrefetch pf;
+#pragma unroll
+    for (int m = 0; m < LS_PF_LISTS; ++m) {
+        const int        c = wave_id() + m * TK_WAVES;
+        const TopkEntry* e = entries + (size_t)(c < splits ? c : 0) * TK_CCAP;
+#pragma unroll
+        for (int r = 0; r < LS_PF_ROUNDS; ++r) {
+            pf.e[m][r] = e[r * WAVE + lane_id()];
+        }
+    }
+    return pf;
+}
+
+// The union of a row's lists at or above the row's bound -> s.cand, cut to the k largest keys (and ties).
+// Returns the count, or -1 when a workgroup of the gather gave up on its list.
+// `my_header`: header of list t, loaded by thread t < splits (requested with the prefetch). `draw_bits`: the
+// row's uniform draw, held by thread 0; it is handed to every thread through the barrier that publishes the
+// headers.
+template<int DT>
+__device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits, const TopkChunkHeader& my_header,
+                                                const TopkEntry* entries, uint32_t* thr_out,
+                                                const LeanListPrefetch& pf, int* draw_bits)
+{
+    const int t = threadIdx.x;
+    // headers through LDS: one load per list, every thread then looks at all of them
+    TopkChunkHeader* hdr = reinterpret_cast<TopkChunkHeader*>(&s.stage.raw[0][0]);
+    static_assert(sizeof(s.stage.raw) >= TK_MAXSPLIT * sizeof(TopkChunkHeader), "headers fit the staging area");
+    if (t < splits) {
+        hdr[t] = my_header;
+    }
+    if (t == 0) {
+        s.n_cand  = 0;
+        s.misc[0] = *draw_bits;
+    }
+    __syncthreads();
+    *draw_bits = s.misc[0];
+    uint32_t T0       = min_valid_key<DT>();
+    bool     overflow = false;
+    int      total    = 0;
+    for (int c = 0; c < splits; ++c) {
+        const TopkChunkHeader h = hdr[c];
+        overflow                = overflow || (h.flags & 2u) != 0u;
+        total += (int)h.count;
+        if ((h.flags & 1u) && h.threshold > T0) {
+            T0 = h.threshold;
+        }
+    }
+    if (overflow) {
+        return -1;
+    }
+    FTK_STAMP(1);
+    // what was requested up front: one slot reservation per wave
+    unsigned long long keepm[LS_PF_LISTS][LS_PF_ROUNDS];
+    int                wave_total = 0;
+#pragma unroll
+    for (int m = 0; m < LS_PF_LISTS; ++m) {
+        const int c   = wave_id() + m * TK_WAVES;
+        const int cnt = c < splits ? (int)hdr[c].count : 0;
+#pragma unroll
+        for (int r = 0; r < LS_PF_ROUNDS; ++r) {
+            keepm[m][r] = __ballot(r * WAVE + lane_id() < cnt && pf.e[m][r].key >= T0);
+            wave_total += (int)__builtin_popcountll(keepm[m][r]);
+        }
+    }
+    int wave_base = 0;
+    if (lane_id() == 0 && wave_total > 0) {
+        wave_base = atomicAdd(&s.n_cand, wave_total);
+    }
+    wave_base = __builtin_amdgcn_readfirstlane(wave_base);
+#pragma unroll
+    for (int m = 0; m < LS_PF_LISTS; ++m) {
+#pragma unroll
+        for (int r = 0; r < LS_PF_ROUNDS; ++r) {
+            const unsigned long long mk = keepm[m][r];
+            if ((mk >> lane_id()) & 1ull) {
+                const int slot = wave_base
+                                 + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mk >> 32),
+                                                                  __builtin_amdgcn_mbcnt_lo((uint32_t)mk, 0u));
+                if (slot < TK_CCAP) {
+                    s.cand.key[slot] = pf.e[m][r].key;
+                    s.cand.idx[slot] = pf.e[m][r].idx;
+                }
+            }
+            wave_base += (int)__builtin_popcountll(mk);
+        }
+    }
+    // the rest: lists beyond the eighth, entries beyond the first 256 of a list
+    for (int c = wave_id(); c < splits; c += TK_WAVES) {
+        const int        cnt   = (int)hdr[c].count;
+        const TopkEntry* e     = entries + (size_t)c * TK_CCAP;
+        const int        begin = c < LS_PF_LISTS * TK_WAVES ? LS_PF_ROUNDS * WAVE : 0;
+        for (int i0 = begin; i0 < cnt; i0 += WAVE) {
+            const int                i    = i0 + lane_id();
+            const TopkEntry          en   = i < cnt ? e[i] : TopkEntry{0u, 0u};
+            const bool               keep = i < cnt && en.key >= T0;
+            const unsigned long long mk   = __ballot(keep);
+            int                      base = 0;
+            if (lane_id() == 0 && mk != 0ull) {
+                base = atomicAdd(&s.n_cand, (int)__builtin_popcountll(mk));
+            }
+            base = __builtin_amdgcn_readfirstlane(base);
+            if (keep) {
+                const int slot =
+                    base + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mk >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mk, 0u));
+                if (slot < TK_CCAP) {
+                    s.cand.key[slot] = en.key;
+                    s.cand.idx[slot] = en.idx;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    int n = s.n_cand;
+    __syncthreads();
+    FTK_STAMP(2);
+    (void)total;
+    if (n > TK_CCAP) {
+        return -2;  // the union does not fit the list: the caller merges with the general routine
+    }
+    if (n > k + k / 2 && n <= 4 * TK_THREADS && k <= LG_MAX_K) {
+        // Far more candidates than needed (every workgroup of the gather reports the best of its own columns):
+        // raise the bound to the k-th largest of 256 slot maxima (slot t: entries t, t + 256, ...), which at
+        // least k entries reach, and keep what reaches it. The replay of the tie orders below ranks every
+        // candidate against every other one; this keeps it short.
+        uint32_t mx = 0u;
+        for (int i = t; i < n; i += TK_THREADS) {
+            const uint32_t key = s.cand.key[i];
+            mx                 = key > mx ? key : mx;
+        }
+        uint32_t* slot_key = reinterpret_cast<uint32_t*>(&s.stage.raw[0][0]);
+        slot_key[t]        = mx;
+        lds_barrier();
+        const uint32_t P = lean_kth_of_slots(slot_key, k);
+        lds_barrier();
+        if (P > T0) {
+            T0 = P;
+            n  = topk_prune(s, n, P);
+        }
+        FTK_STAMP(4);
+    }
+    *thr_out = T0;
+    return n;
+}
+
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, FusedLaunch l)
+{
+    constexpr int BMW = 0;  // the recovery paths read whole-row bitmaps from global memory
+    __shared__ TopkShared s;
+    const int             row = blockIdx.x;
+    // everything the row needs is requested before the first decision: the lists (vector loads), the
+    // arguments (scalar loads), the draw
+    TopkEntry*             row_entries = l.entries + (size_t)row * l.row_entries;
+    const LeanListPrefetch pf          = lean_prefetch_lists(l.splits, row_entries);
+    const bool             skip        = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
+    const bool             fin         = row_flag_or(l.finished, row, p.end_ids + row, false);
+    const int              k           = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
+    const float            tp          = row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f);
+    FusedRow<DT, BMW>      r(p, row);
+    if (skip) {
+        return;
+    }
+    if (fin) {
+        if (threadIdx.x == 0) {
+            l.ids[row] = p.end_ids[row];
+        }
+        return;
+    }
+    FTK_STAMP(0);
+    const TopkChunkHeader* headers = l.headers + (size_t)row * l.splits;
+    TopkChunkHeader        my_header{};
+    if ((int)threadIdx.x < l.splits) {
+        my_header = headers[threadIdx.x];
+    }
+    int draw_bits = 0;
+    if (threadIdx.x == 0) {
+        draw_bits = __float_as_int(row_uniform(l.rng, l.uniforms, row));
+    }
+    const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row, p.end_ids);
+    uint32_t          thr = 0u;
+    int               n   = lean_merge_lists<DT>(s, k, l.splits, my_header, row_entries, &thr, pf, &draw_bits);
+    const float       u   = __int_as_float(draw_bits);
+    if (n == -2) {
+        const TopkListPrefetch none{};
+        n = topk_merge_lists<DT>(s, k, l.splits, headers, row_entries, &thr, none);
+    }
+    if (n < 0) {
+        // A workgroup of the gather could not hold its candidates. Walk the whole row again, here, with the
+        // stream that recovers from overfull tiles; only rows it cannot bound either take the literal replay.
+        r.prepare_whole_row();
+        __syncthreads();
+        n = topk_stream<DT, FusedRow<DT, BMW>, 0>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
+    }
+    topk_select_lds<DT, FusedRow<DT, BMW>, true>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u,
+                                                 p.end_ids, out);
+    FTK_STAMP(8);
+}
+
 // Launchers, one translation unit per element type (lean_kernels.hip built with FTK_LEAN_DT = 0, 1, 2).
 // window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large; variant: see lean_occupancy.
 // start / stop: optional events carried by the launch.
 int lean_gather_launch_f32(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
+int lean_select_launch_f32(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+                           hipEvent_t stop);
+int lean_select_launch_f16(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+                           hipEvent_t stop);
+int lean_select_launch_bf16(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+                            hipEvent_t stop);
 int lean_gather_launch_f16(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 int lean_gather_launch_bf16(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
@@ -446,7 +712,8 @@ int lean_gather_launch_bf16(int window, int variant, dim3 grid, hipStream_t st, 
 // workgroups per compute unit a variant of the lean gather is built for
 inline int lean_occupancy(int variant)
 {
-    return variant == 2 ? 8 : 4;
+    (void)variant;
+    return 4;
 }
 
 }  // namespace ftk

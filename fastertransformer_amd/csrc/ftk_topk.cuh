@@ -26,23 +26,8 @@
 #include "ftk_device.cuh"
 #include "ftk_transform.cuh"
 
-// Optional phase timing for kernel development: FTK_PHASE(i) adds the time since the previous mark of
-// this workgroup to slot i (100 MHz constant clock, thread 0 only). Compiled out by default.
-#ifdef FTK_PHASE_TIMING
-static __device__ unsigned long long g_ftk_phase[32];
-#define FTK_PHASE_BEGIN() unsigned long long ftk_phase_t0_ = wall_clock64()
-#define FTK_PHASE(i)                                                                                                   \
-    do {                                                                                                               \
-        const unsigned long long now_ = wall_clock64();                                                                \
-        if (threadIdx.x == 0) {                                                                                        \
-            atomicAdd(&g_ftk_phase[i], now_ - ftk_phase_t0_);                                                          \
-            atomicAdd(&g_ftk_phase[16 + (i)], 1ull);                                                                   \
-        }                                                                                                              \
-        ftk_phase_t0_ = wall_clock64();                                                                                \
-    } while (0)
-#else
-#define FTK_PHASE_BEGIN()
-#define FTK_PHASE(i)
+#ifndef FTK_STAMP
+#define FTK_STAMP(i)
 #endif
 
 namespace ftk {
@@ -290,13 +275,23 @@ __device__ __forceinline__ int topk_prune(TopkShared& s, int n, uint32_t thr)
         s.n_cand = 0;
     }
     lds_barrier();
+    // one slot reservation per wave and batch of 64 entries (a ballot and a prefix count place the lanes)
 #pragma unroll
     for (int r = 0; r < TK_CCAP / TK_THREADS; ++r) {
-        const int i = t + r * TK_THREADS;
-        if (i < n && ck[r] >= thr) {
-            const int slot   = atomicAdd(&s.n_cand, 1);
-            s.cand.key[slot] = ck[r];
-            s.cand.idx[slot] = ci[r];
+        if (r * TK_THREADS < n) {
+            const bool               keep = t + r * TK_THREADS < n && ck[r] >= thr;
+            const unsigned long long m    = __ballot(keep);
+            int                      base = 0;
+            if (lane_id() == 0 && m != 0ull) {
+                base = atomicAdd(&s.n_cand, (int)__builtin_popcountll(m));
+            }
+            base = __builtin_amdgcn_readfirstlane(base);
+            if (keep) {
+                const int slot =
+                    base + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                s.cand.key[slot] = ck[r];
+                s.cand.idx[slot] = ci[r];
+            }
         }
     }
     lds_barrier();
@@ -439,6 +434,78 @@ __device__ __forceinline__ int topk_tighten(TopkShared& s, int n, int k, uint32_
     return topk_prune(s, n, *thr);
 }
 
+// Keep the candidates that at most k-1 others beat (the k largest keys and every tie with the k-th); in place,
+// order not preserved; returns how many remain. n <= 4 * TK_THREADS. An entry is dropped exactly when k or more
+// keys are strictly greater, so nothing the reference could pick is lost. Every thread counts, for up to four
+// entries of its own, the keys above them: the list is read four keys at a time (all lanes read the same
+// address), several reads in flight.
+__device__ __forceinline__ int topk_cut_to_k(TopkShared& s, int n, int k)
+{
+    constexpr int PER = 4;
+    const int     t   = threadIdx.x;
+    const int     per = (n + TK_THREADS - 1) / TK_THREADS;  // entries per thread that exist at all (uniform)
+    uint32_t      ck[PER], ci[PER];
+    int           above[PER];
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+        const int i = t + r * TK_THREADS;
+        ck[r]       = (r < per && i < n) ? s.cand.key[i] : 0xFFFFFFFFu;
+        ci[r]       = (r < per && i < n) ? s.cand.idx[i] : 0u;
+        above[r]    = 0;
+    }
+    const int n16 = (n + 15) & ~15;
+    if (t < n16 - n) {
+        s.cand.key[n + t] = 0u;  // padding that is above nothing
+    }
+    if (t == 0) {
+        s.n_cand = 0;
+    }
+    lds_barrier();
+    for (int j0 = 0; j0 < n16; j0 += 16) {
+        uint4 kk[4];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            kk[b] = *reinterpret_cast<const uint4*>(&s.cand.key[j0 + 4 * b]);
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t kj[4] = {kk[b].x, kk[b].y, kk[b].z, kk[b].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    if (r < per) {
+                        above[r] += kj[e] > ck[r] ? 1 : 0;
+                    }
+                }
+            }
+        }
+    }
+    lds_barrier();  // every thread has read the list: it can be rewritten
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+        if (r < per) {
+            const bool               keep = t + r * TK_THREADS < n && above[r] < k;
+            const unsigned long long m    = __ballot(keep);
+            int                      base = 0;
+            if (lane_id() == 0 && m != 0ull) {
+                base = atomicAdd(&s.n_cand, (int)__builtin_popcountll(m));
+            }
+            base = __builtin_amdgcn_readfirstlane(base);
+            if (keep) {
+                const int slot =
+                    base + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                s.cand.key[slot] = ck[r];
+                s.cand.idx[slot] = ci[r];
+            }
+        }
+    }
+    lds_barrier();
+    const int m = s.n_cand;
+    lds_barrier();
+    return m;
+}
+
 // -------------------------------------------------------------------------------------------
 // stream: tiles [tile_begin, tile_end) of one row -> candidate list in LDS
 // -------------------------------------------------------------------------------------------
@@ -565,7 +632,6 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         }
     };
 
-    FTK_PHASE_BEGIN();
     if (t == 0) {
         s.n_cand = 0;
     }
@@ -585,7 +651,6 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         }
         return rowctx.vector_bits(first, EPV);
     };
-    FTK_PHASE(1);
 
     // ---- initial bound from the first tile: maxima over the vectors that take the fast transform
     // (leaving the others out only lowers the bound).
@@ -685,7 +750,6 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
             }
         }
     }
-    FTK_PHASE(2);
     thr         = (uint32_t)__builtin_amdgcn_readfirstlane((int)thr);  // uniform: keep it in a scalar register
     float thr_f = key_to_float(thr);  // x >= thr_f  <=>  order_key(x) >= thr (NaN fails both)
     // The first tile is examined a second time below. Keep the compiler from carrying the converted
@@ -916,7 +980,6 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
             }
         }
         drain();
-        FTK_PHASE(3);
         // the next tile is requested before the bookkeeping of this one
         if (tile + 1 < tile_end) {
             load_tile(tile + 1);
@@ -930,12 +993,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         if (n_now > TK_CCAP) {
             const int tlo = max(0, vec0 * EPV - a);
             const int thi = max(tlo, min(vocab, (vec0 + TILE_VECS) * EPV - a));
-#ifdef FTK_NO_RARE
-            (void)tlo; (void)thi;
-            n = -1;
-#else
             n             = topk_stream_rare<DT, Row>(rowctx, s, k, n, tlo, thi, thr);
-#endif
             if (n < 0) {
                 return -1;
             }
@@ -952,7 +1010,6 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
         else {
             n = n_now;
         }
-        FTK_PHASE(4);
     }
     *thr_out = thr;
     return n;
@@ -970,7 +1027,6 @@ __device__ __forceinline__ void topk_dump_list(TopkShared& s, int n, int k, int 
                                                TopkChunkHeader* header, TopkEntry* entries)
 {
     const int t = threadIdx.x;
-    FTK_PHASE_BEGIN();
     uint32_t share = 0u;
     if (n > k && (n > TK_RAW_DUMP || n * splits > TK_CCAP)) {  // the union of raw lists fits the merge's list
         n                = topk_tighten(s, n, k, &thr);
@@ -990,7 +1046,6 @@ __device__ __forceinline__ void topk_dump_list(TopkShared& s, int n, int k, int 
         h.share     = share;
         *header     = h;
     }
-    FTK_PHASE(5);
 }
 
 // -------------------------------------------------------------------------------------------
@@ -1026,46 +1081,55 @@ __device__ __forceinline__ TopkOutputs topk_outputs(int* ids, int* sequence_leng
 }
 
 // thread 0 only: weights w[0..n) in selection order -> sampled position (sampling_topk_kernels.cu:282-311).
-// `w` is 16-byte aligned LDS, zero padded to a multiple of 4 (adding +0 to a non-negative sum is exact),
-// so the strictly sequential sum runs from registers loaded four at a time.
+// `w` is 16-byte aligned LDS, zero padded to a multiple of 4 (adding +0 to a non-negative sum is exact).
+// Both passes are strictly sequential in fp32, as in the reference; 32 weights are fetched at a time so that
+// the chain of additions never waits for LDS.
 __device__ __forceinline__ int topk_sample_walk(const float* w, int n, float u, float p, float* s_sum_out)
 {
     const float4* w4    = reinterpret_cast<const float4*>(w);
     const int     n4    = (n + 3) >> 2;
     float         s_sum = 0.0f;
-#pragma unroll 4
-    for (int i = 0; i < n4; ++i) {
-        const float4 v = w4[i];
-        s_sum          = s_sum + v.x;
-        s_sum          = s_sum + v.y;
-        s_sum          = s_sum + v.z;
-        s_sum          = s_sum + v.w;
-    }
-    // the subtractions depend on each other, the loads do not: sixteen weights are fetched at a time
-    // (reading a few entries past n is harmless, they are not used)
-    float rand_num = u * p * s_sum;
-    int   pick     = -1;
-    for (int i0 = 0; i0 < n && pick < 0; i0 += 16) {
-        float4 v[4];
+    for (int i0 = 0; i0 < n4; i0 += 8) {
+        float4 v[8];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            v[b] = w4[(i0 >> 2) + b];
+        for (int b = 0; b < 8; ++b) {
+            v[b] = i0 + b < n4 ? w4[i0 + b] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
-        const float x[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
-                             v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const int i = i0 + j;
-            if (pick < 0 && i < n) {
-                rand_num = rand_num - x[j];
-                if (rand_num <= 0.0f || i == n - 1) {
-                    pick = i;
+        for (int b = 0; b < 8; ++b) {
+            s_sum = s_sum + v[b].x;
+            s_sum = s_sum + v[b].y;
+            s_sum = s_sum + v[b].z;
+            s_sum = s_sum + v[b].w;
+        }
+    }
+    // the running difference never recovers once it is <= 0 (the weights are non-negative), so the first
+    // position where it is <= 0 is found without branching: keep subtracting, remember the first hit
+    float rand_num = u * p * s_sum;
+    int   pick     = n - 1;
+    bool  found    = false;
+    for (int i0 = 0; i0 < n4 && !found; i0 += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            v[b] = i0 + b < n4 ? w4[i0 + b] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const float x[4] = {v[b].x, v[b].y, v[b].z, v[b].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = (i0 + b) * 4 + j;
+                rand_num    = found ? rand_num : rand_num - x[j];
+                if (!found && i < n && rand_num <= 0.0f) {
+                    pick  = i;
+                    found = true;
                 }
             }
         }
     }
     *s_sum_out = s_sum;
-    return pick < 0 ? n - 1 : pick;
+    return pick;
 }
 
 __device__ __forceinline__ void topk_emit(const TopkOutputs& o, int row, int id, bool probs_in, float w, float s_sum,
@@ -1194,13 +1258,12 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
     const int BS1     = 1 << bs1_log;
     const int BS2     = max_top_k <= 32 ? 128 : 256;
     int       n_list  = 0;  // length of the final ordered list: values in s.w (as fp32), ids in s.idx
-    FTK_PHASE_BEGIN();
 
     if (n >= 0) {
         if (n > TK_THREADS && n > k) {
             n = topk_tighten<DEEP>(s, n, k, &thr);
         }
-        FTK_PHASE(9);
+        FTK_STAMP(5);
         // candidates -> stage-1 composite keys, in place
         //   slice(3) | ~key(32) | BS1-1-t (8) | j (21),   i = (j*8 + slice)*BS1 + t
         constexpr int PER = TK_CCAP / TK_THREADS;
@@ -1228,7 +1291,6 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
             }
         }
         lds_barrier();
-        FTK_PHASE(10);
         int slice_start[8];
         {
             int acc = 0;
@@ -1361,7 +1423,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
         __syncthreads();
     }
 
-    FTK_PHASE(11);
+    FTK_STAMP(6);
     // ---- weights (sampling_topk_kernels.cu:264-279): exp(x - max) on logits, the value itself on
     // probabilities; the list is padded with zero weights to a multiple of 4 for the vectorised walk
     const float x0 = n_list > 0 ? s.sel.w[0] : 0.0f;
@@ -1371,7 +1433,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
         s.sel.w[i]        = i < n_list ? (probs_in ? x : det_expf(x - x0)) : 0.0f;
     }
     __syncthreads();
-    FTK_PHASE(12);
+    FTK_STAMP(7);
     if (t == 0) {
         if (n_list == 0) {
             topk_emit(out, row, 0, probs_in, 0.0f, 0.0f, end_ids, false);
@@ -1382,7 +1444,6 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
             topk_emit(out, row, s.sel.idx[pick] % vocab, probs_in, s.sel.w[pick], s_sum, end_ids, true);
         }
     }
-    FTK_PHASE(13);
 }
 
 // What a select workgroup asks for before it knows anything about its row: wave w takes the first
@@ -1414,7 +1475,6 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
                                                 const TopkListPrefetch& pf)
 {
     const int t = threadIdx.x;
-    FTK_PHASE_BEGIN();
     // Row-wide lower bound T0 of the k-th largest key, the larger of two valid ones: the largest
     // `threshold` of a chunk that holds >= k elements, and the smallest `share` when every chunk has one.
     // A list is complete above its own threshold (lists of chunks with fewer than k selectable elements
@@ -1430,13 +1490,13 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
             T0 = h.threshold;
         }
     }
+    FTK_STAMP(1);
     if (overflow) {
         return -1;
     }
     if (min_share > T0) {
         T0 = min_share;  // 0 when some chunk has no share bound
     }
-    FTK_PHASE(7);
     // one wave per chunk list
     auto gather = [&](uint32_t thr) -> int {
         if (t == 0) {
@@ -1485,7 +1545,7 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
         return total;
     };
     int n = gather(T0);
-    FTK_PHASE(8);
+    FTK_STAMP(2);
     if (n > TK_CCAP) {
         // large k over many chunks: find the exact k-th largest key by bisection over the lists
         auto count_ge = [&](uint32_t thr) -> int {
@@ -1514,6 +1574,12 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
     }
     if (n > TK_CCAP) {
         return -1;  // thousands of identical values around the k-th
+    }
+    if (n > k + k / 4 && n <= 4 * TK_THREADS) {
+        // Cut the union to its k largest keys (and their ties) before the tie orders are replayed: the replay
+        // ranks every candidate against every other one with 64-bit keys, twice.
+        n = topk_cut_to_k(s, n, k);
+        FTK_STAMP(4);
     }
     *thr_out = T0;
     return n;

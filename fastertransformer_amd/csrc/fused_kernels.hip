@@ -64,96 +64,6 @@ history_bitmap_kernel(uint32_t* __restrict__ bitmaps, int bitmap_words, const in
     }
 }
 
-template<int DT, int BMW, int MANY = 0>
-__global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
-fused_row_kernel(FusedParams p, FusedLaunch l)
-{
-    __shared__ TopkShared s;
-    const int             row = blockIdx.x;
-    if (p.skip_decode != nullptr && p.skip_decode[row]) {
-        return;
-    }
-    if (l.finished != nullptr && l.finished[row]) {
-        if (threadIdx.x == 0) {
-            l.ids[row] = p.end_ids[row];  // a finished row emits its end id without looking at the logits
-        }
-        return;
-    }
-    const int    k  = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    const float  tp = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
-    FTK_PHASE_BEGIN();
-    const float  u  = fused_row_draw(s, l, row);
-    const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row, p.end_ids);
-    FusedRow<DT, BMW> r(p, row);
-    FTK_PHASE(0);
-    uint32_t     thr = 0u;
-    const int    n   = topk_stream<DT, FusedRow<DT, BMW>, MANY>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
-    topk_select_lds<DT>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, l.entries + (size_t)row * l.row_entries, false, u,
-                        p.end_ids, out);
-}
-
-template<int DT, int BMW, int MANY = 0>
-__global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : BMW <= FUSED_BITMAP_WORDS_SMALL ? TK_MIN_WGS : (TK_MIN_WGS * 3 + 3) / 4)
-fused_gather_kernel(FusedParams p, FusedLaunch l)
-{
-    __shared__ TopkShared s;
-    const int             row   = blockIdx.y;
-    const int             chunk = blockIdx.x;
-    if (p.skip_decode != nullptr && p.skip_decode[row]) {
-        return;
-    }
-    if (p.finished_in != nullptr && p.finished_in[row]) {
-        return;
-    }
-    const int    k = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    FusedRow<DT, BMW> r(p, row);
-    const int    tiles = topk_row_tiles<DT>(r.rowp, p.Vp);
-    const int    t0    = min(tiles, chunk * l.tiles_per_wg);
-    const int    t1    = min(tiles, t0 + l.tiles_per_wg);
-    uint32_t     thr   = 0u;
-    const int    n     = topk_stream<DT, FusedRow<DT, BMW>, MANY>(r, s, p.Vp, k, t0, t1, &thr);
-    topk_dump_list(s, n, k, l.splits, thr, l.headers + (size_t)row * l.splits + chunk,
-                   l.entries + (size_t)row * l.row_entries + (size_t)chunk * TK_CCAP);
-}
-
-template<int DT>
-__global__ void __launch_bounds__(TK_THREADS) fused_select_kernel(FusedParams p, FusedLaunch l)
-{
-    constexpr int BMW = 0;  // the literal replay reads whole-row bitmaps from global memory
-    __shared__ TopkShared s;
-    const int             row = blockIdx.x;
-    // everything the row needs is requested before the first decision: the arguments (scalar loads), the
-    // chunk lists (vector loads), the draw
-    TopkEntry*             row_entries = l.entries + (size_t)row * l.row_entries;
-    const TopkListPrefetch pf          = topk_prefetch_lists(l.splits, row_entries);
-    const bool   skip = p.skip_decode != nullptr && p.skip_decode[row];
-    const bool   fin  = l.finished != nullptr && l.finished[row];
-    const int    k    = p.top_ks != nullptr ? p.top_ks[row] : p.max_top_k;
-    const float  tp   = p.top_ps != nullptr ? p.top_ps[row] : 1.0f;
-    FusedRow<DT, BMW> r(p, row);
-    if (skip) {
-        return;
-    }
-    if (fin) {
-        if (threadIdx.x == 0) {
-            l.ids[row] = p.end_ids[row];
-        }
-        return;
-    }
-    const float  u  = fused_row_draw(s, l, row);
-    const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row, p.end_ids);
-    uint32_t     thr         = 0u;
-    int          n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr, pf);
-    if (n < 0 && topk_many_level(p.max_top_k) == 0) {
-        // A workgroup of the gather could not hold its candidates. Walk the whole row again, here, with the
-        // stream that recovers from overfull tiles; only rows it cannot bound either take the literal replay.
-        r.prepare_whole_row();
-        __syncthreads();
-        n = topk_stream<DT, FusedRow<DT, BMW>, 0>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);
-    }
-    topk_select_lds<DT, FusedRow<DT, BMW>, true>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
-}
-
 }  // namespace ftk
 
 using namespace ftk;
@@ -182,18 +92,6 @@ void launch_timed(int which, K kernel, dim3 grid, dim3 block, hipStream_t st, Ar
     }
 }
 }  // namespace
-
-#ifdef FTK_PHASE_TIMING
-extern "C" int ftk_debug_read_phases_fused(unsigned long long* out, int reset)
-{
-    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ftk_phase), sizeof(unsigned long long) * 32);
-    if (e == hipSuccess && reset) {
-        unsigned long long z[32] = {};
-        e = hipMemcpyToSymbol(HIP_SYMBOL(g_ftk_phase), z, sizeof(z));
-    }
-    return (int)e;
-}
-#endif
 
 extern "C" int ftk_profile_enable(int max_launches)
 {
@@ -367,23 +265,37 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     l.subs_per_wg     = 0;
     l.headers         = (TopkChunkHeader*)(ws + bitmap_bytes);
     l.entries         = (TopkEntry*)(l.headers + (size_t)rows * plan.splits);
+    // events carried by a launch when per-kernel timing is on
+    auto take_events = [&](int which, hipEvent_t* e0, hipEvent_t* e1) {
+        KernelTimer& tm = g_timers[which];
+        *e0 = *e1 = nullptr;
+        if (g_profile && tm.used < (int)tm.start.size()) {
+            *e0 = tm.start[tm.used];
+            *e1 = tm.stop[tm.used];
+            tm.used++;
+        }
+    };
+    auto launch_general = [&](int kind, int window, dim3 grid) -> int {
+        hipEvent_t e0, e1;
+        take_events(kind == FUSED_KIND_SELECT ? 2 : 1, &e0, &e1);
+        if (a->dtype == FTK_DTYPE_F32) {
+            return fused_launch_f32(kind, window, many, grid, st, p, l, e0, e1);
+        }
+        if (a->dtype == FTK_DTYPE_F16) {
+            return fused_launch_f16(kind, window, many, grid, st, p, l, e0, e1);
+        }
+        return fused_launch_bf16(kind, window, many, grid, st, p, l, e0, e1);
+    };
+    const int window = p.bitmaps_ready ? 0 : (p.lds_window == 2 ? 2 : 1);
+    int       rc;
     if (lean_mode != 0) {
         l.splits       = lplan.splits;
         l.subs_per_wg  = lplan.subs_per_wg;
         l.row_entries  = (size_t)lplan.splits * TK_CCAP;
         l.entries      = (TopkEntry*)(l.headers + (size_t)rows * lplan.splits);
         const dim3 lgrid(lplan.splits, rows);
-        const int  window = p.bitmaps_ready ? 0 : (p.lds_window == 2 ? 2 : 1);
-        hipEvent_t e0 = nullptr, e1 = nullptr;
-        {
-            KernelTimer& tm = g_timers[1];
-            if (g_profile && tm.used < (int)tm.start.size()) {
-                e0 = tm.start[tm.used];
-                e1 = tm.stop[tm.used];
-                tm.used++;
-            }
-        }
-        int rc;
+        hipEvent_t e0, e1;
+        take_events(1, &e0, &e1);
         if (a->dtype == FTK_DTYPE_F32) {
             rc = lean_gather_launch_f32(window, lean_mode, lgrid, st, p, l, e0, e1);
         }
@@ -396,68 +308,23 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         if (rc != 0) {
             return rc;
         }
-        FTK_LAUNCH_CHECK();
-        FTK_DISPATCH_DTYPE(a->dtype,
-                           launch_timed(2, fused_select_kernel<DT>, dim3(rows), dim3(TK_THREADS), st, p, l));
-        FTK_LAUNCH_CHECK();
-        return 0;
+        take_events(2, &e0, &e1);
+        if (a->dtype == FTK_DTYPE_F32) {
+            return lean_select_launch_f32(rows, st, p, l, e0, e1);
+        }
+        if (a->dtype == FTK_DTYPE_F16) {
+            return lean_select_launch_f16(rows, st, p, l, e0, e1);
+        }
+        return lean_select_launch_bf16(rows, st, p, l, e0, e1);
     }
     if (plan.splits == 1) {
-        const dim3 grid1(rows), block(TK_THREADS);
-        if (many == 2) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 2>, grid1,
-                                                      block, st, p, l));
-        }
-        else if (many == 1) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 1>, grid1,
-                                                      block, st, p, l));
-        }
-        else if (p.bitmaps_ready) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>, grid1, block,
-                                                      st, p, l));
-        }
-        else if (p.lds_window == 2) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_LARGE>, grid1, block,
-                                                      st, p, l));
-        }
-        else {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_row_kernel<DT, FUSED_BITMAP_WORDS_SMALL>, grid1, block,
-                                                      st, p, l));
-        }
-        FTK_LAUNCH_CHECK();
-        return 0;
+        return launch_general(FUSED_KIND_ROW, window, dim3(rows));
     }
-    dim3 grid(plan.splits, rows);
-    {
-        const dim3 block(TK_THREADS);
-        if (many == 2) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 2>, grid,
-                                                      block, st, p, l));
-        }
-        else if (many == 1) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL, 1>, grid,
-                                                      block, st, p, l));
-        }
-        else if (p.bitmaps_ready) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>, grid, block,
-                                                      st, p, l));
-        }
-        else if (p.lds_window == 2) {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_LARGE>, grid, block,
-                                                      st, p, l));
-        }
-        else {
-            FTK_DISPATCH_DTYPE(a->dtype, launch_timed(1, fused_gather_kernel<DT, FUSED_BITMAP_WORDS_SMALL>, grid, block,
-                                                      st, p, l));
-        }
+    rc = launch_general(FUSED_KIND_GATHER, window, dim3(plan.splits, rows));
+    if (rc != 0) {
+        return rc;
     }
-    FTK_LAUNCH_CHECK();
-    {
-        FTK_DISPATCH_DTYPE(a->dtype,
-                           launch_timed(2, fused_select_kernel<DT>, dim3(rows), dim3(TK_THREADS), st, p, l));
-    }
-    FTK_LAUNCH_CHECK();
-    return 0;
+    return launch_general(FUSED_KIND_SELECT, 0, dim3(rows));
 }
 
 // ---- the fused step for callers that cannot allocate ------------------------------------------------

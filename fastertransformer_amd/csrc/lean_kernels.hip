@@ -46,9 +46,28 @@ int lean_gather_launch_bf16
      hipEvent_t stop)
 {
     if (variant == 2) {
-        return lean_launch_window<8, 2>(window, grid, st, p, l, start, stop);
+        return lean_launch_window<4, 3>(window, grid, st, p, l, start, stop);
     }
-    return lean_launch_window<4, 4>(window, grid, st, p, l, start, stop);
+    return lean_launch_window<4, 2>(window, grid, st, p, l, start, stop);
+}
+
+#if FTK_LEAN_DT == 0
+int lean_select_launch_f32
+#elif FTK_LEAN_DT == 1
+int lean_select_launch_f16
+#else
+int lean_select_launch_bf16
+#endif
+    (int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start, hipEvent_t stop)
+{
+    if (start != nullptr) {
+        hipExtLaunchKernelGGL((lean_select_kernel<FTK_LEAN_DT>), dim3(rows), dim3(TK_THREADS), 0, st, start, stop, 0, p,
+                              l);
+    }
+    else {
+        hipLaunchKernelGGL((lean_select_kernel<FTK_LEAN_DT>), dim3(rows), dim3(TK_THREADS), 0, st, p, l);
+    }
+    return (int)hipGetLastError();
 }
 
 }  // namespace ftk

@@ -83,7 +83,6 @@ __global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : TK_MI
     __shared__ TopkShared s;
     const int             row   = blockIdx.y;
     const int             chunk = blockIdx.x;
-    FTK_PHASE_BEGIN();
     if (a.skip_decode != nullptr && a.skip_decode[row]) {
         return;
     }
@@ -93,7 +92,6 @@ __global__ void __launch_bounds__(TK_THREADS, MANY > 0 ? TK_MIN_WGS_MANY : TK_MI
     const int      k = a.top_ks != nullptr ? a.top_ks[row] : a.max_top_k;
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
-    FTK_PHASE(0);
     const int tiles = topk_row_tiles<DT>(r.rowp, a.vocab);
     const int t0    = min(tiles, chunk * a.tiles_per_wg);
     const int t1    = min(tiles, t0 + a.tiles_per_wg);
@@ -124,12 +122,10 @@ __global__ void __launch_bounds__(TK_THREADS) topk_select_kernel(TopkKernelArgs 
         }
         return;
     }
-    FTK_PHASE_BEGIN();
     const float    u = topk_row_draw(s, a.rng, a.uniforms, row);
     const TopkOutputs out = topk_outputs(a.ids, a.sequence_length, a.finished, a.cum_log_probs, a.output_log_probs, row, a.end_ids);
     PlainRowAt<DT> r;
     r.rowp = (const typename Storage<DT>::T*)a.log_probs + (size_t)row * a.vocab;
-    FTK_PHASE(6);
     uint32_t   thr = 0u;
     const int  n   = topk_merge_lists<DT>(s, k, a.splits, a.headers + (size_t)row * a.splits, row_entries, &thr, pf);
     topk_select_lds<DT, PlainRowAt<DT>, true>(r, s, n, thr, row, a.vocab, k, p, a.max_top_k, row_entries,
@@ -141,18 +137,6 @@ __global__ void __launch_bounds__(TK_THREADS) topk_select_kernel(TopkKernelArgs 
 using namespace ftk;
 
 extern "C" {
-
-#ifdef FTK_PHASE_TIMING
-int ftk_debug_read_phases(unsigned long long* out, int reset)
-{
-    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(g_ftk_phase), sizeof(unsigned long long) * 32);
-    if (e == hipSuccess && reset) {
-        unsigned long long z[32] = {};
-        e = hipMemcpyToSymbol(HIP_SYMBOL(g_ftk_phase), z, sizeof(z));
-    }
-    return (int)e;
-}
-#endif
 
 int ftk_invoke_batch_topk_sampling(int dtype, void* workspace, size_t* workspace_size, const void* log_probs, int* ids,
                                    int* sequence_length, bool* finished, float* cum_log_probs,
