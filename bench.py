@@ -22,6 +22,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+PLAIN_READ = "plain_read_b256_v128256_f32"
 # HBM bytes per launch of the dominant kernel on the headline workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by a copy kernel of known size (summary under profiles/)
 TRAFFIC_BYTES_PER_LAUNCH = 152029196
@@ -44,6 +45,10 @@ WORKLOADS = {
     "decode_step_b256_v51200_f16_topk1-1024_topp0.9_temp0.8_rep1.1": dict(
         dtype="f16", batch=256, vocab=51200, vocab_padded=51200, top_k=(1, 4, 16, 40, 64, 1024), top_p=0.9,
         temperature=0.8, repetition_penalty=1.1, prompt=64, sigma=2.5),
+    # secondary line (only with --workload): the fused step at batch 1024 (fp16, vocabulary 152064), no log-probs
+    "decode_step_b1024_v152064_f16_topk64_topp0.9_temp0.8_rep1.1": dict(
+        dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
+        repetition_penalty=1.1, prompt=64, sigma=2.5),
     "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs": dict(
         dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=8, sigma=2.5),
@@ -56,7 +61,7 @@ def algorithmic_bytes(w, step):
     return w["batch"] * w["vocab_padded"] * elem + w["batch"] * history * 4 + w["batch"] * 32
 
 
-def run_gpu(name, w, steps, warmup, nbuf=4):
+def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     import torch
     import fastertransformer_amd as fa
     from fastertransformer_amd import ops
@@ -130,6 +135,15 @@ def run_gpu(name, w, steps, warmup, nbuf=4):
         kernel_ms.append((tot.value / n.value) if n.value else 0.0)
     ops.check(lib.ftk_profile_enable(0))
     assert checksum == int(output_ids[H + warmup:H + total].to(torch.int64).sum().item()), "the two passes differ"
+    oracle = None
+    if check_oracle:
+        # one more step, outside every timed region, repeated on the CPU oracle from the same state
+        from helpers import to_numpy
+        state = (to_numpy(finished), to_numpy(seq_len))
+        one_step(total)
+        torch.cuda.synchronize()
+        oracle = check_step_against_oracle(w, bufs[total % nbuf], draws[total % nbuf], output_ids, H + total, H,
+                                           top_ks, state)
 
     ms_per_step = wall * 1e3 / steps
     mid_step = H + warmup + steps // 2
@@ -144,8 +158,54 @@ def run_gpu(name, w, steps, warmup, nbuf=4):
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=TRAFFIC_BYTES_PER_LAUNCH, kernel=dominant, algorithmic_bytes_per_launch=alg),
         step_gbs=alg / (gpu_ms / steps * 1e-3) / 1e9,
-        sampled_ids_checksum=checksum,
+        sampled_ids_checksum=checksum, oracle_check=oracle,
     )
+
+
+def check_step_against_oracle(w, logits, draws, output_ids, step, H, top_ks, state):
+    """One decode step of the benchmark repeated on the CPU oracle (same logits, draws, token history, finished
+    flags and lengths): the sampled ids of every row must be identical. Returns what was compared."""
+    import ft_oracle as O
+    from helpers import to_numpy
+    odt = {"f32": O.F32, "f16": O.F16, "bf16": O.BF16}[w["dtype"]]
+    B, V, Vp = w["batch"], w["vocab"], w["vocab_padded"]
+    ids = to_numpy(output_ids)
+    got = ids[step].copy()
+    history = ids.copy()
+    history[step:] = 0
+    layer = O.OracleDynamicDecodeLayer(odt, V, Vp)
+    layer.setup(B, [int(k) for k in top_ks], [w["top_p"]], [w["temperature"]], [w["repetition_penalty"]])
+    finished, seq = state[0].copy(), state[1].copy()
+    end = np.full(B, V - 1, np.int32)
+    x = to_numpy(logits.reshape(B, Vp), odt)
+    layer.forward(x, end, history, step, H, to_numpy(draws), finished=finished, sequence_length=seq)
+    want = history[step]
+    assert np.array_equal(got, want), "sampled ids differ from the oracle in %d of %d rows" % (
+        int((got != want).sum()), B)
+    return dict(rows=B, step=int(step), ids_checksum=int(want.astype(np.int64).sum()), identical=True)
+
+
+def run_plain_read(steps, warmup, nbuf=4):
+    """The yardstick: a kernel that only fetches 256 x 128256 fp32 with the streaming kernel's launch shape
+    (ftk_measure_plain_read), buffers in rotation like the decode step's logits."""
+    import torch
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+    torch.cuda.set_device(0)
+    B, V = 256, 128256
+    bufs = [torch.randn((B, V), device="cuda:0") for _ in range(nbuf)]
+    sink = torch.zeros(8192, device="cuda:0")
+    lib = fa.ftk()
+    nbytes = B * V * 4
+    ms = C.c_float(0.0)
+    times = []
+    for i in range(warmup + steps):
+        ops.check(lib.ftk_measure_plain_read(bufs[i % nbuf].data_ptr(), nbytes, sink.data_ptr(), sink.numel(),
+                                             ops.current_stream(), C.addressof(ms)))
+        if i >= warmup:
+            times.append(ms.value)
+    avg = sum(times) / len(times)
+    return dict(bytes=nbytes, ms=avg, best_ms=min(times), gbs=nbytes / (avg * 1e-3) / 1e9)
 
 
 def run_gpu_topp(name, w, steps, warmup, nbuf=3):
@@ -256,14 +316,13 @@ def run_gpu_loop(name, w, steps, warmup, nbuf=2):
                 sampled_ids_checksum=int(output_ids[H + warmup:H + total].to(torch.int64).sum().item()))
 
 
-def run_cpu_baseline(w, budget_s=12.0):
-    """the oracle (a scalar, single-threaded restatement of the reference algorithm) on rows of the same
-    workload, until `budget_s` seconds of CPU work have been spent"""
+def _oracle_rows_per_second(w, rows, budget_s, seed):
+    """the oracle's DynamicDecodeLayer on `rows`-row batches of the workload for about `budget_s` seconds of this
+    thread's time; returns (rows done, seconds)"""
     import ft_oracle as O
     dt = {"f32": O.F32, "f16": O.F16, "bf16": O.BF16}[w["dtype"]]
     V, Vp, H = w["vocab"], w["vocab_padded"], w["prompt"]
-    rows = 16
-    rng = np.random.default_rng(99)
+    rng = np.random.default_rng(seed)
     layer = O.OracleDynamicDecodeLayer(dt, V, Vp)
     layer.setup(rows, [w["top_k"]], [w["top_p"]], [w["temperature"]], [w["repetition_penalty"]])
     max_steps = 4096
@@ -273,7 +332,7 @@ def run_cpu_baseline(w, budget_s=12.0):
     seq = np.full(rows, H - 1, np.int32)
     end = np.full(rows, V - 1, np.int32)
     # a few logits batches generated up front and reused, so that the loop times the oracle and nothing else
-    batches = [O.to_storage((rng.standard_normal((rows, Vp)) * w["sigma"]).astype(np.float32), dt) for _ in range(4)]
+    batches = [O.to_storage((rng.standard_normal((rows, Vp)) * w["sigma"]).astype(np.float32), dt) for _ in range(2)]
     done, spent, step = 0, 0.0, H
     while spent < budget_s and step < H + max_steps:
         logits = batches[(step - H) % len(batches)].copy()
@@ -284,9 +343,33 @@ def run_cpu_baseline(w, budget_s=12.0):
         spent += time.perf_counter() - t0
         done += rows
         step += 1
-    return dict(value=done / spent, unit="tokens/s", cores=1, kind="port",
-                sample="%d rows of the same workload (%d decode steps of a %d-row batch, V=%d), %.1f s of CPU time"
-                       % (done, step - H, rows, V, spent))
+    return done, spent
+
+
+def run_cpu_baseline(w, budget_s=8.0):
+    """The CPU baseline beside the GPU number: the oracle (a scalar restatement of the reference algorithm; the
+    reference's own host functions live inside CUDA unit tests and cannot be built here) on rows of the same
+    workload, first on one core, then with one thread per core, every thread on rows of its own (rows are
+    independent; the oracle's C code runs outside the interpreter lock). Bounded: about `budget_s` seconds each."""
+    from concurrent.futures import ThreadPoolExecutor
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1))
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    rows = 8
+    done1, spent1 = _oracle_rows_per_second(w, rows, budget_s, 99)
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(max_workers=cores) as pool:
+        parts = list(pool.map(lambda i: _oracle_rows_per_second(w, rows, budget_s, 100 + i), range(cores)))
+    wall = time.perf_counter() - t0
+    done_all = sum(p[0] for p in parts)
+    busy = max(p[1] for p in parts)  # the threads run side by side: the slowest one bounds the rate
+    return dict(value=done_all / busy, unit="tokens/s", cores=cores, kind="port",
+                single_core_value=done1 / spent1,
+                sample="%d-row batches of the same workload (V=%d): %d rows in %.1f s on one core, then %d rows in "
+                       "%.1f s with one thread on each of %d cores (%.1f s wall including input generation)"
+                       % (rows, w["vocab"], done1, spent1, done_all, busy, cores, wall))
 
 
 def main():
@@ -298,7 +381,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run five plain device copies of 128 MiB, the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE counter readings are scaled by")
-    ap.add_argument("--workload", default=next(iter(WORKLOADS)), choices=list(WORKLOADS),
+    ap.add_argument("--workload", default=next(iter(WORKLOADS)), choices=list(WORKLOADS) + [PLAIN_READ],
                     help="default: the headline decode step; the others print a secondary line of their own")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -306,6 +389,17 @@ def main():
               "exchange); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     name = a.workload
+    if name == PLAIN_READ:
+        r = run_plain_read(a.steps, a.warmup)
+        print(json.dumps({
+            "metric": "HBM GB/s of a kernel that only reads 256 x 128256 fp32 (the streaming kernel's launch shape)",
+            "value": r["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": r["ms"], "best_ms": r["best_ms"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": name},
+            "roofline": {"bound": "hbm", "achieved": r["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": r["gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": "read_yardstick_kernel",
+                         "algorithmic_bytes_per_launch": r["bytes"]}}))
+        return
     w = WORKLOADS[name]
     if name.startswith("topp_step"):
         r = run_gpu_topp(name, w, a.steps, a.warmup)
@@ -329,7 +423,7 @@ def main():
                        "top_p": w["top_p"]},
             "sampled_ids_checksum": r["sampled_ids_checksum"]}))
         return
-    r = run_gpu(name, w, a.steps, a.warmup)
+    r = run_gpu(name, w, a.steps, a.warmup, check_oracle=(name == next(iter(WORKLOADS))))
     if name != next(iter(WORKLOADS)):
         r["roofline"]["traffic"] = None  # the counter runs cover the headline workload only
         print(json.dumps({
@@ -338,7 +432,8 @@ def main():
             "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
             "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": w["dtype"], "data": "synthetic",
-            "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"], "top_k": list(w["top_k"]),
+            "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"],
+                       "top_k": list(w["top_k"]) if isinstance(w["top_k"], tuple) else w["top_k"],
                        "top_p": w["top_p"], "temperature": w["temperature"],
                        "repetition_penalty": w["repetition_penalty"], "history": w["prompt"]},
             "roofline": r["roofline"], "gpu_ms_per_step": r["gpu_ms_per_step"], "kernel_ms": r["kernel_ms"],
@@ -362,6 +457,7 @@ def main():
         "roofline": r["roofline"],
         "gpu_ms_per_step": r["gpu_ms_per_step"], "kernel_ms": r["kernel_ms"], "step_hbm_gbs": r["step_gbs"],
         "step_hbm_frac": r["step_gbs"] / HBM_PEAK_GBS, "sampled_ids_checksum": r["sampled_ids_checksum"],
+        "oracle_check": r["oracle_check"],
     }
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline(w)

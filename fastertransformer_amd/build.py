@@ -1,6 +1,8 @@
 """Builds the native libraries of the sampling engine in-tree.
 
   fastertransformer_amd/lib/libftk_sampling.so  HIP kernels + C ABI (include/ftk_sampling.h), gfx950
+  fastertransformer_amd/lib/libftk_sampling_hooks.so  the same with the test hooks of include/ftk_test_hooks.h
+                                                (loaded by the test-suite only)
   fastertransformer_amd/lib/libft_decode.so     host C++ layers (DynamicDecodeLayer, TopK/TopPSamplingLayer)
                                                 + the handle API used by bindings
   fastertransformer_amd/lib/libth_transformer.so  torch.classes.FasterTransformer.DynamicDecodeOp (PyTorch-ROCm
@@ -48,6 +50,10 @@ HIP_FLAGS = [
 ]
 
 
+HOOK_UNITS = [("fused_kernels.hip", "fused_kernels.o"), ("topp_kernels.hip", "topp_kernels.o"),
+              ("criteria_kernels.hip", "criteria_kernels.o")]
+
+
 def _run(cmd):
     print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
@@ -90,6 +96,20 @@ def build(force=True, verbose=True, with_torch=True):
         list(pool.map(_run, jobs))
     kernels_so = os.path.join(LIB, "libftk_sampling.so")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", kernels_so] + objs)
+    # The hooks build for the test-suite (include/ftk_test_hooks.h): the three translation units that carry
+    # hooks are compiled again with -DFTK_TEST_HOOKS, everything else is shared with the product library.
+    hook_objs = list(objs)
+    hook_jobs = []
+    for src, obj_name in HOOK_UNITS:
+        path = os.path.join(CSRC, src)
+        obj = os.path.join(LIB, obj_name.replace(".o", "_hooks.o"))
+        if force or _newer(obj, [path] + sorted(_includes(path))):
+            hook_jobs.append([HIPCC] + HIP_FLAGS + ["-DFTK_TEST_HOOKS", "-c", path, "-o", obj])
+        hook_objs[hook_objs.index(os.path.join(LIB, obj_name))] = obj
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        list(pool.map(_run, hook_jobs))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", os.path.join(LIB, "libftk_sampling_hooks.so")]
+         + hook_objs)
 
     host_sources, th_sources = [], []
     for d, _, files in os.walk(SRC):

@@ -5,48 +5,46 @@
 
 #include "ftk_device.cuh"
 #include "ftk_sampling.h"
+#ifdef FTK_TEST_HOOKS
+#include "ftk_test_hooks.h"
+#endif
 #include "ftk_words.cuh"
 
 namespace ftk {
 
-// src/fastertransformer/kernels/ban_bad_words.cu:22-86. grid (ceil(L/block), rows); one thread per
-// word slot.
+// src/fastertransformer/kernels/ban_bad_words.cu:22-86. grid (ceil(L/block), rows); one thread per word slot.
+// `id_offset`: the window's first row in the batch (the column of row r's history is id_offset + r).
 template<int DT>
 __global__ void ban_bad_words_kernel(typename Storage<DT>::T* __restrict__ logits, const int* __restrict__ output_ids,
-                                     const int* __restrict__ parent_ids, int batch_size, int beam_width,
-                                     const int* __restrict__ bad_words, int bad_words_len, bool share_words,
-                                     int id_offset, int vocab_size_padded, int step)
+                                     int batch_size, const int* __restrict__ bad_words, int bad_words_len,
+                                     bool share_words, int id_offset, int vocab_size_padded, int step)
 {
     typedef Storage<DT> S;
-    const int           id        = blockIdx.x * blockDim.x + threadIdx.x;
-    const int           batch_idx = blockIdx.y / beam_width;
-    const int           beam_idx  = blockIdx.y % beam_width;
-    if (id >= bad_words_len) {
+    const int           w   = blockIdx.x * blockDim.x + threadIdx.x;
+    const int           row = blockIdx.y;
+    if (w >= bad_words_len) {
         return;
     }
-    const int* base = share_words ? bad_words : bad_words + (size_t)batch_idx * 2 * bad_words_len;
-    const int  tok  = banned_token(base, bad_words_len, id, output_ids, parent_ids, batch_size, beam_width,
-                                   id_offset + batch_idx * beam_width, beam_idx, step);
-    if (0 < tok && tok < vocab_size_padded) {
-        logits[((size_t)batch_idx * beam_width + beam_idx) * vocab_size_padded + tok] = S::st(-__builtin_inff());
+    const WordList words = word_list(share_words ? bad_words : bad_words + (size_t)row * 2 * bad_words_len, bad_words_len);
+    const int      tok   = banned_token(words, w, output_ids + id_offset + row, (size_t)batch_size, step);
+    if (0 < tok && tok < vocab_size_padded) {  // token 0 is never banned, as in the reference
+        logits[(size_t)row * vocab_size_padded + tok] = S::st(-__builtin_inff());
     }
 }
 
 // src/fastertransformer/kernels/stop_criteria_kernels.cu:24-81
-__global__ void stop_words_kernel(const int* __restrict__ output_ids, const int* __restrict__ parent_ids,
-                                  const int* __restrict__ stop_words, bool* __restrict__ finished, int id_offset,
-                                  int stop_words_len, int batch_size, int beam_width, int step)
+__global__ void stop_words_kernel(const int* __restrict__ output_ids, const int* __restrict__ stop_words,
+                                  bool* __restrict__ finished, int id_offset, int stop_words_len, int batch_size,
+                                  int step)
 {
-    const int id        = blockIdx.x * blockDim.x + threadIdx.x;
-    const int batch_idx = blockIdx.y / beam_width;
-    const int beam_idx  = blockIdx.y % beam_width;
-    if (id >= stop_words_len) {
+    const int w   = blockIdx.x * blockDim.x + threadIdx.x;
+    const int row = blockIdx.y;
+    if (w >= stop_words_len) {
         return;
     }
-    const int* base = stop_words + (size_t)batch_idx * 2 * stop_words_len;
-    if (stop_word_matches(base, stop_words_len, id, output_ids, parent_ids, batch_size, beam_width,
-                          id_offset + batch_idx * beam_width, beam_idx, step)) {
-        finished[batch_idx * beam_width + beam_idx] = true;
+    const WordList words = word_list(stop_words + (size_t)row * 2 * stop_words_len, stop_words_len);
+    if (stop_word_matches(words, w, output_ids + id_offset + row, (size_t)batch_size, step)) {
+        finished[row] = true;
     }
 }
 
@@ -79,6 +77,7 @@ __global__ void rng_init_kernel(RngState* states, int n, unsigned long long seed
     }
 }
 
+#ifdef FTK_TEST_HOOKS
 __global__ void test_math_kernel(int kind, const float* __restrict__ in, float* __restrict__ out, size_t n)
 {
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
@@ -106,6 +105,7 @@ __global__ void test_rng_kernel(RngState* states, float* out, int batch, int n_d
         }
     }
 }
+#endif  // FTK_TEST_HOOKS
 
 }  // namespace ftk
 
@@ -164,14 +164,15 @@ int ftk_invoke_ban_bad_words(int dtype, void* logits, const int* output_ids_buf,
     if (bad_words_len == 0 || local_batch_size <= 0) {
         return 0;
     }
-    if (beam_width > 1 && parent_ids_buf == nullptr) {
-        return FTK_ERR_ARGUMENT;
+    (void)parent_ids_buf;
+    if (beam_width != 1) {
+        return FTK_ERR_ARGUMENT;  // sampling only: one hypothesis per row
     }
     const int block = (int)min((size_t)256, ((bad_words_len + 63) / 64) * 64);
-    dim3      grid((unsigned)((bad_words_len + block - 1) / block), (unsigned)(local_batch_size * beam_width));
+    dim3      grid((unsigned)((bad_words_len + block - 1) / block), (unsigned)local_batch_size);
     FTK_DISPATCH_DTYPE(dtype, ban_bad_words_kernel<DT><<<grid, block, 0, (hipStream_t)stream>>>(
-                                  (Storage<DT>::T*)logits, output_ids_buf, parent_ids_buf, batch_size, beam_width,
-                                  bad_words, (int)bad_words_len, share_words, id_offset, vocab_size_padded, (int)step));
+                                  (Storage<DT>::T*)logits, output_ids_buf, batch_size, bad_words, (int)bad_words_len,
+                                  share_words, id_offset, vocab_size_padded, (int)step));
     FTK_LAUNCH_CHECK();
     return 0;
 }
@@ -183,14 +184,14 @@ int ftk_invoke_stop_words_criterion_rows(const int* output_ids, const int* paren
     if (stop_words_len == 0 || num_rows <= 0) {
         return 0;
     }
-    if (beam_width > 1 && parent_ids == nullptr) {
-        return FTK_ERR_ARGUMENT;
+    (void)parent_ids;
+    if (beam_width != 1) {
+        return FTK_ERR_ARGUMENT;  // sampling only: one hypothesis per row
     }
     const int block = (int)min((size_t)256, ((stop_words_len + 63) / 64) * 64);
-    dim3      grid((unsigned)((stop_words_len + block - 1) / block), (unsigned)(num_rows * beam_width));
-    stop_words_kernel<<<grid, block, 0, (hipStream_t)stream>>>(output_ids, parent_ids, stop_words, finished,
-                                                               (int)id_offset, (int)stop_words_len, batch_size,
-                                                               beam_width, step);
+    dim3      grid((unsigned)((stop_words_len + block - 1) / block), (unsigned)num_rows);
+    stop_words_kernel<<<grid, block, 0, (hipStream_t)stream>>>(output_ids, stop_words, finished, (int)id_offset,
+                                                               (int)stop_words_len, batch_size, step);
     FTK_LAUNCH_CHECK();
     return 0;
 }
@@ -238,6 +239,8 @@ int ftk_invoke_length_criterion(bool* finished, bool* should_stop, int* h_pinned
     return 0;
 }
 
+#ifdef FTK_TEST_HOOKS
+// ---- test hooks (declared in include/ftk_test_hooks.h; only the hooks build of the library has them)
 float ftk_host_expf(float x)
 {
     return det_expf(x);
@@ -274,5 +277,6 @@ int ftk_test_rng_uniform(ftk_rng_state* states, float* out, int batch_size, int 
     FTK_LAUNCH_CHECK();
     return 0;
 }
+#endif  // FTK_TEST_HOOKS
 
 }  // extern "C"

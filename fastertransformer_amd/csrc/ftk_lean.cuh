@@ -14,7 +14,7 @@
 //     evaluated exactly, by the wave that parked them, when its parking list fills up;
 //   - the bound is the k-th largest of 256 values of distinct elements - first the thread maxima over the
 //     first two sub-tiles, later the largest candidate each lane has evaluated - found by every wave on its
-//     own with 24 rounds of ballots (one workgroup barrier per bound, no sort);
+//     own with 16 rounds of ballots (one workgroup barrier per bound, no sort);
 //   - candidates go straight to the workgroup's list in the workspace.
 // A workgroup that cannot keep its list inside the workspace slot says so in the header; the merging kernel
 // then walks that row again with the general stream.
@@ -62,8 +62,10 @@ inline LeanPlan lean_plan(int vocab, int rows, int elem_bytes, int fill)
     return p;
 }
 
-// The largest value P, to within its low eight bits, such that at least k of the 256 keys are >= P
-// (0 when fewer than k keys are non-zero). Every wave calls it on the same keys and gets the same answer.
+// The largest value P, to within its low sixteen bits, such that at least k of the 256 keys are >= P
+// (0 when fewer than k keys are non-zero): sign, exponent and seven bits of mantissa decide, which admits a
+// few per cent more candidates than the exact k-th largest would. Every wave calls it on the same keys and
+// gets the same answer.
 __device__ __forceinline__ uint32_t lean_kth_of_slots(const uint32_t* keys, int k)
 {
     uint32_t kk[LG_WAVES];
@@ -73,7 +75,7 @@ __device__ __forceinline__ uint32_t lean_kth_of_slots(const uint32_t* keys, int 
     }
     uint32_t P = 0u;
 #pragma unroll
-    for (int bit = 31; bit >= 8; --bit) {
+    for (int bit = 31; bit >= 16; --bit) {
         const uint32_t cand = P | (1u << bit);
         int            c    = 0;
 #pragma unroll
@@ -133,7 +135,7 @@ __device__ __forceinline__ uint4 lean_stream_load(const uint4* p)
 
 constexpr int LG_HIST_U = 8;  // history ids a thread requests before the logits (2048 positions per workgroup)
 
-template<int DT, int BMW, int OCC, int R, int EXP = 0>
+template<int DT, int BMW, int OCC, int R>
 __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParams p, FusedLaunch l)
 {
     typedef Storage<DT>   S;
@@ -160,7 +162,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 
     // The token history comes first (it is time-major: every id is a cache line of its own), so that the
     // bitmap of penalised columns is built while the logits are still on their way.
-    const bool hist = !(EXP & 1) && BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
+    const bool hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
     int        hist_ids[LG_HIST_U];
     if (hist) {
 #pragma unroll
@@ -275,11 +277,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     // ---- first bound: the k-th largest of the thread maxima over the first two sub-tiles. Only vectors whose
     // elements all take the plain transform count (no history column, not the masked end id), so every
     // maximum is the final value of an element.
-    if (EXP & 2) {
-        set_threshold(order_key((EXP & 32) ? 10.0f : 7.4f));
-        valid = true;
-    }
-    else if (nsub > 0) {
+    if (nsub > 0) {
         float tmax = NEG_INF;
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
@@ -328,7 +326,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-        const int staged = (EXP & 16) ? 0 : wcount;
+        const int staged = wcount;
         for (int e0 = 0; e0 < staged; e0 += WAVE) {
             const int  e    = e0 + ((lane - rot) & (WAVE - 1));
             const bool have = e < staged;
@@ -430,7 +428,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 if (q + R < nsub) {
                     load(r, q + R);
                 }
-                const bool tighten = !(EXP & 8) && q + 1 == next_tighten && q + 1 < nsub;
+                const bool tighten = q + 1 == next_tighten && q + 1 < nsub;
                 if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
                     drain();
                 }
@@ -545,7 +543,6 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
     if (overflow) {
         return -1;
     }
-    FTK_STAMP(1);
     // what was requested up front: one slot reservation per wave
     unsigned long long keepm[LS_PF_LISTS][LS_PF_ROUNDS];
     int                wave_total = 0;
@@ -609,7 +606,6 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
     __syncthreads();
     int n = s.n_cand;
     __syncthreads();
-    FTK_STAMP(2);
     (void)total;
     if (n > TK_CCAP) {
         return -2;  // the union does not fit the list: the caller merges with the general routine
@@ -633,7 +629,6 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
             T0 = P;
             n  = topk_prune(s, n, P);
         }
-        FTK_STAMP(4);
     }
     *thr_out = T0;
     return n;
@@ -663,7 +658,6 @@ __global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, 
         }
         return;
     }
-    FTK_STAMP(0);
     const TopkChunkHeader* headers = l.headers + (size_t)row * l.splits;
     TopkChunkHeader        my_header{};
     if ((int)threadIdx.x < l.splits) {
@@ -690,13 +684,12 @@ __global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, 
     }
     topk_select_lds<DT, FusedRow<DT, BMW>, true>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u,
                                                  p.end_ids, out);
-    FTK_STAMP(8);
 }
 
 // Launchers, one translation unit per element type (lean_kernels.hip built with FTK_LEAN_DT = 0, 1, 2).
-// window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large; variant: see lean_occupancy.
+// window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large.
 // start / stop: optional events carried by the launch.
-int lean_gather_launch_f32(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_f32(int window, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 int lean_select_launch_f32(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                            hipEvent_t stop);
@@ -704,16 +697,13 @@ int lean_select_launch_f16(int rows, hipStream_t st, const FusedParams& p, const
                            hipEvent_t stop);
 int lean_select_launch_bf16(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                             hipEvent_t stop);
-int lean_gather_launch_f16(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_f16(int window, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
-int lean_gather_launch_bf16(int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_bf16(int window, dim3 grid, hipStream_t st, const FusedParams& p,
                             const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 
-// workgroups per compute unit a variant of the lean gather is built for
-inline int lean_occupancy(int variant)
-{
-    (void)variant;
-    return 4;
-}
+// workgroups per compute unit the lean gather is built for, and sub-tiles in flight per thread
+constexpr int LG_OCCUPANCY = 4;
+constexpr int LG_RING      = 2;
 
 }  // namespace ftk

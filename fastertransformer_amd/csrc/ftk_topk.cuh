@@ -26,10 +26,6 @@
 #include "ftk_device.cuh"
 #include "ftk_transform.cuh"
 
-#ifndef FTK_STAMP
-#define FTK_STAMP(i)
-#endif
-
 namespace ftk {
 
 #ifndef FTK_TK_THREADS
@@ -1081,7 +1077,7 @@ __device__ __forceinline__ TopkOutputs topk_outputs(int* ids, int* sequence_leng
 }
 
 // thread 0 only: weights w[0..n) in selection order -> sampled position (sampling_topk_kernels.cu:282-311).
-// `w` is 16-byte aligned LDS, zero padded to a multiple of 4 (adding +0 to a non-negative sum is exact).
+// `w` is 16-byte aligned LDS, zero padded to a multiple of 32 (adding +0 to a non-negative sum is exact).
 // Both passes are strictly sequential in fp32, as in the reference; 32 weights are fetched at a time so that
 // the chain of additions never waits for LDS.
 __device__ __forceinline__ int topk_sample_walk(const float* w, int n, float u, float p, float* s_sum_out)
@@ -1093,7 +1089,7 @@ __device__ __forceinline__ int topk_sample_walk(const float* w, int n, float u, 
         float4 v[8];
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            v[b] = i0 + b < n4 ? w4[i0 + b] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            v[b] = w4[i0 + b];
         }
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
@@ -1103,31 +1099,30 @@ __device__ __forceinline__ int topk_sample_walk(const float* w, int n, float u, 
             s_sum = s_sum + v[b].w;
         }
     }
-    // the running difference never recovers once it is <= 0 (the weights are non-negative), so the first
-    // position where it is <= 0 is found without branching: keep subtracting, remember the first hit
+    // The running difference never rises again (the weights are non-negative), so the first position where it
+    // is <= 0 is the number of positions where it is still > 0 (or not a number, as in the reference, whose
+    // `<= 0` test a NaN never passes): counted without branches, the subtractions are the only dependent chain.
     float rand_num = u * p * s_sum;
-    int   pick     = n - 1;
-    bool  found    = false;
-    for (int i0 = 0; i0 < n4 && !found; i0 += 8) {
+    int   ahead    = 0;
+    for (int i0 = 0; i0 < n4; i0 += 8) {
         float4 v[8];
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            v[b] = i0 + b < n4 ? w4[i0 + b] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            v[b] = w4[i0 + b];
         }
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            const float x[4] = {v[b].x, v[b].y, v[b].z, v[b].w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int i = (i0 + b) * 4 + j;
-                rand_num    = found ? rand_num : rand_num - x[j];
-                if (!found && i < n && rand_num <= 0.0f) {
-                    pick  = i;
-                    found = true;
-                }
-            }
+            rand_num = rand_num - v[b].x;
+            ahead += rand_num <= 0.0f ? 0 : 1;
+            rand_num = rand_num - v[b].y;
+            ahead += rand_num <= 0.0f ? 0 : 1;
+            rand_num = rand_num - v[b].z;
+            ahead += rand_num <= 0.0f ? 0 : 1;
+            rand_num = rand_num - v[b].w;
+            ahead += rand_num <= 0.0f ? 0 : 1;
         }
     }
+    const int pick = ahead < n - 1 ? ahead : n - 1;
     *s_sum_out = s_sum;
     return pick;
 }
@@ -1263,119 +1258,171 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
         if (n > TK_THREADS && n > k) {
             n = topk_tighten<DEEP>(s, n, k, &thr);
         }
-        FTK_STAMP(5);
-        // candidates -> stage-1 composite keys, in place
-        //   slice(3) | ~key(32) | BS1-1-t (8) | j (21),   i = (j*8 + slice)*BS1 + t
-        constexpr int PER = TK_CCAP / TK_THREADS;
-        uint32_t      ck[PER], ci[PER];
-#pragma unroll
-        for (int r = 0; r < PER; ++r) {
-            const int i = t + r * TK_THREADS;
-            ck[r]       = i < n ? s.cand.key[i] : 0u;
-            ci[r]       = i < n ? s.cand.idx[i] : 0u;
-        }
-        if (t < 8) {
-            s.slice_count[t] = 0;
-        }
-        lds_barrier();
-#pragma unroll
-        for (int r = 0; r < PER; ++r) {
-            const int i = t + r * TK_THREADS;
-            if (i < n) {
-                const int blk   = (int)(ci[r] >> bs1_log);
-                const int tt    = (int)(ci[r] & (uint32_t)(BS1 - 1));
-                const int slice = blk & 7;
-                atomicAdd(&s.slice_count[slice], 1);
-                s.keys[i] = ((unsigned long long)slice << 61) | ((unsigned long long)(~ck[r]) << 29)
-                            | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
-            }
-        }
-        lds_barrier();
-        int slice_start[8];
-        {
-            int acc = 0;
-#pragma unroll
-            for (int sl = 0; sl < 8; ++sl) {
-                slice_start[sl] = acc;
-                acc += s.slice_count[sl];
-            }
-        }
-        // decode a stage-1 composite at sorted position q into (vocabulary index, stage-2 composite)
-        //   stage 2: ~key(32) | BS2-1-pos%BS2 (8) | pos/BS2 (12) | payload (12),  pos = slice*k + rank
-        auto stage2_key = [&](unsigned long long c, int q, int payload, int* idx_out) -> unsigned long long {
-            const int      slice = (int)(c >> 61);
-            const uint32_t ikey  = (uint32_t)(c >> 29);
-            const int      tt    = BS1 - 1 - (int)((c >> 21) & 0xFFull);
-            const int      j     = (int)(c & 0x1FFFFFull);
-            int            start = 0;
-#pragma unroll
-            for (int sl = 0; sl < 8; ++sl) {
-                start = sl == slice ? slice_start[sl] : start;
-            }
-            const int r = q - start;
-            *idx_out    = (j * 8 + slice) * BS1 + tt;
-            if (r >= k) {
-                return ~0ull;
-            }
-            const int pos = slice * k + r;
-            return ((unsigned long long)ikey << 32) | ((unsigned long long)(BS2 - 1 - pos % BS2) << 24)
-                   | ((unsigned long long)(pos / BS2) << 12) | (unsigned long long)payload;
-        };
-
         if (n <= TK_THREADS) {
-            // ---- small candidate sets (the usual case): rank by counting, one candidate per thread.
-            // Composite keys are unique, so "number of smaller keys" is the sorted position.
-            // (keys are read two at a time; an odd list is padded with a key that never counts)
-            const unsigned long long mine = t < n ? s.keys[t] : ~0ull;
-            // sixteen keys per round; DEEP: all eight loads in flight before the first compare
-            const int n16 = (n + 15) & ~15;
-            auto      rank = [&](unsigned long long key) -> int {
-                int q = 0;
-                if constexpr (DEEP) {
-                    for (int j0 = 0; j0 < n16; j0 += 16) {
-                        ulonglong2 kk[8];
-#pragma unroll
-                        for (int b = 0; b < 8; ++b) {
-                            kk[b] = *reinterpret_cast<const ulonglong2*>(&s.keys[j0 + 2 * b]);
-                        }
-#pragma unroll
-                        for (int b = 0; b < 8; ++b) {
-                            q += kk[b].x < key ? 1 : 0;
-                            q += kk[b].y < key ? 1 : 0;
-                        }
-                    }
-                }
-                else {
-#pragma unroll 4
-                    for (int j = 0; j < n16; j += 2) {
-                        const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&s.keys[j]);
-                        q += kk.x < key ? 1 : 0;
-                        q += kk.y < key ? 1 : 0;
-                    }
-                }
-                return q;
-            };
-            if (t >= n && t < n16) {
-                s.keys[t] = ~0ull;  // padding that never counts
+            // ---- small candidate sets (the usual case): both tie orders by counting, no sort.
+            //   stage 1: slice(3) | ~key(32) | BS1-1-t (8) | j (21),   i = (j*8 + slice)*BS1 + t
+            //   stage 2: ~key(32) | BS2-1-pos%BS2 (8) | pos/BS2 (12) | 0,   pos = slice*k + rank in slice
+            // Composite keys are unique, so "number of smaller keys" is the sorted position, and the rank inside
+            // a slice is that minus the number of keys of lower slices. The all-pairs counting is spread over
+            // all threads: with CP = n rounded up to a power of two, thread t counts for candidate t % CP over
+            // part t / CP of the list, and the partial counts meet in LDS.
+            const uint32_t my_key = t < n ? s.cand.key[t] : 0u;
+            const uint32_t my_idx = t < n ? s.cand.idx[t] : 0u;
+            unsigned long long* A   = s.keys;                        // stage-1 keys  [0, 256)
+            unsigned long long* B   = s.keys + TK_THREADS;           // stage-2 keys  [256, 512)
+            int*                cnt = reinterpret_cast<int*>(s.keys + 2 * TK_THREADS);  // 3 x 256 partial counts
+            const int           n2  = (n + 1) & ~1;
+            int                 CP  = 2;
+            while (CP < n) {
+                CP <<= 1;
+            }
+            const int parts = TK_THREADS / CP;  // CP <= 256
+            const int c     = t & (CP - 1);
+            const int part  = t / CP;
+            // pairs of list entries [jlo, jhi) belong to this thread's part
+            const int pairs = n2 >> 1;
+            const int per   = (pairs + parts - 1) / parts;
+            const int jlo   = min(pairs, part * per) * 2;
+            const int jhi   = min(pairs, part * per + per) * 2;
+            lds_barrier();  // every candidate is in registers: the list's memory can be reused
+            unsigned long long mine = ~0ull;
+            if (t < n) {
+                const int blk   = (int)(my_idx >> bs1_log);
+                const int tt    = (int)(my_idx & (uint32_t)(BS1 - 1));
+                const int slice = blk & 7;
+                mine = ((unsigned long long)slice << 61) | ((unsigned long long)(~my_key) << 29)
+                       | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
+            }
+            if (t < n2) {
+                A[t] = mine;  // (an odd list is padded with a key that never counts)
+            }
+            cnt[t]                  = 0;
+            cnt[TK_THREADS + t]     = 0;
+            cnt[2 * TK_THREADS + t] = 0;
+            if (t == 0) {
+                s.misc[1] = 0;
             }
             lds_barrier();
-            const int                q      = rank(mine);
-            int                      my_idx = 0;
-            const unsigned long long k2     = t < n ? stage2_key(mine, q, 0, &my_idx) : ~0ull;
+            {
+                const unsigned long long key  = c < n ? A[c] : ~0ull;
+                const unsigned long long base = key & (7ull << 61);  // below it: the keys of lower slices
+                int                      q = 0, qs = 0;
+#pragma unroll 4
+                for (int j = jlo; j < jhi; j += 2) {
+                    const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&A[j]);
+                    q += kk.x < key ? 1 : 0;
+                    q += kk.y < key ? 1 : 0;
+                    qs += kk.x < base ? 1 : 0;
+                    qs += kk.y < base ? 1 : 0;
+                }
+                if (c < n && jhi > jlo) {
+                    atomicAdd(&cnt[c], q);
+                    atomicAdd(&cnt[TK_THREADS + c], qs);
+                }
+            }
             lds_barrier();
-            s.keys[t] = k2;
+            unsigned long long k2 = ~0ull;
+            if (t < n) {
+                const int slice = (int)(mine >> 61);
+                const int r     = cnt[t] - cnt[TK_THREADS + t];  // rank inside the slice
+                if (r < k) {
+                    const int pos = slice * k + r;
+                    k2 = ((unsigned long long)(uint32_t)(mine >> 29) << 32)
+                         | ((unsigned long long)(BS2 - 1 - pos % BS2) << 24) | ((unsigned long long)(pos / BS2) << 12);
+                }
+            }
+            if (t < n2) {
+                B[t] = k2;
+            }
             lds_barrier();
-            const int q2 = rank(k2);
-            const bool kept = k2 != ~0ull;
-            n_list          = block_sum_i<TK_WAVES>(kept ? 1 : 0, (int*)s.red32);
-            n_list          = n_list < k ? n_list : k;
-            if (kept && q2 < n_list) {
-                s.sel.w[q2]   = key_to_float(~(uint32_t)(k2 >> 32));
-                s.sel.idx[q2] = my_idx;
+            {
+                const unsigned long long key = c < n ? B[c] : ~0ull;
+                int                      q = 0, kept = 0;
+#pragma unroll 4
+                for (int j = jlo; j < jhi; j += 2) {
+                    const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&B[j]);
+                    q += kk.x < key ? 1 : 0;
+                    q += kk.y < key ? 1 : 0;
+                    kept += kk.x != ~0ull ? 1 : 0;
+                    kept += kk.y != ~0ull ? 1 : 0;
+                }
+                if (c < n && jhi > jlo) {
+                    atomicAdd(&cnt[2 * TK_THREADS + c], q);
+                }
+                if (c == 0 && jhi > jlo) {
+                    atomicAdd(&s.misc[1], kept);  // entries that stage 1 kept, over all parts
+                }
+            }
+            lds_barrier();
+            n_list = min(k, s.misc[1]);
+            if (t < n && k2 != ~0ull) {
+                const int q2 = cnt[2 * TK_THREADS + t];
+                if (q2 < n_list) {
+                    s.sel.w[q2]   = key_to_float(~(uint32_t)(k2 >> 32));
+                    s.sel.idx[q2] = (int)my_idx;
+                }
             }
             __syncthreads();
         }
         else {
+            // candidates -> stage-1 composite keys, in place
+            //   slice(3) | ~key(32) | BS1-1-t (8) | j (21),   i = (j*8 + slice)*BS1 + t
+            constexpr int PER = TK_CCAP / TK_THREADS;
+            uint32_t      ck[PER], ci[PER];
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                const int i = t + r * TK_THREADS;
+                ck[r]       = i < n ? s.cand.key[i] : 0u;
+                ci[r]       = i < n ? s.cand.idx[i] : 0u;
+            }
+            if (t < 8) {
+                s.slice_count[t] = 0;
+            }
+            lds_barrier();
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                const int i = t + r * TK_THREADS;
+                if (i < n) {
+                    const int blk   = (int)(ci[r] >> bs1_log);
+                    const int tt    = (int)(ci[r] & (uint32_t)(BS1 - 1));
+                    const int slice = blk & 7;
+                    atomicAdd(&s.slice_count[slice], 1);
+                    s.keys[i] = ((unsigned long long)slice << 61) | ((unsigned long long)(~ck[r]) << 29)
+                                | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
+                }
+            }
+            lds_barrier();
+            int slice_start[8];
+            {
+                int acc = 0;
+#pragma unroll
+                for (int sl = 0; sl < 8; ++sl) {
+                    slice_start[sl] = acc;
+                    acc += s.slice_count[sl];
+                }
+            }
+            // decode a stage-1 composite at sorted position q into (vocabulary index, stage-2 composite)
+            //   stage 2: ~key(32) | BS2-1-pos%BS2 (8) | pos/BS2 (12) | payload (12),  pos = slice*k + rank
+            auto stage2_key = [&](unsigned long long c, int q, int payload, int* idx_out) -> unsigned long long {
+                const int      slice = (int)(c >> 61);
+                const uint32_t ikey  = (uint32_t)(c >> 29);
+                const int      tt    = BS1 - 1 - (int)((c >> 21) & 0xFFull);
+                const int      j     = (int)(c & 0x1FFFFFull);
+                int            start = 0;
+#pragma unroll
+                for (int sl = 0; sl < 8; ++sl) {
+                    start = sl == slice ? slice_start[sl] : start;
+                }
+                const int r = q - start;
+                *idx_out    = (j * 8 + slice) * BS1 + tt;
+                if (r >= k) {
+                    return ~0ull;
+                }
+                const int pos = slice * k + r;
+                return ((unsigned long long)ikey << 32) | ((unsigned long long)(BS2 - 1 - pos % BS2) << 24)
+                       | ((unsigned long long)(pos / BS2) << 12) | (unsigned long long)payload;
+            };
+
             // ---- large candidate sets: two bitonic sorts (of exactly n keys: no padding to a power of two)
             block_sort_u64<TK_THREADS>(s.keys, n);
             for (int qi = t; qi < n; qi += TK_THREADS) {
@@ -1423,17 +1470,15 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
         __syncthreads();
     }
 
-    FTK_STAMP(6);
     // ---- weights (sampling_topk_kernels.cu:264-279): exp(x - max) on logits, the value itself on
-    // probabilities; the list is padded with zero weights to a multiple of 4 for the vectorised walk
+    // probabilities; the list is padded with zero weights to a multiple of 32 for the walk, which reads 32 at a time
     const float x0 = n_list > 0 ? s.sel.w[0] : 0.0f;
     __syncthreads();
-    for (int i = t; i < ((n_list + 3) & ~3); i += TK_THREADS) {
+    for (int i = t; i < ((n_list + 31) & ~31); i += TK_THREADS) {
         const float x = i < n_list ? s.sel.w[i] : 0.0f;
         s.sel.w[i]        = i < n_list ? (probs_in ? x : det_expf(x - x0)) : 0.0f;
     }
     __syncthreads();
-    FTK_STAMP(7);
     if (t == 0) {
         if (n_list == 0) {
             topk_emit(out, row, 0, probs_in, 0.0f, 0.0f, end_ids, false);
@@ -1490,7 +1535,6 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
             T0 = h.threshold;
         }
     }
-    FTK_STAMP(1);
     if (overflow) {
         return -1;
     }
@@ -1545,7 +1589,6 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
         return total;
     };
     int n = gather(T0);
-    FTK_STAMP(2);
     if (n > TK_CCAP) {
         // large k over many chunks: find the exact k-th largest key by bisection over the lists
         auto count_ge = [&](uint32_t thr) -> int {
@@ -1579,7 +1622,6 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
         // Cut the union to its k largest keys (and their ties) before the tie orders are replayed: the replay
         // ranks every candidate against every other one with 64-bit keys, twice.
         n = topk_cut_to_k(s, n, k);
-        FTK_STAMP(4);
     }
     *thr_out = T0;
     return n;

@@ -1,80 +1,75 @@
-// n-gram matching against the time-major token history, shared by the stand-alone bad-word /
-// stop-word kernels and the fused decode kernels.
+// Word lists (bad words, stop words) matched against the time-major token history.
 //
-// Word-list layout (examples/pytorch/gpt/utils/word_list.py:36-67): `words` points at [2, L] ints;
-// row 0 holds all n-grams' token ids back to back (0-padded), row 1 the inclusive end offset of
-// each n-gram (-1-padded). Word i spans ids [off[i-1] (or 0), off[i]).
+// Layout (examples/pytorch/gpt/utils/word_list.py:36-67): a list is [2, L] ints; row 0 holds the token ids of
+// all n-grams back to back (0-padded), row 1 the inclusive end offset of each n-gram (-1-padded): n-gram w
+// spans ids [end[w-1] (or 0), end[w]). The history of a row is a column of output_ids [max_seq, batch].
+// Sampling only: one hypothesis per row, so there is no parent-id chain to follow.
 #pragma once
 #include "ftk_device.cuh"
 
 namespace ftk {
 
-// src/fastertransformer/kernels/ban_bad_words.cu:35-85. Returns the token id to ban, or -1.
-// `row_index` = id_offset + batch_idx * beam_width (column of the history matrix for beam 0).
-__device__ __forceinline__ int banned_token(const int* __restrict__ words, int words_len, int word,
-                                            const int* __restrict__ output_ids, const int* __restrict__ parent_ids,
-                                            int batch_size, int beam_width, int row_index, int beam_idx, int step)
-{
-    const int* offsets = words + words_len;
-    if (offsets[word] < 0) {
-        return -1;
-    }
-    const int item_end   = offsets[word];
-    const int item_start = word > 0 ? offsets[word - 1] : 0;
-    const int item_size  = item_end - item_start;
-    bool      ban        = item_size == 1;
-    if (item_size > 1 && step >= item_size - 1) {
-        ban            = true;
-        int parent_id  = beam_idx;
-        for (int t = item_size - 2; t >= 0; --t) {
-            const size_t pos = (size_t)(step - (item_size - 1) + t) * batch_size * beam_width + row_index + parent_id;
-            if (output_ids[pos] != words[item_start + t]) {
-                ban = false;
-                break;
-            }
-            if (beam_width > 1) {
-                parent_id = parent_ids[pos];
-                if (parent_id < 0 || parent_id >= beam_width) {
-                    ban = false;
-                    break;
-                }
-            }
-        }
-    }
-    return ban ? words[item_end - 1] : -1;
-}
-
-// src/fastertransformer/kernels/stop_criteria_kernels.cu:34-80: the token written at `step` is the
-// last token of the n-gram and is compared first.
-__device__ __forceinline__ bool stop_word_matches(const int* __restrict__ words, int words_len, int word,
-                                                  const int* __restrict__ output_ids,
-                                                  const int* __restrict__ parent_ids, int batch_size, int beam_width,
-                                                  int row_index, int beam_idx, int step)
-{
-    const int* offsets = words + words_len;
-    if (offsets[word] < 0) {
-        return false;
-    }
-    const int item_end   = offsets[word];
-    const int item_start = word > 0 ? offsets[word - 1] : 0;
-    const int item_size  = item_end - item_start;
-    if (step + 1 < item_size) {
-        return false;
-    }
-    int parent_id = beam_idx;
-    for (int t = item_size - 1; t >= 0; --t) {
-        const size_t pos = (size_t)(step - (item_size - 1) + t) * batch_size * beam_width + row_index + parent_id;
-        if (output_ids[pos] != words[item_start + t]) {
+struct WordList {
+    const int* ids;   // row 0
+    const int* ends;  // row 1
+    // n-gram `w`: first id and length; false for an unused slot
+    __device__ __forceinline__ bool ngram(int w, const int** first, int* count) const
+    {
+        const int end = ends[w];
+        if (end < 0) {
             return false;
         }
-        if (beam_width > 1) {
-            parent_id = parent_ids[pos];
-            if (parent_id < 0 || parent_id >= beam_width) {
-                return false;
-            }
+        const int begin = w > 0 ? ends[w - 1] : 0;
+        *first          = ids + begin;
+        *count          = end - begin;
+        return true;
+    }
+};
+
+__device__ __forceinline__ WordList word_list(const int* base, int len)
+{
+    return WordList{base, base + len};
+}
+
+// Do the `count` tokens written at times last-count+1 .. last of history column `column` (element (t, row) at
+// column[t * stride]) equal tokens[0 .. count)? Compared from the most recent token backwards, as both
+// reference kernels do; an n-gram longer than the history does not match.
+__device__ __forceinline__ bool history_ends_with(const int* __restrict__ tokens, int count,
+                                                  const int* __restrict__ column, size_t stride, int last)
+{
+    if (count > last + 1) {
+        return false;
+    }
+    for (int t = count - 1; t >= 0; --t) {
+        if (column[(size_t)(last - (count - 1) + t) * stride] != tokens[t]) {
+            return false;
         }
     }
     return true;
+}
+
+// src/fastertransformer/kernels/ban_bad_words.cu:35-85: the last token of an n-gram is banned when the
+// n-gram has one token, or when the history before `step` ends with its first n-1 tokens. Returns that token
+// or -1.
+__device__ __forceinline__ int banned_token(const WordList& words, int w, const int* __restrict__ column,
+                                            size_t stride, int step)
+{
+    const int* first;
+    int        count;
+    if (!words.ngram(w, &first, &count) || count < 1) {
+        return -1;
+    }
+    return history_ends_with(first, count - 1, column, stride, step - 1) ? first[count - 1] : -1;
+}
+
+// src/fastertransformer/kernels/stop_criteria_kernels.cu:34-80: the history up to and including the token
+// written at `step` ends with the n-gram.
+__device__ __forceinline__ bool stop_word_matches(const WordList& words, int w, const int* __restrict__ column,
+                                                  size_t stride, int step)
+{
+    const int* first;
+    int        count;
+    return words.ngram(w, &first, &count) && history_ends_with(first, count, column, stride, step);
 }
 
 }  // namespace ftk

@@ -89,13 +89,11 @@ __global__ void __launch_bounds__(TK_THREADS) fused_select_kernel(FusedParams p,
         }
         return;
     }
-    FTK_STAMP(0);
     const float  u  = fused_row_draw(s, l, row);
     const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row, p.end_ids);
     uint32_t     thr         = 0u;
     const int    n = topk_merge_lists<DT>(s, k, l.splits, l.headers + (size_t)row * l.splits, row_entries, &thr, pf);
     topk_select_lds<DT, FusedRow<DT, BMW>, true>(r, s, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u, p.end_ids, out);
-    FTK_STAMP(8);
 }
 
 

@@ -14,11 +14,13 @@
 //                           bitmap over the vocabulary (who gets the repetition / presence penalty)
 #include <hip/hip_ext.h>
 
-#include <cstdlib>
 #include <mutex>
 #include <vector>
 
 #include "ftk_sampling.h"
+#ifdef FTK_TEST_HOOKS
+#include "ftk_test_hooks.h"
+#endif
 #include "ftk_fused.cuh"
 #include "ftk_lean.cuh"
 
@@ -148,17 +150,18 @@ extern "C" int ftk_profile_read(int kernel, double* total_ms, int* launches)
     return 0;
 }
 
-// Which build of the lean gather a launch takes: 0 switches it off (every launch takes the general stream),
-// 1 = four workgroups per compute unit with four sub-tiles in flight per thread, 2 = eight with two.
-// Read once from FTK_LEAN.
-static int lean_variant()
+#ifdef FTK_TEST_HOOKS
+// Test hook (hooks build of the library only): non-zero sends every launch through the general stream, so
+// that it can be compared with the lean gather on the shapes the lean gather normally takes.
+static int g_fused_force_general = 0;
+extern "C" void ftk_test_set_fused_force_general(int v)
 {
-    static const int v = []() {
-        const char* e = std::getenv("FTK_LEAN");
-        return e != nullptr ? std::atoi(e) : 1;
-    }();
-    return v;
+    g_fused_force_general = v;
 }
+#else
+static constexpr int g_fused_force_general = 0;
+#endif
+
 extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
 {
     if (a == nullptr) {
@@ -177,8 +180,8 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const int      bitmap_words = (a->vocab_size_padded + 31) / 32 + 1;  // +1: vector_bits may peek one word ahead
     const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
     // Launches with a small k and no bias take the lean gather, which cuts a row differently.
-    const int      lean_mode = many == 0 && a->embedding_bias == nullptr ? lean_variant() : 0;
-    const LeanPlan lplan     = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * lean_occupancy(lean_mode));
+    const int      lean_mode = many == 0 && a->embedding_bias == nullptr && !g_fused_force_general ? 1 : 0;
+    const LeanPlan lplan     = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * LG_OCCUPANCY);
     const size_t   lean_bytes =
         (size_t)(rows > 0 ? rows : 0) * lplan.splits * (sizeof(TopkChunkHeader) + (size_t)TK_CCAP * sizeof(TopkEntry));
     const size_t   need = bitmap_bytes + (lean_mode != 0 && lean_bytes > plan.bytes ? lean_bytes : plan.bytes);
@@ -297,13 +300,13 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         hipEvent_t e0, e1;
         take_events(1, &e0, &e1);
         if (a->dtype == FTK_DTYPE_F32) {
-            rc = lean_gather_launch_f32(window, lean_mode, lgrid, st, p, l, e0, e1);
+            rc = lean_gather_launch_f32(window, lgrid, st, p, l, e0, e1);
         }
         else if (a->dtype == FTK_DTYPE_F16) {
-            rc = lean_gather_launch_f16(window, lean_mode, lgrid, st, p, l, e0, e1);
+            rc = lean_gather_launch_f16(window, lgrid, st, p, l, e0, e1);
         }
         else {
-            rc = lean_gather_launch_bf16(window, lean_mode, lgrid, st, p, l, e0, e1);
+            rc = lean_gather_launch_bf16(window, lgrid, st, p, l, e0, e1);
         }
         if (rc != 0) {
             return rc;
@@ -325,6 +328,100 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         return rc;
     }
     return launch_general(FUSED_KIND_SELECT, 0, dim3(rows));
+}
+
+// ---- plain read of a buffer: the yardstick of the streaming kernels ------------------------------------
+// What the gather would cost if it did nothing but fetch: the same launch shape (256-thread workgroups, four
+// per compute unit, each walking a contiguous share in sub-tiles of four 16-byte vectors per thread with two
+// sub-tiles in flight, non-temporal loads), one maximum per vector, one float written per workgroup.
+namespace ftk {
+__global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY)
+read_yardstick_kernel(const uint4* __restrict__ data, size_t nvec, size_t vec_per_wg, float* __restrict__ sink)
+{
+    const int    t  = threadIdx.x;
+    const size_t vb = (size_t)blockIdx.x * vec_per_wg;
+    const size_t ve = vb + vec_per_wg < nvec ? vb + vec_per_wg : nvec;
+    if (vb >= ve) {
+        return;
+    }
+    const int nsub = (int)((ve - vb + LG_SUB_VECS - 1) / LG_SUB_VECS);
+    uint4     raw[LG_RING][LG_NV];
+    auto      load = [&](int slot, int q) {
+#pragma unroll
+        for (int j = 0; j < LG_NV; ++j) {
+            size_t vi = vb + (size_t)q * LG_SUB_VECS + j * LG_THREADS + t;
+            vi        = vi < ve ? vi : ve - 1;
+            raw[slot][j] = lean_stream_load(data + vi);
+        }
+    };
+#pragma unroll
+    for (int r = 0; r < LG_RING; ++r) {
+        if (r < nsub) {
+            load(r, r);
+        }
+    }
+    float m = -__builtin_inff();
+    for (int q0 = 0; q0 < nsub; q0 += LG_RING) {
+#pragma unroll
+        for (int r = 0; r < LG_RING; ++r) {
+            const int q = q0 + r;
+            if (q < nsub) {
+#pragma unroll
+                for (int j = 0; j < LG_NV; ++j) {
+                    m = __builtin_fmaxf(m, lean_raw_max<DT_F32>(raw[r][j]));
+                }
+                if (q + LG_RING < nsub) {
+                    load(r, q + LG_RING);
+                }
+            }
+        }
+    }
+    m = wave_max(m);
+    if (lane_id() == 0) {
+        sink[blockIdx.x * LG_WAVES + wave_id()] = m;
+    }
+}
+}  // namespace ftk
+
+extern "C" int ftk_measure_plain_read(const void* data, size_t bytes, float* sink, size_t sink_floats,
+                                      ftk_stream_t stream, float* elapsed_ms)
+{
+    const int    wgs  = 256 * LG_OCCUPANCY;
+    const size_t nvec = bytes / sizeof(uint4);
+    if (data == nullptr || sink == nullptr || nvec == 0 || ((uintptr_t)data & 15u) != 0
+        || sink_floats < (size_t)wgs * LG_WAVES) {
+        return FTK_ERR_ARGUMENT;
+    }
+    const size_t vec_per_wg = ((nvec + wgs - 1) / wgs + LG_THREADS - 1) / LG_THREADS * LG_THREADS;
+    hipStream_t  st         = (hipStream_t)stream;
+    if (elapsed_ms == nullptr) {
+        hipLaunchKernelGGL(read_yardstick_kernel, dim3(wgs), dim3(LG_THREADS), 0, st, (const uint4*)data, nvec,
+                           vec_per_wg, sink);
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
+    hipEvent_t e0, e1;
+    hipError_t e = hipEventCreate(&e0);
+    if (e != hipSuccess) {
+        return (int)e;
+    }
+    e = hipEventCreate(&e1);
+    if (e != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return (int)e;
+    }
+    hipExtLaunchKernelGGL(read_yardstick_kernel, dim3(wgs), dim3(LG_THREADS), 0, st, e0, e1, 0, (const uint4*)data,
+                          nvec, vec_per_wg, sink);
+    e = hipGetLastError();
+    if (e == hipSuccess) {
+        e = hipEventSynchronize(e1);
+    }
+    if (e == hipSuccess) {
+        e = hipEventElapsedTime(elapsed_ms, e0, e1);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return (int)e;
 }
 
 // ---- the fused step for callers that cannot allocate ------------------------------------------------

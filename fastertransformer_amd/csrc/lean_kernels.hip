@@ -42,13 +42,10 @@ int lean_gather_launch_f16
 #else
 int lean_gather_launch_bf16
 #endif
-    (int window, int variant, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+    (int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
      hipEvent_t stop)
 {
-    if (variant == 2) {
-        return lean_launch_window<4, 3>(window, grid, st, p, l, start, stop);
-    }
-    return lean_launch_window<4, 2>(window, grid, st, p, l, start, stop);
+    return lean_launch_window<LG_OCCUPANCY, LG_RING>(window, grid, st, p, l, start, stop);
 }
 
 #if FTK_LEAN_DT == 0

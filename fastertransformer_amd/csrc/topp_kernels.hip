@@ -10,6 +10,9 @@
 // The replacement orders only the part of a row in front of the draw (see the top-p section).
 #include "ftk_device.cuh"
 #include "ftk_sampling.h"
+#ifdef FTK_TEST_HOOKS
+#include "ftk_test_hooks.h"
+#endif
 #include "ftk_transform.cuh"
 
 namespace ftk {
@@ -1440,12 +1443,17 @@ int ftk_invoke_topp_initialize(int* topp_id_val_buf, int* topp_offset_buf, int* 
     return 0;
 }
 
-// Test hook: a non-zero value routes every row through the radix-sort fallback.
+#ifdef FTK_TEST_HOOKS
+// Test hook (hooks build of the library only): a non-zero value routes every row through the radix-sort
+// fallback, so that it can be exercised on small inputs.
 static int g_topp_force_deep = 0;
 void       ftk_test_set_topp_force_deep(int v)
 {
     g_topp_force_deep = v;
 }
+#else
+static constexpr int g_topp_force_deep = 0;
+#endif
 
 int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace_size, size_t* cub_temp_storage_size,
                                    int* output_ids, int* sequence_length, bool* finished, float* cum_log_probs,

@@ -49,22 +49,28 @@ _SIGNATURES = {
     "ftk_invoke_length_criterion": [_vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_fused_topk_step": [_vp, _vp],
     "ftk_fused_topk_step_static": [_vp, _vp],
+    "ftk_measure_plain_read": [_vp, _sz, _vp, _sz, _vp, _vp],
     "ftk_invoke_log_prob_from_logits": [_i, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _b],
     "ftk_invoke_decoding_initialize": [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_invoke_plus_scalar": [_vp, _i, _i, _vp],
     "ftk_invoke_transpose_axis01": [_vp, _vp, _vp, _i, _i, _vp],
+    "ftk_error_string": [_i],
+    "ftk_profile_enable": [_i],
+    "ftk_profile_read": [_i, _vp, _vp],
+}
+# include/ftk_test_hooks.h: only libftk_sampling_hooks.so (the test build) exports these
+_HOOK_SIGNATURES = {
     "ftk_host_expf": [_f],
     "ftk_host_logf": [_f],
     "ftk_test_device_math": [_i, _vp, _vp, _sz, _vp],
     "ftk_test_rng_uniform": [_vp, _vp, _i, _i, _vp],
     "ftk_test_set_topp_force_deep": [_i],
+    "ftk_test_set_fused_force_general": [_i],
     "ftk_host_philox4x32_10": [_vp, _vp, _vp],
-    "ftk_error_string": [_i],
-    "ftk_profile_enable": [_i],
-    "ftk_profile_read": [_i, _vp, _vp],
 }
 _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_char_p,
-             "ftk_test_set_topp_force_deep": None, "ftk_host_philox4x32_10": None}
+             "ftk_test_set_topp_force_deep": None, "ftk_test_set_fused_force_general": None,
+             "ftk_host_philox4x32_10": None}
 
 
 # error codes of include/ftk_sampling.h (positive values are hipError_t)
@@ -75,6 +81,11 @@ FUSED_STATIC_WORKSPACE_BYTES = 32 << 20
 def exported_symbols():
     """names every entry point include/ftk_sampling.h declares"""
     return sorted(_SIGNATURES)
+
+
+def hook_symbols():
+    """names every entry point include/ftk_test_hooks.h declares"""
+    return sorted(_HOOK_SIGNATURES)
 
 
 def ftk():
@@ -92,6 +103,27 @@ def ftk():
             fn.restype = _RESTYPES.get(name, _i)
         _ftk = lib
     return _ftk
+
+
+_hooks = None
+
+
+def ftk_hooks():
+    """libftk_sampling_hooks.so: the test build of the kernel library (every product entry point plus the hooks
+    of include/ftk_test_hooks.h). Its symbols stay local, so it does not get in the way of the product library."""
+    global _hooks
+    if _hooks is None:
+        path = os.path.join(lib_dir(), "libftk_sampling_hooks.so")
+        if not os.path.exists(path):
+            raise FtkError("%s is missing: run `python -m fastertransformer_amd.build`" % path)
+        lib = C.CDLL(path, mode=C.RTLD_LOCAL)
+        for table in (_SIGNATURES, _HOOK_SIGNATURES):
+            for name, argtypes in table.items():
+                fn = getattr(lib, name)
+                fn.argtypes = argtypes
+                fn.restype = _RESTYPES.get(name, _i)
+        _hooks = lib
+    return _hooks
 
 
 class FtTensor(C.Structure):
@@ -154,8 +186,7 @@ class FusedTopkArgs(C.Structure):
         ("dtype", _i), ("logits", _vp), ("embedding_bias", _vp), ("vocab_size", _i), ("vocab_size_padded", _i),
         ("batch_size", _i), ("local_batch_size", _i), ("step", _i), ("max_input_length", _i),
         ("temperatures", _vp), ("penalties", _vp), ("penalty_type", _i), ("min_lengths", _vp), ("end_ids", _vp),
-        ("input_lengths", _vp), ("output_ids", _vp), ("bad_words", _vp), ("bad_words_len", _i),
-        ("bad_words_shared", _i), ("id_offset", _i), ("top_ks", _vp), ("top_ps", _vp), ("max_top_k", _i),
+        ("input_lengths", _vp), ("output_ids", _vp), ("top_ks", _vp), ("top_ps", _vp), ("max_top_k", _i),
         ("skip_decode", _vp), ("rng_state", _vp), ("uniform_draws", _vp), ("ids", _vp), ("sequence_length", _vp),
         ("finished", _vp), ("workspace", _vp), ("workspace_size", _sz),
     ]

@@ -1,0 +1,5 @@
+// Header name of the reference (src/fastertransformer/kernels/ban_bad_words.h), kept so that a call site's
+// #include line resolves unchanged. The launchers it declares there (invokeBanBadWords)
+// are declared, for this engine, in sampling_kernels.h.
+#pragma once
+#include "src/fastertransformer/kernels/sampling_kernels.h"

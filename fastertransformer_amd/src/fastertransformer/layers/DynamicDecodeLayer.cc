@@ -82,118 +82,127 @@ void DynamicDecodeLayer<T>::forward(std::unordered_map<std::string, Tensor>*    
     forward(&output_map, &input_map);
 }
 
+namespace {
+
+// The rows [first, first + count) of a tensor whose leading dimension is the batch: a view, no copy.
+Tensor rowWindow(const Tensor& t, size_t first, size_t count)
+{
+    std::vector<size_t> shape = t.shape;
+    size_t              inner = 1;
+    for (size_t d = 1; d < shape.size(); ++d) {
+        inner *= shape[d];
+    }
+    shape[0] = count;
+    return t.slice(shape, first * inner);
+}
+
+// What the two sampling layers see of a step: tensors with one entry per row are cut to the micro-batch window,
+// the others are handed over as they are. (Key names: layers/DynamicDecodeLayer.cc:193-235 of the reference.)
+const char* const kRowInputs[]   = {"logits", "end_id", "input_lengths", "uniform_draws"};
+const char* const kWholeInputs[] = {"step", "max_input_length", "embedding_bias"};
+const char* const kRowOutputs[]  = {"sequence_length", "finished", "cum_log_probs"};
+
+}  // namespace
+
 // reference: DynamicDecodeLayer<T>::forward, layers/DynamicDecodeLayer.cc:191-474 (tensor names and
 // shapes are documented there, :193-235). Extension: input "uniform_draws" [batch] float on the GPU,
 // one draw in (0, 1] per row, replaces the generator for this step.
 template<typename T>
 void DynamicDecodeLayer<T>::forward(TensorMap* output_tensors, TensorMap* input_tensors)
 {
-    const int ite  = (int)input_tensors->at("ite").getVal<uint>();
-    const int step = input_tensors->at("step").getVal<int>();
-    FT_CHECK(input_tensors->at("logits").shape.size() == 3);
+    const Tensor& logits = input_tensors->at("logits");
+    FT_CHECK(logits.shape.size() == 3);
+    FT_CHECK_WITH_INFO(logits.shape[1] == 1, "this engine implements the sampling path only (beam_width must be 1)");
+    const int    ite   = (int)input_tensors->at("ite").getVal<uint>();
+    const int    step  = input_tensors->at("step").getVal<int>();
+    const size_t batch = logits.shape[0];
+    const size_t rows  = (size_t)input_tensors->at("local_batch_size").getVal<int>();
+    const size_t first = (size_t)ite * rows;  // the window: rows [first, first + rows) of the batch
+    FT_CHECK_WITH_INFO(first + rows <= batch, "ite / local_batch_size window exceeds the batch");
 
-    const size_t batch_size       = input_tensors->at("logits").shape[0];
-    const size_t beam_width       = input_tensors->at("logits").shape[1];
-    const size_t local_batch_size = (size_t)input_tensors->at("local_batch_size").getVal<int>();
-    FT_CHECK_WITH_INFO(beam_width == 1, "this engine implements the sampling path only (beam_width must be 1)");
-    FT_CHECK_WITH_INFO((ite + 1) * local_batch_size <= batch_size, "ite / local_batch_size window exceeds the batch");
-    const size_t local_batch_offset = ite * local_batch_size;
+    banBadWords(output_tensors, input_tensors, first, rows, step);
 
-    if (input_tensors->isExist("bad_words_list")) {
-        const auto& bad_words = input_tensors->at("bad_words_list");
-        FT_CHECK_WITH_INFO(bad_words.shape.size() == 2 || bad_words.shape.size() == 3,
-                           "Bad words dimension must be 2 or 3.");
-        const bool is_matrix = bad_words.shape.size() == 2;
-        if (!is_matrix) {
-            FT_CHECK_WITH_INFO(bad_words.shape[0] == batch_size,
-                               fmtstr("Shape of dim 0 of bad words is invalid. It must be equal to batch size."
-                                      " However, it is %d and the batch size is %d.",
-                                      (int)bad_words.shape[0], (int)batch_size));
+    // Every row belongs to exactly one of the two layers (k > 0 or greedy: top-k; k == 0 && p > 0: top-p);
+    // both get the same window.
+    TensorMap window_in({{"ite", Tensor{MEMORY_CPU, TYPE_INT32, {1}, &ite}}});
+    for (const char* key : kWholeInputs) {
+        if (input_tensors->isExist(key)) {
+            window_in.insert({key, input_tensors->at(key)});
         }
-        const bool   shared_bad_words = is_matrix || bad_words.shape[0] == 1;
-        const size_t bad_words_len    = bad_words.shape[is_matrix ? 1 : 2];
-        invokeBanBadWords((T*)input_tensors->at("logits").getPtrWithOffset(local_batch_offset * vocab_size_padded_),
-                          output_tensors->at("output_ids").getPtr<const int>(), (const int*)nullptr, (int)batch_size,
-                          (int)local_batch_size, (int)beam_width,
-                          shared_bad_words ?
-                              bad_words.getPtr<const int>() :
-                              bad_words.getPtrWithOffset<const int>(local_batch_offset * 2 * bad_words_len),
-                          shared_bad_words, bad_words_len, (int)local_batch_offset, (int)vocab_size_padded_,
-                          (size_t)step, stream_);
     }
-
-    {
-        Tensor logits = input_tensors->at("logits");
-        Tensor end_id = input_tensors->at("end_id");
-
-        TensorMap decode_input_tensors(
-            {{"logits", logits.slice({local_batch_size, beam_width, logits.shape[2]},
-                                     local_batch_offset * logits.shape[2])},
-             {"step", input_tensors->at("step")},
-             {"max_input_length", input_tensors->at("max_input_length")},
-             {"end_id", end_id.slice({local_batch_size}, local_batch_offset)},
-             {"ite", Tensor{MEMORY_CPU, TYPE_INT32, {1}, &ite}}});
-        if (input_tensors->isExist("embedding_bias")) {
-            decode_input_tensors.insert({"embedding_bias", input_tensors->at("embedding_bias")});
+    for (const char* key : kRowInputs) {
+        if (input_tensors->isExist(key)) {
+            window_in.insert({key, rowWindow(input_tensors->at(key), first, rows)});
         }
-        if (input_tensors->isExist("input_lengths")) {
-            Tensor input_lengths = input_tensors->at("input_lengths");
-            decode_input_tensors.insert(
-                {"input_lengths", input_lengths.slice({local_batch_size, beam_width}, local_batch_offset)});
-        }
-        if (input_tensors->isExist("uniform_draws")) {
-            Tensor draws = input_tensors->at("uniform_draws");
-            decode_input_tensors.insert({"uniform_draws", draws.slice({local_batch_size}, local_batch_offset)});
-        }
-
-        TensorMap decode_output_tensors({{"output_ids", output_tensors->at("output_ids")}});
-        if (output_tensors->isExist("sequence_length")) {
-            Tensor sequence_length = output_tensors->at("sequence_length");
-            decode_output_tensors.insert(
-                {"sequence_length", sequence_length.slice({local_batch_size * beam_width}, local_batch_offset)});
-        }
-        if (output_tensors->isExist("finished")) {
-            Tensor finished = output_tensors->at("finished");
-            decode_output_tensors.insert(
-                {"finished", finished.slice({local_batch_size * beam_width}, local_batch_offset)});
-        }
-        if (output_tensors->isExist("cum_log_probs")) {
-            Tensor cum_log_probs = output_tensors->at("cum_log_probs");
-            decode_output_tensors.insert(
-                {"cum_log_probs", cum_log_probs.slice({local_batch_size * beam_width}, local_batch_offset)});
-        }
-        if (output_tensors->isExist("output_log_probs")) {
-            Tensor       output_log_probs = output_tensors->at("output_log_probs");
-            const int    max_input_length = input_tensors->at("max_input_length").getVal<int>();
-            const size_t step_offset      = (size_t)(step - max_input_length) * batch_size * beam_width;
-            decode_output_tensors.insert(
-                {"output_log_probs",
-                 output_log_probs.slice({output_log_probs.shape[0] - (step - max_input_length),
-                                         local_batch_size * beam_width},
-                                        step_offset + local_batch_offset)});
-        }
-        // every row belongs to exactly one of the two layers (k > 0 or greedy: top-k; k == 0 && p > 0: top-p)
-        topk_decode_->forward(&decode_output_tensors, &decode_input_tensors);
-        topp_decode_->forward(&decode_output_tensors, &decode_input_tensors);
     }
+    TensorMap window_out({{"output_ids", output_tensors->at("output_ids")}});
+    for (const char* key : kRowOutputs) {
+        if (output_tensors->isExist(key)) {
+            window_out.insert({key, rowWindow(output_tensors->at(key), first, rows)});
+        }
+    }
+    if (output_tensors->isExist("output_log_probs")) {
+        // [generated length, batch]: the layers write row 0 of what they are given, so the view starts at this
+        // step's row and this window's column (layers/DynamicDecodeLayer.cc:427-435)
+        const Tensor& lp        = output_tensors->at("output_log_probs");
+        const size_t  generated = (size_t)(step - input_tensors->at("max_input_length").getVal<int>());
+        window_out.insert({"output_log_probs", lp.slice({lp.shape[0] - generated, rows}, generated * batch + first)});
+    }
+    topk_decode_->forward(&window_out, &window_in);
+    topp_decode_->forward(&window_out, &window_in);
 
+    stopCriteria(output_tensors, input_tensors, first, rows, step);
+}
+
+// Bad words are masked on the caller's logits before either layer looks at them (layers/DynamicDecodeLayer.cc:
+// 248-281): a [2, L] list serves every row (so does [1, 2, L] at batch 1); [batch, 2, L] has a list per row.
+template<typename T>
+void DynamicDecodeLayer<T>::banBadWords(TensorMap* output_tensors, TensorMap* input_tensors, size_t first, size_t rows,
+                                        int step)
+{
+    if (!input_tensors->isExist("bad_words_list")) {
+        return;
+    }
+    const Tensor& words = input_tensors->at("bad_words_list");
+    const size_t  rank  = words.shape.size();
+    const size_t  batch = input_tensors->at("logits").shape[0];
+    FT_CHECK_WITH_INFO(rank == 2 || rank == 3, "Bad words dimension must be 2 or 3.");
+    FT_CHECK_WITH_INFO(rank == 2 || words.shape[0] == batch,
+                       fmtstr("Shape of dim 0 of bad words is invalid. It must be equal to batch size."
+                              " However, it is %d and the batch size is %d.",
+                              (int)words.shape[0], (int)batch));
+    const bool   one_list = rank == 2 || words.shape[0] == 1;
+    const size_t length   = words.shape[rank - 1];
+    const int*   lists    = one_list ? words.getPtr<const int>() : words.getPtrWithOffset<const int>(first * 2 * length);
+    invokeBanBadWords((T*)input_tensors->at("logits").getPtrWithOffset(first * vocab_size_padded_),
+                      output_tensors->at("output_ids").getPtr<const int>(), (const int*)nullptr, (int)batch, (int)rows,
+                      1, lists, one_list, length, (int)first, (int)vocab_size_padded_, (size_t)step, stream_);
+}
+
+// After sampling: stop words on the rows of this window (layers/DynamicDecodeLayer.cc:449-462; the reference
+// examines `batch` rows from the window's start, which runs past the window), then the length criterion on the
+// whole batch, which also tells the host whether every row is finished (:464-473).
+template<typename T>
+void DynamicDecodeLayer<T>::stopCriteria(TensorMap* output_tensors, TensorMap* input_tensors, size_t first,
+                                         size_t rows, int step)
+{
+    const size_t batch = input_tensors->at("logits").shape[0];
     if (input_tensors->isExist("stop_words_list")) {
-        const size_t stop_words_length = input_tensors->at("stop_words_list").shape[2];
+        const Tensor& words  = input_tensors->at("stop_words_list");
+        const size_t  length = words.shape[2];
         FT_CHECK_WITH_INFO(output_tensors->at("finished", Tensor()).getPtr<bool>() != nullptr,
                            "stop_words_list needs the finished output");
-        // only the rows of this window are examined
         check_ftk(ftk_invoke_stop_words_criterion_rows(
             output_tensors->at("output_ids").getPtr<const int>(), nullptr,
-            input_tensors->at("stop_words_list").getPtrWithOffset<const int>(local_batch_offset * 2 * stop_words_length),
-            output_tensors->at("finished").getPtrWithOffset<bool>(local_batch_offset), local_batch_offset,
-            stop_words_length, (int)batch_size, (int)local_batch_size, (int)beam_width, step, stream_));
+            words.getPtrWithOffset<const int>(first * 2 * length),
+            output_tensors->at("finished").getPtrWithOffset<bool>(first), first, length, (int)batch, (int)rows, 1, step,
+            stream_));
     }
-
     if (input_tensors->isExist("sequence_limit_length")) {
         invokeLengthCriterion(output_tensors->at("finished").getPtr<bool>(),
                               output_tensors->at("should_stop").getPtr<bool>(), h_pinned_finished_sum_,
-                              input_tensors->at("sequence_limit_length").getPtr<const uint32_t>(), (int)batch_size,
-                              (int)beam_width, step, stream_);
+                              input_tensors->at("sequence_limit_length").getPtr<const uint32_t>(), (int)batch, 1, step,
+                              stream_);
     }
 }
 

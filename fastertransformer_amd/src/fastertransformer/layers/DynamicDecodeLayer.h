@@ -16,6 +16,9 @@ protected:
     void allocateBuffer() override;
     void freeBuffer() override;
     void initialize();
+    // the two parts of a step around the sampling layers; `first` / `rows`: the micro-batch window
+    void banBadWords(TensorMap* output_tensors, TensorMap* input_tensors, size_t first, size_t rows, int step);
+    void stopCriteria(TensorMap* output_tensors, TensorMap* input_tensors, size_t first, size_t rows, int step);
 
     TopKSamplingLayer<T>* topk_decode_ = nullptr;
     TopPSamplingLayer<T>* topp_decode_ = nullptr;

@@ -129,9 +129,11 @@ void BaseSamplingLayer<T>::setup(const size_t batch_size, const size_t beam_widt
             states[i].seed   = random_seeds.getVal<unsigned long long>(random_seeds.size() == 1 ? 0 : i);
             states[i].offset = 0;
         }
-        // synchronous copy: `states` is a temporary
-        check_hip_error(hipMemcpy(curandstate_buf_, states.data(), sizeof(ftk_rng_state) * batch_size,
-                                  hipMemcpyHostToDevice));
+        // on the layer's stream, so that it is ordered against steps still queued there; `states` is a
+        // temporary, so the copy is waited for
+        check_hip_error(hipMemcpyAsync(curandstate_buf_, states.data(), sizeof(ftk_rng_state) * batch_size,
+                                       hipMemcpyHostToDevice, stream_));
+        check_hip_error(hipStreamSynchronize(stream_));
     }
     else {
         invokeCurandInitialize(curandstate_buf_, batch_size, 0, stream_);

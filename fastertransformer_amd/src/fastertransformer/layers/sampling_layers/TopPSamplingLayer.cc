@@ -71,8 +71,10 @@ void TopPSamplingLayer<T>::setup(const size_t batch_size, const size_t beam_widt
         }
         const Tensor t = runtime_args->at(key);
         FT_CHECK_WITH_INFO(t.size() == batch_size, fmtstr("%s must be of shape [batch_size]", key));
-        check_hip_error(hipMemcpy(dst, t.data, elem * batch_size,
-                                  t.where == MEMORY_GPU ? hipMemcpyDeviceToHost : hipMemcpyHostToHost));
+        // ordered after whatever produced the tensor on this layer's stream, then waited for
+        check_hip_error(hipMemcpyAsync(dst, t.data, elem * batch_size,
+                                       t.where == MEMORY_GPU ? hipMemcpyDeviceToHost : hipMemcpyHostToHost, stream_));
+        check_hip_error(hipStreamSynchronize(stream_));
     };
     fetch("top_p_decay", decay.data(), sizeof(float));
     fetch("top_p_min", pmin.data(), sizeof(float));
@@ -150,6 +152,16 @@ void TopPSamplingLayer<T>::runSampling(TensorMap* output_tensors, TensorMap* inp
     float* output_log_probs = output_tensors->at("output_log_probs", Tensor()).template getPtr<float>();
     int*   ids = output_tensors->at("output_ids").template getPtrWithOffset<int>((size_t)step * batch_size + off);
 
+    // The chunking of a row depends on the number of rows in the call, so a window smaller than the setup batch
+    // can need a slightly larger workspace: ask for this window's size and grow on demand.
+    size_t need = 0, unused = 0;
+    invokeTopPSampling<T>(nullptr, need, unused, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                          nullptr, nullptr, curandstate_buf_, local_batch_size, vocab_size_padded_, nullptr,
+                          runtime_max_top_p_, stream_, cuda_device_prop_, skip_decode_buf_);
+    if (need > sampling_workspace_size_) {
+        sampling_workspace_      = allocator_->reMalloc(sampling_workspace_, need, false);
+        sampling_workspace_size_ = need;
+    }
     invokeBatchTopPSampling<T>(sampling_workspace_, sampling_workspace_size_, cub_temp_storage_size_, ids,
                                output_tensors->at("sequence_length", Tensor()).template getPtr<int>(), finished,
                                cum_log_probs, output_log_probs, logits, nullptr, nullptr, nullptr,

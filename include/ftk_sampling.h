@@ -172,8 +172,10 @@ int ftk_invoke_length_criterion(bool* finished, bool* should_stop, int* h_pinned
  * One call = the kernel sequence BaseSamplingLayer<T>::forward + TopKSamplingLayer<T>::runSampling
  * issue for the rows a top-k layer owns (layers/sampling_layers/BaseSamplingLayer.cc:255-359,
  * layers/sampling_layers/TopKSamplingLayer.cu:189-268) when no log-prob output is requested:
- * bad words, temperature(+bias), repetition/presence penalty, min-length, end/pad mask, top-k
- * selection and sampling, with the logits read from HBM once and never written. */
+ * temperature(+bias), repetition/presence penalty, min-length, end/pad mask, top-k selection and sampling,
+ * with the logits read from HBM once and never written (the reference leaves them penalised). Bad words are
+ * not part of it: DynamicDecodeLayer masks them on the logits before the sampling layers run
+ * (ftk_invoke_ban_bad_words), here as in the reference. */
 typedef struct ftk_fused_topk_args {
     int         dtype;
     const void* logits;         /* [local_batch, vocab_size_padded], not modified */
@@ -190,10 +192,6 @@ typedef struct ftk_fused_topk_args {
     const int*   end_ids;        /* [local] */
     const int*   input_lengths;  /* [local] or NULL */
     const int*   output_ids;     /* history base + window offset: element (t, row) at output_ids[t*batch_size+row] */
-    const int*   bad_words;      /* [2, L] or [local, 2, L] or NULL */
-    int          bad_words_len;
-    int          bad_words_shared;
-    int          id_offset; /* kept for symmetry with invokeBanBadWords; rows are already windowed */
     const int*   top_ks;    /* [local] */
     const float* top_ps;    /* [local] */
     int          max_top_k;
@@ -222,6 +220,14 @@ int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
  * are safe back to back. */
 #define FTK_FUSED_STATIC_WORKSPACE_BYTES (32u << 20)
 int ftk_fused_topk_step_static(ftk_fused_topk_args* args, ftk_stream_t stream);
+
+/* Measurement aid without a counterpart in the reference: reads `bytes` (16-byte aligned, a multiple of 16 is
+ * used) once with the launch shape and load instructions of the fused step's streaming kernel and nothing else
+ * (one maximum per 16 bytes; one float per wave goes to `sink`, which needs at least 4096 floats). It is the
+ * yardstick the streaming kernel's duration is compared with. elapsed_ms != NULL: the launch carries a pair of
+ * events, the call waits for the kernel and returns its duration. */
+int ftk_measure_plain_read(const void* data, size_t bytes, float* sink, size_t sink_floats, ftk_stream_t stream,
+                           float* elapsed_ms);
 
 /* ---- the steps either side of the sampling path -------------------------------------------- */
 /* kernels/logprob_kernels.cu:137-183 invokeLogProbFromLogits<T>: cum_log_probs[b] = sum over step < lengths[b]-1 of
@@ -257,18 +263,6 @@ int ftk_invoke_transpose_axis01(int* out, const int* in, const int* in_skipping_
  * events) and resets the count. kernel: 0 = history bitmap, 1 = gather (the streaming pass), 2 = select. */
 int ftk_profile_enable(int max_launches);
 int ftk_profile_read(int kernel, double* total_ms, int* launches);
-
-/* ---- test hooks (host-side instances of the shared arithmetic, and device probes) ----------- */
-float ftk_host_expf(float x);
-float ftk_host_logf(float x);
-/* kind 0: det_expf, 1: det_logf, 2: float->half->float, 3: float->bf16->float; n elements on device */
-int ftk_test_device_math(int kind, const float* in, float* out, size_t n, ftk_stream_t stream);
-/* draws `n_draws` uniforms per row into out[row*n_draws + i], advancing the states */
-int ftk_test_rng_uniform(ftk_rng_state* states, float* out, int batch_size, int n_draws, ftk_stream_t stream);
-/* non-zero: every top-p row takes the radix-sort fallback (exercises it on small inputs) */
-void ftk_test_set_topp_force_deep(int enable);
-/* raw Philox-4x32-10 block for known-answer tests (host) */
-void ftk_host_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,33 @@
+/*
+ * Test hooks of the sampling engine. They exist only in libftk_sampling_hooks.so, a second build of
+ * libftk_sampling.so compiled with -DFTK_TEST_HOOKS for the test-suite; the product library does not export
+ * them and has none of the process-wide switches they set. None of them has a counterpart in the reference.
+ */
+#ifndef FTK_TEST_HOOKS_H
+#define FTK_TEST_HOOKS_H
+
+#include "ftk_sampling.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* host-side instances of the arithmetic shared by all kernels */
+float ftk_host_expf(float x);
+float ftk_host_logf(float x);
+/* raw Philox-4x32-10 block for known-answer tests (host) */
+void ftk_host_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+/* kind 0: det_expf, 1: det_logf, 2: float->half->float, 3: float->bf16->float, 4: 1/(x+1e-6), 5: subnormal
+ * arithmetic; n elements on device */
+int ftk_test_device_math(int kind, const float* in, float* out, size_t n, ftk_stream_t stream);
+/* draws `n_draws` uniforms per row into out[row*n_draws + i], advancing the states */
+int ftk_test_rng_uniform(ftk_rng_state* states, float* out, int batch_size, int n_draws, ftk_stream_t stream);
+/* non-zero: every top-p row takes the radix-sort fallback (exercises it on small inputs); process-wide */
+void ftk_test_set_topp_force_deep(int enable);
+/* non-zero: every fused step takes the general stream, also where the lean gather would run; process-wide */
+void ftk_test_set_fused_force_general(int enable);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FTK_TEST_HOOKS_H */

@@ -82,3 +82,47 @@ def uniforms(rng, n):
     u = rng.random(n).astype(np.float32)
     u = np.where(u == 0.0, np.float32(1.0), u)
     return u.astype(np.float32)
+
+
+def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=None):
+    """One fused decode step straight through the C ABI (temperature 0.8, repetition penalty 1.1 over `history`,
+    top-k `k`, top-p 0.9, injected draws). entry: "caller" = ftk_fused_topk_step with a workspace of the queried
+    size, "static" = ftk_fused_topk_step_static. Returns (ids, sequence_length, finished, rc, needed bytes)."""
+    import ctypes as C
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+    dev = "cuda"
+    out_ids = torch.zeros((H + 1, B), dtype=torch.int32, device=dev)
+    out_ids[:H] = history
+    finished = finished0.clone()
+    seq = seqlen0.clone()
+    temps = torch.full((B,), 0.8, device=dev)
+    pens = torch.full((B,), 1.1, device=dev)
+    end_ids = torch.full((B,), V - 1, dtype=torch.int32, device=dev)
+    top_ks = torch.full((B,), k, dtype=torch.int32, device=dev)
+    top_ps = torch.full((B,), 0.9, device=dev)
+    a = ops.FusedTopkArgs()
+    a.dtype, a.logits, a.embedding_bias = dt, logits.data_ptr(), None
+    a.vocab_size = a.vocab_size_padded = V
+    a.batch_size = a.local_batch_size = B
+    a.step, a.max_input_length = H, H
+    a.temperatures, a.penalties, a.penalty_type = temps.data_ptr(), pens.data_ptr(), ops.PENALTY_MULTIPLICATIVE
+    a.end_ids, a.output_ids = end_ids.data_ptr(), out_ids.data_ptr()
+    a.top_ks, a.top_ps, a.max_top_k = top_ks.data_ptr(), top_ps.data_ptr(), k
+    a.uniform_draws = draws.data_ptr()
+    a.ids = out_ids.data_ptr() + 4 * H * B
+    a.sequence_length, a.finished = seq.data_ptr(), finished.data_ptr()
+    lib = fa.ftk() if lib is None else lib
+    stream = ops.current_stream()
+    ws = None
+    if entry == "caller":
+        a.workspace = None
+        ops.check(lib.ftk_fused_topk_step(C.addressof(a), stream), "size query")
+        ws = torch.empty(a.workspace_size, dtype=torch.uint8, device=dev)
+        a.workspace = ws.data_ptr()
+        rc = lib.ftk_fused_topk_step(C.addressof(a), stream)
+    else:
+        a.workspace, a.workspace_size = None, 0
+        rc = lib.ftk_fused_topk_step_static(C.addressof(a), stream)
+    torch.cuda.synchronize()
+    return out_ids[H].cpu().numpy(), seq.cpu().numpy(), finished.cpu().numpy(), rc, a.workspace_size

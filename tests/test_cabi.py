@@ -44,6 +44,21 @@ def test_kernel_library_exports_every_declared_function():
     assert sorted(ops.exported_symbols()) == declared
 
 
+def test_test_hooks_live_in_their_own_library_only():
+    """include/ftk_test_hooks.h is served by libftk_sampling_hooks.so (the test build); the product library has
+    neither the hooks nor the process-wide switches behind them"""
+    _ensure_built()
+    from fastertransformer_amd import ops
+    declared = [n for n in _declared_functions("ftk_test_hooks.h")]
+    assert sorted(ops.hook_symbols()) == declared and len(declared) >= 7
+    hooks, product = ops.ftk_hooks(), ops.ftk()
+    for name in declared:
+        assert hasattr(hooks, name), name
+        assert not hasattr(product, name), name
+    for name in ops.exported_symbols():  # the hooks build is a complete library
+        assert hasattr(hooks, name), name
+
+
 def test_decode_library_exports_every_declared_function():
     _ensure_built()
     from fastertransformer_amd import ops
@@ -95,7 +110,7 @@ def test_workspace_queries_and_argument_errors():
 def test_shared_arithmetic_matches_the_oracle_bit_for_bit():
     _ensure_built()
     from fastertransformer_amd import ops
-    lib = ops.ftk()
+    lib = ops.ftk_hooks()
     rng = np.random.default_rng(2)
     x = np.concatenate([rng.uniform(-90, 90, 5000), [0.0, -0.0, -np.inf, 88.7, -103.9]]).astype(np.float32)
     got = np.array([lib.ftk_host_expf(C.c_float(float(v))) for v in x], np.float32)
@@ -109,7 +124,7 @@ def test_philox_known_answers():
     """Random123 known-answer vectors for Philox-4x32-10"""
     _ensure_built()
     from fastertransformer_amd import ops
-    lib = ops.ftk()
+    lib = ops.ftk_hooks()
     vectors = [
         ((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
         ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),

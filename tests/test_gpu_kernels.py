@@ -29,7 +29,8 @@ def _sync(torch):
 
 
 def test_device_math_matches_host_bitwise(env):
-    torch, lib, ops = env
+    torch, _, ops = env
+    lib = ops.ftk_hooks()
     rng = np.random.default_rng(1)
     x = np.concatenate([rng.uniform(-104, 89, 400000), rng.uniform(-1, 1, 50000),
                         -np.abs(rng.standard_normal(200000)) * 10, [0.0, -0.0, -103.9, 88.7, -200.0, 100.0]])
@@ -49,7 +50,8 @@ def test_device_math_matches_host_bitwise(env):
 
 
 def test_device_conversions_division_subnormals(env):
-    torch, lib, ops = env
+    torch, _, ops = env
+    lib = ops.ftk_hooks()
     rng = np.random.default_rng(2)
     x = np.concatenate([rng.standard_normal(300000) * 100, rng.uniform(-7e4, 7e4, 100000),
                         rng.standard_normal(100000) * 1e-5, rng.standard_normal(100000) * 1e-7,
@@ -340,6 +342,8 @@ def test_topk_domain_error(env):
 
 def _run_topp(env, dt, probs, p_arr, end_ids, u, finished=None, seq=None, skip=None, logprobs=False, force_deep=False):
     torch, lib, ops = env
+    if force_deep:
+        lib = ops.ftk_hooks()  # the switch exists in the test build of the library only
     batch, Vp = probs.shape
     d_probs = to_torch(probs, dt)
     d_ids = torch.full((batch,), -7, dtype=torch.int32, device="cuda")
@@ -355,7 +359,8 @@ def _run_topp(env, dt, probs, p_arr, end_ids, u, finished=None, seq=None, skip=N
                                                  None, None, None, None, None, None, None, None, batch, Vp, None, 1.0,
                                                  None, None, None))
     ws = torch.empty(max(ws_size.value, 16), dtype=torch.uint8, device="cuda")
-    lib.ftk_test_set_topp_force_deep(int(force_deep))
+    if force_deep:
+        lib.ftk_test_set_topp_force_deep(1)
     try:
         ops.check(lib.ftk_invoke_batch_topp_sampling(dt, ws.data_ptr(), C.addressof(ws_size), C.addressof(cub),
                                                      d_ids.data_ptr(), ops.ptr(d_seq), ops.ptr(d_fin), ops.ptr(d_cum),
@@ -365,7 +370,8 @@ def _run_topp(env, dt, probs, p_arr, end_ids, u, finished=None, seq=None, skip=N
                                                      ops.ptr(d_skip)))
         _sync(torch)
     finally:
-        lib.ftk_test_set_topp_force_deep(0)
+        if force_deep:
+            lib.ftk_test_set_topp_force_deep(0)
     return (to_numpy(d_ids), to_numpy(d_fin) if d_fin is not None else None,
             to_numpy(d_seq) if d_seq is not None else None, to_numpy(d_cum) if logprobs else None,
             to_numpy(d_out) if logprobs else None)
@@ -544,7 +550,8 @@ def test_stop_words_and_length_criterion(env):
 
 
 def test_rng_determinism_and_range(env):
-    torch, lib, ops = env
+    torch, _, ops = env
+    lib = ops.ftk_hooks()
     batch, n = 64, 500
     st = torch.zeros(batch * 2, dtype=torch.int64, device="cuda")
     ops.check(lib.ftk_invoke_curand_initialize(st.data_ptr(), batch, 1234, ops.current_stream()))
@@ -761,3 +768,33 @@ def test_topk_sampling_random_shapes(env, dt, seed):
             O.add_bias_softmax(dt, src, None, end_ids, None, batch, V, V)
         args = (dt, src, k_arr, p_arr, max_k, end_ids, u, finished.copy(), seq, skip, logprobs)
         _compare_topk(_run_topk(env, *args), _oracle_topk(*args), dt)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_fused_step_lean_gather_equals_general_stream(env, dt):
+    """The two streaming kernels of the fused step on the same launch: the lean gather (what a launch with k <= 128
+    and no bias takes) and the general stream, forced through the hook of the test build. Sampled ids, lengths
+    and flags must be identical, at a batch that splits rows over several workgroups and at one that does not."""
+    from helpers import run_fused_step
+    torch, _, ops = env
+    hooks = ops.ftk_hooks()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(31 + dt)
+    V, H, k = 100003, 40, 50
+    for B in (24, 1030):
+        logits = (torch.randn((B, V), generator=gen, device="cuda") * 2.0).to(ops.torch_dtype(dt))
+        history = torch.randint(0, V, (H, B), generator=gen, device="cuda", dtype=torch.int32)
+        draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
+        finished0 = torch.zeros(B, dtype=torch.bool, device="cuda")
+        finished0[1] = True
+        seqlen0 = torch.full((B,), H - 1, dtype=torch.int32, device="cuda")
+        lean = run_fused_step("caller", torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks)
+        hooks.ftk_test_set_fused_force_general(1)
+        try:
+            general = run_fused_step("caller", torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0,
+                                     lib=hooks)
+        finally:
+            hooks.ftk_test_set_fused_force_general(0)
+        assert lean[3] == 0 and general[3] == 0
+        for a, b in zip(lean[:3], general[:3]):
+            assert np.array_equal(a, b)

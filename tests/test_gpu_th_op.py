@@ -185,7 +185,7 @@ def test_matches_the_oracle_layer(th):
     oracle."""
     import ctypes as C
     from fastertransformer_amd import ops
-    host = ops.ftk()
+    host = ops.ftk_hooks()
 
     def draw(seed, i):
         c = (C.c_uint32 * 4)(i, 0, 0, 0)
