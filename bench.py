@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 PLAIN_READ = "plain_read_b256_v128256_f32"
 # HBM bytes per launch of the dominant kernel on the headline workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by a copy kernel of known size (summary under profiles/)
-TRAFFIC_BYTES_PER_LAUNCH = 152029196
+TRAFFIC_BYTES_PER_LAUNCH = 134055870
 
 WORKLOADS = {
     # the configuration the headline metric is quoted on
@@ -150,8 +150,10 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     alg = algorithmic_bytes(w, mid_step)
     gather_ms = kernel_ms[1]
     achieved = alg / (gather_ms * 1e-3) / 1e9 if gather_ms > 0 else 0.0
-    # batches of at least 1024 rows run the one-launch row kernel; smaller ones stream, then select
-    dominant = "fused_gather_kernel" if kernel_ms[2] > 0 else "fused_row_kernel"
+    # launches whose largest k is at most 128 (and no bias) stream with the lean gather; the others with the general
+    # stream, in one launch from 1024 rows on
+    lean = max(int(k) for k in top_ks) <= 128
+    dominant = "lean_gather_kernel" if lean else ("fused_gather_kernel" if kernel_ms[2] > 0 else "fused_row_kernel")
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
         kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2]),
