@@ -32,6 +32,9 @@ KERNEL_UNITS = [
     ("fused_kernels.hip", "fused_kernels.o", []),
     ("topp_kernels.hip", "topp_kernels.o", []),
     ("topk_kernels.hip", "topk_kernels.o", []),
+    ("logprob_kernels.hip", "logprob_kernels_f32.o", ["-DFTK_LP_DT=0"]),
+    ("logprob_kernels.hip", "logprob_kernels_f16.o", ["-DFTK_LP_DT=1"]),
+    ("logprob_kernels.hip", "logprob_kernels_bf16.o", ["-DFTK_LP_DT=2"]),
     ("lean_kernels.hip", "lean_kernels_f32.o", ["-DFTK_LEAN_DT=0"]),
     ("lean_kernels.hip", "lean_kernels_f16.o", ["-DFTK_LEAN_DT=1"]),
     ("lean_kernels.hip", "lean_kernels_bf16.o", ["-DFTK_LEAN_DT=2"]),

@@ -121,6 +121,8 @@ const char* ftk_error_string(int code)
         case FTK_ERR_TOPK_DOMAIN: return "top-k kernel supports 1<=k<=1024";
         case FTK_ERR_ARGUMENT: return "invalid argument";
         case FTK_ERR_WORKSPACE: return "workspace too small";
+        case FTK_ERR_UNSUPPORTED:
+            return "log-prob outputs are not covered by the fused step for this configuration: run the kernel sequence";
         case FTK_ERR_STATIC_WORKSPACE:
             return "the step needs more workspace than the library's fixed array (FTK_FUSED_STATIC_WORKSPACE_BYTES): "
                    "use ftk_fused_topk_step with a caller workspace";

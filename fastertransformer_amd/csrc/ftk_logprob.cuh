@@ -1,0 +1,587 @@
+// Fused decode step for rows of the top-k layer when cum_log_probs / output_log_probs are requested.
+//
+// The reference then turns the penalised logits into probabilities over the whole row before it samples
+// (src/fastertransformer/layers/sampling_layers/TopKSamplingLayer.cu:220-266: invokeAddBiasSoftMax, then the
+// top-k kernels on probabilities, whose log-prob outputs are log p and log p - log S). Its kernel sequence
+// moves the row nine times (temperature R+W, penalties, softmax 3R+3W, top-k k+2 R). Here the row is read
+// twice and never written:
+//   lp_rowmax_kernel - streams the row once (the launch shape of the lean gather), applies temperature,
+//                      history penalty and the min-length mask in registers and leaves the exact maximum of
+//                      every workgroup's share in the workspace;
+//   lp_row_kernel    - one workgroup per row streams it again, with the same arithmetic, and
+//                        * sums e_v = T(exp(y_v - max)) in the order of the reference's softmax
+//                          (sampling_topp_kernels.cu:1308-1344: thread t of 1024 adds columns t, t + 1024, ...
+//                          one after the other; reduce_kernel_utils.cuh:73-103: xor butterflies 16..1 inside
+//                          32-lane groups, then over the 32 group sums), so the sum has the reference's bits:
+//                          a thread owns four neighbouring chains and walks them with 16-byte (fp32) or 8-byte
+//                          (16-bit types) loads that are 1024 columns apart;
+//                        * gathers the candidates of the top-k selection by e_v, with a bound lowered by what
+//                          the division and rounding to T can merge, so that every column whose probability
+//                          ties with the k-th largest is among them;
+//                        * turns the candidates' e_v into probabilities T(e_v / (sum + 1e-6)), replays the
+//                          reference's tie orders on them and samples (topk_select_lds with probabilities in).
+// Rows it cannot bound take the literal replay on probabilities computed on the fly.
+// Preconditions (checked by the host, which otherwise reports FTK_ERR_UNSUPPORTED and the layer runs the kernel
+// sequence): no embedding bias, largest k <= 128, vocabulary >= 1024 (the reference's block is min(V, 1024)
+// threads), rows aligned to 16 bytes.
+#pragma once
+#include <type_traits>
+
+#include "ftk_lean.cuh"
+
+namespace ftk {
+
+constexpr int LP_THREADS = 256;
+constexpr int LP_CHAINS  = 4;     // neighbouring summation chains per thread
+constexpr int LP_BLOCK   = 1024;  // chains per row: the reference's block size
+constexpr int LP_RING    = 8;     // loads in flight per thread
+constexpr int LP_HEAD    = 4;     // rounds examined before the first bound exists
+static_assert(LP_THREADS * LP_CHAINS == LP_BLOCK, "a workgroup owns all chains of its row");
+
+struct LogProbLaunch {
+    float* cum_log_probs;     // [rows] or null
+    float* output_log_probs;  // [rows] or null
+    float* partial_max;       // [rows][splits]
+    int    splits;            // workgroups per row of lp_rowmax_kernel
+};
+
+// ---- pass 1 --------------------------------------------------------------------------------------------
+template<int DT, int BMW>
+__global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(FusedParams p, FusedLaunch l, LogProbLaunch lp)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         EPV = (int)(16 / sizeof(T));
+    constexpr int         R   = LG_RING;
+    __shared__ float      red[LG_WAVES];
+    const int             t     = threadIdx.x;
+    const int             row   = blockIdx.y;
+    const int             chunk = blockIdx.x;
+    const T*              rowp  = (const T*)p.logits + (size_t)row * p.Vp;  // 16-byte aligned (host check)
+    const uint4*          base  = reinterpret_cast<const uint4*>(rowp);
+    const int             vhi   = p.V / EPV;  // whole vectors below column V
+    const int             vb    = min(vhi, chunk * l.subs_per_wg * LG_SUB_VECS);
+    const int             ve    = min(vhi, vb + l.subs_per_wg * LG_SUB_VECS);
+    const int             nvec  = ve - vb;
+    const int             nsub  = (nvec + LG_SUB_VECS - 1) / LG_SUB_VECS;
+
+    const bool hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
+    int        hist_ids[LG_HIST_U];
+    if (hist) {
+#pragma unroll
+        for (int u = 0; u < LG_HIST_U; ++u) {
+            const int pos = t + u * LG_THREADS;
+            hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
+        }
+    }
+    uint4 raw[R][LG_NV];
+    auto  load = [&](int slot, int q) {
+#pragma unroll
+        for (int j = 0; j < LG_NV; ++j) {
+            const int vi = min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1);
+            raw[slot][j] = lean_stream_load(base + vi);
+        }
+    };
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (r < nsub) {
+            load(r, r);
+        }
+    }
+    const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
+    const bool        fin  = row_flag_or(p.finished_in, row, p.end_ids + row, false);
+    FusedRow<DT, BMW> rowctx(p, row);
+    if (skip || fin) {
+        return;
+    }
+    const bool last_wg = chunk == (int)gridDim.x - 1;
+    const int  lo_col  = vb * EPV;
+    const int  hi_col  = last_wg ? p.V : ve * EPV;
+    if (hist) {
+        uint32_t* window = fused_lds_bitmap<FusedRow<DT, BMW>::LDS_WORDS>();
+        const int origin = lo_col & ~31;
+        const int words  = min(FusedRow<DT, BMW>::LDS_WORDS, (hi_col - origin + 31) / 32 + 1);
+        for (int i = t; i < words; i += LG_THREADS) {
+            window[i] = 0u;
+        }
+        lds_barrier();
+        auto mark = [&](int pos, int id) {
+            if (id >= lo_col && id < hi_col && rowctx.history_position_counts(pos)) {
+                atomicOr(&window[(id - origin) >> 5], 1u << ((id - origin) & 31));
+            }
+        };
+#pragma unroll
+        for (int u = 0; u < LG_HIST_U; ++u) {
+            mark(t + u * LG_THREADS, hist_ids[u]);
+        }
+        for (int pos = t + LG_HIST_U * LG_THREADS; pos < p.step; pos += LG_THREADS) {
+            mark(pos, p.output_ids[(size_t)pos * p.batch_size + row]);
+        }
+        rowctx.bm_mode   = 1;
+        rowctx.bm_origin = origin;
+    }
+    lds_barrier();
+    const bool  bitsv   = rowctx.has_vector_bits();
+    const float mul     = rowctx.fast_mul;
+    const bool  ordered = mul > 0.0f && mul < __builtin_inff();  // the plain transform keeps the order
+    const float NEG_INF = -__builtin_inff();
+    float       m       = NEG_INF;
+    // the exact value of a vector's largest element: plain vectors through their raw maximum (rounding to T and
+    // a positive multiplier keep the order), the others element by element
+    auto vector_max = [&](const uint4& v, int first) -> float {
+        uint32_t bits = 0u;
+        if (bitsv) {
+            if (BMW > 0) {
+                const int rel = first - rowctx.bm_origin;
+                bits          = (rowctx.bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
+            }
+            else {
+                bits = rowctx.vector_bits(first, EPV);
+            }
+        }
+        const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - first);
+        if (bits == 0u && rel_end >= (uint32_t)EPV && ordered) {
+            return rowctx.fast(lean_raw_max<DT>(v));
+        }
+        float vm = NEG_INF;
+#pragma unroll
+        for (int c = 0; c < EPV; ++c) {
+            float x = rowctx.fast(vector_element<DT>(v, c));
+            if ((bits >> c) & 1u) {
+                x = rowctx.flagged(x);
+            }
+            if ((uint32_t)c == rel_end) {
+                x = -S::max_t();
+            }
+            vm = __builtin_fmaxf(vm, x);
+        }
+        return vm;
+    };
+    for (int q0 = 0; q0 < nsub; q0 += R) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int q = q0 + r;
+            if (q < nsub) {
+#pragma unroll
+                for (int j = 0; j < LG_NV; ++j) {
+                    const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
+                    const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV);
+                    m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
+                }
+                if (q + R < nsub) {
+                    load(r, q + R);
+                }
+            }
+        }
+    }
+    if (last_wg) {
+        // the columns behind the last whole vector
+        for (int v = vhi * EPV + t; v < p.V; v += LG_THREADS) {
+            m = __builtin_fmaxf(m, topk_value_at<DT>(rowctx, v));
+        }
+    }
+    m = wave_max(m);
+    if (lane_id() == 0) {
+        red[wave_id()] = m;
+    }
+    lds_barrier();
+    if (t == 0) {
+        float r = red[0];
+#pragma unroll
+        for (int w = 1; w < LG_WAVES; ++w) {
+            r = __builtin_fmaxf(r, red[w]);
+        }
+        lp.partial_max[(size_t)row * lp.splits + chunk] = r;
+    }
+}
+
+// ---- pass 2 --------------------------------------------------------------------------------------------
+// Row accessor of the recovery paths: the key of column v is that of its probability.
+template<int DT>
+struct ProbRow {
+    typedef Storage<DT>       S;
+    typedef typename S::T     T;
+    FusedRow<DT, 0>*          base;
+    float                     row_max;
+    float                     denom;  // sum + 1e-6
+    __device__ __forceinline__ void prepare_whole_row()
+    {
+        base->prepare_whole_row();
+    }
+    __device__ __forceinline__ float prob_of(float y) const
+    {
+        const float e = round_t<DT>(det_expf(y - row_max));
+        return round_t<DT>(e / denom);
+    }
+    __device__ __forceinline__ uint32_t key_at(int v) const
+    {
+        const uint32_t bit = base->bm_mode != 0 ? base->vector_bits(v, 1) : 0u;
+        return order_key(prob_of(base->slow(v, S::ld(base->rowp[v]), bit)));
+    }
+};
+
+// element c of a thread's chunk (four neighbouring columns) as fp32
+template<int DT>
+__device__ __forceinline__ float lp_chunk_element(const uint4& v, int c)
+{
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    return __uint_as_float(w[c]);
+}
+template<int DT>
+__device__ __forceinline__ float lp_chunk_element(const uint2& v, int c)
+{
+    const uint32_t w[2] = {v.x, v.y};
+    return Storage<DT>::ld((uint16_t)(c & 1 ? w[c >> 1] >> 16 : w[c >> 1] & 0xFFFFu));
+}
+
+// Ties after the division: two e values give the same probability T(e / denom) only if they differ by less than
+// a unit in the last place of that probability times denom. While the k-th largest probability is a normal
+// number of T that is at most 2^-(mantissa bits - 1) of e (four half-units, to be safe): candidates are gathered
+// down to e_bound * (1 - LP_TIE_REL). When it is subnormal the unit no longer shrinks with the value, ties reach
+// arbitrarily far down, and the row takes the literal replay (lp_ties_bounded tells).
+template<int DT>
+__device__ __forceinline__ float lp_tie_rel()
+{
+    return DT == DT_F32 ? 2.384185791015625e-07f : (DT == DT_F16 ? 0.001953125f : 0.015625f);
+}
+template<int DT>
+__device__ __forceinline__ bool lp_ties_bounded(float e_bound, float denom)
+{
+    const float smallest_normal = DT == DT_F16 ? 6.103515625e-05f : 1.17549435e-38f;
+    return e_bound >= 2.0f * smallest_normal * denom;
+}
+
+template<int DT, int BMW>
+__global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, FusedLaunch l, LogProbLaunch lp)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    // a thread's load: LP_CHAINS neighbouring columns
+    typedef typename std::conditional<sizeof(T) == 4, uint4, uint2>::type Chunk;
+    __shared__ TopkShared s;
+    __shared__ uint32_t   slot_key[2][LP_THREADS];
+    __shared__ float      warp_sum[32];
+    const int             t   = threadIdx.x;
+    const int             row = blockIdx.x;
+    const T*              rowp = (const T*)p.logits + (size_t)row * p.Vp;
+    const Chunk*          base = reinterpret_cast<const Chunk*>(rowp);
+    const int             rounds = (p.V + LP_BLOCK - 1) / LP_BLOCK;  // columns >= V are masked: e = 0 exactly
+
+    // history first, then the first loads of the row, then the arguments
+    const bool hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
+    int        hist_ids[LG_HIST_U];
+    if (hist) {
+#pragma unroll
+        for (int u = 0; u < LG_HIST_U; ++u) {
+            const int pos = t + u * LP_THREADS;
+            hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
+        }
+    }
+    Chunk raw[LP_RING];
+    auto  load = [&](int slot, int n) {
+        // the last round may reach past the row: such a thread reads its chunk of the round before (never used).
+        // Rows are 16-byte aligned, so a chunk that starts inside the padded row lies inside it.
+        const int col = n * LP_BLOCK + t * LP_CHAINS;
+        raw[slot]     = base[(col < p.Vp ? col : col - LP_BLOCK) / LP_CHAINS];
+    };
+#pragma unroll
+    for (int r = 0; r < LP_RING; ++r) {
+        if (r < rounds) {
+            load(r, r);
+        }
+    }
+    const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
+    const bool        fin  = row_flag_or(l.finished, row, p.end_ids + row, false);
+    const int         k    = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
+    const float       tp   = row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f);
+    FusedRow<DT, BMW> rowctx(p, row);
+    if (skip) {
+        return;
+    }
+    if (fin) {
+        if (t == 0) {
+            l.ids[row] = p.end_ids[row];  // a finished row emits its end id: no draw, no log-prob, no length update
+        }
+        return;
+    }
+    int draw_bits = 0;
+    if (t == 0) {
+        draw_bits = __float_as_int(row_uniform(l.rng, l.uniforms, row));
+    }
+    const TopkOutputs out =
+        topk_outputs(l.ids, l.sequence_length, l.finished, lp.cum_log_probs, lp.output_log_probs, row, p.end_ids);
+    // the row's maximum: pass 1 left one per workgroup; pad columns count as -MAX_T
+    float row_max = -3.402823466e+38f;
+    for (int c = 0; c < lp.splits; ++c) {
+        row_max = __builtin_fmaxf(row_max, lp.partial_max[(size_t)row * lp.splits + c]);
+    }
+    if (p.V < p.Vp) {
+        row_max = __builtin_fmaxf(row_max, -S::max_t());
+    }
+    row_max = uniform_f(row_max);
+    if (t == 0) {
+        s.n_cand  = 0;
+        s.misc[0] = draw_bits;
+    }
+    constexpr int LP_BM_OVERLAY = (int)(sizeof(s.sel) / sizeof(uint32_t));
+    constexpr int LP_BM_TAIL    = BMW > LP_BM_OVERLAY ? BMW - LP_BM_OVERLAY : 1;
+    __shared__ uint32_t bitmap_tail[LP_BM_TAIL];
+    if (hist) {
+        uint32_t* head_words = reinterpret_cast<uint32_t*>(&s.sel);
+        const int words      = min(BMW, (p.V + 31) / 32 + 1);
+        for (int i = t; i < words; i += LP_THREADS) {
+            (i < LP_BM_OVERLAY ? head_words[i] : bitmap_tail[i - LP_BM_OVERLAY]) = 0u;
+        }
+        lds_barrier();
+        auto mark = [&](int pos, int id) {
+            if (id >= 0 && id < p.V && rowctx.history_position_counts(pos)) {
+                const int w = id >> 5;
+                atomicOr(w < LP_BM_OVERLAY ? &head_words[w] : &bitmap_tail[w - LP_BM_OVERLAY], 1u << (id & 31));
+            }
+        };
+#pragma unroll
+        for (int u = 0; u < LG_HIST_U; ++u) {
+            mark(t + u * LP_THREADS, hist_ids[u]);
+        }
+        for (int pos = t + LG_HIST_U * LP_THREADS; pos < p.step; pos += LP_THREADS) {
+            mark(pos, p.output_ids[(size_t)pos * p.batch_size + row]);
+        }
+    }
+    lds_barrier();
+    const float u     = __int_as_float(s.misc[0]);
+    const bool  bitsv = hist || rowctx.has_vector_bits();
+    const uint32_t KMIN = min_valid_key<DT>();
+
+    // The row's history bitmap lives in LDS that nothing else uses while the row streams: the ordered-list area
+    // of the select phase holds its first words, a small array of its own the rest (four workgroups then fit a
+    // compute unit even with the window of the largest vocabularies).
+    auto bitmap_word = [&](int w) -> uint32_t {
+        if constexpr (BMW > 0) {
+            return w < LP_BM_OVERLAY ? reinterpret_cast<const uint32_t*>(&s.sel)[w] : bitmap_tail[w - LP_BM_OVERLAY];
+        }
+        else {
+            return rowctx.bm_word(w);
+        }
+    };
+    // e values of the LP_CHAINS columns a chunk holds (first column `col`); columns >= V give 0
+    auto e_values = [&](const Chunk& v, int col, float* e) {
+        uint32_t bits = 0u;
+        if (bitsv) {
+            if (BMW > 0) {
+                bits = (bitmap_word(col >> 5) >> (col & 31)) & ((1u << LP_CHAINS) - 1u);
+            }
+            else {
+                bits = rowctx.vector_bits(col, LP_CHAINS);
+            }
+        }
+        float y[LP_CHAINS];
+#pragma unroll
+        for (int c = 0; c < LP_CHAINS; ++c) {
+            y[c] = rowctx.fast(lp_chunk_element<DT>(v, c));
+        }
+        // rare: a column of the history, the masked end id, the end of the vocabulary
+        const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - col);
+        if (bits != 0u || rel_end < (uint32_t)LP_CHAINS || col + LP_CHAINS > p.V) {
+#pragma unroll
+            for (int c = 0; c < LP_CHAINS; ++c) {
+                if ((bits >> c) & 1u) {
+                    y[c] = rowctx.flagged(y[c]);
+                }
+                if ((uint32_t)c == rel_end || col + c >= p.V) {
+                    y[c] = -S::max_t();
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < LP_CHAINS; ++c) {
+            e[c] = round_t<DT>(det_expf(y[c] - row_max));
+        }
+        if (col + LP_CHAINS > p.V) {
+#pragma unroll
+            for (int c = 0; c < LP_CHAINS; ++c) {
+                e[c] = col + c < p.V ? e[c] : 0.0f;  // (what lies behind the vocabulary adds nothing)
+            }
+        }
+    };
+
+    float    acc[LP_CHAINS] = {0.0f, 0.0f, 0.0f, 0.0f};  // the chains' running sums
+    uint32_t thr            = KMIN;                      // candidates: e with key >= thr_low
+    float    thr_low        = key_to_float(KMIN);
+    uint32_t dmax           = 0u;  // largest key this thread has put on the list
+    bool     valid          = false;
+    int      par            = 0;
+    auto     set_threshold  = [&](uint32_t key) {
+        thr           = key;
+        const float e = key_to_float(key);
+        thr_low       = uniform_f(e - e * lp_tie_rel<DT>());
+    };
+    auto push = [&](float e, int col) {
+        const uint32_t key  = order_key(e);
+        const int      slot = atomicAdd(&s.n_cand, 1);
+        if (slot < TK_CCAP) {
+            s.cand.key[slot] = key;
+            s.cand.idx[slot] = (uint32_t)col;
+        }
+        dmax = key > dmax ? key : dmax;
+    };
+    auto rebound = [&](uint32_t mine) {
+        slot_key[par][t] = mine;
+        lds_barrier();
+        const uint32_t P = lean_kth_of_slots(slot_key[par], k);
+        par ^= 1;
+        if (P > thr && P > order_key(0.0f)) {  // at least k columns with e > 0 at or above it
+            set_threshold(P);
+            valid = true;
+        }
+    };
+
+    // ---- head: the first rounds are summed and kept; their largest e per thread gives the first bound
+    float head_e[LP_HEAD][LP_CHAINS];
+    const int head = min(rounds, LP_HEAD);
+    {
+        float tmax = 0.0f;
+#pragma unroll
+        for (int n = 0; n < LP_HEAD; ++n) {
+            if (n < head) {
+                e_values(raw[n], n * LP_BLOCK + t * LP_CHAINS, head_e[n]);
+#pragma unroll
+                for (int c = 0; c < LP_CHAINS; ++c) {
+                    acc[c] = acc[c] + head_e[n][c];
+                    tmax   = __builtin_fmaxf(tmax, head_e[n][c]);
+                }
+                if (n + LP_RING < rounds) {
+                    load(n, n + LP_RING);
+                }
+            }
+        }
+        rebound(order_key(tmax));
+#pragma unroll
+        for (int n = 0; n < LP_HEAD; ++n) {
+            if (n < head) {
+#pragma unroll
+                for (int c = 0; c < LP_CHAINS; ++c) {
+                    const int col = n * LP_BLOCK + t * LP_CHAINS + c;
+                    if (head_e[n][c] >= thr_low && col < p.V) {
+                        push(head_e[n][c], col);
+                    }
+                }
+            }
+        }
+    }
+    // ---- the rest of the row; the bound is raised again after 8, 16, 32, ... rounds
+    static_assert(LP_RING % LP_HEAD == 0 && LP_RING > LP_HEAD, "the ring continues where the head stopped");
+    int next_tighten = 2 * LP_HEAD;
+    for (int n0 = LP_HEAD; n0 < rounds; n0 += LP_RING) {
+#pragma unroll
+        for (int r = 0; r < LP_RING; ++r) {
+            const int n = n0 + r;
+            if (n < rounds) {
+                const int slot = (LP_HEAD + r) % LP_RING;
+                float     e[LP_CHAINS];
+                const int col0 = n * LP_BLOCK + t * LP_CHAINS;
+                e_values(raw[slot], col0, e);
+#pragma unroll
+                for (int c = 0; c < LP_CHAINS; ++c) {
+                    acc[c] = acc[c] + e[c];
+                    if (e[c] >= thr_low && col0 + c < p.V) {
+                        push(e[c], col0 + c);
+                    }
+                }
+                if (n + LP_RING < rounds) {
+                    load(slot, n + LP_RING);
+                }
+                if (n + 1 == next_tighten && n + 1 < rounds) {
+                    next_tighten *= 2;
+                    rebound(dmax);
+                }
+            }
+        }
+    }
+    // ---- the sum, in the reference's order: chain t = 4 * thread + c; butterflies with masks 16, 8, 4 run
+    // between the eight threads of a 32-chain group, masks 2 and 1 inside a thread
+#pragma unroll
+    for (int o = 4; o >= 1; o >>= 1) {
+#pragma unroll
+        for (int c = 0; c < LP_CHAINS; ++c) {
+            acc[c] = acc[c] + __shfl_xor(acc[c], o, WAVE);
+        }
+    }
+    acc[0] = acc[0] + acc[2];
+    acc[1] = acc[1] + acc[3];
+    acc[0] = acc[0] + acc[1];
+    if ((t & 7) == 0) {
+        warp_sum[t >> 3] = acc[0];
+    }
+    __syncthreads();
+    float total = t < 32 ? warp_sum[t] : 0.0f;
+    if (t < WAVE) {
+#pragma unroll
+        for (int o = 16; o >= 1; o >>= 1) {
+            total = total + __shfl_xor(total, o, WAVE);
+        }
+        if (t == 0) {
+            warp_sum[0] = total;
+        }
+    }
+    __syncthreads();
+    const float denom = uniform_f(warp_sum[0] + 1e-6f);
+    int         n     = s.n_cand;
+    __syncthreads();
+    // ---- candidates: e -> probability
+    if (n > TK_CCAP || !valid || !lp_ties_bounded<DT>(key_to_float(thr), denom)) {
+        // The list is incomplete, or fewer than k columns have a non-zero e (then columns of probability zero
+        // are picked too, by the reference's tie rules), or the k-th largest probability may be subnormal
+        // (ties without bound): the literal replay, on probabilities.
+        n = -1;
+    }
+    else {
+        int positive = 0;
+        for (int i = t; i < n; i += LP_THREADS) {
+            const uint32_t key = order_key(round_t<DT>(key_to_float(s.cand.key[i]) / denom));
+            s.cand.key[i]      = key;
+            positive += key > order_key(0.0f) ? 1 : 0;
+        }
+        positive = block_sum_i<LP_THREADS / WAVE>(positive, (int*)s.red32);
+        if (positive < k) {
+            // probabilities that round to zero reach into the top k: they tie with every other zero of the row
+            n = -1;
+        }
+        else if (n > k + k / 2 && n <= 4 * TK_THREADS) {
+            // keep what reaches the k-th largest of 256 slot maxima (at least k candidates do, and everything
+            // that ties with the k-th largest probability does)
+            uint32_t mx = 0u;
+            for (int i = t; i < n; i += TK_THREADS) {
+                const uint32_t key = s.cand.key[i];
+                mx                 = key > mx ? key : mx;
+            }
+            slot_key[par][t] = mx;
+            lds_barrier();
+            const uint32_t P = lean_kth_of_slots(slot_key[par], k);
+            lds_barrier();
+            if (P > KMIN) {
+                n = topk_prune(s, n, P);
+            }
+        }
+    }
+    FusedRow<DT, 0> r0(p, row);
+    ProbRow<DT>     prow{&r0, row_max, denom};
+    topk_select_lds<DT, ProbRow<DT>, true>(prow, s, n, KMIN, row, p.Vp, k, tp, p.max_top_k,
+                                           l.entries + (size_t)row * l.row_entries, true, u, p.end_ids, out);
+}
+
+// Launchers, one translation unit per element type (logprob_kernels.hip built with FTK_LP_DT = 0, 1, 2).
+// window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large.
+int lp_rowmax_launch_f32(int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                         const LogProbLaunch& lp);
+int lp_rowmax_launch_f16(int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                         const LogProbLaunch& lp);
+int lp_rowmax_launch_bf16(int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                          const LogProbLaunch& lp);
+int lp_row_launch_f32(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                      const LogProbLaunch& lp);
+int lp_row_launch_f16(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                      const LogProbLaunch& lp);
+int lp_row_launch_bf16(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                       const LogProbLaunch& lp);
+
+}  // namespace ftk

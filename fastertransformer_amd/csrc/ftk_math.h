@@ -74,11 +74,17 @@ FTK_HD float det_expf(float x)
     const float z = r * r;
     float       y = fma_rn(p, z, r) + 1.0f;
     const int   ni = (int)n;
+#if defined(__HIP_DEVICE_COMPILE__)
+    // one exact scaling by 2^ni (a single rounding when the result is subnormal): the same value as the two
+    // multiplications of the host branch, in one instruction
+    return __builtin_ldexpf(y, ni);
+#else
     const int   n1 = ni / 2;
     const int   n2 = ni - n1;
     y              = y * u2f((uint32_t)(n1 + 127) << 23);
     y              = y * u2f((uint32_t)(n2 + 127) << 23);
     return y;
+#endif
 }
 
 // Cephes logf: x = m 2^e, m in [sqrt(1/2), sqrt 2), f = m - 1, log x = f - f^2/2 + f^3 P(f) + e ln2.

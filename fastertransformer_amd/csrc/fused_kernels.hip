@@ -23,6 +23,7 @@
 #endif
 #include "ftk_fused.cuh"
 #include "ftk_lean.cuh"
+#include "ftk_logprob.cuh"
 
 namespace ftk {
 
@@ -69,6 +70,14 @@ history_bitmap_kernel(uint32_t* __restrict__ bitmaps, int bitmap_words, const in
 }  // namespace ftk
 
 using namespace ftk;
+
+#define FTK_HIP_CHECK(call)                                                                                            \
+    do {                                                                                                               \
+        const hipError_t e_ = (call);                                                                                  \
+        if (e_ != hipSuccess) {                                                                                        \
+            return (int)e_;                                                                                            \
+        }                                                                                                              \
+    } while (0)
 
 // ---- optional per-kernel timing (HIP events on the caller's stream) ------------------------------
 namespace {
@@ -181,6 +190,14 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
     // Launches with a small k and no bias take the lean gather, which cuts a row differently.
     const int      lean_mode = many == 0 && a->embedding_bias == nullptr && !g_fused_force_general ? 1 : 0;
+    // Log-prob outputs: the two-read step covers what the lean gather covers, for vocabularies of at least 1024
+    // columns (the reference's softmax block) in rows that start on 16-byte boundaries.
+    const bool want_log_probs = a->cum_log_probs != nullptr || a->output_log_probs != nullptr;
+    if (want_log_probs
+        && (lean_mode == 0 || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
+            || ((uintptr_t)a->logits & 15u) != 0)) {
+        return FTK_ERR_UNSUPPORTED;
+    }
     const LeanPlan lplan     = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * LG_OCCUPANCY);
     const size_t   lean_bytes =
         (size_t)(rows > 0 ? rows : 0) * lplan.splits * (sizeof(TopkChunkHeader) + (size_t)TK_CCAP * sizeof(TopkEntry));
@@ -237,9 +254,9 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         const int    epv        = 16 / elem;
         const size_t range_cols = lean_mode != 0 ? (size_t)lplan.subs_per_wg * LG_SUB_VECS * epv + 2 * epv :
                                                    (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
-        const size_t words      = range_cols / 32 + 4;
+        const size_t words      = (want_log_probs ? (size_t)a->vocab_size : range_cols) / 32 + 4;
         const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && many == 0
-                           && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1
+                           && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1 && !want_log_probs
                                || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
         if (local) {
             p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
@@ -297,6 +314,38 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         l.row_entries  = (size_t)lplan.splits * TK_CCAP;
         l.entries      = (TopkEntry*)(l.headers + (size_t)rows * lplan.splits);
         const dim3 lgrid(lplan.splits, rows);
+        if (want_log_probs) {
+            LogProbLaunch lp;
+            lp.cum_log_probs    = a->cum_log_probs;
+            lp.output_log_probs = a->output_log_probs;
+            lp.partial_max      = (float*)l.headers;  // one float per list header slot: the lists are not used
+            lp.splits           = lplan.splits;
+            hipEvent_t e0, e1;
+            take_events(1, &e0, &e1);
+            if (e0 != nullptr) {
+                FTK_HIP_CHECK(hipEventRecord(e0, st));
+            }
+            rc = a->dtype == FTK_DTYPE_F32 ? lp_rowmax_launch_f32(window, lgrid, st, p, l, lp) :
+                 a->dtype == FTK_DTYPE_F16 ? lp_rowmax_launch_f16(window, lgrid, st, p, l, lp) :
+                                             lp_rowmax_launch_bf16(window, lgrid, st, p, l, lp);
+            if (rc != 0) {
+                return rc;
+            }
+            if (e1 != nullptr) {
+                FTK_HIP_CHECK(hipEventRecord(e1, st));
+            }
+            take_events(2, &e0, &e1);
+            if (e0 != nullptr) {
+                FTK_HIP_CHECK(hipEventRecord(e0, st));
+            }
+            rc = a->dtype == FTK_DTYPE_F32 ? lp_row_launch_f32(window, rows, st, p, l, lp) :
+                 a->dtype == FTK_DTYPE_F16 ? lp_row_launch_f16(window, rows, st, p, l, lp) :
+                                             lp_row_launch_bf16(window, rows, st, p, l, lp);
+            if (rc == 0 && e1 != nullptr) {
+                FTK_HIP_CHECK(hipEventRecord(e1, st));
+            }
+            return rc;
+        }
         hipEvent_t e0, e1;
         take_events(1, &e0, &e1);
         if (a->dtype == FTK_DTYPE_F32) {

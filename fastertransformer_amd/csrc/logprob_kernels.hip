@@ -1,0 +1,60 @@
+// Instances of the two-read log-prob step (ftk_logprob.cuh) for one element type: this file is compiled once
+// per type with -DFTK_LP_DT=0 (f32), 1 (f16), 2 (bf16).
+#include <type_traits>
+
+#include "ftk_logprob.cuh"
+
+#ifndef FTK_LP_DT
+#error "build with -DFTK_LP_DT=0|1|2"
+#endif
+
+namespace ftk {
+
+#if FTK_LP_DT == 0
+int lp_rowmax_launch_f32
+#elif FTK_LP_DT == 1
+int lp_rowmax_launch_f16
+#else
+int lp_rowmax_launch_bf16
+#endif
+    (int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, const LogProbLaunch& lp)
+{
+    constexpr int DT = FTK_LP_DT;
+    if (window == 0) {
+        hipLaunchKernelGGL((lp_rowmax_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>), grid, dim3(LG_THREADS), 0, st, p, l, lp);
+    }
+    else if (window == 2) {
+        hipLaunchKernelGGL((lp_rowmax_kernel<DT, FUSED_BITMAP_WORDS_LARGE>), grid, dim3(LG_THREADS), 0, st, p, l, lp);
+    }
+    else {
+        hipLaunchKernelGGL((lp_rowmax_kernel<DT, FUSED_BITMAP_WORDS_SMALL>), grid, dim3(LG_THREADS), 0, st, p, l, lp);
+    }
+    return (int)hipGetLastError();
+}
+
+#if FTK_LP_DT == 0
+int lp_row_launch_f32
+#elif FTK_LP_DT == 1
+int lp_row_launch_f16
+#else
+int lp_row_launch_bf16
+#endif
+    (int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, const LogProbLaunch& lp)
+{
+    constexpr int DT = FTK_LP_DT;
+    if (window == 0) {
+        hipLaunchKernelGGL((lp_row_kernel<DT, FUSED_BITMAP_WORDS_GLOBAL>), dim3(rows), dim3(LP_THREADS), 0, st, p, l,
+                           lp);
+    }
+    else if (window == 2) {
+        hipLaunchKernelGGL((lp_row_kernel<DT, FUSED_BITMAP_WORDS_LARGE>), dim3(rows), dim3(LP_THREADS), 0, st, p, l,
+                           lp);
+    }
+    else {
+        hipLaunchKernelGGL((lp_row_kernel<DT, FUSED_BITMAP_WORDS_SMALL>), dim3(rows), dim3(LP_THREADS), 0, st, p, l,
+                           lp);
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace ftk

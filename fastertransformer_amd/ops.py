@@ -75,6 +75,7 @@ _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_c
 
 # error codes of include/ftk_sampling.h (positive values are hipError_t)
 FTK_ERR_DTYPE, FTK_ERR_TOPK_DOMAIN, FTK_ERR_ARGUMENT, FTK_ERR_WORKSPACE, FTK_ERR_STATIC_WORKSPACE = -1, -2, -3, -4, -5
+FTK_ERR_UNSUPPORTED = -6
 FUSED_STATIC_WORKSPACE_BYTES = 32 << 20
 
 
@@ -188,7 +189,8 @@ class FusedTopkArgs(C.Structure):
         ("temperatures", _vp), ("penalties", _vp), ("penalty_type", _i), ("min_lengths", _vp), ("end_ids", _vp),
         ("input_lengths", _vp), ("output_ids", _vp), ("top_ks", _vp), ("top_ps", _vp), ("max_top_k", _i),
         ("skip_decode", _vp), ("rng_state", _vp), ("uniform_draws", _vp), ("ids", _vp), ("sequence_length", _vp),
-        ("finished", _vp), ("workspace", _vp), ("workspace_size", _sz),
+        ("finished", _vp), ("cum_log_probs", _vp), ("output_log_probs", _vp), ("workspace", _vp),
+        ("workspace_size", _sz),
     ]
 
 

@@ -131,23 +131,23 @@ void TopKSamplingLayer<T>::ensureWorkspace(int local_batch_size)
     }
 }
 
+// FT_SAMPLING_DISABLE_FUSED=1 forces the kernel-by-kernel sequence of the reference (read at every step, so
+// that one process can run both).
 static bool fusedDisabled()
 {
-    static const bool disabled = []() {
-        const char* env = std::getenv("FT_SAMPLING_DISABLE_FUSED");
-        return env != nullptr && env[0] == '1';
-    }();
-    return disabled;
+    const char* env = std::getenv("FT_SAMPLING_DISABLE_FUSED");
+    return env != nullptr && env[0] == '1';
 }
 
-// One streaming pass over the logits for the whole penalty + mask + top-k pipeline. Taken when no
-// log-prob output is requested (those need the full-row softmax first) and no extension penalty is set.
+// One streaming pass over the logits for the whole penalty + mask + top-k pipeline - two passes when log-prob
+// outputs are requested, which need the probabilities of the whole row. Not taken with the frequency-penalty
+// extension, nor for the configurations the fused step reports as unsupported with log-probs.
 template<typename T>
 bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_tensors)
 {
     float* cum_log_probs    = output_tensors->at("cum_log_probs", Tensor()).template getPtr<float>();
     float* output_log_probs = output_tensors->at("output_log_probs", Tensor()).template getPtr<float>();
-    if (fusedDisabled() || cum_log_probs != nullptr || output_log_probs != nullptr || this->has_frequency_penalty_) {
+    if (fusedDisabled() || this->has_frequency_penalty_) {
         return false;
     }
     const int batch_size       = output_tensors->at("output_ids").shape[1];
@@ -202,9 +202,15 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
     a.ids = output_tensors->at("output_ids").template getPtrWithOffset<int>((size_t)step * batch_size + off);
     a.sequence_length = output_tensors->at("sequence_length", Tensor()).template getPtr<int>();
     a.finished        = output_tensors->at("finished", Tensor()).template getPtr<bool>();
+    a.cum_log_probs    = cum_log_probs;
+    a.output_log_probs = output_log_probs;
     // size query (null workspace), grow if this window needs more than setup() reserved
     a.workspace = nullptr;
-    check_ftk(ftk_fused_topk_step(&a, stream_));
+    const int query = ftk_fused_topk_step(&a, stream_);
+    if (query == FTK_ERR_UNSUPPORTED) {
+        return false;  // log-probs with a bias, a large k, a tiny vocabulary or unaligned rows: the kernel sequence
+    }
+    check_ftk(query);
     if (a.workspace_size > sampling_workspace_size_) {
         sampling_workspace_      = allocator_->reMalloc(sampling_workspace_, a.workspace_size, false);
         sampling_workspace_size_ = a.workspace_size;

@@ -37,7 +37,8 @@ enum {
     FTK_ERR_TOPK_DOMAIN = -2, /* top-k outside [1, 1024]: std::domain_error in sampling_topk_kernels.cu:393-394 */
     FTK_ERR_ARGUMENT    = -3, /* null / inconsistent argument */
     FTK_ERR_WORKSPACE   = -4, /* workspace smaller than the queried size */
-    FTK_ERR_STATIC_WORKSPACE = -5 /* ftk_fused_topk_step_static: the step needs more than the library's fixed array */
+    FTK_ERR_STATIC_WORKSPACE = -5, /* ftk_fused_topk_step_static: the step needs more than the library's fixed array */
+    FTK_ERR_UNSUPPORTED = -6 /* ftk_fused_topk_step: log-prob outputs for a configuration the fused step does not cover */
 };
 
 /* Per-row generator state; replaces curandState_t (48 bytes) in every signature. Row b draws
@@ -171,9 +172,10 @@ int ftk_invoke_length_criterion(bool* finished, bool* should_stop, int* h_pinned
 /* ---- fused decode step ---------------------------------------------------------------------
  * One call = the kernel sequence BaseSamplingLayer<T>::forward + TopKSamplingLayer<T>::runSampling
  * issue for the rows a top-k layer owns (layers/sampling_layers/BaseSamplingLayer.cc:255-359,
- * layers/sampling_layers/TopKSamplingLayer.cu:189-268) when no log-prob output is requested:
- * temperature(+bias), repetition/presence penalty, min-length, end/pad mask, top-k selection and sampling,
- * with the logits read from HBM once and never written (the reference leaves them penalised). Bad words are
+ * layers/sampling_layers/TopKSamplingLayer.cu:189-268): temperature(+bias), repetition/presence penalty,
+ * min-length, end/pad mask, (softmax when log-probs are requested,) top-k selection and sampling, with the
+ * logits read from HBM once - twice with log-probs - and never written (the reference leaves them penalised,
+ * or turned into probabilities). Bad words are
  * not part of it: DynamicDecodeLayer masks them on the logits before the sampling layers run
  * (ftk_invoke_ban_bad_words), here as in the reference. */
 typedef struct ftk_fused_topk_args {
@@ -202,6 +204,13 @@ typedef struct ftk_fused_topk_args {
     int*  ids;             /* [local]: output_ids + step*batch_size + window offset */
     int*  sequence_length; /* [local] or NULL */
     bool* finished;        /* [local] or NULL */
+    /* Log-prob outputs (both NULL: none). With either one the step takes the probabilities of the whole row as
+     * the reference does (softmax after the penalties, top-k on probabilities): cum_log_probs[b] += log p,
+     * output_log_probs[b] = log p - log(sum of the k probabilities). Covered for launches without embedding
+     * bias, largest k <= 128, vocab_size >= 1024 and 16-byte aligned rows; anything else returns
+     * FTK_ERR_UNSUPPORTED (also for the size query) and launches nothing: run the kernel sequence instead. */
+    float* cum_log_probs;    /* [local] or NULL */
+    float* output_log_probs; /* [local] or NULL: the row of this step */
     void*  workspace;
     size_t workspace_size;
 } ftk_fused_topk_args;

@@ -1,9 +1,30 @@
 """Drives the product's DynamicDecodeLayer (GPU, through the C handle API) and the oracle's layer
 restatement (CPU) with the same named tensors, step by step, and compares every output."""
+import contextlib
+import os
+
 import numpy as np
 
 import ft_oracle as O
 from helpers import bits, to_numpy, to_torch
+
+
+@contextlib.contextmanager
+def kernel_sequence(enabled=True):
+    """Inside: the product's top-k layer runs the reference's kernel-by-kernel sequence (which mutates the caller's
+    logits like the reference) instead of its fused step (which leaves them alone)."""
+    key, old = "FT_SAMPLING_DISABLE_FUSED", os.environ.get("FT_SAMPLING_DISABLE_FUSED")
+    if enabled:
+        os.environ[key] = "1"
+    else:
+        os.environ.pop(key, None)
+    try:
+        yield
+    finally:
+        if old is None:
+            os.environ.pop(key, None)
+        else:
+            os.environ[key] = old
 
 
 class Case:

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import ft_oracle as O
-from decode_harness import Case, OracleRunner, ProductRunner, compare
+from decode_harness import Case, OracleRunner, ProductRunner, compare, kernel_sequence
 from helpers import DTYPES, DTYPE_NAMES, make_logits, make_word_list, to_numpy, to_torch, uniforms
 
 pytestmark = pytest.mark.gpu
@@ -192,8 +192,12 @@ def test_config5_full_loop(dt):
         xf[rng.random(B) < 0.15, end] = 30.0  # some rows finish early
         return O.to_storage(xf, dt)
 
-    snap = _run_case(c, rng, 12, logits_fn, check_logits=True)
-    assert snap["finished"].all() and bool(snap["should_stop"][0])
+    # the fused step with log-probs (two reads of the logits, none mutated), then the reference's kernel sequence,
+    # whose in-place results (penalised logits turned into probabilities) must match the oracle's bit for bit
+    for sequence in (False, True):
+        with kernel_sequence(sequence):
+            snap = _run_case(c, rng, 12, logits_fn, check_logits=sequence)
+        assert snap["finished"].all() and bool(snap["should_stop"][0])
 
 
 def test_headline_step_topk_topp_penalty_fused():
@@ -384,3 +388,67 @@ def test_fused_step_large_k_with_bias_and_history(dt, max_k):
                  prompt=_history(rng, H, B, V, zipf=1.3), input_lengths=rng.integers(H // 2, H + 1, B),
                  end_ids=rng.integers(0, V, B).astype(np.int32), **kw)
         _run_case(c, rng, 3, lambda i: make_logits(rng, dt, B, V, Vp, 2.0), check_logits=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("seed", [0, 1])
+def test_fused_step_with_log_probs_random_scenarios(dt, seed):
+    """The two-read fused step (log-probs requested): random batches, vocabularies from 1024 columns up (aligned
+    and padded), per-row k up to 128 with and without top-p, temperature, repetition or presence penalty over short
+    and long histories, min length, rows that finish; ids / flags / lengths bit-exact, log-probs to tolerance."""
+    rng = np.random.default_rng(7000 + 10 * dt + seed)
+    for case in range(4):
+        B = int(rng.choice([1, 5, 33, 300]))
+        V = int(rng.choice([1024, int(rng.integers(1025, 9000)), int(rng.integers(30000, 160000))]))
+        Vp = (V + 7) // 8 * 8 + int(rng.choice([0, 8, 64]))
+        H = int(rng.choice([3, 40, 300]))
+        max_k = int(rng.choice([1, 8, 64, 128]))
+        ks = rng.integers(1, max_k + 1, B).astype(np.uint32)
+        ks[0] = max_k
+        ps = np.where(rng.random(B) < 0.5, 1.0, rng.uniform(0.2, 0.99, B)).astype(np.float32)
+        kw = {}
+        if rng.random() < 0.7:
+            kw["temperature"] = rng.uniform(0.5, 1.6, B)
+        pen = int(rng.integers(0, 3))
+        if pen == 1:
+            kw["repetition_penalty"] = rng.uniform(1.0, 1.6, B)
+        elif pen == 2:
+            kw["presence_penalty"] = rng.uniform(0.0, 1.5, B)
+        if rng.random() < 0.5:
+            kw["min_length"] = rng.integers(0, 4, B)
+        end = rng.integers(0, V, B).astype(np.int32)
+        c = Case(dt, B, V, Vp, max_input_length=H, gen_len=3, runtime_top_k=ks, runtime_top_p=ps,
+                 prompt=_history(rng, H, B, V, zipf=1.3 if rng.random() < 0.5 else None),
+                 input_lengths=rng.integers(1, H + 1, B), end_ids=end, with_cum=True, with_out_lp=True, **kw)
+        scale = float(rng.uniform(0.5, 4.0))
+
+        def logits_fn(i):
+            x = O.to_f32(make_logits(rng, dt, B, V, Vp, scale), dt)
+            rows = rng.random(B) < 0.2
+            x[rows, end[rows]] = 40.0  # these rows finish
+            return O.to_storage(x, dt)
+
+        _run_case(c, rng, 3, logits_fn, check_logits=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_fused_step_with_log_probs_ties_and_flat_rows(dt):
+    """Rows where probabilities tie or vanish: logits from a handful of distinct values, a flat row (every
+    probability equal; zero after rounding in fp16 at this vocabulary), one dominant column (all other
+    probabilities round to zero), and rows where fewer than k columns have a non-zero probability. The picks must
+    follow the reference's tie rules on probabilities."""
+    rng = np.random.default_rng(7100 + dt)
+    B, V, H = 12, 70016, 4
+    x = rng.standard_normal((B, V)).astype(np.float32)
+    x[0:3] = rng.choice(np.array([-2.0, 0.5, 1.0, 1.5], np.float32), (3, V))   # few distinct values
+    x[3] = 0.25                                                                 # flat
+    x[4] = -20.0
+    x[4, 777] = 30.0                                                            # one column takes everything
+    x[5] = -60.0
+    x[5, rng.integers(0, V, 20)] = rng.uniform(0, 3, 20)                        # 20 live columns, k = 64
+    x[6:9] = np.round(x[6:9] * 4) / 4                                           # quarter steps: many ties
+    c = Case(dt, B, V, V, max_input_length=H, gen_len=2, runtime_top_k=[64], runtime_top_p=[0.95],
+             temperature=[0.9], repetition_penalty=[1.2], prompt=_history(rng, H, B, V), with_cum=True,
+             with_out_lp=True)
+    xs = O.to_storage(x, dt)
+    _run_case(c, rng, 2, lambda i: xs, check_logits=False)
