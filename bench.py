@@ -129,7 +129,7 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
         one_step(i)
     torch.cuda.synchronize()
     kernel_ms = []
-    for k in range(3):
+    for k in range(4):
         tot, n = C.c_double(0.0), C.c_int(0)
         ops.check(lib.ftk_profile_read(k, C.addressof(tot), C.addressof(n)))
         kernel_ms.append((tot.value / n.value) if n.value else 0.0)
@@ -156,7 +156,7 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     dominant = "lean_gather_kernel" if lean else ("fused_gather_kernel" if kernel_ms[2] > 0 else "fused_row_kernel")
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
-        kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2]),
+        kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2], maxima=kernel_ms[3]),
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
                       traffic=TRAFFIC_BYTES_PER_LAUNCH, kernel=dominant, algorithmic_bytes_per_launch=alg),
         step_gbs=alg / (gpu_ms / steps * 1e-3) / 1e9,

@@ -359,6 +359,10 @@ struct FusedLaunch {
     size_t           row_entries;
     TopkChunkHeader* headers;
     TopkEntry*       entries;
+    // two-read selection for a large k (lean_gather_kernel, slots and preset modes): per row and workgroup,
+    // 256 * slot_u maxima of disjoint groups of columns
+    uint32_t* slots;
+    int       slot_u;
 };
 
 __device__ __forceinline__ float fused_row_draw(TopkShared& s, const FusedLaunch& l, int row)

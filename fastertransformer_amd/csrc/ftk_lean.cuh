@@ -135,7 +135,25 @@ __device__ __forceinline__ uint4 lean_stream_load(const uint4* p)
 
 constexpr int LG_HIST_U = 8;  // history ids a thread requests before the logits (2048 positions per workgroup)
 
-template<int DT, int BMW, int OCC, int R>
+// What a launch of lean_gather_kernel does.
+//   STREAM: one read of the row. Every workgroup bounds the k-th largest of its own columns as it goes
+//           (k <= LG_MAX_K).
+//   SLOTS / PRESET: two reads, for any k up to 1024. The first launch (SLOTS) only takes maxima: 256 * slot_u
+//           per workgroup, each over a group of columns of its own. The k-th largest of a row's maxima bounds
+//           the row's k-th largest value from below, and with two to four times k maxima only little more than
+//           k columns reach it. The second launch (PRESET) finds that bound first and gathers against it.
+enum { LG_MODE_STREAM = 0, LG_MODE_SLOTS = 1, LG_MODE_PRESET = 2 };
+constexpr int LG_SLOT_U_MAX    = 4;   // maxima a thread delivers: one per vector of a sub-tile
+constexpr int LG_SLOT_KEYS_MAX = 32;  // maxima of a row a thread of the PRESET launch holds: splits * slot_u
+
+// slot_u for a row cut into `splits`; 0: too many workgroups per row for the two-read selection
+inline int lean_slot_u(int splits)
+{
+    const int u = LG_SLOT_KEYS_MAX / (splits > 0 ? splits : 1);
+    return u >= 4 ? 4 : (u >= 2 ? 2 : u);
+}
+
+template<int DT, int BMW, int OCC, int R, int MODE>
 __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParams p, FusedLaunch l)
 {
     typedef Storage<DT>   S;
@@ -183,6 +201,17 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     for (int r = 0; r < R; ++r) {
         if (r < nsub) {
             load(r, r);
+        }
+    }
+
+    // PRESET: the row's maxima from the SLOTS launch, thread t looks at slot t of every group
+    uint32_t  slot_keys[MODE == LG_MODE_PRESET ? LG_SLOT_KEYS_MAX : 1];
+    const int n_slot_keys = MODE == LG_MODE_PRESET ? (int)gridDim.x * l.slot_u : 0;
+    if constexpr (MODE == LG_MODE_PRESET) {
+        const uint32_t* mine = l.slots + (size_t)row * gridDim.x * l.slot_u * LG_THREADS + t;
+#pragma unroll
+        for (int i = 0; i < LG_SLOT_KEYS_MAX; ++i) {
+            slot_keys[i] = i < n_slot_keys ? mine[(size_t)i * LG_THREADS] : 0u;
         }
     }
 
@@ -274,10 +303,102 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     };
     set_threshold(KMIN);
 
+    // flags of the vector that starts at column `first`: one bit per column of the history
+    auto vector_flags = [&](int first) -> uint32_t {
+        if (aligned_bits) {
+            const int brel = max(first - rowctx.bm_origin, 0);
+            return (rowctx.bm_word(brel >> 5) >> (brel & 31)) & ((1u << EPV) - 1u);
+        }
+        return bitsv ? rowctx.vector_bits(first, EPV) : 0u;
+    };
+
+    if constexpr (MODE == LG_MODE_SLOTS) {
+        // ---- maxima only. Vectors whose elements all take the plain transform count (no history column, not
+        // the masked end id): the transform keeps the order, so the maximum of the stored values gives the
+        // largest final value of the group.
+        float sm[LG_NV];
+#pragma unroll
+        for (int j = 0; j < LG_NV; ++j) {
+            sm[j] = NEG_INF;
+        }
+        for (int q0 = 0; q0 < nsub; q0 += R) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int q = q0 + r;
+                if (q < nsub) {
+#pragma unroll
+                    for (int j = 0; j < LG_NV; ++j) {
+                        const int  rel   = q * LG_SUB_VECS + j * LG_THREADS + t;
+                        const int  first = (vb + rel) * EPV - a;
+                        const bool clean = rel < nvec && rowctx.plain_vector(first, EPV) && vector_flags(first) == 0u;
+                        sm[j] = __builtin_fmaxf(sm[j], clean ? lean_raw_max<DT>(raw[r][j]) : NEG_INF);
+                    }
+                    if (q + R < nsub) {
+                        load(r, q + R);
+                    }
+                }
+            }
+        }
+        uint32_t key[LG_NV];
+#pragma unroll
+        for (int j = 0; j < LG_NV; ++j) {
+            key[j] = all_hit ? 0u : order_key(rowctx.fast(sm[j]));
+        }
+        uint32_t* dst = l.slots + ((size_t)row * gridDim.x + chunk) * l.slot_u * LG_THREADS + t;
+        if (l.slot_u == 4) {
+#pragma unroll
+            for (int j = 0; j < LG_NV; ++j) {
+                dst[j * LG_THREADS] = key[j];
+            }
+        }
+        else if (l.slot_u == 2) {
+            dst[0]          = max(key[0], key[1]);
+            dst[LG_THREADS] = max(key[2], key[3]);
+        }
+        else {
+            dst[0] = max(max(key[0], key[1]), max(key[2], key[3]));
+        }
+        return;
+    }
+
+    if constexpr (MODE == LG_MODE_PRESET) {
+        // ---- the bound of the row: the largest P, to within its low sixteen bits, that at least k of the
+        // row's maxima reach. Every workgroup of the row finds the same one.
+        uint32_t P  = 0u;
+        int      pp = 0;
+#pragma unroll 1
+        for (int bit = 31; bit >= 16; --bit) {
+            const uint32_t cand = P | (1u << bit);
+            int            c    = 0;
+#pragma unroll
+            for (int i = 0; i < LG_SLOT_KEYS_MAX; ++i) {
+                if (i < n_slot_keys) {
+                    c += slot_keys[i] >= cand ? 1 : 0;
+                }
+            }
+            c = wave_sum_i(c);
+            if (lane == 0) {
+                s.slot_key[pp][wv] = (uint32_t)c;
+            }
+            lds_barrier();
+            int total = 0;
+#pragma unroll
+            for (int g = 0; g < LG_WAVES; ++g) {
+                total += (int)s.slot_key[pp][g];
+            }
+            pp ^= 1;
+            P = total >= k ? cand : P;
+        }
+        if (P >= KMIN) {
+            set_threshold(P);
+            valid = true;
+        }
+    }
+
     // ---- first bound: the k-th largest of the thread maxima over the first two sub-tiles. Only vectors whose
     // elements all take the plain transform count (no history column, not the masked end id), so every
     // maximum is the final value of an element.
-    if (nsub > 0) {
+    if (MODE == LG_MODE_STREAM && nsub > 0) {
         float tmax = NEG_INF;
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
@@ -286,15 +407,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 for (int j = 0; j < LG_NV; ++j) {
                     const int  rel   = sb * LG_SUB_VECS + j * LG_THREADS + t;
                     const int  first = (vb + rel) * EPV - a;
-                    uint32_t   bits  = 0u;
-                    if (aligned_bits) {
-                        const int brel = max(first - rowctx.bm_origin, 0);
-                        bits           = (rowctx.bm_word(brel >> 5) >> (brel & 31)) & ((1u << EPV) - 1u);
-                    }
-                    else if (bitsv) {
-                        bits = rowctx.vector_bits(first, EPV);
-                    }
-                    const bool clean = rel < nvec && rowctx.plain_vector(first, EPV) && bits == 0u;
+                    const bool clean = rel < nvec && rowctx.plain_vector(first, EPV) && vector_flags(first) == 0u;
                     float vm = NEG_INF;
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) {
@@ -428,7 +541,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 if (q + R < nsub) {
                     load(r, q + R);
                 }
-                const bool tighten = q + 1 == next_tighten && q + 1 < nsub;
+                const bool tighten = MODE == LG_MODE_STREAM && q + 1 == next_tighten && q + 1 < nsub;
                 if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
                     drain();
                 }
@@ -610,7 +723,7 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
     if (n > TK_CCAP) {
         return -2;  // the union does not fit the list: the caller merges with the general routine
     }
-    if (n > k + k / 2 && n <= 4 * TK_THREADS && k <= LG_MAX_K) {
+    if (n > k + k / 2 && n <= 4 * TK_THREADS && k <= LG_MAX_K && k <= TK_THREADS) {
         // Far more candidates than needed (every workgroup of the gather reports the best of its own columns):
         // raise the bound to the k-th largest of 256 slot maxima (slot t: entries t, t + 256, ...), which at
         // least k entries reach, and keep what reaches it. The replay of the tie orders below ranks every
@@ -687,9 +800,9 @@ __global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, 
 }
 
 // Launchers, one translation unit per element type (lean_kernels.hip built with FTK_LEAN_DT = 0, 1, 2).
-// window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large.
+// mode: LG_MODE_*; window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large.
 // start / stop: optional events carried by the launch.
-int lean_gather_launch_f32(int window, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_f32(int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 int lean_select_launch_f32(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                            hipEvent_t stop);
@@ -697,9 +810,9 @@ int lean_select_launch_f16(int rows, hipStream_t st, const FusedParams& p, const
                            hipEvent_t stop);
 int lean_select_launch_bf16(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                             hipEvent_t stop);
-int lean_gather_launch_f16(int window, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_f16(int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
-int lean_gather_launch_bf16(int window, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_bf16(int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p,
                             const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 
 // workgroups per compute unit the lean gather is built for, and sub-tiles in flight per thread

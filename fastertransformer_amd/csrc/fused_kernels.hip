@@ -85,7 +85,7 @@ struct KernelTimer {
     std::vector<hipEvent_t> start, stop;
     int                     used = 0;
 };
-KernelTimer g_timers[3];
+KernelTimer g_timers[4];
 bool        g_profile = false;
 
 // Launches `kernel`; when timing is on, the launch itself carries a start and a stop event, so the
@@ -136,7 +136,7 @@ extern "C" int ftk_profile_enable(int max_launches)
 
 extern "C" int ftk_profile_read(int kernel, double* total_ms, int* launches)
 {
-    if (kernel < 0 || kernel > 2 || total_ms == nullptr || launches == nullptr) {
+    if (kernel < 0 || kernel > 3 || total_ms == nullptr || launches == nullptr) {
         return FTK_ERR_ARGUMENT;
     }
     KernelTimer& t = g_timers[kernel];
@@ -188,19 +188,27 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const int      many         = topk_many_level(a->max_top_k);  // > 0: the large-k kernels (whole-row bitmaps only)
     const int      bitmap_words = (a->vocab_size_padded + 31) / 32 + 1;  // +1: vector_bits may peek one word ahead
     const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
-    // Launches with a small k and no bias take the lean gather, which cuts a row differently.
-    const int      lean_mode = many == 0 && a->embedding_bias == nullptr && !g_fused_force_general ? 1 : 0;
+    // Launches without a bias take the lean gather, which cuts a row differently: in one read of the logits
+    // for a small k (lean_mode 1), in two for a large one (2) where a row yields at least twice k maxima.
+    const LeanPlan lplan      = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * LG_OCCUPANCY);
+    const int      slot_u     = lean_slot_u(lplan.splits);
+    const bool     lean_ok    = a->embedding_bias == nullptr && !g_fused_force_general;
+    const bool     two_reads  = lean_ok && many > 0 && slot_u > 0
+                           && (size_t)lplan.splits * slot_u * LG_THREADS >= (size_t)2 * a->max_top_k
+                           && (size_t)a->vocab_size / (16 / elem) >= (size_t)lplan.splits * slot_u * LG_THREADS;
+    const int      lean_mode  = lean_ok && many == 0 ? 1 : (two_reads ? 2 : 0);
     // Log-prob outputs: the two-read step covers what the lean gather covers, for vocabularies of at least 1024
     // columns (the reference's softmax block) in rows that start on 16-byte boundaries.
     const bool want_log_probs = a->cum_log_probs != nullptr || a->output_log_probs != nullptr;
     if (want_log_probs
-        && (lean_mode == 0 || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
+        && (lean_mode != 1 || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
             || ((uintptr_t)a->logits & 15u) != 0)) {
         return FTK_ERR_UNSUPPORTED;
     }
-    const LeanPlan lplan     = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * LG_OCCUPANCY);
+    const size_t   slot_bytes = lean_mode == 2 ? (size_t)lplan.splits * slot_u * LG_THREADS * sizeof(uint32_t) : 0;
     const size_t   lean_bytes =
-        (size_t)(rows > 0 ? rows : 0) * lplan.splits * (sizeof(TopkChunkHeader) + (size_t)TK_CCAP * sizeof(TopkEntry));
+        (size_t)(rows > 0 ? rows : 0)
+        * (lplan.splits * (sizeof(TopkChunkHeader) + (size_t)TK_CCAP * sizeof(TopkEntry)) + slot_bytes);
     const size_t   need = bitmap_bytes + (lean_mode != 0 && lean_bytes > plan.bytes ? lean_bytes : plan.bytes);
     if (a->workspace == nullptr) {
         a->workspace_size = need;
@@ -255,7 +263,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         const size_t range_cols = lean_mode != 0 ? (size_t)lplan.subs_per_wg * LG_SUB_VECS * epv + 2 * epv :
                                                    (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
         const size_t words      = (want_log_probs ? (size_t)a->vocab_size : range_cols) / 32 + 4;
-        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && many == 0
+        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && (many == 0 || lean_mode == 2)
                            && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1 && !want_log_probs
                                || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
         if (local) {
@@ -285,6 +293,8 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     l.subs_per_wg     = 0;
     l.headers         = (TopkChunkHeader*)(ws + bitmap_bytes);
     l.entries         = (TopkEntry*)(l.headers + (size_t)rows * plan.splits);
+    l.slots           = nullptr;
+    l.slot_u          = 0;
     // events carried by a launch when per-kernel timing is on
     auto take_events = [&](int which, hipEvent_t* e0, hipEvent_t* e1) {
         KernelTimer& tm = g_timers[which];
@@ -346,20 +356,30 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             }
             return rc;
         }
-        hipEvent_t e0, e1;
-        take_events(1, &e0, &e1);
-        if (a->dtype == FTK_DTYPE_F32) {
-            rc = lean_gather_launch_f32(window, lgrid, st, p, l, e0, e1);
+        auto launch_lean = [&](int mode, int timer) -> int {
+            hipEvent_t e0, e1;
+            take_events(timer, &e0, &e1);
+            if (a->dtype == FTK_DTYPE_F32) {
+                return lean_gather_launch_f32(mode, window, lgrid, st, p, l, e0, e1);
+            }
+            if (a->dtype == FTK_DTYPE_F16) {
+                return lean_gather_launch_f16(mode, window, lgrid, st, p, l, e0, e1);
+            }
+            return lean_gather_launch_bf16(mode, window, lgrid, st, p, l, e0, e1);
+        };
+        if (lean_mode == 2) {
+            l.slots  = (uint32_t*)(l.entries + (size_t)rows * l.row_entries);
+            l.slot_u = slot_u;
+            rc       = launch_lean(LG_MODE_SLOTS, 3);
+            if (rc != 0) {
+                return rc;
+            }
         }
-        else if (a->dtype == FTK_DTYPE_F16) {
-            rc = lean_gather_launch_f16(window, lgrid, st, p, l, e0, e1);
-        }
-        else {
-            rc = lean_gather_launch_bf16(window, lgrid, st, p, l, e0, e1);
-        }
+        rc = launch_lean(lean_mode == 2 ? LG_MODE_PRESET : LG_MODE_STREAM, 1);
         if (rc != 0) {
             return rc;
         }
+        hipEvent_t e0, e1;
         take_events(2, &e0, &e1);
         if (a->dtype == FTK_DTYPE_F32) {
             return lean_select_launch_f32(rows, st, p, l, e0, e1);

@@ -8,31 +8,31 @@
 
 namespace ftk {
 
-template<int BMW, int OCC, int R>
+template<int BMW, int OCC, int R, int MODE>
 static int lean_launch_one(dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                            hipEvent_t stop)
 {
     if (start != nullptr) {
-        hipExtLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R>), grid, dim3(LG_THREADS), 0, st, start,
+        hipExtLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R, MODE>), grid, dim3(LG_THREADS), 0, st, start,
                               stop, 0, p, l);
     }
     else {
-        hipLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R>), grid, dim3(LG_THREADS), 0, st, p, l);
+        hipLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R, MODE>), grid, dim3(LG_THREADS), 0, st, p, l);
     }
     return (int)hipGetLastError();
 }
 
-template<int OCC, int R>
+template<int OCC, int R, int MODE>
 static int lean_launch_window(int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
                               hipEvent_t start, hipEvent_t stop)
 {
     if (window == 0) {
-        return lean_launch_one<FUSED_BITMAP_WORDS_GLOBAL, OCC, R>(grid, st, p, l, start, stop);
+        return lean_launch_one<FUSED_BITMAP_WORDS_GLOBAL, OCC, R, MODE>(grid, st, p, l, start, stop);
     }
     if (window == 2) {
-        return lean_launch_one<FUSED_BITMAP_WORDS_LARGE, OCC, R>(grid, st, p, l, start, stop);
+        return lean_launch_one<FUSED_BITMAP_WORDS_LARGE, OCC, R, MODE>(grid, st, p, l, start, stop);
     }
-    return lean_launch_one<FUSED_BITMAP_WORDS_SMALL, OCC, R>(grid, st, p, l, start, stop);
+    return lean_launch_one<FUSED_BITMAP_WORDS_SMALL, OCC, R, MODE>(grid, st, p, l, start, stop);
 }
 
 #if FTK_LEAN_DT == 0
@@ -42,10 +42,16 @@ int lean_gather_launch_f16
 #else
 int lean_gather_launch_bf16
 #endif
-    (int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+    (int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
      hipEvent_t stop)
 {
-    return lean_launch_window<LG_OCCUPANCY, LG_RING>(window, grid, st, p, l, start, stop);
+    if (mode == LG_MODE_SLOTS) {
+        return lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_SLOTS>(window, grid, st, p, l, start, stop);
+    }
+    if (mode == LG_MODE_PRESET) {
+        return lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_PRESET>(window, grid, st, p, l, start, stop);
+    }
+    return lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_STREAM>(window, grid, st, p, l, start, stop);
 }
 
 #if FTK_LEAN_DT == 0

@@ -269,7 +269,8 @@ int ftk_invoke_transpose_axis01(int* out, const int* in, const int* in_skipping_
  * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
  * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on
  * the caller's stream (n = 0 switches it off); ftk_profile_read sums them (it synchronises on the
- * events) and resets the count. kernel: 0 = history bitmap, 1 = gather (the streaming pass), 2 = select. */
+ * events) and resets the count. kernel: 0 = history bitmap, 1 = gather (the streaming pass), 2 = select,
+ * 3 = the first of two reads a launch with a large k makes (the maxima that bound the row's k-th largest). */
 int ftk_profile_enable(int max_launches);
 int ftk_profile_read(int kernel, double* total_ms, int* launches);
 
