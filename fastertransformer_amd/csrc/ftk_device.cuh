@@ -196,6 +196,181 @@ __device__ __forceinline__ void block_sort_u64(unsigned long long* keys, int n)
     }
 }
 
+// The same result as block_sort_u64 for n <= 256 * PER keys, by a block of 256 threads, with the keys in
+// registers: thread t holds the PER keys of positions t * PER .. t * PER + PER - 1 of the network. Partners
+// less than PER apart are in the thread's own registers, partners in the same wave come through lane
+// exchanges, and only the stages that pair up different waves go through LDS (in `keys` itself, which must
+// hold 256 * PER entries). The positions from n on count as the largest key.
+template<int PER>
+__device__ __forceinline__ void block_sort_u64_regs(unsigned long long* keys, int n)
+{
+    constexpr int THREADS = 256;
+    constexpr int N       = THREADS * PER;
+    static_assert(PER == 2 || PER == 4 || PER == 8, "keys per thread");
+    const int          t = (int)threadIdx.x;
+    unsigned long long k[PER];
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+        const int e = r * THREADS + t;  // any assignment will do for unsorted input: this one has no bank conflicts
+        k[r]        = e < n ? keys[e] : ~0ull;
+    }
+    // compare-exchange with a key of another thread: `keep_min` says which of the two this thread keeps
+    auto exchange = [&](unsigned long long mine, unsigned long long other, bool keep_min) -> unsigned long long {
+        const bool other_smaller = other < mine;
+        return other_smaller == keep_min ? other : mine;
+    };
+#pragma unroll 1
+    for (int size = 2; size <= N; size <<= 1) {
+        // ascending where the position has the `size` bit clear (the whole thread agrees once size >= 2 * PER)
+#pragma unroll 1
+        for (int j = size >> 1; j >= PER; j >>= 1) {
+            const int  tj       = j / PER;  // distance of the partner thread
+            const bool asc      = ((t * PER) & size) == 0;
+            const bool keep_min = ((t & tj) == 0) == asc;
+            if (tj < WAVE) {
+                // every key of the partner lane is requested before the first one is used
+                int lo[PER], hi[PER];
+                if (tj == 1) {
+#pragma unroll
+                    for (int r = 0; r < PER; ++r) {  // quad_perm [1, 0, 3, 2]
+                        lo[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)k[r], 0xB1, 0xF, 0xF, false);
+                        hi[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(k[r] >> 32), 0xB1, 0xF, 0xF, false);
+                    }
+                }
+                else if (tj == 2) {
+#pragma unroll
+                    for (int r = 0; r < PER; ++r) {  // quad_perm [2, 3, 0, 1]
+                        lo[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)k[r], 0x4E, 0xF, 0xF, false);
+                        hi[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(k[r] >> 32), 0x4E, 0xF, 0xF, false);
+                    }
+                }
+                else {
+                    const int from = (lane_id() ^ tj) << 2;
+#pragma unroll
+                    for (int r = 0; r < PER; ++r) {
+                        lo[r] = __builtin_amdgcn_ds_bpermute(from, (int)(uint32_t)k[r]);
+                        hi[r] = __builtin_amdgcn_ds_bpermute(from, (int)(uint32_t)(k[r] >> 32));
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    const unsigned long long other = ((unsigned long long)(uint32_t)hi[r] << 32) | (uint32_t)lo[r];
+                    k[r]                           = exchange(k[r], other, keep_min);
+                }
+            }
+            else {
+                __syncthreads();  // earlier reads of `keys` are done
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    keys[r * THREADS + t] = k[r];
+                }
+                __syncthreads();
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    k[r] = exchange(k[r], keys[r * THREADS + (t ^ tj)], keep_min);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = PER >> 1; j > 0; j >>= 1) {
+            if (j < size) {
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    if ((r & j) == 0) {
+                        const bool               asc = ((t * PER + r) & size) == 0;
+                        const unsigned long long a = k[r], b = k[r | j];
+                        const bool               swap = (b < a) == asc;
+                        k[r]     = swap ? b : a;
+                        k[r | j] = swap ? a : b;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+        const int e = t * PER + r;
+        if (e < n) {
+            keys[e] = k[r];
+        }
+    }
+    __syncthreads();
+}
+
+// Ascending sort of 64 * PER keys held by one wave, PER per lane: afterwards lane l holds positions
+// l * PER .. l * PER + PER - 1 of the sorted sequence. No LDS, no barrier.
+template<int PER>
+__device__ __forceinline__ void wave_sort_keys_u64(unsigned long long (&k)[PER])
+{
+    constexpr int N = WAVE * PER;
+    const int     l = lane_id();
+#pragma unroll 1
+    for (int size = 2; size <= N; size <<= 1) {
+#pragma unroll 1
+        for (int j = size >> 1; j >= PER; j >>= 1) {
+            const int  lj       = j / PER;
+            const bool asc      = ((l * PER) & size) == 0;
+            const bool keep_min = ((l & lj) == 0) == asc;
+            int        lo[PER], hi[PER];
+            if (lj == 1) {
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {  // quad_perm [1, 0, 3, 2]
+                    lo[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)k[r], 0xB1, 0xF, 0xF, false);
+                    hi[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(k[r] >> 32), 0xB1, 0xF, 0xF, false);
+                }
+            }
+            else if (lj == 2) {
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {  // quad_perm [2, 3, 0, 1]
+                    lo[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)k[r], 0x4E, 0xF, 0xF, false);
+                    hi[r] = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(k[r] >> 32), 0x4E, 0xF, 0xF, false);
+                }
+            }
+            else {
+                const int from = (l ^ lj) << 2;
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    lo[r] = __builtin_amdgcn_ds_bpermute(from, (int)(uint32_t)k[r]);
+                    hi[r] = __builtin_amdgcn_ds_bpermute(from, (int)(uint32_t)(k[r] >> 32));
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                const unsigned long long other = ((unsigned long long)(uint32_t)hi[r] << 32) | (uint32_t)lo[r];
+                k[r]                           = ((other < k[r]) == keep_min) ? other : k[r];
+            }
+        }
+#pragma unroll
+        for (int j = PER >> 1; j > 0; j >>= 1) {
+            if (j < size) {
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    if ((r & j) == 0) {
+                        const bool               asc = ((l * PER + r) & size) == 0;
+                        const unsigned long long a = k[r], b = k[r | j];
+                        const bool               swap = (b < a) == asc;
+                        k[r]     = swap ? b : a;
+                        k[r | j] = swap ? a : b;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Ascending sort of n <= 2048 keys in LDS (`keys` holds 2048 entries) by a block of 256 threads. One copy per
+// kernel: the callers are not on the path of the common, small lists.
+__device__ __noinline__ void block_sort_u64_2048(unsigned long long* keys, int n)
+{
+    if (n <= 1024) {
+        block_sort_u64_regs<4>(keys, n);
+    }
+    else {
+        block_sort_u64_regs<8>(keys, n);
+    }
+}
+
 // ---- Philox-4x32-10 (counter-based generator; replaces cuRAND's XORWOW) ---------------------
 FTK_HD void philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1, uint32_t out[4])
 {

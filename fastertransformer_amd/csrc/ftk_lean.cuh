@@ -691,27 +691,36 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
             wave_base += (int)__builtin_popcountll(mk);
         }
     }
-    // the rest: lists beyond the eighth, entries beyond the first 256 of a list
+    // the rest: lists beyond the eighth, entries beyond the first 256 of a list; four rounds of loads in flight
     for (int c = wave_id(); c < splits; c += TK_WAVES) {
         const int        cnt   = (int)hdr[c].count;
         const TopkEntry* e     = entries + (size_t)c * TK_CCAP;
         const int        begin = c < LS_PF_LISTS * TK_WAVES ? LS_PF_ROUNDS * WAVE : 0;
-        for (int i0 = begin; i0 < cnt; i0 += WAVE) {
-            const int                i    = i0 + lane_id();
-            const TopkEntry          en   = i < cnt ? e[i] : TopkEntry{0u, 0u};
-            const bool               keep = i < cnt && en.key >= T0;
-            const unsigned long long mk   = __ballot(keep);
-            int                      base = 0;
-            if (lane_id() == 0 && mk != 0ull) {
-                base = atomicAdd(&s.n_cand, (int)__builtin_popcountll(mk));
+        for (int i0 = begin; i0 < cnt; i0 += 4 * WAVE) {
+            TopkEntry en[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = i0 + r * WAVE + lane_id();
+                en[r]       = e[min(i, TK_CCAP - 1)];
             }
-            base = __builtin_amdgcn_readfirstlane(base);
-            if (keep) {
-                const int slot =
-                    base + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mk >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mk, 0u));
-                if (slot < TK_CCAP) {
-                    s.cand.key[slot] = en.key;
-                    s.cand.idx[slot] = en.idx;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int                i    = i0 + r * WAVE + lane_id();
+                const bool               keep = i < cnt && en[r].key >= T0;
+                const unsigned long long mk   = __ballot(keep);
+                int                      base = 0;
+                if (lane_id() == 0 && mk != 0ull) {
+                    base = atomicAdd(&s.n_cand, (int)__builtin_popcountll(mk));
+                }
+                base = __builtin_amdgcn_readfirstlane(base);
+                if (keep) {
+                    const int slot = base
+                                     + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(mk >> 32),
+                                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)mk, 0u));
+                    if (slot < TK_CCAP) {
+                        s.cand.key[slot] = en[r].key;
+                        s.cand.idx[slot] = en[r].idx;
+                    }
                 }
             }
         }
@@ -786,7 +795,7 @@ __global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, 
     const float       u   = __int_as_float(draw_bits);
     if (n == -2) {
         const TopkListPrefetch none{};
-        n = topk_merge_lists<DT>(s, k, l.splits, headers, row_entries, &thr, none);
+        n = topk_merge_lists<DT>(s, k, l.splits, headers, row_entries, &thr, none, false);
     }
     if (n < 0) {
         // A workgroup of the gather could not hold its candidates. Walk the whole row again, here, with the

@@ -39,6 +39,7 @@ constexpr int TK_MIN_WGS  = 1024 / TK_THREADS;  // workgroups per compute unit t
 constexpr int TK_MIN_WGS_MANY = TK_MIN_WGS / 2;
 constexpr int TK_NVT      = 16;    // 16-byte vectors per thread and tile: 64 KB per workgroup in flight
 constexpr int TK_CCAP     = 2048;  // candidates a workgroup can hold
+constexpr int TK_SLICE_CAP = TK_CCAP / 8;  // ... of one stage-1 slice, for the per-slice sort of the select
 constexpr int TK_MAXSPLIT = 64;
 constexpr int TK_FILL_WGS = 256 * TK_MIN_WGS;  // workgroups wanted in flight: every compute unit full
 constexpr int TK_STAGE    = 512 / TK_WAVES;    // vectors a wave can park per tile
@@ -1100,26 +1101,36 @@ __device__ __forceinline__ int topk_sample_walk(const float* w, int n, float u, 
         }
     }
     // The running difference never rises again (the weights are non-negative), so the first position where it
-    // is <= 0 is the number of positions where it is still > 0 (or not a number, as in the reference, whose
-    // `<= 0` test a NaN never passes): counted without branches, the subtractions are the only dependent chain.
+    // is <= 0 is the number of positions in front of it, where it is still > 0 (or not a number, as in the
+    // reference, whose `<= 0` test a NaN never passes). A batch of 32 whose last difference is still positive has
+    // no such position: only the subtractions, one dependent chain, are paid for it. The batch where the walk
+    // ends is looked at position by position.
     float rand_num = u * p * s_sum;
     int   ahead    = 0;
-    for (int i0 = 0; i0 < n4; i0 += 8) {
+    bool  walking  = true;
+    for (int i0 = 0; i0 < n4 && walking; i0 += 8) {
         float4 v[8];
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
             v[b] = w4[i0 + b];
         }
+        float r[32];
 #pragma unroll
         for (int b = 0; b < 8; ++b) {
-            rand_num = rand_num - v[b].x;
-            ahead += rand_num <= 0.0f ? 0 : 1;
-            rand_num = rand_num - v[b].y;
-            ahead += rand_num <= 0.0f ? 0 : 1;
-            rand_num = rand_num - v[b].z;
-            ahead += rand_num <= 0.0f ? 0 : 1;
-            rand_num = rand_num - v[b].w;
-            ahead += rand_num <= 0.0f ? 0 : 1;
+            r[4 * b + 0] = rand_num = rand_num - v[b].x;
+            r[4 * b + 1] = rand_num = rand_num - v[b].y;
+            r[4 * b + 2] = rand_num = rand_num - v[b].z;
+            r[4 * b + 3] = rand_num = rand_num - v[b].w;
+        }
+        if (r[31] > 0.0f) {
+            ahead += 32;
+        }
+        else {
+#pragma unroll
+            for (int e = 0; e < 32; ++e) {
+                walking = walking && !(r[e] <= 0.0f);
+                ahead += walking ? 1 : 0;
+            }
         }
     }
     const int pick = ahead < n - 1 ? ahead : n - 1;
@@ -1255,8 +1266,8 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
     int       n_list  = 0;  // length of the final ordered list: values in s.w (as fp32), ids in s.idx
 
     if (n >= 0) {
-        if (n > TK_THREADS && n > k) {
-            n = topk_tighten<DEEP>(s, n, k, &thr);
+        if (n > TK_THREADS && n > k && k <= TK_THREADS) {
+            n = topk_tighten<DEEP>(s, n, k, &thr);  // (a larger k goes to the sorts below, which take any n)
         }
         if (n <= TK_THREADS) {
             // ---- small candidate sets (the usual case): both tie orders by counting, no sort.
@@ -1379,28 +1390,227 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 s.slice_count[t] = 0;
             }
             lds_barrier();
+            unsigned long long comp[PER];  // stage-1 keys of this thread's candidates
+            int                cs[PER];    // ... and their slots among the candidates of their slice
 #pragma unroll
             for (int r = 0; r < PER; ++r) {
                 const int i = t + r * TK_THREADS;
+                comp[r]     = ~0ull;
+                cs[r]       = 0;
                 if (i < n) {
                     const int blk   = (int)(ci[r] >> bs1_log);
                     const int tt    = (int)(ci[r] & (uint32_t)(BS1 - 1));
                     const int slice = blk & 7;
-                    atomicAdd(&s.slice_count[slice], 1);
-                    s.keys[i] = ((unsigned long long)slice << 61) | ((unsigned long long)(~ck[r]) << 29)
-                                | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
+                    cs[r]           = atomicAdd(&s.slice_count[slice], 1);
+                    comp[r] = ((unsigned long long)slice << 61) | ((unsigned long long)(~ck[r]) << 29)
+                              | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
                 }
             }
             lds_barrier();
             int slice_start[8];
+            int most = 0;
             {
                 int acc = 0;
 #pragma unroll
                 for (int sl = 0; sl < 8; ++sl) {
                     slice_start[sl] = acc;
                     acc += s.slice_count[sl];
+                    most = max(most, s.slice_count[sl]);
                 }
             }
+            if (most <= TK_SLICE_CAP) {
+                // ---- the usual case: no slice holds more than 256 candidates. Stage 1 is a sort per slice, two
+                // slices per wave, in registers, which leaves eight sorted runs; stage 2 (below) merges them.
+                unsigned long long* bucket = s.keys;  // [8][TK_SLICE_CAP], unused slots hold the largest key
+#pragma unroll
+                for (int r = 0; r < PER; ++r) {
+                    const int i = t + r * TK_THREADS;  // (TK_CCAP slots: slice r, slot t)
+                    if (t >= s.slice_count[r]) {
+                        bucket[i] = ~0ull;
+                    }
+                    if (i < n) {
+                        bucket[(int)(comp[r] >> 61) * TK_SLICE_CAP + cs[r]] = comp[r];
+                    }
+                }
+                lds_barrier();
+                static_assert(TK_SLICE_CAP == 4 * WAVE && TK_WAVES == 4, "a wave sorts two slices, four keys per lane");
+#pragma unroll 1
+                for (int h = 0; h < 2; ++h) {
+                    unsigned long long* b = bucket + (wave_id() * 2 + h) * TK_SLICE_CAP;
+                    unsigned long long  kk[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        kk[r] = b[r * WAVE + lane_id()];
+                    }
+                    wave_sort_keys_u64<4>(kk);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        b[lane_id() * 4 + r] = kk[r];
+                    }
+                }
+                lds_barrier();
+                int kept[8];  // entries of a run that stage 1 keeps
+                int total_kept = 0;
+#pragma unroll
+                for (int sl = 0; sl < 8; ++sl) {
+                    kept[sl] = min(s.slice_count[sl], k);
+                    total_kept += kept[sl];
+                }
+                n_list = min(k, total_kept);
+                // the second tie rule as a number: smaller comes first
+                const int bs2_log = max_top_k <= 32 ? 7 : 8;  // BS2 is a power of two
+                auto      tie2    = [&](int slice, int r) -> int {
+                    const int pos = slice * k + r;
+                    return ((BS2 - 1 - (pos & (BS2 - 1))) << 12) | (pos >> bs2_log);
+                };
+                // ---- stage 2. Each run is first put into the order of its stage-2 keys, which moves entries
+                // among the entries of equal value of their run only; thread t handles entry t of every run. Then
+                // the eight runs are merged in three rounds of pairwise merges.
+                //   stage-2 key: ~key(32) | BS2-1-pos%BS2 (8) | pos/BS2 (12) | slot of the entry in its run (12)
+                unsigned long long c2[8];
+                int                newpos[8];
+                {
+                    uint32_t ikey[8];
+                    int      mine[8], before[8], smaller[8];
+#pragma unroll
+                    for (int o = 0; o < 8; ++o) {
+                        const unsigned long long c = bucket[o * TK_SLICE_CAP + t];
+                        ikey[o]                    = (uint32_t)(c >> 29);
+                        mine[o]                    = tie2(o, t);
+                        before[o]                  = 0;
+                        smaller[o]                 = 0;
+                        const int tt               = BS1 - 1 - (int)((c >> 21) & 0xFFull);
+                        const int j                = (int)(c & 0x1FFFFFull);
+                        if (t < kept[o]) {
+                            s.sel.idx[o * TK_SLICE_CAP + t] = (j * 8 + o) * BS1 + tt;
+                        }
+                    }
+                    // neighbours of equal value at distance d, to the left and to the right, all runs together
+                    uint32_t open_left = 0xFFu, open_right = 0xFFu;
+                    for (int d = 1; (open_left | open_right) != 0u; ++d) {
+                        unsigned long long vl[8], vr[8];
+#pragma unroll
+                        for (int o = 0; o < 8; ++o) {
+                            vl[o] = bucket[o * TK_SLICE_CAP + max(t - d, 0)];
+                            vr[o] = bucket[o * TK_SLICE_CAP + min(t + d, TK_SLICE_CAP - 1)];
+                        }
+#pragma unroll
+                        for (int o = 0; o < 8; ++o) {
+                            const bool l = ((open_left >> o) & 1u) != 0u && t < kept[o] && t - d >= 0
+                                           && (uint32_t)(vl[o] >> 29) == ikey[o];
+                            const bool r = ((open_right >> o) & 1u) != 0u && t + d < kept[o]
+                                           && (uint32_t)(vr[o] >> 29) == ikey[o];
+                            before[o] += l ? 1 : 0;
+                            smaller[o] += (l && tie2(o, t - d) < mine[o] ? 1 : 0) + (r && tie2(o, t + d) < mine[o] ? 1 : 0);
+                            open_left  = l ? open_left : (open_left & ~(1u << o));
+                            open_right = r ? open_right : (open_right & ~(1u << o));
+                        }
+                    }
+#pragma unroll
+                    for (int o = 0; o < 8; ++o) {
+                        newpos[o] = t - before[o] + smaller[o];
+                        c2[o]     = ((unsigned long long)ikey[o] << 32) | ((unsigned long long)mine[o] << 12)
+                                | (unsigned long long)(o * TK_SLICE_CAP + t);
+                    }
+                }
+                lds_barrier();  // every entry of the runs has been read
+#pragma unroll
+                for (int o = 0; o < 8; ++o) {
+                    if (t < kept[o]) {
+                        bucket[o * TK_SLICE_CAP + newpos[o]] = c2[o];
+                    }
+                }
+                if (t < 8) {
+                    s.slice_count[t] = min(s.slice_count[t], k);  // run lengths for the merges
+                }
+                lds_barrier();
+                // Pairwise merges in place: a thread finds where its eight outputs start in the two runs
+                // (one binary search along the diagonal), merges them into registers, and writes them once
+                // everybody has read. Run lengths alternate between two small arrays.
+                int* len_a = s.slice_count;
+                int* len_b = reinterpret_cast<int*>(s.red32);
+#pragma unroll 1
+                for (int round = 0; round < 3; ++round) {
+                    const int cap  = (2 * TK_SLICE_CAP) << round;  // slots of a pair of runs
+                    const int tpp  = cap / 8;                      // threads per pair
+                    const int pair = t / tpp;
+                    const int d    = (t % tpp) * 8;                // first output of this thread
+                    const int nx = len_a[2 * pair], ny = len_a[2 * pair + 1];
+                    const unsigned long long* X = bucket + pair * cap;
+                    const unsigned long long* Y = X + cap / 2;
+                    int lo = max(0, d - ny), hi = min(d, nx);
+#pragma unroll 1
+                    for (int step = 0; step < 11; ++step) {  // at most 1024 entries on either side
+                        const int                mid = (lo + hi) >> 1;
+                        const unsigned long long xv  = X[min(mid, cap / 2 - 1)];
+                        const unsigned long long yv  = Y[min(max(d - 1 - mid, 0), cap / 2 - 1)];
+                        const bool               go  = lo < hi;
+                        const bool               up  = xv < yv;  // X[mid] comes before Y[d - 1 - mid]: take more of X
+                        lo                           = go && up ? mid + 1 : lo;
+                        hi                           = go && !up ? mid : hi;
+                    }
+                    int                xi = lo, yj = d - lo;
+                    unsigned long long out[8];
+                    unsigned long long xa = xi < nx ? X[xi] : ~0ull;
+                    unsigned long long yb = yj < ny ? Y[yj] : ~0ull;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const bool take_x = xa < yb;
+                        out[e]            = take_x ? xa : yb;
+                        xi += take_x ? 1 : 0;
+                        yj += take_x ? 0 : 1;
+                        const unsigned long long nxt =
+                            take_x ? (xi < nx ? X[min(xi, cap / 2 - 1)] : ~0ull) : (yj < ny ? Y[min(yj, cap / 2 - 1)] : ~0ull);
+                        xa = take_x ? nxt : xa;
+                        yb = take_x ? yb : nxt;
+                    }
+                    lds_barrier();
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (d + e < nx + ny) {
+                            bucket[pair * cap + d + e] = out[e];
+                        }
+                    }
+                    if (t % tpp == 0) {
+                        len_b[pair] = nx + ny;
+                    }
+                    lds_barrier();
+                    int* swap = len_a;
+                    len_a     = len_b;
+                    len_b     = swap;
+                }
+                // the first n_list entries, resolved into vocabulary index and value
+                {
+                    constexpr int LPT = 1024 / TK_THREADS;  // list entries per thread (k <= 1024)
+                    int           my_idx[LPT];
+                    float         my_val[LPT];
+#pragma unroll
+                    for (int r = 0; r < LPT; ++r) {
+                        const int i = t + r * TK_THREADS;
+                        my_idx[r]   = i < n_list ? s.sel.idx[(int)(bucket[i] & 0xFFFull)] : 0;
+                        my_val[r]   = i < n_list ? key_to_float(~(uint32_t)(bucket[i] >> 32)) : 0.0f;
+                    }
+                    __syncthreads();
+#pragma unroll
+                    for (int r = 0; r < LPT; ++r) {
+                        const int i = t + r * TK_THREADS;
+                        if (i < n_list) {
+                            s.sel.idx[i] = my_idx[r];
+                            s.sel.w[i]   = my_val[r];
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+            else {
+#pragma unroll
+            for (int r = 0; r < PER; ++r) {
+                const int i = t + r * TK_THREADS;
+                if (i < n) {
+                    s.keys[i] = comp[r];
+                }
+            }
+            __syncthreads();
             // decode a stage-1 composite at sorted position q into (vocabulary index, stage-2 composite)
             //   stage 2: ~key(32) | BS2-1-pos%BS2 (8) | pos/BS2 (12) | payload (12),  pos = slice*k + rank
             auto stage2_key = [&](unsigned long long c, int q, int payload, int* idx_out) -> unsigned long long {
@@ -1424,7 +1634,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
             };
 
             // ---- large candidate sets: two bitonic sorts (of exactly n keys: no padding to a power of two)
-            block_sort_u64<TK_THREADS>(s.keys, n);
+            block_sort_u64_2048(s.keys, n);
             for (int qi = t; qi < n; qi += TK_THREADS) {
                 int                      idx;
                 const unsigned long long nk = stage2_key(s.keys[qi], qi, qi, &idx);
@@ -1432,7 +1642,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 s.keys[qi]                  = nk;
             }
             __syncthreads();
-            block_sort_u64<TK_THREADS>(s.keys, n);
+            block_sort_u64_2048(s.keys, n);
             {
                 int cnt = 0;
                 for (int i = t; i < min(k, n); i += TK_THREADS) {
@@ -1460,6 +1670,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
                 }
             }
             __syncthreads();
+            }
         }
     }
     else {
@@ -1513,11 +1724,11 @@ __device__ __forceinline__ TopkListPrefetch topk_prefetch_lists(int splits, cons
 
 // Rows split over several workgroups: merge their lists from the workspace into s.cand.
 // Returns the candidate count, or -1 for the literal replay; *thr_out is a valid bound when the result
-// is >= k.
+// is >= k. `pf`: what topk_prefetch_lists returned at the top of the kernel (have_pf false: nothing was requested).
 template<int DT>
 __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits, const TopkChunkHeader* headers,
                                                 const TopkEntry* entries, uint32_t* thr_out,
-                                                const TopkListPrefetch& pf)
+                                                const TopkListPrefetch& pf, bool have_pf = true)
 {
     const int t = threadIdx.x;
     // Row-wide lower bound T0 of the k-th largest key, the larger of two valid ones: the largest
@@ -1555,7 +1766,7 @@ __device__ __forceinline__ int topk_merge_lists(TopkShared& s, int k, int splits
                 // the first rounds of a wave's first list were requested at the top of the kernel
                 TopkEntry en = TopkEntry{0u, 0u};
                 if (i < cnt) {
-                    if (ch == wave_id() && i0 < TK_PREFETCH * WAVE) {
+                    if (have_pf && ch == wave_id() && i0 < TK_PREFETCH * WAVE) {
                         en = pf.first[0];
 #pragma unroll
                         for (int r = 1; r < TK_PREFETCH; ++r) {

@@ -164,3 +164,24 @@ def test_rows_whose_late_columns_dominate(dt):
              temperature=[0.9], repetition_penalty=[1.2], prompt=_history(rng, H, B, V))
     xs = O.to_storage(x, dt)
     _run(c, rng, 2, lambda i: xs, check_logits=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_large_k_two_reads_and_lopsided_slices(dt):
+    """Launches whose largest k is beyond 128 read the logits twice (maxima of column groups bound the k-th
+    largest, then a gather against that bound) and order the candidates slice by slice. Rows here: k from 1 to
+    1024 over plain noise with many equal values (fp16 / bf16), rows whose large values all sit in the columns of
+    one stage-1 slice (more than 256 candidates in it: the whole-list sorts take over), and constant rows."""
+    rng = np.random.default_rng(900 + dt)
+    B, V, H = 64, 51200, 5
+    x = rng.standard_normal((B, V), dtype=np.float32) * np.float32(2.0)
+    cols = np.arange(V)
+    one_slice = ((cols >> 8) & 7) == 3          # BS1 = 256 for k > 16
+    x[1::8][:, one_slice] += 9.0                # every candidate of these rows lies in slice 3
+    x[2::8] = np.round(x[2::8])                 # few distinct values: long runs of equal candidates
+    x[3::8] = 1.5                               # a constant row
+    ks = np.array([1024, 1000, 777, 300, 129, 64, 7, 1] * (B // 8), dtype=np.uint32)
+    c = Case(dt, B, V, V, max_input_length=H, gen_len=2, runtime_top_k=ks, runtime_top_p=[0.9],
+             temperature=[0.8], repetition_penalty=[1.1], prompt=_history(rng, H, B, V))
+    xs = O.to_storage(x, dt)
+    _run(c, rng, 2, lambda i: xs, check_logits=False)
