@@ -37,11 +37,8 @@ WORKLOADS = {
     "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9": dict(
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=0, top_p=(0.5, 0.99), top_p_decay=0.9,
         top_p_min=0.3, top_p_reset_id=13, zipf_s=1.1, noise=0.5, prompt=0),
-    # secondary line (only with --workload): the full decode loop at batch 1024 (fp16, vocabulary 152064), per-step latency with
-    # cum_log_probs / output_log_probs and the length criterion on (the kernel-by-kernel path: log-probs need the
-    # probabilities of the whole row)
     # secondary line (only with --workload): the fused step with a per-row k drawn from {1, 4, 16, 40, 64, 1024}
-    # (fp16, vocabulary 51200): the rows with k = 1024 set the pace of the launch
+    # (fp16, vocabulary 51200): the rows with k = 1024 set the pace of the launch, which reads the logits twice
     "decode_step_b256_v51200_f16_topk1-1024_topp0.9_temp0.8_rep1.1": dict(
         dtype="f16", batch=256, vocab=51200, vocab_padded=51200, top_k=(1, 4, 16, 40, 64, 1024), top_p=0.9,
         temperature=0.8, repetition_penalty=1.1, prompt=64, sigma=2.5),
@@ -49,6 +46,9 @@ WORKLOADS = {
     "decode_step_b1024_v152064_f16_topk64_topp0.9_temp0.8_rep1.1": dict(
         dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=64, sigma=2.5),
+    # secondary line (only with --workload): the full decode loop at batch 1024 (fp16, vocabulary 152064), per-step
+    # latency with cum_log_probs / output_log_probs and the length criterion on (the fused step with log-probs:
+    # row maximum, then one kernel per row that sums, gathers and samples)
     "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs": dict(
         dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=8, sigma=2.5),
@@ -150,15 +150,13 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     alg = algorithmic_bytes(w, mid_step)
     gather_ms = kernel_ms[1]
     achieved = alg / (gather_ms * 1e-3) / 1e9 if gather_ms > 0 else 0.0
-    # launches whose largest k is at most 128 (and no bias) stream with the lean gather; the others with the general
-    # stream, in one launch from 1024 rows on
-    lean = max(int(k) for k in top_ks) <= 128
-    dominant = "lean_gather_kernel" if lean else ("fused_gather_kernel" if kernel_ms[2] > 0 else "fused_row_kernel")
+    # launches without a bias stream with the lean gather (largest k beyond 128: twice, maxima first)
+    dominant = "lean_gather_kernel"
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
         kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2], maxima=kernel_ms[3]),
         roofline=dict(bound="hbm", achieved=achieved, peak=HBM_PEAK_GBS, unit="GB/s", frac=achieved / HBM_PEAK_GBS,
-                      traffic=TRAFFIC_BYTES_PER_LAUNCH, kernel=dominant, algorithmic_bytes_per_launch=alg),
+                      traffic=TRAFFIC_BYTES_PER_LAUNCH if name == next(iter(WORKLOADS)) else None, kernel=dominant, algorithmic_bytes_per_launch=alg),
         step_gbs=alg / (gpu_ms / steps * 1e-3) / 1e9,
         sampled_ids_checksum=checksum, oracle_check=oracle,
     )
