@@ -1,4 +1,5 @@
-// Streaming candidate gather of the fused decode step for launches whose largest k is at most 128.
+// Streaming candidate gather of the fused decode step for launches without an embedding bias: in one read of
+// the logits when the largest k is at most 128, in two (maxima first, see LG_MODE_*) for a larger k.
 //
 // Same contract as the stream of ftk_topk.cuh (reference behaviour: topk_stage1 of
 // src/fastertransformer/kernels/sampling_topk_kernels.cu:130-202 after the penalty kernels of
