@@ -185,3 +185,17 @@ def test_large_k_two_reads_and_lopsided_slices(dt):
              temperature=[0.8], repetition_penalty=[1.1], prompt=_history(rng, H, B, V))
     xs = O.to_storage(x, dt)
     _run(c, rng, 2, lambda i: xs, check_logits=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("B,k", [(1, 128), (3, 100), (2, 1024), (5, 400)])
+def test_few_rows_many_lists_per_row(dt, B, k):
+    """A handful of rows of a long vocabulary: every row is cut into the largest number of workgroups, each of which
+    reports at least k candidates of its own, so the union of a row's lists is longer than the 2048 entries the
+    select kernel holds at once (k = 128 and 100) and is cut by the general merge; with k beyond 128 the same
+    geometry goes through the two reads with two maxima per thread."""
+    rng = np.random.default_rng(7000 + 10 * B + dt)
+    V, H = 128256, 4
+    c = Case(dt, B, V, V, max_input_length=H, gen_len=2, runtime_top_k=[k], runtime_top_p=[0.95],
+             temperature=[0.7], repetition_penalty=[1.3], prompt=_history(rng, H, B, V))
+    _run(c, rng, 2, lambda i: _normal(rng, dt, B, V, 3.0), check_logits=False)
