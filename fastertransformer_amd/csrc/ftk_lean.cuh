@@ -633,7 +633,8 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
     const int t = threadIdx.x;
     // headers through LDS: one load per list, every thread then looks at all of them
     TopkChunkHeader* hdr = reinterpret_cast<TopkChunkHeader*>(&s.stage.raw[0][0]);
-    static_assert(sizeof(s.stage.raw) >= TK_MAXSPLIT * sizeof(TopkChunkHeader), "headers fit the staging area");
+    static_assert(sizeof(s.stage.raw) >= TK_MAXSPLIT * sizeof(TopkChunkHeader) + TK_THREADS * sizeof(uint32_t),
+                  "headers and 256 slot maxima fit the staging area");
     if (t < splits) {
         hdr[t] = my_header;
     }
@@ -656,6 +657,38 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
     }
     if (overflow) {
         return -1;
+    }
+    if (total > TK_CCAP && k <= LG_MAX_K) {
+        // Many lists that each hold the best of their own columns: together they may not fit the list in LDS.
+        // Raise the bound first: every thread takes the largest key among the entries it is about to look at
+        // (they are entries of its own), and at least k of these 256 maxima reach the k-th largest of them.
+        uint32_t mx = 0u;
+#pragma unroll
+        for (int m = 0; m < LS_PF_LISTS; ++m) {
+            const int c   = wave_id() + m * TK_WAVES;
+            const int cnt = c < splits ? (int)hdr[c].count : 0;
+#pragma unroll
+            for (int r = 0; r < LS_PF_ROUNDS; ++r) {
+                const uint32_t key = r * WAVE + lane_id() < cnt ? pf.e[m][r].key : 0u;
+                mx                 = key > mx ? key : mx;
+            }
+        }
+        for (int c = wave_id(); c < splits; c += TK_WAVES) {
+            const int        cnt   = (int)hdr[c].count;
+            const TopkEntry* e     = entries + (size_t)c * TK_CCAP;
+            const int        begin = c < LS_PF_LISTS * TK_WAVES ? LS_PF_ROUNDS * WAVE : 0;
+            for (int i = begin + lane_id(); i < cnt; i += WAVE) {
+                const uint32_t key = e[i].key;
+                mx                 = key > mx ? key : mx;
+            }
+        }
+        uint32_t* slot_key = reinterpret_cast<uint32_t*>(&s.stage.raw[0][0]) + 4 * TK_MAXSPLIT;  // behind the headers
+        slot_key[t]        = mx;
+        lds_barrier();
+        const uint32_t P = lean_kth_of_slots(slot_key, k);
+        if (P > T0) {
+            T0 = P;
+        }
     }
     // what was requested up front: one slot reservation per wave
     unsigned long long keepm[LS_PF_LISTS][LS_PF_ROUNDS];
