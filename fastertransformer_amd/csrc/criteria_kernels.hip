@@ -90,6 +90,7 @@ __global__ void test_math_kernel(int kind, const float* __restrict__ in, float* 
             case 3: y = bf16_bits_to_float(float_to_bf16_bits(x)); break;
             case 4: y = 1.0f / (x + 1e-6f); break;             // correctly rounded division
             case 5: y = x * 1.1754944e-38f + x * 0.5f * 1.1754944e-38f; break;  // subnormal arithmetic
+            case 6: y = det_expf_nonpos(x); break;
             default: y = x;
         }
         out[i] = y;

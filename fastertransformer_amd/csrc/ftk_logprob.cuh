@@ -394,7 +394,7 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
         }
 #pragma unroll
         for (int c = 0; c < LP_CHAINS; ++c) {
-            e[c] = round_t<DT>(det_expf(y[c] - row_max));
+            e[c] = round_t<DT>(det_expf_nonpos(y[c] - row_max));
         }
         if (col + LP_CHAINS > p.V) {
 #pragma unroll

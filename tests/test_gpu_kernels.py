@@ -84,6 +84,28 @@ def test_device_conversions_division_subnormals(env):
     assert np.array_equal(to_numpy(d_out).view(np.uint32), ref.view(np.uint32))
 
 
+def test_device_exp_of_non_positive_arguments(env):
+    """The exp without range checks that the log-prob step uses on y - max: bit for bit the oracle's exp on every
+    non-positive argument, including the band around the underflow cut-off, -inf, -0 and NaN."""
+    torch, _, ops = env
+    lib = ops.ftk_hooks()
+    rng = np.random.default_rng(77)
+    x = np.concatenate([-np.abs(rng.standard_normal(400000) * 30), -rng.uniform(0.0, 110.0, 400000),
+                        -rng.uniform(103.0, 105.0, 200000), -np.abs(rng.standard_normal(100000)) * 1e-6,
+                        [0.0, -0.0, -103.97283, -103.972832, -103.9728, -104.0, -104.00001, -150.0, -1e30,
+                         -np.inf]]).astype(np.float32)
+    d_in = to_torch(x)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(6, d_in.data_ptr(), d_out.data_ptr(), x.size, ops.current_stream()))
+    _sync(torch)
+    assert np.array_equal(to_numpy(d_out).view(np.uint32), O.expf(x).view(np.uint32))
+    nan = to_torch(np.array([np.nan], np.float32))
+    out = torch.empty_like(nan)
+    ops.check(lib.ftk_test_device_math(6, nan.data_ptr(), out.data_ptr(), 1, ops.current_stream()))
+    _sync(torch)
+    assert np.isnan(to_numpy(out)[0])
+
+
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
 @pytest.mark.parametrize("V,Vp", [(4, 4), (50001, 50001), (50001, 50008), (32000, 32000), (1000, 1024)])
 @pytest.mark.parametrize("with_bias", [False, True])
