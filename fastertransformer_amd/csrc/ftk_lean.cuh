@@ -1,5 +1,5 @@
 // Streaming candidate gather of the fused decode step for launches without an embedding bias: in one read of
-// the logits when the largest k is at most 128, in two (maxima first, see LG_MODE_*) for a larger k.
+// the logits when the largest k is at most 192, in two (maxima first, see LG_MODE_*) for a larger k.
 //
 // Same contract as the stream of ftk_topk.cuh (reference behaviour: topk_stage1 of
 // src/fastertransformer/kernels/sampling_topk_kernels.cu:130-202 after the penalty kernels of
@@ -32,7 +32,7 @@ constexpr int LG_NV       = 4;                   // 16-byte vectors per thread a
 constexpr int LG_SUB_VECS = LG_THREADS * LG_NV;  // a sub-tile: 16 KB
 constexpr int LG_DRAIN_AT = 64;                  // parked vectors at which a wave evaluates them (checked once per sub-tile)
 constexpr int LG_STAGE    = LG_DRAIN_AT + LG_NV * WAVE;  // vectors a wave can park between two evaluations
-constexpr int LG_MAX_K    = TK_STAGE;            // the launches that take the general stream start above this
+constexpr int LG_MAX_K    = 192;  // largest k of a launch that reads the logits once (the bound is the k-th of 256 values)
 
 struct LeanShared {
     uint4    stage_raw[LG_WAVES][LG_STAGE];
@@ -138,7 +138,7 @@ constexpr int LG_HIST_U = 8;  // history ids a thread requests before the logits
 
 // What a launch of lean_gather_kernel does.
 //   STREAM: one read of the row. Every workgroup bounds the k-th largest of its own columns as it goes
-//           (k <= LG_MAX_K).
+//           (k <= LG_MAX_K: the bound is the k-th largest of 256 values, which gets loose as k approaches 256).
 //   SLOTS / PRESET: two reads, for any k up to 1024. The first launch (SLOTS) only takes maxima: 256 * slot_u
 //           per workgroup, each over a group of columns of its own. The k-th largest of a row's maxima bounds
 //           the row's k-th largest value from below, and with two to four times k maxima only little more than

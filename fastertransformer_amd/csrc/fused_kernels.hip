@@ -193,15 +193,16 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const LeanPlan lplan      = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * LG_OCCUPANCY);
     const int      slot_u     = lean_slot_u(lplan.splits);
     const bool     lean_ok    = a->embedding_bias == nullptr && !g_fused_force_general;
-    const bool     two_reads  = lean_ok && many > 0 && slot_u > 0
+    const bool     one_read   = lean_ok && a->max_top_k <= LG_MAX_K;
+    const bool     two_reads  = lean_ok && !one_read && slot_u > 0
                            && (size_t)lplan.splits * slot_u * LG_THREADS >= (size_t)2 * a->max_top_k
                            && (size_t)a->vocab_size / (16 / elem) >= (size_t)lplan.splits * slot_u * LG_THREADS;
-    const int      lean_mode  = lean_ok && many == 0 ? 1 : (two_reads ? 2 : 0);
+    const int      lean_mode  = one_read ? 1 : (two_reads ? 2 : 0);
     // Log-prob outputs: the two-read step covers what the lean gather covers, for vocabularies of at least 1024
     // columns (the reference's softmax block) in rows that start on 16-byte boundaries.
     const bool want_log_probs = a->cum_log_probs != nullptr || a->output_log_probs != nullptr;
     if (want_log_probs
-        && (lean_mode != 1 || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
+        && (lean_mode != 1 || a->max_top_k > TK_STAGE || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
             || ((uintptr_t)a->logits & 15u) != 0)) {
         return FTK_ERR_UNSUPPORTED;
     }
@@ -263,7 +264,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         const size_t range_cols = lean_mode != 0 ? (size_t)lplan.subs_per_wg * LG_SUB_VECS * epv + 2 * epv :
                                                    (size_t)plan.tiles_per_wg * TK_THREADS * TK_NVT * epv + epv;
         const size_t words      = (want_log_probs ? (size_t)a->vocab_size : range_cols) / 32 + 4;
-        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && (many == 0 || lean_mode == 2)
+        const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && (many == 0 || lean_mode != 0)
                            && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1 && !want_log_probs
                                || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
         if (local) {

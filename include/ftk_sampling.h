@@ -174,7 +174,7 @@ int ftk_invoke_length_criterion(bool* finished, bool* should_stop, int* h_pinned
  * issue for the rows a top-k layer owns (layers/sampling_layers/BaseSamplingLayer.cc:255-359,
  * layers/sampling_layers/TopKSamplingLayer.cu:189-268): temperature(+bias), repetition/presence penalty,
  * min-length, end/pad mask, (softmax when log-probs are requested,) top-k selection and sampling, with the
- * logits read from HBM once - twice with log-probs or a k above 128 - and never written (the reference leaves them penalised,
+ * logits read from HBM once - twice with log-probs or a k above 192 - and never written (the reference leaves them penalised,
  * or turned into probabilities). Bad words are
  * not part of it: DynamicDecodeLayer masks them on the logits before the sampling layers run
  * (ftk_invoke_ban_bad_words), here as in the reference. */

@@ -188,12 +188,12 @@ def test_large_k_two_reads_and_lopsided_slices(dt):
 
 
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
-@pytest.mark.parametrize("B,k", [(1, 128), (3, 100), (2, 1024), (5, 400)])
+@pytest.mark.parametrize("B,k", [(1, 128), (3, 100), (4, 192), (70, 150), (2, 1024), (5, 400), (3, 193)])
 def test_few_rows_many_lists_per_row(dt, B, k):
     """A handful of rows of a long vocabulary: every row is cut into the largest number of workgroups, each of which
     reports at least k candidates of its own, so the union of a row's lists is longer than the 2048 entries the
-    select kernel holds at once (k = 128 and 100) and is cut by the general merge; with k beyond 128 the same
-    geometry goes through the two reads with two maxima per thread."""
+    select kernel holds at once (k up to 192, one read of the logits) and the bound is raised before the lists are
+    merged; with k beyond 192 the same geometry goes through the two reads with two maxima per thread."""
     rng = np.random.default_rng(7000 + 10 * B + dt)
     V, H = 128256, 4
     c = Case(dt, B, V, V, max_input_length=H, gen_len=2, runtime_top_k=[k], runtime_top_p=[0.95],
