@@ -116,40 +116,50 @@ repetition_kernel(typename Storage<DT>::T* __restrict__ logits, const float* __r
 }
 
 // ---- presence + frequency penalty (extension) -----------------------------------------------
-// History staged in LDS; the first occurrence of an id counts its occurrences and applies the
-// penalty. O(step^2 / threads) compares, fine for the few-thousand-token histories it is meant for.
+// One workgroup per row. The ids of the history are counted in an open-addressing table in LDS (`slots` entries,
+// a power of two of at least twice the history length): every distinct id ends up in one slot with its number
+// of occurrences, and the slot's owner applies the penalty once, from the unpenalised value.
 template<int DT>
 __global__ void __launch_bounds__(REP_THREADS)
 frequency_kernel(typename Storage<DT>::T* __restrict__ logits, const float* __restrict__ presence,
                  const float* __restrict__ frequency, const int* __restrict__ output_ids, int batch_size,
-                 int vocab_stride, const int* __restrict__ input_lengths, int max_input_length, int step)
+                 int vocab_stride, const int* __restrict__ input_lengths, int max_input_length, int step, int slots)
 {
-    typedef Storage<DT>     S;
-    extern __shared__ int   hist[];
-    const int               row          = blockIdx.x;
-    const int               input_length = input_lengths != nullptr ? input_lengths[row] : max_input_length;
-    typename S::T*          rowp         = logits + (size_t)row * vocab_stride;
+    typedef Storage<DT>   S;
+    extern __shared__ int table[];  // ids [slots], counts [slots]
+    int*                  ids          = table;
+    int*                  counts       = table + slots;
+    const int             row          = blockIdx.x;
+    const int             input_length = input_lengths != nullptr ? input_lengths[row] : max_input_length;
+    typename S::T*        rowp         = logits + (size_t)row * vocab_stride;
+    for (int i = threadIdx.x; i < slots; i += REP_THREADS) {
+        ids[i]    = -1;
+        counts[i] = 0;
+    }
+    __syncthreads();
+    const int shift = __builtin_clz((unsigned)slots) + 1;  // the top log2(slots) bits of the product
     for (int t = threadIdx.x; t < step; t += REP_THREADS) {
         const bool pad = t >= input_length && t < max_input_length;
         const int  id  = output_ids[(size_t)t * batch_size + row];
-        hist[t]        = (pad || id < 0 || id >= vocab_stride) ? -1 : id;
+        if (pad || id < 0 || id >= vocab_stride) {
+            continue;
+        }
+        int h = (int)(((unsigned)id * 2654435761u) >> shift);
+        for (;;) {  // (the table is at most half full: an empty slot is always found)
+            const int old = atomicCAS(&ids[h], -1, id);
+            if (old == -1 || old == id) {
+                atomicAdd(&counts[h], 1);
+                break;
+            }
+            h = (h + 1) & (slots - 1);
+        }
     }
     __syncthreads();
     const float pres = presence[row], freq = frequency[row];
-    for (int t = threadIdx.x; t < step; t += REP_THREADS) {
-        const int id = hist[t];
-        if (id < 0) {
-            continue;
-        }
-        int  count = 0;
-        bool first = true;
-        for (int u = 0; u < step; ++u) {
-            const bool same = hist[u] == id;
-            count += same ? 1 : 0;
-            first = first && !(same && u < t);
-        }
-        if (first) {
-            rowp[id] = S::st(frequency_value(S::ld(rowp[id]), pres, freq, count));
+    for (int i = threadIdx.x; i < slots; i += REP_THREADS) {
+        const int id = ids[i];
+        if (id >= 0) {
+            rowp[id] = S::st(frequency_value(S::ld(rowp[id]), pres, freq, counts[i]));
         }
     }
 }
@@ -275,13 +285,29 @@ int ftk_invoke_batch_apply_frequency_penalty(int dtype, void* logits, const floa
     if (local_batch_size <= 0 || step <= 0) {
         return 0;
     }
-    const size_t smem = (size_t)step * sizeof(int);
-    if (smem > 64 * 1024) {
-        return FTK_ERR_ARGUMENT;  // history longer than 16384 tokens does not fit the staging buffer
+    // a table at most half full where that fits 128 KB of LDS, otherwise the smallest power of two above the
+    // history length (distinct ids are fewer than slots, so the probing always ends)
+    constexpr int MAX_SLOTS = 16384;
+    int           slots     = 256;
+    while (slots < 2 * step && slots < MAX_SLOTS) {
+        slots <<= 1;
     }
-    FTK_DISPATCH_DTYPE(dtype, frequency_kernel<DT><<<local_batch_size, REP_THREADS, smem, (hipStream_t)stream>>>(
-                                  (Storage<DT>::T*)logits, presence, frequency, output_ids, batch_size, vocab_size,
-                                  input_lengths, max_input_length, step));
+    if (step >= slots) {
+        return FTK_ERR_ARGUMENT;  // a history of 16384 tokens or more does not fit the counting table
+    }
+    const size_t smem = (size_t)slots * 2 * sizeof(int);
+    FTK_DISPATCH_DTYPE(dtype, {
+        if (smem > 64 * 1024) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&frequency_kernel<DT>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) {
+                return (int)e;
+            }
+        }
+        frequency_kernel<DT><<<local_batch_size, REP_THREADS, smem, (hipStream_t)stream>>>(
+            (Storage<DT>::T*)logits, presence, frequency, output_ids, batch_size, vocab_size, input_lengths,
+            max_input_length, step, slots);
+    });
     FTK_LAUNCH_CHECK();
     return 0;
 }

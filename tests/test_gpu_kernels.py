@@ -172,10 +172,13 @@ def test_repetition_penalty(env, dt, ptype, V, max_input, step):
 
 
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
-def test_frequency_penalty_extension(env, dt):
+@pytest.mark.parametrize("step", [1, 700, 2048, 9000, 16383])
+def test_frequency_penalty_extension(env, dt, step):
+    """step 700 / 2048: a counting table at most half full; 9000 / 16383: the largest table, nearly full at the end;
+    16384 tokens and more are refused."""
     torch, lib, ops = env
     rng = np.random.default_rng(11)
-    batch, V, step, max_input = 4, 32000, 700, 16
+    batch, V, max_input = 4, 32000, min(16, step)
     logits = make_logits(rng, dt, batch, V, V, scale=2.0)
     out_ids = np.minimum(rng.zipf(1.2, (step, batch)), V - 1).astype(np.int32)
     input_lengths = rng.integers(1, max_input + 1, batch).astype(np.int32)
@@ -190,6 +193,9 @@ def test_frequency_penalty_extension(env, dt):
                                                            max_input, step, ops.current_stream()))
     _sync(torch)
     assert np.array_equal(bits(to_numpy(d, dt), dt), bits(ref, dt))
+    assert lib.ftk_invoke_batch_apply_frequency_penalty(dt, d.data_ptr(), d_pres.data_ptr(), d_freq.data_ptr(),
+                                                        d_ids.data_ptr(), batch, batch, V, d_len.data_ptr(),
+                                                        max_input, 16384, ops.current_stream()) == ops.FTK_ERR_ARGUMENT
 
 
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
