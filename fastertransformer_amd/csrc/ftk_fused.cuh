@@ -262,7 +262,12 @@ struct FusedRow {
     }
     __device__ __forceinline__ bool plain_vector(int first, int n) const
     {
-        return bias == nullptr && first + n <= V && !(masked_end_id >= first && masked_end_id < first + n);
+        return bias == nullptr && interior_vector(first, n);
+    }
+    // columns of the vocabulary proper, none of them the masked end id (a bias may still apply)
+    __device__ __forceinline__ bool interior_vector(int first, int n) const
+    {
+        return first + n <= V && !(masked_end_id >= first && masked_end_id < first + n);
     }
     __device__ __forceinline__ bool has_vector_bits() const
     {

@@ -154,7 +154,8 @@ inline int lean_slot_u(int splits)
     return u >= 4 ? 4 : (u >= 2 ? 2 : u);
 }
 
-template<int DT, int BMW, int OCC, int R, int MODE>
+// BIAS: the launch has an embedding bias (a variant of its own: the common kernels do not carry its registers).
+template<int DT, int BMW, int OCC, int R, int MODE, bool BIAS>
 __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParams p, FusedLaunch l)
 {
     typedef Storage<DT>   S;
@@ -190,13 +191,39 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
             hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
         }
     }
-    uint4 raw[R][LG_NV];
-    auto  load = [&](int slot, int q) {
+    // An embedding bias (rows and bias on 16-byte boundaries: the launcher checks) is read alongside: the same
+    // vector of every row, so it comes from the caches.
+    constexpr bool has_bias  = BIAS;
+    const uint4*   bias_base = reinterpret_cast<const uint4*>(p.bias);
+    uint4          raw[R][LG_NV];
+    uint4          rawb[BIAS ? R : 1][LG_NV];
+    auto         load = [&](int slot, int q) {
 #pragma unroll
         for (int j = 0; j < LG_NV; ++j) {
             const int vi = min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1);  // past the end: a harmless vector
             raw[slot][j] = lean_stream_load(base + vi);
+            if constexpr (BIAS) {
+                rawb[slot][j] = bias_base[vi];
+            }
         }
+    };
+    // largest element of a vector before the temperature: as stored, or stored + bias (unrounded for 16-bit
+    // types: the thresholds allow for that rounding)
+    auto vector_max = [&](const uint4& v, const uint4& b) -> float {
+        if (!has_bias) {
+            return lean_raw_max<DT>(v);
+        }
+        float m = -__builtin_inff();
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+            m = __builtin_fmaxf(m, vector_element<DT>(v, e) + vector_element<DT>(b, e));
+        }
+        return m;
+    };
+    // element e of a vector as the temperature sees it: T(stored + bias)
+    auto biased_element = [&](const uint4& v, const uint4& b, int e) -> float {
+        const float x = vector_element<DT>(v, e);
+        return has_bias ? round_t<DT>(x + vector_element<DT>(b, e)) : x;
     };
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -279,6 +306,9 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
         // rounding to T can lift a product by half a unit of T, and a history penalty that raises values
         // (a multiplicative one below 1, a negative additive one) can lift it further.
         float h = lean_below_rounding<DT>(thr_f);
+        if (has_bias) {
+            h = lean_below_rounding<DT>(h);  // stored + bias is rounded to T as well
+        }
         if (bitsv) {
             const float pen = rowctx.penalty;
             float       g   = h;
@@ -331,8 +361,18 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                     for (int j = 0; j < LG_NV; ++j) {
                         const int  rel   = q * LG_SUB_VECS + j * LG_THREADS + t;
                         const int  first = (vb + rel) * EPV - a;
-                        const bool clean = rel < nvec && rowctx.plain_vector(first, EPV) && vector_flags(first) == 0u;
-                        sm[j] = __builtin_fmaxf(sm[j], clean ? lean_raw_max<DT>(raw[r][j]) : NEG_INF);
+                        const bool clean = rel < nvec && rowctx.interior_vector(first, EPV) && vector_flags(first) == 0u;
+                        float      vm    = NEG_INF;
+                        if (has_bias) {
+#pragma unroll
+                            for (int e = 0; e < EPV; ++e) {
+                                vm = __builtin_fmaxf(vm, biased_element(raw[r][j], rawb[BIAS ? r : 0][j], e));
+                            }
+                        }
+                        else {
+                            vm = lean_raw_max<DT>(raw[r][j]);
+                        }
+                        sm[j] = __builtin_fmaxf(sm[j], clean ? vm : NEG_INF);
                     }
                     if (q + R < nsub) {
                         load(r, q + R);
@@ -408,11 +448,11 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 for (int j = 0; j < LG_NV; ++j) {
                     const int  rel   = sb * LG_SUB_VECS + j * LG_THREADS + t;
                     const int  first = (vb + rel) * EPV - a;
-                    const bool clean = rel < nvec && rowctx.plain_vector(first, EPV) && vector_flags(first) == 0u;
+                    const bool clean = rel < nvec && rowctx.interior_vector(first, EPV) && vector_flags(first) == 0u;
                     float vm = NEG_INF;
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) {
-                        vm = __builtin_fmaxf(vm, rowctx.fast(vector_element<DT>(raw[sb][j], e)));
+                        vm = __builtin_fmaxf(vm, rowctx.fast(biased_element(raw[sb][j], rawb[BIAS ? sb : 0][j], e)));
                     }
                     tmax = __builtin_fmaxf(tmax, clean ? vm : NEG_INF);
                 }
@@ -450,6 +490,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
             if (have) {
                 const uint4 v = s.stage_raw[wv][e];
                 first         = s.stage_first[wv][e];
+                const uint4 bias_vec = has_bias ? bias_base[first / EPV] : v;  // (first is a multiple of EPV with a bias)
                 uint32_t bits = 0u;
                 if (aligned_bits) {
                     const int rel = first - rowctx.bm_origin;
@@ -460,7 +501,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 }
 #pragma unroll
                 for (int c = 0; c < EPV; ++c) {
-                    x[c] = rowctx.fast(vector_element<DT>(v, c));
+                    x[c] = rowctx.fast(biased_element(v, bias_vec, c));
                 }
                 if (bits != 0u) {  // rare: a column of the history
 #pragma unroll
@@ -536,7 +577,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 #pragma unroll
                 for (int j = 0; j < LG_NV; ++j) {
                     const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
-                    const float m   = lean_raw_max<DT>(raw[r][j]) * mul;
+                    const float m   = vector_max(raw[r][j], rawb[BIAS ? r : 0][j]) * mul;
                     park((all_hit || m >= thr_hot) && rel < nvec, raw[r][j], (vb + rel) * EPV - a);
                 }
                 if (q + R < nsub) {

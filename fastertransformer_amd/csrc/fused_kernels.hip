@@ -188,11 +188,16 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     const int      many         = topk_many_level(a->max_top_k);  // > 0: the large-k kernels (whole-row bitmaps only)
     const int      bitmap_words = (a->vocab_size_padded + 31) / 32 + 1;  // +1: vector_bits may peek one word ahead
     const size_t   bitmap_bytes = ((size_t)rows * bitmap_words * sizeof(uint32_t) + 255) / 256 * 256;
-    // Launches without a bias take the lean gather, which cuts a row differently: in one read of the logits
-    // for a small k (lean_mode 1), in two for a large one (2) where a row yields at least twice k maxima.
+    // Almost every launch takes the lean gather, which cuts a row differently from the general stream: in one
+    // read of the logits for a small k (lean_mode 1), in two for a large one (2) where a row yields at least
+    // twice k maxima.
     const LeanPlan lplan      = lean_plan(a->vocab_size, rows > 0 ? rows : 1, elem, 256 * LG_OCCUPANCY);
     const int      slot_u     = lean_slot_u(lplan.splits);
-    const bool     lean_ok    = a->embedding_bias == nullptr && !g_fused_force_general;
+    // (an embedding bias is read in 16-byte vectors next to the row: both must start on 16-byte boundaries)
+    const bool     bias_ok    = a->embedding_bias == nullptr
+                         || (((uintptr_t)a->embedding_bias | (uintptr_t)a->logits) & 15u) == 0
+                                && ((size_t)a->vocab_size_padded * elem) % 16 == 0;
+    const bool     lean_ok    = bias_ok && !g_fused_force_general;
     const bool     one_read   = lean_ok && a->max_top_k <= LG_MAX_K;
     const bool     two_reads  = lean_ok && !one_read && slot_u > 0
                            && (size_t)lplan.splits * slot_u * LG_THREADS >= (size_t)2 * a->max_top_k
@@ -202,7 +207,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     // columns (the reference's softmax block) in rows that start on 16-byte boundaries.
     const bool want_log_probs = a->cum_log_probs != nullptr || a->output_log_probs != nullptr;
     if (want_log_probs
-        && (lean_mode != 1 || a->max_top_k > TK_STAGE || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
+        && (lean_mode != 1 || a->embedding_bias != nullptr || a->max_top_k > TK_STAGE || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
             || ((uintptr_t)a->logits & 15u) != 0)) {
         return FTK_ERR_UNSUPPORTED;
     }

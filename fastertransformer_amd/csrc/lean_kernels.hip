@@ -8,31 +8,31 @@
 
 namespace ftk {
 
-template<int BMW, int OCC, int R, int MODE>
+template<int BMW, int OCC, int R, int MODE, bool BIAS>
 static int lean_launch_one(dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                            hipEvent_t stop)
 {
     if (start != nullptr) {
-        hipExtLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R, MODE>), grid, dim3(LG_THREADS), 0, st, start,
+        hipExtLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R, MODE, BIAS>), grid, dim3(LG_THREADS), 0, st, start,
                               stop, 0, p, l);
     }
     else {
-        hipLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R, MODE>), grid, dim3(LG_THREADS), 0, st, p, l);
+        hipLaunchKernelGGL((lean_gather_kernel<FTK_LEAN_DT, BMW, OCC, R, MODE, BIAS>), grid, dim3(LG_THREADS), 0, st, p, l);
     }
     return (int)hipGetLastError();
 }
 
-template<int OCC, int R, int MODE>
+template<int OCC, int R, int MODE, bool BIAS>
 static int lean_launch_window(int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
                               hipEvent_t start, hipEvent_t stop)
 {
     if (window == 0) {
-        return lean_launch_one<FUSED_BITMAP_WORDS_GLOBAL, OCC, R, MODE>(grid, st, p, l, start, stop);
+        return lean_launch_one<FUSED_BITMAP_WORDS_GLOBAL, OCC, R, MODE, BIAS>(grid, st, p, l, start, stop);
     }
     if (window == 2) {
-        return lean_launch_one<FUSED_BITMAP_WORDS_LARGE, OCC, R, MODE>(grid, st, p, l, start, stop);
+        return lean_launch_one<FUSED_BITMAP_WORDS_LARGE, OCC, R, MODE, BIAS>(grid, st, p, l, start, stop);
     }
-    return lean_launch_one<FUSED_BITMAP_WORDS_SMALL, OCC, R, MODE>(grid, st, p, l, start, stop);
+    return lean_launch_one<FUSED_BITMAP_WORDS_SMALL, OCC, R, MODE, BIAS>(grid, st, p, l, start, stop);
 }
 
 #if FTK_LEAN_DT == 0
@@ -45,13 +45,17 @@ int lean_gather_launch_bf16
     (int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
      hipEvent_t stop)
 {
+    const bool bias = p.bias != nullptr;
     if (mode == LG_MODE_SLOTS) {
-        return lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_SLOTS>(window, grid, st, p, l, start, stop);
+        return bias ? lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_SLOTS, true>(window, grid, st, p, l, start, stop) :
+                      lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_SLOTS, false>(window, grid, st, p, l, start, stop);
     }
     if (mode == LG_MODE_PRESET) {
-        return lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_PRESET>(window, grid, st, p, l, start, stop);
+        return bias ? lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_PRESET, true>(window, grid, st, p, l, start, stop) :
+                      lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_PRESET, false>(window, grid, st, p, l, start, stop);
     }
-    return lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_STREAM>(window, grid, st, p, l, start, stop);
+    return bias ? lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_STREAM, true>(window, grid, st, p, l, start, stop) :
+                  lean_launch_window<LG_OCCUPANCY, LG_RING, LG_MODE_STREAM, false>(window, grid, st, p, l, start, stop);
 }
 
 #if FTK_LEAN_DT == 0

@@ -199,3 +199,16 @@ def test_few_rows_many_lists_per_row(dt, B, k):
     c = Case(dt, B, V, V, max_input_length=H, gen_len=2, runtime_top_k=[k], runtime_top_p=[0.95],
              temperature=[0.7], repetition_penalty=[1.3], prompt=_history(rng, H, B, V))
     _run(c, rng, 2, lambda i: _normal(rng, dt, B, V, 3.0), check_logits=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("k", [50, 600])
+def test_embedding_bias_through_the_fused_step(dt, k):
+    """An embedding bias (added before the temperature, rounded to T) with rows and bias on 16-byte boundaries goes
+    through the same streaming kernels as rows without one: one read of the logits (k = 50) and two (k = 600)."""
+    rng = np.random.default_rng(8100 + dt + k)
+    B, V, H = 48, 65536 + 8 * 5, 6
+    bias = O.to_storage(rng.standard_normal(V).astype(np.float32) * np.float32(1.5), dt)
+    c = Case(dt, B, V, V, max_input_length=H, gen_len=2, runtime_top_k=[k], runtime_top_p=[0.9], temperature=[0.7],
+             repetition_penalty=[1.2], embedding_bias=bias, prompt=_history(rng, H, B, V))
+    _run(c, rng, 2, lambda i: _normal(rng, dt, B, V, 2.0), check_logits=False)
