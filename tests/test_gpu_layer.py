@@ -452,3 +452,81 @@ def test_fused_step_with_log_probs_ties_and_flat_rows(dt):
              with_out_lp=True)
     xs = O.to_storage(x, dt)
     _run_case(c, rng, 2, lambda i: xs, check_logits=False)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_scenarios_over_every_step_variant(seed):
+    """Random decode scenarios through the layer against the oracle, ids / flags / lengths bit-exact: all three
+    element types, 1 to 70 rows, short to long vocabularies (aligned, padded, odd), per-row k with a largest k from
+    1 to 1024 (one read of the logits, two reads, general stream), rows owned by the top-p layer mixed in,
+    temperature, repetition / presence / frequency penalties over histories of 1 to 2100 tokens, min length,
+    embedding bias, log-prob outputs, windows of the batch, and value patterns that overflow candidate lists
+    (few distinct values, constant rows, ramps, all large values in one stage-1 slice)."""
+    for case in range(20):
+        rng = np.random.default_rng(100000 + 1000 * seed + case)
+        dt = int(rng.integers(0, 3))
+        long_row = rng.random() < 0.3
+        B = int(rng.choice([1, 2, 3, 5])) if long_row else int(rng.choice([1, 2, 7, 33, 70]))
+        V = int(rng.integers(70000, 270000)) if long_row else \
+            int(rng.choice([int(rng.integers(300, 3000)), int(rng.integers(3000, 20000)), int(rng.integers(20000, 70000))]))
+        Vp = (V + 7) // 8 * 8 + int(rng.choice([0, 8, 64])) if rng.random() < 0.7 else V + int(rng.integers(0, 5))
+        H = int(rng.choice([1, 3, 40, 300, 2100]))
+        max_k = int(rng.choice([1, 8, 64, 128, 150, 192, 193, 300, 700, 1024]))
+        ks = rng.integers(1, max_k + 1, B).astype(np.uint32)
+        ks[0] = max_k
+        ps = np.where(rng.random(B) < 0.5, 1.0, rng.uniform(0.2, 0.99, B)).astype(np.float32)
+        if B > 1 and rng.random() < 0.3:  # some rows belong to the top-p layer
+            tp = rng.random(B) < 0.4
+            tp[0] = False
+            ks[tp] = 0
+            ps[tp] = rng.uniform(0.3, 0.95, int(tp.sum())).astype(np.float32)
+        kw = {}
+        if rng.random() < 0.7:
+            kw["temperature"] = rng.uniform(0.5, 1.6, B)
+        pen = int(rng.integers(0, 4))
+        if pen == 1:
+            kw["repetition_penalty"] = rng.uniform(0.7, 1.6, B)
+        elif pen == 2:
+            kw["presence_penalty"] = rng.uniform(-0.5, 1.5, B)
+        elif pen == 3:
+            kw["presence_penalty"] = rng.uniform(0.0, 1.5, B)
+            kw["frequency_penalty"] = rng.uniform(0.0, 0.5, B)
+        if rng.random() < 0.5:
+            kw["min_length"] = rng.integers(0, 4, B)
+        if rng.random() < 0.3:
+            kw["embedding_bias"] = O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt)
+        lp = rng.random() < 0.3
+        local = B // 7 if B % 7 == 0 and rng.random() < 0.4 else None
+        end = rng.integers(0, V, B).astype(np.int32)
+        c = Case(dt, B, V, Vp, max_input_length=H, gen_len=2, runtime_top_k=ks, runtime_top_p=ps,
+                 prompt=_history(rng, H, B, V, zipf=1.3 if rng.random() < 0.5 else None),
+                 input_lengths=rng.integers(1, H + 1, B), end_ids=end, with_cum=lp, with_out_lp=lp, local_batch=local,
+                 **kw)
+        scale = float(rng.uniform(0.5, 4.0))
+        kind = rng.choice(["normal", "normal", "rounded", "ramp", "few", "const", "blocks"])
+
+        def logits_fn(i):
+            x = O.to_f32(make_logits(rng, dt, B, V, Vp, scale), dt)
+            if kind == "rounded":
+                x = np.round(x * 2) / 2
+            elif kind == "ramp":
+                x[:, :V] += np.linspace(-5, 5, V, dtype=np.float32)
+            elif kind == "few":
+                x = rng.choice(np.array([-1.0, 0.0, 0.5, 2.0, 2.5], np.float32), x.shape)
+            elif kind == "const":
+                x[:] = 0.75
+                x[:, ::997] = 1.0
+            elif kind == "blocks":
+                x[:, ((np.arange(x.shape[1]) >> 8) & 7) == 5] += 8.0
+            rows = rng.random(B) < 0.2
+            x[rows, end[rows]] = 40.0  # these rows finish
+            return O.to_storage(x, dt)
+
+        p, o = ProductRunner(c), OracleRunner(c)
+        for i in range(2):
+            step = H + i
+            logits, u = logits_fn(i), uniforms(rng, B)
+            for ite in range(1 if local is None else B // local):
+                p.step(step, logits, u, ite=ite)
+                o.step(step, logits, u, ite=ite)
+            compare(p.snapshot(), o.snapshot(), dt, False, where="seed %d case %d step %d" % (seed, case, step))
