@@ -49,6 +49,8 @@ KERNEL_UNITS = [
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # private arrays stay out of LDS: the kernels' LDS budgets (workgroups per compute unit) are planned by hand
+    "-mllvm", "-disable-promote-alloca-to-lds=1",
     "-Wno-unused-result", "-I", CSRC, "-I", INCLUDE,
 ]
 

@@ -154,18 +154,55 @@ inline int lean_slot_u(int splits)
     return u >= 4 ? 4 : (u >= 2 ? 2 : u);
 }
 
+constexpr int LS_PF_LISTS  = 2;  // lists a wave requests up front (wave w: lists w and w + 4)
+constexpr int LS_PF_ROUNDS = 4;  // 64 entries each: the first 256 entries of a list
+
+struct LeanListPrefetch {
+    TopkEntry e[LS_PF_LISTS][LS_PF_ROUNDS];
+};
+
+// Requested at the top of the kernel, before anything is known about the row: the loads are in flight while
+// the row's arguments and the list headers arrive. Reads stay inside the row's slots of the workspace.
+__device__ __forceinline__ LeanListPrefetch lean_prefetch_lists(int splits, const TopkEntry* entries)
+{
+    LeanListPrefetch pf;
+#pragma unroll
+    for (int m = 0; m < LS_PF_LISTS; ++m) {
+        const int        c = wave_id() + m * TK_WAVES;
+        const TopkEntry* e = entries + (size_t)(c < splits ? c : 0) * TK_CCAP;
+#pragma unroll
+        for (int r = 0; r < LS_PF_ROUNDS; ++r) {
+            pf.e[m][r] = e[r * WAVE + lane_id()];
+        }
+    }
+    return pf;
+}
+
+template<int DT>
+__device__ __forceinline__ void lean_select_row(TopkShared& s, const FusedParams& p, const FusedLaunch& l, int row, int k,
+                                                float tp, const LeanListPrefetch& pf);
+
+union LeanTopkShared {
+    LeanShared lean;  // while the row is read
+    TopkShared topk;  // while a row's list is ordered and sampled (ROWSEL)
+};
+
 // BIAS: the launch has an embedding bias (a variant of its own: the common kernels do not carry its registers).
-template<int DT, int BMW, int OCC, int R, int MODE, bool BIAS>
+// ROWSEL: every row belongs to one workgroup (gridDim.x == 1), which goes on to order its list and sample:
+// the step is this one launch, and the selection of one row overlaps with the reading of others.
+template<int DT, int BMW, int OCC, int R, int MODE, bool BIAS, bool ROWSEL>
 __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParams p, FusedLaunch l)
 {
     typedef Storage<DT>   S;
     typedef typename S::T T;
     constexpr int         EPV = (int)(16 / sizeof(T));
     static_assert(R >= 2, "the first bound reads two sub-tiles");
-    __shared__ LeanShared s;
-    const int             t     = threadIdx.x;
-    const int             row   = blockIdx.y;
-    const int             chunk = blockIdx.x;
+    static_assert(!ROWSEL || LG_THREADS == TK_THREADS, "the selection runs in the gather's workgroup");
+    __shared__ LeanTopkShared sh;
+    LeanShared&               s     = sh.lean;
+    const int                 t     = threadIdx.x;
+    const int                 row   = blockIdx.y;
+    const int                 chunk = blockIdx.x;
     const int             lane  = lane_id();
     const int             wv    = wave_id();
 
@@ -248,8 +285,12 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
     const bool        fin  = row_flag_or(p.finished_in, row, p.end_ids + row, false);
     const int         k    = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
+    const float       tp   = ROWSEL ? row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f) : 1.0f;
     FusedRow<DT, BMW> rowctx(p, row);
     if (skip || fin) {
+        if (ROWSEL && fin && !skip && t == 0) {
+            l.ids[row] = p.end_ids[row];  // (what the select kernel does for a finished row)
+        }
         return;
     }
     if (t == 0) {
@@ -632,35 +673,17 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
         h.share     = 0u;
         l.headers[(size_t)row * l.splits + chunk] = h;
     }
+    if constexpr (ROWSEL) {
+        __syncthreads();  // list and header are written; the gather's view of the shared memory is dead
+        const TopkEntry*       row_entries = l.entries + (size_t)row * l.row_entries;
+        const LeanListPrefetch pf          = lean_prefetch_lists(l.splits, row_entries);
+        lean_select_row<DT>(sh.topk, p, l, row, k, tp, pf);
+    }
 }
 
 // -------------------------------------------------------------------------------------------
 // merge + select for the lists of the lean gather
 // -------------------------------------------------------------------------------------------
-constexpr int LS_PF_LISTS  = 2;  // lists a wave requests up front (wave w: lists w and w + 4)
-constexpr int LS_PF_ROUNDS = 4;  // 64 entries each: the first 256 entries of a list
-
-struct LeanListPrefetch {
-    TopkEntry e[LS_PF_LISTS][LS_PF_ROUNDS];
-};
-
-// Requested at the top of the kernel, before anything is known about the row: the loads are in flight while
-// the row's arguments and the list headers arrive. Reads stay inside the row's slots of the workspace.
-__device__ __forceinline__ LeanListPrefetch lean_prefetch_lists(int splits, const TopkEntry* entries)
-{
-    LeanListPrefetch pf;
-#pragma unroll
-    for (int m = 0; m < LS_PF_LISTS; ++m) {
-        const int        c = wave_id() + m * TK_WAVES;
-        const TopkEntry* e = entries + (size_t)(c < splits ? c : 0) * TK_CCAP;
-#pragma unroll
-        for (int r = 0; r < LS_PF_ROUNDS; ++r) {
-            pf.e[m][r] = e[r * WAVE + lane_id()];
-        }
-    }
-    return pf;
-}
-
 // The union of a row's lists at or above the row's bound -> s.cand, cut to the k largest keys (and ties).
 // Returns the count, or -1 when a workgroup of the gather gave up on its list.
 // `my_header`: header of list t, loaded by thread t < splits (requested with the prefetch). `draw_bits`: the
@@ -831,31 +854,15 @@ __device__ __forceinline__ int lean_merge_lists(TopkShared& s, int k, int splits
     return n;
 }
 
+// Merge the lists of a row, replay the tie orders, sample, write the row's outputs. Every thread of the workgroup
+// calls it, for a row that takes part; `k`, `tp`: the row's top-k and top-p; `pf`: lean_prefetch_lists of the row.
 template<int DT>
-__global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, FusedLaunch l)
+__device__ __forceinline__ void lean_select_row(TopkShared& s, const FusedParams& p, const FusedLaunch& l, int row, int k,
+                                                float tp, const LeanListPrefetch& pf)
 {
-    constexpr int BMW = 0;  // the recovery paths read whole-row bitmaps from global memory
-    __shared__ TopkShared s;
-    const int             row = blockIdx.x;
-    // everything the row needs is requested before the first decision: the lists (vector loads), the
-    // arguments (scalar loads), the draw
+    constexpr int          BMW         = 0;  // the recovery paths read whole-row bitmaps from global memory
     TopkEntry*             row_entries = l.entries + (size_t)row * l.row_entries;
-    const LeanListPrefetch pf          = lean_prefetch_lists(l.splits, row_entries);
-    const bool             skip        = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
-    const bool             fin         = row_flag_or(l.finished, row, p.end_ids + row, false);
-    const int              k           = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
-    const float            tp          = row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f);
-    FusedRow<DT, BMW>      r(p, row);
-    if (skip) {
-        return;
-    }
-    if (fin) {
-        if (threadIdx.x == 0) {
-            l.ids[row] = p.end_ids[row];
-        }
-        return;
-    }
-    const TopkChunkHeader* headers = l.headers + (size_t)row * l.splits;
+    const TopkChunkHeader* headers     = l.headers + (size_t)row * l.splits;
     TopkChunkHeader        my_header{};
     if ((int)threadIdx.x < l.splits) {
         my_header = headers[threadIdx.x];
@@ -864,6 +871,7 @@ __global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, 
     if (threadIdx.x == 0) {
         draw_bits = __float_as_int(row_uniform(l.rng, l.uniforms, row));
     }
+    FusedRow<DT, BMW> r(p, row);
     const TopkOutputs out = topk_outputs(l.ids, l.sequence_length, l.finished, nullptr, nullptr, row, p.end_ids);
     uint32_t          thr = 0u;
     int               n   = lean_merge_lists<DT>(s, k, l.splits, my_header, row_entries, &thr, pf, &draw_bits);
@@ -883,10 +891,35 @@ __global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, 
                                                  p.end_ids, out);
 }
 
+template<int DT>
+__global__ void __launch_bounds__(TK_THREADS) lean_select_kernel(FusedParams p, FusedLaunch l)
+{
+    __shared__ TopkShared s;
+    const int             row = blockIdx.x;
+    // everything the row needs is requested before the first decision: the lists (vector loads), the
+    // arguments (scalar loads)
+    const LeanListPrefetch pf   = lean_prefetch_lists(l.splits, l.entries + (size_t)row * l.row_entries);
+    const bool             skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
+    const bool             fin  = row_flag_or(l.finished, row, p.end_ids + row, false);
+    const int              k    = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
+    const float            tp   = row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f);
+    if (skip) {
+        return;
+    }
+    if (fin) {
+        if (threadIdx.x == 0) {
+            l.ids[row] = p.end_ids[row];
+        }
+        return;
+    }
+    lean_select_row<DT>(s, p, l, row, k, tp, pf);
+}
+
 // Launchers, one translation unit per element type (lean_kernels.hip built with FTK_LEAN_DT = 0, 1, 2).
-// mode: LG_MODE_*; window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large.
+// mode: LG_MODE_*; row_select: one workgroup per row that also orders and samples (LG_MODE_STREAM without a
+// bias only); window: 0 = history bitmaps in global memory, 1 = small LDS window, 2 = large.
 // start / stop: optional events carried by the launch.
-int lean_gather_launch_f32(int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_f32(int mode, bool row_select, int window, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 int lean_select_launch_f32(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                            hipEvent_t stop);
@@ -894,9 +927,9 @@ int lean_select_launch_f16(int rows, hipStream_t st, const FusedParams& p, const
                            hipEvent_t stop);
 int lean_select_launch_bf16(int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
                             hipEvent_t stop);
-int lean_gather_launch_f16(int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_f16(int mode, bool row_select, int window, dim3 grid, hipStream_t st, const FusedParams& p,
                            const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
-int lean_gather_launch_bf16(int mode, int window, dim3 grid, hipStream_t st, const FusedParams& p,
+int lean_gather_launch_bf16(int mode, bool row_select, int window, dim3 grid, hipStream_t st, const FusedParams& p,
                             const FusedLaunch& l, hipEvent_t start, hipEvent_t stop);
 
 // workgroups per compute unit the lean gather is built for, and sub-tiles in flight per thread

@@ -167,8 +167,15 @@ extern "C" void ftk_test_set_fused_force_general(int v)
 {
     g_fused_force_general = v;
 }
+// Test hook: non-zero keeps the selection in a launch of its own also where one workgroup per row could do both.
+static int g_fused_two_launches = 0;
+extern "C" void ftk_test_set_fused_two_launches(int v)
+{
+    g_fused_two_launches = v;
+}
 #else
 static constexpr int g_fused_force_general = 0;
+static constexpr int g_fused_two_launches  = 0;
 #endif
 
 extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
@@ -362,16 +369,19 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             }
             return rc;
         }
+        // one workgroup per row: it also orders and samples, the step is one launch
+        const bool row_select =
+            lean_mode == 1 && lplan.splits == 1 && a->embedding_bias == nullptr && g_fused_two_launches == 0;
         auto launch_lean = [&](int mode, int timer) -> int {
             hipEvent_t e0, e1;
             take_events(timer, &e0, &e1);
             if (a->dtype == FTK_DTYPE_F32) {
-                return lean_gather_launch_f32(mode, window, lgrid, st, p, l, e0, e1);
+                return lean_gather_launch_f32(mode, row_select, window, lgrid, st, p, l, e0, e1);
             }
             if (a->dtype == FTK_DTYPE_F16) {
-                return lean_gather_launch_f16(mode, window, lgrid, st, p, l, e0, e1);
+                return lean_gather_launch_f16(mode, row_select, window, lgrid, st, p, l, e0, e1);
             }
-            return lean_gather_launch_bf16(mode, window, lgrid, st, p, l, e0, e1);
+            return lean_gather_launch_bf16(mode, row_select, window, lgrid, st, p, l, e0, e1);
         };
         if (lean_mode == 2) {
             l.slots  = (uint32_t*)(l.entries + (size_t)rows * l.row_entries);
@@ -382,7 +392,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             }
         }
         rc = launch_lean(lean_mode == 2 ? LG_MODE_PRESET : LG_MODE_STREAM, 1);
-        if (rc != 0) {
+        if (rc != 0 || row_select) {
             return rc;
         }
         hipEvent_t e0, e1;

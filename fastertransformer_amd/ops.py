@@ -66,10 +66,12 @@ _HOOK_SIGNATURES = {
     "ftk_test_rng_uniform": [_vp, _vp, _i, _i, _vp],
     "ftk_test_set_topp_force_deep": [_i],
     "ftk_test_set_fused_force_general": [_i],
+    "ftk_test_set_fused_two_launches": [_i],
     "ftk_host_philox4x32_10": [_vp, _vp, _vp],
 }
 _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_char_p,
              "ftk_test_set_topp_force_deep": None, "ftk_test_set_fused_force_general": None,
+             "ftk_test_set_fused_two_launches": None,
              "ftk_host_philox4x32_10": None}
 
 

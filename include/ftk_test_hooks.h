@@ -26,6 +26,9 @@ int ftk_test_rng_uniform(ftk_rng_state* states, float* out, int batch_size, int 
 void ftk_test_set_topp_force_deep(int enable);
 /* non-zero: every fused step takes the general stream, also where the lean gather would run; process-wide */
 void ftk_test_set_fused_force_general(int enable);
+/* non-zero: the fused step keeps gather and selection in two launches also where one workgroup per row could do
+   both in one; process-wide */
+void ftk_test_set_fused_two_launches(int enable);
 
 #ifdef __cplusplus
 }

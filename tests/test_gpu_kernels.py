@@ -826,3 +826,32 @@ def test_fused_step_lean_gather_equals_general_stream(env, dt):
         assert lean[3] == 0 and general[3] == 0
         for a, b in zip(lean[:3], general[:3]):
             assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_fused_step_one_launch_equals_two_launches(env, dt):
+    """Batches that give every row to one workgroup finish the step in the gather's launch (the workgroup goes on to
+    order its list and sample). The same launch with the selection kept in a kernel of its own, forced through the
+    hook of the test build, must give identical ids, lengths and flags: many short rows, long rows, and a row that
+    is finished on entry."""
+    from helpers import run_fused_step
+    torch, _, ops = env
+    hooks = ops.ftk_hooks()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(77 + dt)
+    for B, V, H, k in ((3000, 9000, 12, 40), (1100, 70001, 30, 64), (5, 3000, 4, 128)):
+        logits = (torch.randn((B, V), generator=gen, device="cuda") * 2.0).to(ops.torch_dtype(dt))
+        history = torch.randint(0, V, (H, B), generator=gen, device="cuda", dtype=torch.int32)
+        draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
+        finished0 = torch.zeros(B, dtype=torch.bool, device="cuda")
+        finished0[1] = True
+        seqlen0 = torch.full((B,), H - 1, dtype=torch.int32, device="cuda")
+        one = run_fused_step("caller", torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks)
+        hooks.ftk_test_set_fused_two_launches(1)
+        try:
+            two = run_fused_step("caller", torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks)
+        finally:
+            hooks.ftk_test_set_fused_two_launches(0)
+        assert one[3] == 0 and two[3] == 0
+        for a, b in zip(one[:3], two[:3]):
+            assert np.array_equal(a, b)
