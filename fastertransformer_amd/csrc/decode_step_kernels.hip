@@ -177,6 +177,65 @@ __global__ void decoding_initialize_kernel(bool* __restrict__ finished, int* __r
     }
 }
 
+// The hypotheses of a batch entry (at most 2 * beam_width of them, num_beams valid) ranked by score, the best
+// beam_width copied out without their first token. One workgroup per batch entry; a rank is the hypothesis with
+// the largest remaining score, the smallest index among equals (the reference scans from index 0).
+constexpr int FIN_THREADS = 256;
+
+__global__ void __launch_bounds__(FIN_THREADS)
+finalize_kernel(int* __restrict__ output_ids, int* __restrict__ sequence_lengths, float* __restrict__ cum_log_probs,
+                float* __restrict__ output_log_probs, const int* __restrict__ topk_output_ids,
+                const int* __restrict__ topk_sequence_lengths, const float* __restrict__ scores,
+                const float* __restrict__ topk_cum_log_probs, const float* __restrict__ topk_log_probs,
+                const int* __restrict__ num_beams, int beam_width, int max_seq_len)
+{
+    extern __shared__ int        fin_shared[];  // rank [beam_width], scores [2 * beam_width]
+    __shared__ unsigned long long red[16];
+    int*                         rank     = fin_shared;
+    float*                       s_scores = reinterpret_cast<float*>(fin_shared + beam_width);
+    const int                    b        = blockIdx.x;
+    const int                    t        = threadIdx.x;
+    const int                    hyps     = 2 * beam_width;
+    const int                    valid    = min(num_beams[b], hyps);
+    for (int j = t; j < hyps; j += FIN_THREADS) {
+        s_scores[j] = j < valid ? scores[(size_t)b * hyps + j] : -3.402823466e+38f;
+    }
+    __syncthreads();
+    for (int i = 0; i < beam_width; ++i) {
+        // largest score, then smallest index: one 64-bit maximum over (order-preserving score, ~index)
+        unsigned long long best = 0ull;
+        for (int j = t; j < hyps; j += FIN_THREADS) {
+            const unsigned long long key = ((unsigned long long)order_key(s_scores[j]) << 32) | (uint32_t)(~j);
+            best                         = key > best ? key : best;
+        }
+        best = block_max<unsigned long long, FIN_THREADS / WAVE>(best, red, 0ull);
+        if (t == 0) {
+            const int j = (int)~(uint32_t)best;
+            rank[i]     = j;
+            s_scores[j] = -3.402823466e+38f;
+        }
+        __syncthreads();
+    }
+    for (int i = t; i < beam_width; i += FIN_THREADS) {
+        const size_t src                             = (size_t)b * hyps + rank[i];
+        sequence_lengths[(size_t)b * beam_width + i] = topk_sequence_lengths[src];
+        if (cum_log_probs != nullptr) {
+            cum_log_probs[(size_t)b * beam_width + i] = topk_cum_log_probs[src];
+        }
+    }
+    for (int beam = 0; beam < beam_width; ++beam) {
+        const size_t src = ((size_t)b * hyps + rank[beam]) * (max_seq_len + 1) + 1;  // (+1: the start token is dropped)
+        const size_t dst = ((size_t)b * beam_width + beam) * max_seq_len;
+        const int    len = topk_sequence_lengths[(size_t)b * hyps + rank[beam]];
+        for (int i = t; i < len; i += FIN_THREADS) {
+            output_ids[dst + i] = topk_output_ids[src + i];
+            if (output_log_probs != nullptr) {
+                output_log_probs[dst + i] = topk_log_probs[src + i];
+            }
+        }
+    }
+}
+
 __global__ void plus_scalar_kernel(int* __restrict__ buf, int val, int size)
 {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < size; i += blockDim.x * gridDim.x) {
@@ -299,6 +358,29 @@ int ftk_invoke_transpose_axis01(int* out, const int* in, const int* in_skipping_
     }
     dim3 grid((dim1 + TR_TILE - 1) / TR_TILE, (dim0 + TR_TILE - 1) / TR_TILE);
     transpose_axis01_kernel<<<grid, TR_TILE * 8, 0, (hipStream_t)stream>>>(out, in, in_skipping_dim1, dim0, dim1);
+    FTK_LAUNCH_CHECK();
+    return 0;
+}
+
+int ftk_invoke_finalize(int* output_ids, int* sequence_lengths, float* cum_log_probs, float* output_log_probs,
+                        const int* topk_output_ids, const int* topk_sequence_lengths, const float* scores,
+                        const float* topk_cum_log_probs, const float* topk_log_probs, const int* num_beams,
+                        int beam_width, int max_seq_len, int batch_size, ftk_stream_t stream)
+{
+    if (batch_size <= 0) {
+        return 0;
+    }
+    if (output_ids == nullptr || sequence_lengths == nullptr || topk_output_ids == nullptr
+        || topk_sequence_lengths == nullptr || scores == nullptr || num_beams == nullptr
+        || (cum_log_probs != nullptr && topk_cum_log_probs == nullptr)
+        || (output_log_probs != nullptr && topk_log_probs == nullptr) || beam_width < 1 || beam_width * 2 >= 1024
+        || max_seq_len < 0) {
+        return FTK_ERR_ARGUMENT;  // (the reference asserts 2 * beam_width < 1024)
+    }
+    const size_t smem = (size_t)beam_width * sizeof(int) + (size_t)beam_width * 2 * sizeof(float);
+    finalize_kernel<<<batch_size, FIN_THREADS, smem, (hipStream_t)stream>>>(
+        output_ids, sequence_lengths, cum_log_probs, output_log_probs, topk_output_ids, topk_sequence_lengths, scores,
+        topk_cum_log_probs, topk_log_probs, num_beams, beam_width, max_seq_len);
     FTK_LAUNCH_CHECK();
     return 0;
 }

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "ftk_invoke_decoding_initialize": [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_invoke_plus_scalar": [_vp, _i, _i, _vp],
     "ftk_invoke_transpose_axis01": [_vp, _vp, _vp, _i, _i, _vp],
+    "ftk_invoke_finalize": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_error_string": [_i],
     "ftk_profile_enable": [_i],
     "ftk_profile_read": [_i, _vp, _vp],

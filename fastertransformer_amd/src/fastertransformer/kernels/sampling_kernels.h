@@ -267,4 +267,15 @@ inline void invokeTransposeAxis01(int* out, int* in, const int* in_skipping_dim1
     check_ftk(ftk_invoke_transpose_axis01(out, in, in_skipping_dim1, dim0, dim1, stream));
 }
 
+// kernels/decoding_kernels.cu:787-813
+inline void invokeFinalize(int* output_ids, int* sequence_lengths, float* cum_log_probs, float* output_log_probs,
+                           const int* topk_output_ids, const int* topk_sequence_lengths, const float* scores,
+                           const float* topk_cum_log_probs, const float* topk_log_probs, const int* num_beams,
+                           const int beam_width, const int max_seq_len, const int batch_size, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_finalize(output_ids, sequence_lengths, cum_log_probs, output_log_probs, topk_output_ids,
+                                  topk_sequence_lengths, scores, topk_cum_log_probs, topk_log_probs, num_beams,
+                                  beam_width, max_seq_len, batch_size, stream));
+}
+
 }  // namespace fastertransformer

@@ -265,6 +265,19 @@ int ftk_invoke_plus_scalar(int* buf, int val, int size, ftk_stream_t stream);
 int ftk_invoke_transpose_axis01(int* out, const int* in, const int* in_skipping_dim1, int dim0, int dim1,
                                 ftk_stream_t stream);
 
+/* kernels/decoding_kernels.cu:697-813 invokeFinalize: per batch entry, the (at most 2 * beam_width, num_beams[b]
+ * valid) finished hypotheses ranked by score - largest first, the smaller index among equal scores - and the best
+ * beam_width of them copied out: sequence_lengths, cum_log_probs (optional), and ids / log-probs (optional) without
+ * their first position. Shapes: output_ids [batch, beam_width, max_seq_len], sequence_lengths and cum_log_probs
+ * [batch, beam_width], output_log_probs like output_ids; topk_output_ids and topk_log_probs
+ * [batch, 2 * beam_width, max_seq_len + 1], topk_sequence_lengths, scores, topk_cum_log_probs
+ * [batch, 2 * beam_width], num_beams [batch]. Hypotheses beyond num_beams[b] count as the lowest score (the
+ * reference reads uninitialised shared memory for them). */
+int ftk_invoke_finalize(int* output_ids, int* sequence_lengths, float* cum_log_probs, float* output_log_probs,
+                        const int* topk_output_ids, const int* topk_sequence_lengths, const float* scores,
+                        const float* topk_cum_log_probs, const float* topk_log_probs, const int* num_beams,
+                        int beam_width, int max_seq_len, int batch_size, ftk_stream_t stream);
+
 /* ---- per-kernel timing of the fused step (the reference's counterpart is its CudaTimer / NVTX ranges,
  * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
  * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on

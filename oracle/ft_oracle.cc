@@ -14,6 +14,8 @@
 //    weight 0 and is never emitted; out-of-range history ids are skipped.
 //  * Lanes that do not exist in a partially filled warp contribute the identity to
 //    blockReduceSum / blockReduceMax (the reference shuffles from them, which is undefined).
+//  * finalize: hypotheses from num_beams[b] on count as the lowest score (the reference scans
+//    shared memory it never wrote for them).
 //  * bfloat16 storage and the frequency penalty have no reference code ("parity unpinned");
 //    they follow the generic `T` branches with fp32 arithmetic and one rounding per store.
 //
@@ -27,8 +29,8 @@
 //  * temperature, repetition / presence, min-length, end mask, softmax, top-p walk and decay:
 //    closed forms in float64 / exact binary cases; storage conversions against numpy and torch;
 //    det_expf / det_logf against float64;
-//  * ban_bad_words, stop words, length criterion: no reference test exists, pinned by brute force
-//    written from the source description only.
+//  * ban_bad_words, stop words, length criterion, finalize: no reference test exists, pinned by brute
+//    force written from the source description only (finalize: a stable descending sort).
 //  PARITY UNPINNED (no reference code or no way to run it here): bfloat16 storage, the frequency
 //  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), and the last-ulp
 //  behaviour of __expf / logf (tolerance 1e-5 relative instead).
@@ -1312,6 +1314,52 @@ void oracle_transpose_axis01(int* out, const int* in, const int* in_skipping_dim
         for (int i1 = 0; i1 < dim1; ++i1) {
             const int off       = in_skipping_dim1 == nullptr ? 0 : in_skipping_dim1[i1] * dim1;
             out[i1 * dim0 + i0] = in[off + i0 * dim1 + i1];
+        }
+    }
+}
+
+// kernels/decoding_kernels.cu:697-785 (finalize): rank i is the hypothesis with the largest remaining score, found
+// by the scan from index 0 (:738-745); hypotheses from num_beams[b] on count as -FLT_MAX here (the reference reads
+// shared memory it never wrote for them). Copies skip the first position of the source rows (:768-771).
+void oracle_finalize(int* output_ids, int* sequence_lengths, float* cum_log_probs, float* output_log_probs,
+                     const int* topk_output_ids, const int* topk_sequence_lengths, const float* scores,
+                     const float* topk_cum_log_probs, const float* topk_log_probs, const int* num_beams,
+                     int beam_width, int max_seq_len, int batch_size)
+{
+    const int hyps = 2 * beam_width;
+    for (int b = 0; b < batch_size; ++b) {
+        std::vector<float> s(hyps, -FLT_MAX);
+        for (int j = 0; j < hyps && j < num_beams[b]; ++j) {
+            s[j] = scores[(size_t)b * hyps + j];
+        }
+        std::vector<int> rank(beam_width, 0);
+        for (int i = 0; i < beam_width; ++i) {
+            float mx = -FLT_MAX;
+            for (int j = 0; j < hyps; ++j) {
+                mx = s[j] > mx ? s[j] : mx;
+            }
+            for (int j = 0; j < hyps; ++j) {
+                if (s[j] == mx) {
+                    rank[i] = j;
+                    s[j]    = -FLT_MAX;
+                    break;
+                }
+            }
+        }
+        for (int i = 0; i < beam_width; ++i) {
+            const size_t src                            = (size_t)b * hyps + rank[i];
+            sequence_lengths[(size_t)b * beam_width + i] = topk_sequence_lengths[src];
+            if (cum_log_probs != nullptr) {
+                cum_log_probs[(size_t)b * beam_width + i] = topk_cum_log_probs[src];
+            }
+            const size_t from = src * (max_seq_len + 1) + 1;
+            const size_t to   = ((size_t)b * beam_width + i) * max_seq_len;
+            for (int t = 0; t < topk_sequence_lengths[src]; ++t) {
+                output_ids[to + t] = topk_output_ids[from + t];
+                if (output_log_probs != nullptr) {
+                    output_log_probs[to + t] = topk_log_probs[from + t];
+                }
+            }
         }
     }
 }

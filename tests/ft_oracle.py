@@ -298,3 +298,17 @@ def transpose_axis01(inp, skipping, dim0, dim1):
     out = np.zeros(dim0 * dim1, np.int32)
     lib().oracle_transpose_axis01(_p(out), _p(inp), _p(skipping), dim0, dim1)
     return out.reshape(dim1, dim0)
+
+
+def finalize(topk_output_ids, topk_sequence_lengths, scores, topk_cum_log_probs, topk_log_probs, num_beams, beam_width,
+             max_seq_len, batch):
+    """invokeFinalize: returns (output_ids [batch, beam, max_seq_len], sequence_lengths, cum_log_probs,
+    output_log_probs); positions past a sequence's length stay zero"""
+    out_ids = np.zeros((batch, beam_width, max_seq_len), np.int32)
+    seq = np.zeros((batch, beam_width), np.int32)
+    cum = np.zeros((batch, beam_width), np.float32) if topk_cum_log_probs is not None else None
+    lp = np.zeros((batch, beam_width, max_seq_len), np.float32) if topk_log_probs is not None else None
+    lib().oracle_finalize(_p(out_ids), _p(seq), _p(cum), _p(lp), _p(topk_output_ids), _p(topk_sequence_lengths),
+                          _p(scores), _p(topk_cum_log_probs), _p(topk_log_probs), _p(num_beams), beam_width,
+                          max_seq_len, batch)
+    return out_ids, seq, cum, lp

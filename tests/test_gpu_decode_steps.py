@@ -132,3 +132,37 @@ def test_plus_scalar_and_transpose():
     assert np.array_equal(to_numpy(d_out), O.transpose_axis01(big, skip, dim0, dim1))
     assert lib.ftk_invoke_transpose_axis01(d_in.data_ptr(), d_in.data_ptr(), None, dim0, dim1,
                                            ops.current_stream()) == ops.FTK_ERR_ARGUMENT
+
+
+@pytest.mark.parametrize("beam_width,ties", [(1, False), (2, True), (4, False), (16, True), (100, True), (511, False)])
+def test_finalize(beam_width, ties):
+    """invokeFinalize against the oracle (ranking of the hypotheses of a batch entry by score, smaller index first
+    among equal scores; copies without the first position), with and without the optional outputs."""
+    import torch
+    from test_oracle import _finalize_case
+    ops, lib = _lib()
+    rng = np.random.default_rng(950 + beam_width)
+    batch, max_seq_len = 7, 41
+    ids, lens, scores, cum, lps, num = _finalize_case(rng, batch, beam_width, max_seq_len, ties)
+    want = O.finalize(ids, lens, scores, cum, lps, num, beam_width, max_seq_len, batch)
+    d = [to_torch(a) for a in (ids, lens, scores, cum, lps, num)]
+    out_ids = torch.zeros((batch, beam_width, max_seq_len), dtype=torch.int32, device="cuda")
+    out_len = torch.zeros((batch, beam_width), dtype=torch.int32, device="cuda")
+    out_cum = torch.zeros((batch, beam_width), dtype=torch.float32, device="cuda")
+    out_lp = torch.zeros((batch, beam_width, max_seq_len), dtype=torch.float32, device="cuda")
+    st = ops.current_stream()
+    ops.check(lib.ftk_invoke_finalize(out_ids.data_ptr(), out_len.data_ptr(), out_cum.data_ptr(), out_lp.data_ptr(),
+                                      d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                                      d[4].data_ptr(), d[5].data_ptr(), beam_width, max_seq_len, batch, st))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_numpy(out_ids), want[0]) and np.array_equal(to_numpy(out_len), want[1])
+    assert np.array_equal(to_numpy(out_cum), want[2]) and np.array_equal(to_numpy(out_lp), want[3])
+    out_ids.zero_()
+    ops.check(lib.ftk_invoke_finalize(out_ids.data_ptr(), out_len.data_ptr(), None, None, d[0].data_ptr(),
+                                      d[1].data_ptr(), d[2].data_ptr(), None, None, d[5].data_ptr(), beam_width,
+                                      max_seq_len, batch, st))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_numpy(out_ids), want[0])
+    assert lib.ftk_invoke_finalize(out_ids.data_ptr(), out_len.data_ptr(), None, None, d[0].data_ptr(),
+                                   d[1].data_ptr(), d[2].data_ptr(), None, None, d[5].data_ptr(), 512, max_seq_len,
+                                   batch, st) == ops.FTK_ERR_ARGUMENT

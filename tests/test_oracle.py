@@ -651,3 +651,49 @@ def test_decode_state_helpers():
     got = O.transpose_axis01(big_in, skip, 37, 53)
     want = np.stack([big_in[skip[i1]:skip[i1] + 37, i1] for i1 in range(53)])
     assert np.array_equal(got, want)
+
+
+def _finalize_case(rng, batch, beam_width, max_seq_len, ties):
+    hyps = 2 * beam_width
+    ids = rng.integers(0, 30000, (batch, hyps, max_seq_len + 1)).astype(np.int32)
+    lens = rng.integers(0, max_seq_len + 1, (batch, hyps)).astype(np.int32)
+    scores = rng.standard_normal((batch, hyps)).astype(np.float32)
+    if ties:
+        scores = np.round(scores)  # many equal scores: the smaller index must win
+    cum = rng.standard_normal((batch, hyps)).astype(np.float32)
+    lps = rng.standard_normal((batch, hyps, max_seq_len + 1)).astype(np.float32)
+    num = rng.integers(beam_width, hyps + 1, batch).astype(np.int32)
+    return ids, lens, scores, cum, lps, num
+
+
+def finalize_by_numpy(ids, lens, scores, cum, lps, num, beam_width, max_seq_len):
+    """the definition, written independently: a stable sort of the valid hypotheses by descending score"""
+    batch = ids.shape[0]
+    out_ids = np.zeros((batch, beam_width, max_seq_len), np.int32)
+    out_lp = np.zeros((batch, beam_width, max_seq_len), np.float32)
+    out_len = np.zeros((batch, beam_width), np.int32)
+    out_cum = np.zeros((batch, beam_width), np.float32)
+    for b in range(batch):
+        order = np.argsort(-scores[b, :num[b]].astype(np.float64), kind="stable")[:beam_width]
+        for i, j in enumerate(order):
+            n = lens[b, j]
+            out_len[b, i], out_cum[b, i] = n, cum[b, j]
+            out_ids[b, i, :n] = ids[b, j, 1:n + 1]
+            out_lp[b, i, :n] = lps[b, j, 1:n + 1]
+    return out_ids, out_len, out_cum, out_lp
+
+
+@pytest.mark.parametrize("beam_width,ties", [(1, False), (2, True), (4, False), (16, True), (100, True)])
+def test_finalize_against_a_stable_sort(beam_width, ties):
+    """invokeFinalize (kernels/decoding_kernels.cu:697-813; no test of it exists in the reference): the oracle's
+    repeated arg-max with the scan from index 0 equals a stable descending sort of the valid hypotheses; the first
+    position of every source row is dropped; optional outputs may be absent."""
+    rng = np.random.default_rng(900 + beam_width)
+    batch, max_seq_len = 5, 23
+    ids, lens, scores, cum, lps, num = _finalize_case(rng, batch, beam_width, max_seq_len, ties)
+    want = finalize_by_numpy(ids, lens, scores, cum, lps, num, beam_width, max_seq_len)
+    got_ids, got_len, got_cum, got_lp = O.finalize(ids, lens, scores, cum, lps, num, beam_width, max_seq_len, batch)
+    assert np.array_equal(got_ids, want[0]) and np.array_equal(got_len, want[1])
+    assert np.array_equal(got_cum, want[2]) and np.array_equal(got_lp, want[3])
+    only_ids = O.finalize(ids, lens, scores, None, None, num, beam_width, max_seq_len, batch)
+    assert np.array_equal(only_ids[0], want[0]) and only_ids[2] is None and only_ids[3] is None
