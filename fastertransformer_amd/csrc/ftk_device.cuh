@@ -45,33 +45,55 @@ __device__ __forceinline__ int wave_id()
 }
 
 // ---- wave / block reductions ----------------------------------------------------------------
+// The value of another lane through DPP (no LDS round trip): CTRL is the dpp_ctrl encoding; every pattern used
+// here has a valid source lane for every lane. Works on 32-bit and 64-bit trivially copyable types.
+template<int CTRL, typename V>
+__device__ __forceinline__ V dpp_from(V v)
+{
+    static_assert(sizeof(V) == 4 || sizeof(V) == 8, "32-bit or 64-bit values");
+    if constexpr (sizeof(V) == 4) {
+        const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false);
+        return __builtin_bit_cast(V, r);
+    }
+    else {
+        const unsigned long long u  = __builtin_bit_cast(unsigned long long, v);
+        const int                lo = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)u, CTRL, 0xF, 0xF, false);
+        const int                hi = __builtin_amdgcn_update_dpp(0, (int)(uint32_t)(u >> 32), CTRL, 0xF, 0xF, false);
+        return __builtin_bit_cast(V, ((unsigned long long)(uint32_t)hi << 32) | (uint32_t)lo);
+    }
+}
+// Reductions whose result does not depend on the order of the operands (maximum, minimum, integer sum), result
+// in every lane: neighbours inside a quad (quad_perm), quads inside a row of 16 lanes (row_ror:4, row_ror:8),
+// then the four rows through two lane exchanges.
+constexpr int DPP_QUAD_XOR1 = 0xB1;   // quad_perm [1, 0, 3, 2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;   // quad_perm [2, 3, 0, 1]
+constexpr int DPP_ROW_ROR4  = 0x124;  // row_ror:4
+constexpr int DPP_ROW_ROR8  = 0x128;  // row_ror:8
+
+template<typename V, typename Op>
+__device__ __forceinline__ V wave_reduce_unordered(V v, Op op)
+{
+    v = op(v, dpp_from<DPP_QUAD_XOR1>(v));
+    v = op(v, dpp_from<DPP_QUAD_XOR2>(v));
+    v = op(v, dpp_from<DPP_ROW_ROR4>(v));
+    v = op(v, dpp_from<DPP_ROW_ROR8>(v));
+    v = op(v, __shfl_xor(v, 16, WAVE));
+    v = op(v, __shfl_xor(v, 32, WAVE));
+    return v;
+}
 template<typename V>
 __device__ __forceinline__ V wave_max(V v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        V other = __shfl_xor(v, o, WAVE);
-        v       = other > v ? other : v;
-    }
-    return v;
+    return wave_reduce_unordered(v, [](V a, V b) { return b > a ? b : a; });
 }
 template<typename V>
 __device__ __forceinline__ V wave_min(V v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        V other = __shfl_xor(v, o, WAVE);
-        v       = other < v ? other : v;
-    }
-    return v;
+    return wave_reduce_unordered(v, [](V a, V b) { return b < a ? b : a; });
 }
 __device__ __forceinline__ int wave_sum_i(int v)
 {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        v += __shfl_xor(v, o, WAVE);
-    }
-    return v;
+    return wave_reduce_unordered(v, [](int a, int b) { return a + b; });
 }
 
 // Block-wide reductions over the threads of the block (multiple of 64, <= 1024). `smem` holds >= 16
