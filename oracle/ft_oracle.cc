@@ -27,11 +27,13 @@
 //    topk_stage2_sampling and of the cub reduction trees, written from the reference sources;
 //    top-k set against numpy on distinct values; inverse CDF and log-probs against float64;
 //  * temperature, repetition / presence, min-length, end mask, softmax, top-p walk and decay:
-//    closed forms in float64 / exact binary cases; storage conversions against numpy and torch;
+//    closed forms in float64 / exact binary cases; the softmax's summation order bit for bit against a
+//    thread-by-thread float32 simulation; storage conversions against numpy and torch;
 //    det_expf / det_logf against float64;
 //  * ban_bad_words, stop words, length criterion, finalize: no reference test exists, pinned by brute
 //    force written from the source description only (finalize: a stable descending sort).
-//  PARITY UNPINNED (no reference code or no way to run it here): bfloat16 storage, the frequency
+//  PARITY UNPINNED (no reference code or no way to run it here): the rounding order of cub's
+//  BLOCK_SCAN_RAKING prefix sums in top-p (cub is not in the reference's tree), bfloat16 storage, the frequency
 //  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), and the last-ulp
 //  behaviour of __expf / logf (tolerance 1e-5 relative instead).
 //

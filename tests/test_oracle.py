@@ -697,3 +697,66 @@ def test_finalize_against_a_stable_sort(beam_width, ties):
     assert np.array_equal(got_cum, want[2]) and np.array_equal(got_lp, want[3])
     only_ids = O.finalize(ids, lens, scores, None, None, num, beam_width, max_seq_len, batch)
     assert np.array_equal(only_ids[0], want[0]) and only_ids[2] is None and only_ids[3] is None
+
+
+def _softmax_by_thread_simulation(x, n, n_padded, max_t):
+    """addBiasSoftMax (sampling_topp_kernels.cu:1308-1344) for one unfinished fp32 row without a bias, written
+    from the reference source independently of the oracle: BLK = min(n, 1024) threads, thread t walks columns
+    t, t + BLK, ...; blockReduceSum (reduce_kernel_utils.cuh:73-103) = xor butterfly 16, 8, 4, 2, 1 inside each warp
+    of 32, lane-0 partials to shared memory, the first warp adds them with the same butterfly. All arithmetic in
+    np.float32, exp from the oracle (the one departure both sides share)."""
+    f32 = np.float32
+    blk = min(n, 1024)
+    vals = np.full(n_padded, -max_t, f32)
+    vals[:n] = x[:n]
+    mx = vals.max()  # (a maximum does not depend on its order)
+    if blk < 1024:
+        mx = max(mx, f32(-1e20))  # blockReduceMax fills missing warps with -1e20f
+    e = O.expf((vals - mx).astype(f32))
+    part = np.zeros(((blk + 31) // 32) * 32, f32)
+    for t in range(blk):
+        s = f32(0.0)
+        for v in range(t, n_padded, blk):
+            s = f32(s + e[v])
+        part[t] = s
+
+    def butterfly(a):  # every lane adds its partner's value, all lanes at once, inside warps of 32
+        a = a.copy()
+        lanes = np.arange(a.size)
+        for mask in (16, 8, 4, 2, 1):
+            a = (a + a[lanes ^ mask]).astype(f32)
+        return a
+    warp_sums = butterfly(part)[0::32]  # lane 0 of every warp
+    second = np.zeros(32, f32)
+    for lane in range(32):
+        if lane < blk / 32.0:  # (threadIdx.x < blockDim.x / 32.f)
+            second[lane] = warp_sums[lane]
+    total = butterfly(second)[0]
+    denom = f32(total + f32(1e-6))
+    return (e / denom).astype(f32), total
+
+
+def test_softmax_summation_order_bit_for_bit():
+    """The order of the softmax's sum decides the last bits of every probability, and sampled ids depend on them.
+    Rows whose terms span many orders of magnitude make the order visible: the oracle must equal the thread-by-thread
+    simulation bit for bit, and on the same rows a plain running sum of the same terms ends in other bits (so the
+    test would catch a different order). Full blocks, a block shorter than 1024 threads with a partial warp, padding."""
+    rng = np.random.default_rng(77)
+    max_t = np.float32(3.4028234663852886e38)
+    seen_other_order_differs = 0
+    for n, n_padded in ((5000, 5000), (4097, 4104), (1000, 1000), (70, 72), (33000, 33024)):
+        x = (rng.standard_normal(n_padded) * 6.0 + rng.integers(-3, 4, n_padded) * 4.0).astype(np.float32)
+        got = x.copy().reshape(1, n_padded)
+        O.add_bias_softmax(O.F32, got, None, np.zeros(1, np.int32), np.zeros(1, np.bool_), 1, n_padded, n)
+        want, total = _softmax_by_thread_simulation(x, n, n_padded, max_t)
+        assert np.array_equal(got[0].view(np.uint32), want.view(np.uint32)), (n, n_padded)
+        # sensitivity: other summation orders of the same terms end in other bits
+        vals = np.full(n_padded, -max_t, np.float32)
+        vals[:n] = x[:n]
+        mx = vals.max() if min(n, 1024) == 1024 else max(vals.max(), np.float32(-1e20))
+        e = O.expf((vals - mx).astype(np.float32))
+        running = np.float32(0.0)
+        for v in e:
+            running = np.float32(running + v)
+        seen_other_order_differs += int(running != total)
+    assert seen_other_order_differs >= 3
