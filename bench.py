@@ -52,6 +52,17 @@ WORKLOADS = {
     "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs": dict(
         dtype="f16", batch=1024, vocab=152064, vocab_padded=152064, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=8, sigma=2.5),
+    # secondary line (only with --workload): the reference's own CPU-runnable case, batch 8 with log-probs
+    "decode_loop_b8_v50257_f32_topk40_rep1.2_logprobs": dict(
+        dtype="f32", batch=8, vocab=50257, vocab_padded=50257, top_k=40, top_p=0.0, temperature=1.0,
+        repetition_penalty=1.2, prompt=64, sigma=2.0, end_id=50256),
+    # secondary line (only with --workload): the penalty- and mask-heavy step: 2048-token Zipf(1.2) history per
+    # row, presence and frequency penalties, min_length beyond the steps taken, 64 bad-word and 16 stop-word
+    # sequences per row, no log-probs
+    "decode_loop_b128_v32000_bf16_hist2048_presence0.5_freq0.3_minlen_badwords_stopwords_topk50": dict(
+        dtype="bf16", batch=128, vocab=32000, vocab_padded=32000, top_k=50, top_p=0.0, temperature=1.0,
+        presence_penalty=0.5, frequency_penalty=0.3, prompt=2048, zipf_history=1.2, min_length_beyond=52,
+        bad_words=(64, 4), stop_words=(16, 3), end_id=2, sigma=2.0, logprobs=False),
 }
 
 
@@ -265,8 +276,9 @@ def run_gpu_topp(name, w, steps, warmup, nbuf=3):
 
 
 def run_gpu_loop(name, w, steps, warmup, nbuf=2):
-    """Decode loop with log-probs and stop criteria; per-step events, logits restored outside them (this path
-    works in place, like the reference)."""
+    """Decode loop with stop criteria and, per workload, log-probs, additive penalties, a minimum length and
+    bad / stop word lists; per-step events, logits restored outside them (this path works in place, like the
+    reference)."""
     import torch
     import fastertransformer_amd as fa
 
@@ -281,24 +293,41 @@ def run_gpu_loop(name, w, steps, warmup, nbuf=2):
     work = torch.empty_like(bufs[0])
     total = steps + warmup
     layer = fa.DynamicDecodeLayer(dt, V, Vp)
-    layer.setup(B, 1, {"runtime_top_k": np.array([w["top_k"]], np.uint32),
-                       "runtime_top_p": np.array([w["top_p"]], np.float32),
-                       "temperature": np.array([w["temperature"]], np.float32),
-                       "repetition_penalty": np.array([w["repetition_penalty"]], np.float32),
-                       "random_seed": np.array([1], np.uint64)})
+    args = {"runtime_top_k": np.array([w["top_k"]], np.uint32), "runtime_top_p": np.array([w["top_p"]], np.float32),
+            "temperature": np.array([w["temperature"]], np.float32), "random_seed": np.array([1], np.uint64)}
+    for key in ("repetition_penalty", "presence_penalty", "frequency_penalty"):
+        if w.get(key) is not None:
+            args[key] = np.array([w[key]], np.float32)
+    if "min_length_beyond" in w:  # the end id stays masked during every measured step
+        args["min_length"] = np.array([H + total + w["min_length_beyond"]], np.int32)
+    layer.setup(B, 1, args)
+    rng = np.random.default_rng(104)
     output_ids = torch.zeros((H + total + 1, B), dtype=torch.int32, device=dev)
-    output_ids[:H] = torch.randint(0, V, (H, B), generator=gen, device=dev, dtype=torch.int32)
+    if "zipf_history" in w:
+        history = np.minimum(rng.zipf(w["zipf_history"], (H, B)), V - 1).astype(np.int32)
+        output_ids[:H] = torch.from_numpy(history).to(dev)
+    else:
+        output_ids[:H] = torch.randint(0, V, (H, B), generator=gen, device=dev, dtype=torch.int32)
     finished = torch.zeros(B, dtype=torch.bool, device=dev)
     seq_len = torch.full((B,), H - 1, dtype=torch.int32, device=dev)
-    cum = torch.zeros(B, device=dev)
-    out_lp = torch.zeros((total + 1, B), device=dev)
-    end_id = torch.full((B,), V - 1, dtype=torch.int32, device=dev)
+    end_id = torch.full((B,), w.get("end_id", V - 1), dtype=torch.int32, device=dev)
     limit = torch.full((B,), H + total + 8, dtype=torch.int32, device=dev)
-    outs = {"output_ids": output_ids, "finished": finished, "sequence_length": seq_len, "cum_log_probs": cum,
-            "output_log_probs": out_lp, "should_stop": np.zeros(1, np.bool_)}
+    outs = {"output_ids": output_ids, "finished": finished, "sequence_length": seq_len,
+            "should_stop": np.zeros(1, np.bool_)}
+    if w.get("logprobs", True):
+        outs["cum_log_probs"] = torch.zeros(B, device=dev)
+        outs["output_log_probs"] = torch.zeros((total + 1, B), device=dev)
     step_arr = np.zeros(1, np.int32)
     fixed = {"step": step_arr, "max_input_length": np.array([H], np.int32), "ite": np.array([0], np.uint32),
              "local_batch_size": np.array([B], np.int32), "end_id": end_id, "sequence_limit_length": limit}
+    from helpers import make_word_list
+    for key, spec in (("bad_words_list", w.get("bad_words")), ("stop_words_list", w.get("stop_words"))):
+        if spec:  # [B, 2, L] word lists in the reference's format, random ids
+            n, longest = spec
+            lists = np.stack([make_word_list(rng, n, longest, V, L=n * longest)[0] for _ in range(B)])
+            fixed[key] = torch.from_numpy(lists).to(dev)
+    if "stop_words_list" in fixed:
+        outs["parent_ids"] = torch.zeros(1, dtype=torch.int32, device=dev)
     ms = []
     for i in range(total):
         step_arr[0] = H + i
@@ -414,13 +443,15 @@ def main():
     if name.startswith("decode_loop"):
         r = run_gpu_loop(name, w, a.steps, a.warmup)
         print(json.dumps({
-            "metric": "per-step latency, decode loop B=1024 V=152064 f16 (top-k + top-p + penalties, log-probs, "
-                      "stop criteria)",
+            "metric": "per-step latency, decode loop B=%d V=%d %s (top-k%s + penalties%s, stop criteria)"
+                      % (w["batch"], w["vocab"], w["dtype"], " + top-p" if w["top_p"] else "",
+                         ", log-probs" if w.get("logprobs", True) else ", bad and stop words, minimum length"),
             "value": r["p50_ms"], "unit": "ms (p50)", "p99_ms": r["p99_ms"], "max_ms": r["max_ms"], "n_gpus": 1,
             "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"], "tokens_per_s": r["tokens_per_s"],
-            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"],
+            "data": "synthetic",
             "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"], "top_k": w["top_k"],
-                       "top_p": w["top_p"]},
+                       "top_p": w["top_p"], "history": w["prompt"]},
             "sampled_ids_checksum": r["sampled_ids_checksum"]}))
         return
     r = run_gpu(name, w, a.steps, a.warmup, check_oracle=(name == next(iter(WORKLOADS))))

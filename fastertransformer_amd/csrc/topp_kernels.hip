@@ -118,10 +118,13 @@ constexpr int SM_THREADS = 1024;
 // The reference block has BLK = min(n, 1024) threads and thread t owns columns t, t+BLK, ...;
 // summation order (reduce_kernel_utils.cuh:73-103) = sequential per thread, xor butterfly
 // (16,8,4,2,1) inside each 32-lane group, lane-0 partials through shared memory, butterfly again.
-template<int DT>
+// STATS_ONLY: stops after the sum and leaves (maximum, denominator) of the row in `stats`; the row itself is
+// not written (softmax_finish_histogram_kernel divides).
+template<int DT, bool STATS_ONLY>
 __global__ void __launch_bounds__(SM_THREADS)
 softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Storage<DT>::T* __restrict__ bias,
-               const int* __restrict__ end_ids, const bool* __restrict__ finished, int n_padded, int n)
+               const int* __restrict__ end_ids, const bool* __restrict__ finished, int n_padded, int n,
+               float2* __restrict__ stats)
 {
     typedef Storage<DT> S;
     __shared__ float    sh[32];
@@ -159,7 +162,7 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
         if (BLK < 1024) {
             mx = __builtin_fmaxf(mx, -1e20f);
         }
-        const float pad_e = round_t<DT>(det_expf(-MAXT - mx));
+        const float pad_e = round_t<DT>(det_expf_nonpos(-MAXT - mx));
         float       sum   = 0.0f;
         if (active) {
             constexpr int U = DT == DT_F32 ? 8 : 16;  // 2-byte loads move half as much per instruction
@@ -172,11 +175,11 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    sum += round_t<DT>(det_expf((x[u] + 0.0f) - mx));
+                    sum += round_t<DT>(det_expf_nonpos((x[u] + 0.0f) - mx));
                 }
             }
             for (; v < n; v += BLK) {
-                sum += round_t<DT>(det_expf((S::ld(rowp[v]) + 0.0f) - mx));
+                sum += round_t<DT>(det_expf_nonpos((S::ld(rowp[v]) + 0.0f) - mx));
             }
             for (; v < n_padded; v += BLK) {
                 sum += pad_e;
@@ -202,8 +205,14 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
         }
         __syncthreads();
         const float denom = sh_bcast + 1e-6f;
+        if constexpr (STATS_ONLY) {
+            if (t == 0) {
+                stats[row] = make_float2(mx, denom);
+            }
+            return;
+        }
         transform_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) {
-            return round_t<DT>(det_expf((x + 0.0f) - mx)) / denom;
+            return round_t<DT>(det_expf_nonpos((x + 0.0f) - mx)) / denom;
         });
         transform_columns<DT, SM_THREADS>(rowp, n, n_padded, [&](int, float) { return pad_e / denom; });
         return;
@@ -223,7 +232,7 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
     float sum = 0.0f;
     if (active) {
         for (int v = t; v < n_padded; v += BLK) {
-            sum += round_t<DT>(det_expf(masked(v) - mx));
+            sum += round_t<DT>(det_expf_nonpos(masked(v) - mx));
         }
     }
 #pragma unroll
@@ -246,9 +255,15 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
     }
     __syncthreads();
     const float denom = sh_bcast + 1e-6f;
+    if constexpr (STATS_ONLY) {
+        if (t == 0) {
+            stats[row] = make_float2(mx, denom);
+        }
+        return;
+    }
     if (active) {
         for (int v = t; v < n_padded; v += BLK) {
-            const float e = round_t<DT>(det_expf(masked(v) - mx));
+            const float e = round_t<DT>(det_expf_nonpos(masked(v) - mx));
             rowp[v]       = S::st(e / denom);
         }
     }
@@ -408,6 +423,98 @@ topp_histogram_kernel(const typename Storage<DT>::T* __restrict__ probs, int voc
     best                    = block_max<unsigned long long, TPH_THREADS / WAVE>(best, red, 0ull);
     if (t == 0) {
         part_best[(size_t)row * S + j] = best;
+    }
+}
+
+// Second half of the softmax for the fused step, (chunks x rows) workgroups: divides every column by the
+// row's denominator (same expression as softmax_kernel, so the stored probabilities are the same bits) and
+// tallies what topp_histogram_kernel would read back from the row, in the same pass.
+template<int DT>
+__global__ void __launch_bounds__(TPH_THREADS)
+softmax_finish_histogram_kernel(typename Storage<DT>::T* __restrict__ logits,
+                                const typename Storage<DT>::T* __restrict__ bias, const int* __restrict__ end_ids,
+                                const bool* __restrict__ finished, const float2* __restrict__ stats, int n_padded,
+                                int n, int chunk, const bool* __restrict__ skip_decode,
+                                uint32_t* __restrict__ part_cnt, uint32_t* __restrict__ part_mass,
+                                unsigned long long* __restrict__ part_best)
+{
+    typedef Storage<DT>           S;
+    __shared__ uint32_t           cnt[TPB_NB];
+    __shared__ uint32_t           mass[TPB_NB];
+    __shared__ unsigned long long red[16];
+    const int                     row    = blockIdx.y;
+    const int                     j      = blockIdx.x;
+    const int                     NS     = gridDim.x;
+    const int                     t      = threadIdx.x;
+    const bool                    tally  = !(skip_decode != nullptr && skip_decode[row]);
+    const bool                    fin    = finished != nullptr ? finished[row] : false;
+    const int                     end_id = fin ? end_ids[row] : -1;
+    const float                   MAXT   = S::max_t();
+    const float2                  st     = stats[row];
+    const float                   mx     = st.x;
+    const float                   denom  = st.y;
+    for (int b = t; b < TPB_NB; b += TPH_THREADS) {
+        cnt[b]  = 0u;
+        mass[b] = 0u;
+    }
+    __syncthreads();
+    const int lo   = (int)min((long long)n_padded, (long long)j * chunk);
+    const int hi   = (int)min((long long)n_padded, (long long)lo + chunk);
+    uint32_t  tmax = 0;
+    int       tidx = 0x7FFFFFFF;
+    auto finish = [&](int v, float y) {
+        // y <= mx (or NaN): the argument of the exponential is never positive
+        const float p = round_t<DT>(det_expf_nonpos(y - mx)) / denom;
+        if (tally) {
+            const float    pr = round_t<DT>(p);
+            const uint32_t k  = order_key(pr);
+            if (k > tmax) {
+                tmax = k;
+                tidx = v;
+            }
+            if (k > ZERO_KEY) {
+                const int b = topp_bucket(k);
+                atomicAdd(&cnt[b], 1u);
+                atomicAdd(&mass[b], (uint32_t)(__builtin_fminf(pr, 1.0f) * 2147483648.0f));
+            }
+        }
+        return p;
+    };
+    typename S::T* rowp = logits + (size_t)row * n_padded;
+    if (!fin && bias == nullptr) {
+        // ordinary rows: no per-column cases in front of the arithmetic
+        const int mid = min(hi, max(lo, n));
+        transform_columns<DT, TPH_THREADS>(rowp, lo, mid, [&](int v, float x) { return finish(v, x + 0.0f); });
+        transform_columns<DT, TPH_THREADS>(rowp, mid, hi, [&](int v, float) { return finish(v, -MAXT); });
+    }
+    else {
+        transform_columns<DT, TPH_THREADS>(rowp, lo, hi, [&](int v, float x) {
+            float y;
+            if (v >= n) {
+                y = -MAXT;
+            }
+            else if (fin) {
+                y = v == end_id ? MAXT : -MAXT;
+            }
+            else {
+                y = round_t<DT>(x + S::ld(bias[v]));
+            }
+            return finish(v, y);
+        });
+    }
+    if (!tally) {
+        return;
+    }
+    __syncthreads();
+    const size_t base = ((size_t)row * NS + j) * TPB_NB;
+    for (int b = t; b < TPB_NB; b += TPH_THREADS) {
+        part_cnt[base + b]  = cnt[b];
+        part_mass[base + b] = mass[b];
+    }
+    unsigned long long best = ((unsigned long long)tmax << 32) | (uint32_t)(~(uint32_t)tidx);
+    best                    = block_max<unsigned long long, TPH_THREADS / WAVE>(best, red, 0ull);
+    if (t == 0) {
+        part_best[(size_t)row * NS + j] = best;
     }
 }
 
@@ -1246,16 +1353,15 @@ __device__ int nth_zero_entry(const typename Storage<DT>::T* __restrict__ rowp, 
 }
 
 template<int DT>
-__global__ void __launch_bounds__(TP_THREADS)
-topp_pick_kernel(const typename Storage<DT>::T* __restrict__ probs, int* __restrict__ ids,
-                 int* __restrict__ sequence_length, bool* __restrict__ finished, float* __restrict__ cum_log_probs,
-                 float* __restrict__ output_log_probs, RngState* rng, const float* __restrict__ uniforms, int vocab,
-                 const int* __restrict__ end_ids, float top_p, const float* __restrict__ top_ps,
-                 const bool* __restrict__ skip_decode, unsigned long long* __restrict__ sorted,
-                 const ToppRowMeta* __restrict__ meta, int force_deep)
+__device__ __forceinline__ void
+topp_pick_row(TopPShared& s, const typename Storage<DT>::T* __restrict__ probs, int* ids,
+              int* __restrict__ sequence_length, bool* __restrict__ finished, float* __restrict__ cum_log_probs,
+              float* __restrict__ output_log_probs, RngState* rng, const float* __restrict__ uniforms, int vocab,
+              const int* __restrict__ end_ids, float top_p, const float* top_ps,
+              const bool* __restrict__ skip_decode, unsigned long long* __restrict__ sorted,
+              const ToppRowMeta* __restrict__ meta, int force_deep)
 {
     typedef Storage<DT>   S;
-    __shared__ TopPShared s;
     const int             row = blockIdx.x;
     const int             t   = threadIdx.x;
     if (skip_decode != nullptr && skip_decode[row]) {
@@ -1379,6 +1485,40 @@ topp_pick_kernel(const typename Storage<DT>::T* __restrict__ probs, int* __restr
     }
 }
 
+// What computeToppDecay (:1381-1412) does to one row; the fused step runs it at the end of the row's pick.
+struct ToppDecayArgs {
+    float*         runtime_top_p;  // NULL: no decay
+    const float*   initial_top_p;
+    const float*   decay;
+    const float*   top_p_min;
+    const int32_t* reset_ids;
+};
+
+template<int DT>
+__global__ void __launch_bounds__(TP_THREADS)
+topp_pick_kernel(const typename Storage<DT>::T* __restrict__ probs, int* ids, int* __restrict__ sequence_length,
+                 bool* __restrict__ finished, float* __restrict__ cum_log_probs, float* __restrict__ output_log_probs,
+                 RngState* rng, const float* __restrict__ uniforms, int vocab, const int* __restrict__ end_ids,
+                 float top_p, const float* top_ps, const bool* __restrict__ skip_decode,
+                 unsigned long long* __restrict__ sorted, const ToppRowMeta* __restrict__ meta, int force_deep,
+                 ToppDecayArgs dec)
+{
+    __shared__ TopPShared s;
+    topp_pick_row<DT>(s, probs, ids, sequence_length, finished, cum_log_probs, output_log_probs, rng, uniforms, vocab,
+                      end_ids, top_p, top_ps, skip_decode, sorted, meta, force_deep);
+    // thread 0 wrote the row's id itself (a skipped row keeps what an earlier kernel left there) and every
+    // thread read the row's top_p before the first barrier of the pick
+    if (dec.runtime_top_p != nullptr && threadIdx.x == 0) {
+        const int row = blockIdx.x;
+        if (ids[row] == dec.reset_ids[row]) {
+            dec.runtime_top_p[row] = dec.initial_top_p[row];
+        }
+        else {
+            dec.runtime_top_p[row] = __builtin_fmaxf(dec.runtime_top_p[row] * dec.decay[row], dec.top_p_min[row]);
+        }
+    }
+}
+
 __global__ void topp_decay_kernel(float* __restrict__ runtime_top_p, const float* __restrict__ initial_top_p,
                                   const int* __restrict__ output_ids, const float* __restrict__ decay,
                                   const float* __restrict__ top_p_min, const int32_t* __restrict__ reset_ids, int n)
@@ -1425,8 +1565,9 @@ int ftk_invoke_add_bias_softmax(int dtype, void* logits, const void* bias, const
     if (m <= 0 || n <= 0) {
         return 0;
     }
-    FTK_DISPATCH_DTYPE(dtype, softmax_kernel<DT><<<m, SM_THREADS, 0, (hipStream_t)stream>>>(
-                                  (Storage<DT>::T*)logits, (const Storage<DT>::T*)bias, end_ids, finished, n_padded, n));
+    FTK_DISPATCH_DTYPE(dtype, (softmax_kernel<DT, false><<<m, SM_THREADS, 0, (hipStream_t)stream>>>(
+                                  (Storage<DT>::T*)logits, (const Storage<DT>::T*)bias, end_ids, finished, n_padded, n,
+                                  nullptr)));
     FTK_LAUNCH_CHECK();
     return 0;
 }
@@ -1455,25 +1596,25 @@ void       ftk_test_set_topp_force_deep(int v)
 static constexpr int g_topp_force_deep = 0;
 #endif
 
-int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace_size, size_t* cub_temp_storage_size,
-                                   int* output_ids, int* sequence_length, bool* finished, float* cum_log_probs,
-                                   float* output_log_probs, const void* log_probs, const int* id_vals,
-                                   int* offset_buf, int* begin_offset_buf, ftk_rng_state* rng_state,
-                                   const float* uniform_draws, int batch_size, size_t vocab_size_padded,
-                                   const int* end_ids, float max_top_p, const float* top_ps, ftk_stream_t stream,
-                                   const bool* skip_decode)
+// Shared by the two entry points below. `softmax_first`: `log_probs` holds logits on entry; the softmax runs as
+// two kernels, the second of which also tallies the histogram, and the decay runs at the end of the pick.
+static int topp_sampling_launch(int dtype, void* workspace, size_t* workspace_size, size_t* cub_temp_storage_size,
+                                int* output_ids, int* sequence_length, bool* finished, float* cum_log_probs,
+                                float* output_log_probs, void* log_probs, ftk_rng_state* rng_state,
+                                const float* uniform_draws, int batch_size, size_t vocab_size_padded,
+                                const int* end_ids, float max_top_p, const float* top_ps, hipStream_t st,
+                                const bool* skip_decode, bool softmax_first, const void* bias, int vocab_size,
+                                ToppDecayArgs dec)
 {
-    (void)id_vals;
-    (void)offset_buf;
-    (void)begin_offset_buf;
     if (dtype < 0 || dtype > 2) {
         return FTK_ERR_DTYPE;
     }
     if (batch_size < 0 || batch_size > 65535) {
         return FTK_ERR_ARGUMENT;
     }
-    const ToppPlan plan = topp_plan(batch_size, vocab_size_padded);
-    const size_t   need = plan.bytes;
+    const ToppPlan plan      = topp_plan(batch_size, vocab_size_padded);
+    const size_t   off_stats = plan.bytes;
+    const size_t   need      = plan.bytes + (softmax_first ? align256((size_t)(batch_size > 0 ? batch_size : 1) * sizeof(float2)) : 0);
     if (workspace == nullptr) {
         if (workspace_size == nullptr) {
             return FTK_ERR_ARGUMENT;
@@ -1496,6 +1637,9 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     if (vocab_size_padded > (size_t)65535 * TP_THREADS) {
         return FTK_ERR_ARGUMENT;
     }
+    if (softmax_first && (vocab_size <= 0 || (size_t)vocab_size > vocab_size_padded)) {
+        return FTK_ERR_ARGUMENT;
+    }
     char*               ws      = (char*)workspace;
     unsigned long long* sorted  = (unsigned long long*)ws;
     uint32_t*           pcnt    = (uint32_t*)(ws + plan.off_pcnt);
@@ -1506,11 +1650,24 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     uint32_t*           segs    = (uint32_t*)(ws + plan.off_seg);
     ToppRowMeta*        meta    = (ToppRowMeta*)(ws + plan.off_meta);
     const int           vocab   = (int)vocab_size_padded;
-    hipStream_t         st      = (hipStream_t)stream;
     const dim3          chunks(plan.splits, batch_size);
-    FTK_DISPATCH_DTYPE(dtype, topp_histogram_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
-                                  (const Storage<DT>::T*)log_probs, vocab, plan.chunk, skip_decode, pcnt, pmass, pbest));
-    FTK_LAUNCH_CHECK();
+    if (softmax_first) {
+        float2* stats = (float2*)(ws + off_stats);
+        FTK_DISPATCH_DTYPE(dtype, (softmax_kernel<DT, true><<<batch_size, SM_THREADS, 0, st>>>(
+                                      (Storage<DT>::T*)log_probs, (const Storage<DT>::T*)bias, end_ids, finished, vocab,
+                                      vocab_size, stats)));
+        FTK_LAUNCH_CHECK();
+        FTK_DISPATCH_DTYPE(dtype, softmax_finish_histogram_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
+                                      (Storage<DT>::T*)log_probs, (const Storage<DT>::T*)bias, end_ids, finished, stats,
+                                      vocab, vocab_size, plan.chunk, skip_decode, pcnt, pmass, pbest));
+        FTK_LAUNCH_CHECK();
+    }
+    else {
+        FTK_DISPATCH_DTYPE(dtype, topp_histogram_kernel<DT><<<chunks, TPH_THREADS, 0, st>>>(
+                                      (const Storage<DT>::T*)log_probs, vocab, plan.chunk, skip_decode, pcnt, pmass,
+                                      pbest));
+        FTK_LAUNCH_CHECK();
+    }
     topp_cut_kernel<<<batch_size, TPC_THREADS, 0, st>>>(plan.splits, pcnt, pmass, pbest, start, boff, segs, meta,
                                                         (const RngState*)rng_state, uniform_draws, max_top_p, top_ps,
                                                         skip_decode);
@@ -1525,9 +1682,47 @@ int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace
     FTK_DISPATCH_DTYPE(dtype, topp_pick_kernel<DT><<<batch_size, TP_THREADS, 0, st>>>(
                                   (const Storage<DT>::T*)log_probs, output_ids, sequence_length, finished,
                                   cum_log_probs, output_log_probs, (RngState*)rng_state, uniform_draws, vocab,
-                                  end_ids, max_top_p, top_ps, skip_decode, sorted, meta, g_topp_force_deep));
+                                  end_ids, max_top_p, top_ps, skip_decode, sorted, meta, g_topp_force_deep, dec));
     FTK_LAUNCH_CHECK();
     return 0;
+}
+
+int ftk_invoke_batch_topp_sampling(int dtype, void* workspace, size_t* workspace_size, size_t* cub_temp_storage_size,
+                                   int* output_ids, int* sequence_length, bool* finished, float* cum_log_probs,
+                                   float* output_log_probs, const void* log_probs, const int* id_vals,
+                                   int* offset_buf, int* begin_offset_buf, ftk_rng_state* rng_state,
+                                   const float* uniform_draws, int batch_size, size_t vocab_size_padded,
+                                   const int* end_ids, float max_top_p, const float* top_ps, ftk_stream_t stream,
+                                   const bool* skip_decode)
+{
+    (void)id_vals;
+    (void)offset_buf;
+    (void)begin_offset_buf;
+    const ToppDecayArgs none = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    return topp_sampling_launch(dtype, workspace, workspace_size, cub_temp_storage_size, output_ids, sequence_length,
+                                finished, cum_log_probs, output_log_probs, const_cast<void*>(log_probs), rng_state,
+                                uniform_draws, batch_size, vocab_size_padded, end_ids, max_top_p, top_ps,
+                                (hipStream_t)stream, skip_decode, false, nullptr, 0, none);
+}
+
+int ftk_fused_topp_step(int dtype, void* workspace, size_t* workspace_size, void* logits, const void* bias,
+                        int vocab_size, size_t vocab_size_padded, int batch_size, const int* end_ids, bool* finished,
+                        int* sequence_length, int* output_ids, float* cum_log_probs, float* output_log_probs,
+                        ftk_rng_state* rng_state, const float* uniform_draws, float max_top_p, float* runtime_top_p,
+                        const float* initial_top_p, const float* top_p_decay, const float* top_p_min,
+                        const int32_t* top_p_reset_ids, const bool* skip_decode, ftk_stream_t stream)
+{
+    ToppDecayArgs dec = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (top_p_decay != nullptr) {
+        if (runtime_top_p == nullptr || initial_top_p == nullptr || top_p_min == nullptr || top_p_reset_ids == nullptr) {
+            return FTK_ERR_ARGUMENT;
+        }
+        dec = ToppDecayArgs{runtime_top_p, initial_top_p, top_p_decay, top_p_min, top_p_reset_ids};
+    }
+    return topp_sampling_launch(dtype, workspace, workspace_size, nullptr, output_ids, sequence_length, finished,
+                                cum_log_probs, output_log_probs, logits, rng_state, uniform_draws, batch_size,
+                                vocab_size_padded, end_ids, max_top_p, runtime_top_p, (hipStream_t)stream,
+                                skip_decode, true, bias, vocab_size, dec);
 }
 
 int ftk_invoke_compute_topp_decay(float* runtime_top_p, const float* runtime_initial_top_p, const int* output_ids,

@@ -140,6 +140,24 @@ void invokeTopPSampling(void* workspace, size_t& workspace_size, size_t& cub_tem
                             (const float*)nullptr, stream, device_prop, skip_decode, uniform_draws);
 }
 
+// One call for the softmax, the top-p sampler and the decay of a step (TopPSamplingLayer<T>::runSampling,
+// layers/sampling_layers/TopPSamplingLayer.cu:256-343); workspace == nullptr asks for the size.
+template<typename T>
+void invokeFusedTopPStep(void* workspace, size_t& workspace_size, T* logits, const T* bias, const int vocab_size,
+                         const size_t vocab_size_padded, const int batch_size, const int* end_ids, bool* finished,
+                         int* sequence_length, int* output_ids, float* cum_log_probs, float* output_log_probs,
+                         curandState_t* curandstate, const float* uniform_draws, const float max_top_p,
+                         float* runtime_top_p, const float* initial_top_p, const float* top_p_decay,
+                         const float* top_p_min, const int32_t* top_p_reset_ids, const bool* skip_decode,
+                         hipStream_t stream)
+{
+    check_ftk(ftk_fused_topp_step(FtkDType<T>::value, workspace, &workspace_size, logits, bias, vocab_size,
+                                  vocab_size_padded, batch_size, end_ids, finished, sequence_length, output_ids,
+                                  cum_log_probs, output_log_probs, curandstate, uniform_draws, max_top_p,
+                                  runtime_top_p, initial_top_p, top_p_decay, top_p_min, top_p_reset_ids, skip_decode,
+                                  stream));
+}
+
 inline void invokeComputeToppDecay(float* runtime_top_p, const float* runtime_initial_top_p, const int* output_ids,
                                    const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
                                    const int local_batch_size, hipStream_t stream)

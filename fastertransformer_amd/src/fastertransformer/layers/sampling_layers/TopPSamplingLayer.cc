@@ -123,10 +123,11 @@ void TopPSamplingLayer<T>::setup(const size_t batch_size, const size_t beam_widt
     const bool any_row = std::any_of(skip_decode_.begin(), skip_decode_.begin() + batch_size,
                                      [](uint8_t s) { return s == 0; });
     if (any_row) {
-        invokeTopPSampling<T>(nullptr, sampling_workspace_size_, cub_temp_storage_size_, nullptr, nullptr, nullptr,
-                              nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, curandstate_buf_,
-                              (int)batch_size, vocab_size_padded_, nullptr, runtime_max_top_p_, stream_,
-                              cuda_device_prop_, skip_decode_buf_);
+        cub_temp_storage_size_ = 0;
+        invokeFusedTopPStep<T>(nullptr, sampling_workspace_size_, nullptr, nullptr, (int)vocab_size_,
+                               vocab_size_padded_, (int)batch_size, nullptr, nullptr, nullptr, nullptr, nullptr,
+                               nullptr, nullptr, nullptr, 0.0f, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                               stream_);
         sampling_workspace_ = allocator_->reMalloc(sampling_workspace_, sampling_workspace_size_, false);
     }
 }
@@ -144,35 +145,30 @@ void TopPSamplingLayer<T>::runSampling(TensorMap* output_tensors, TensorMap* inp
 
     const int* end_ids  = input_tensors->at("end_id").template getPtr<const int>();
     bool*      finished = output_tensors->at("finished", Tensor()).template getPtr<bool>();
-    invokeAddBiasSoftMax(logits, (T*)nullptr, end_ids, finished, local_batch_size, (int)vocab_size_padded_,
-                         (int)vocab_size_, stream_);
-    sync_check_hip_error();
-
     float* cum_log_probs    = output_tensors->at("cum_log_probs", Tensor()).template getPtr<float>();
     float* output_log_probs = output_tensors->at("output_log_probs", Tensor()).template getPtr<float>();
     int*   ids = output_tensors->at("output_ids").template getPtrWithOffset<int>((size_t)step * batch_size + off);
 
-    // The chunking of a row depends on the number of rows in the call, so a window smaller than the setup batch
-    // can need a slightly larger workspace: ask for this window's size and grow on demand.
-    size_t need = 0, unused = 0;
-    invokeTopPSampling<T>(nullptr, need, unused, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                          nullptr, nullptr, curandstate_buf_, local_batch_size, vocab_size_padded_, nullptr,
-                          runtime_max_top_p_, stream_, cuda_device_prop_, skip_decode_buf_);
+    // The reference's three launches per step (softmax, sampler, decay) go out as one call: the sampler's first
+    // pass over the row rides on the softmax's last one and the decay on the sampler's last kernel. The chunking
+    // of a row depends on the number of rows in the call, so a window smaller than the setup batch can need a
+    // slightly larger workspace: ask for this window's size and grow on demand.
+    size_t need = 0;
+    invokeFusedTopPStep<T>(nullptr, need, nullptr, nullptr, (int)vocab_size_, vocab_size_padded_, local_batch_size,
+                           nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, nullptr,
+                           nullptr, nullptr, nullptr, nullptr, nullptr, stream_);
     if (need > sampling_workspace_size_) {
         sampling_workspace_      = allocator_->reMalloc(sampling_workspace_, need, false);
         sampling_workspace_size_ = need;
     }
-    invokeBatchTopPSampling<T>(sampling_workspace_, sampling_workspace_size_, cub_temp_storage_size_, ids,
-                               output_tensors->at("sequence_length", Tensor()).template getPtr<int>(), finished,
-                               cum_log_probs, output_log_probs, logits, nullptr, nullptr, nullptr,
-                               curandstate_buf_ + off, local_batch_size, vocab_size_padded_, end_ids,
-                               runtime_max_top_p_, runtime_top_p_buf_ + off, stream_, cuda_device_prop_,
-                               skip_decode_buf_ + off,
-                               input_tensors->at("uniform_draws", Tensor()).template getPtr<const float>());
-    sync_check_hip_error();
-
-    invokeComputeToppDecay(runtime_top_p_buf_ + off, initial_top_p_buf_ + off, ids, top_p_decay_buf_ + off,
-                           top_p_min_buf_ + off, top_p_reset_ids_buf_ + off, local_batch_size, stream_);
+    invokeFusedTopPStep<T>(sampling_workspace_, sampling_workspace_size_, logits, (const T*)nullptr, (int)vocab_size_,
+                           vocab_size_padded_, local_batch_size, end_ids, finished,
+                           output_tensors->at("sequence_length", Tensor()).template getPtr<int>(), ids, cum_log_probs,
+                           output_log_probs, curandstate_buf_ + off,
+                           input_tensors->at("uniform_draws", Tensor()).template getPtr<const float>(),
+                           runtime_max_top_p_, runtime_top_p_buf_ + off, initial_top_p_buf_ + off,
+                           top_p_decay_buf_ + off, top_p_min_buf_ + off, top_p_reset_ids_buf_ + off,
+                           skip_decode_buf_ + off, stream_);
     sync_check_hip_error();
 }
 

@@ -104,6 +104,20 @@ int ftk_invoke_compute_topp_decay(float* runtime_top_p, const float* runtime_ini
                                   const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
                                   int local_batch_size, ftk_stream_t stream);
 
+/* One call for what TopPSamplingLayer<T>::runSampling issues per step
+ * (layers/sampling_layers/TopPSamplingLayer.cu:256-343): invokeAddBiasSoftMax on `logits` ([batch_size,
+ * vocab_size_padded], left holding the probabilities exactly as ftk_invoke_add_bias_softmax leaves them),
+ * invokeBatchTopPSampling on the result with `runtime_top_p` as top_ps (NULL: max_top_p for every row), and, when
+ * top_p_decay is not NULL, invokeComputeToppDecay on the ids just written. Results are those of the three calls
+ * in sequence; the row is read once less and the histogram of the sampler is taken while the probabilities are
+ * written. workspace == NULL: size query (slightly above ftk_invoke_batch_topp_sampling's). */
+int ftk_fused_topp_step(int dtype, void* workspace, size_t* workspace_size, void* logits, const void* bias,
+                        int vocab_size, size_t vocab_size_padded, int batch_size, const int* end_ids, bool* finished,
+                        int* sequence_length, int* output_ids, float* cum_log_probs, float* output_log_probs,
+                        ftk_rng_state* rng_state, const float* uniform_draws, float max_top_p, float* runtime_top_p,
+                        const float* initial_top_p, const float* top_p_decay, const float* top_p_min,
+                        const int32_t* top_p_reset_ids, const bool* skip_decode, ftk_stream_t stream);
+
 /* ---- kernels/sampling_penalty_kernels.h -------------------------------------------------- */
 
 /* invokeApplyTemperaturePenalty<T>, kernels/sampling_penalty_kernels.cu:75-99 */

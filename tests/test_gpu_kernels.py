@@ -719,6 +719,73 @@ def test_softmax_and_topp_random_shapes(env, dt, seed):
 
 
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_fused_topp_step_against_the_three_calls_of_the_oracle(env, dt, seed):
+    """ftk_fused_topp_step = softmax, top-p sampler and decay in one call: the probabilities left in the logits
+    buffer bit for bit, ids, flags, lengths, log-probs and the decayed top_p, on seeded random shapes with pad
+    columns, finished and skipped rows, with and without an embedding bias."""
+    torch, lib, ops = env
+    rng = np.random.default_rng(7000 + 100 * dt + seed)
+    for case in range(5):
+        V = int(rng.choice([rng.integers(9, 300), rng.integers(300, 9000), rng.integers(9000, 70000)]))
+        Vp = V + int(rng.choice([0, 0, 1, 7, 64]))
+        batch = int(rng.integers(1, 12))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            x = rng.standard_normal((batch, Vp)) * rng.uniform(0.1, 4.0)
+        elif kind == 1:
+            ranks = np.arange(1, Vp + 1, dtype=np.float64)
+            x = np.stack([(-rng.uniform(0.8, 1.5) * np.log(ranks))[rng.permutation(Vp)] for _ in range(batch)])
+            x = x + rng.standard_normal((batch, Vp)) * 0.3
+        else:
+            x = rng.integers(0, 4, (batch, Vp)).astype(np.float64) * rng.uniform(0.2, 2.0)   # few distinct values
+        logits = O.to_storage(x.astype(np.float32), dt)
+        bias = O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt) if case % 2 else None
+        end_ids = rng.integers(0, V, batch).astype(np.int32)
+        finished = rng.random(batch) < 0.15
+        skip = rng.random(batch) < 0.2
+        seq = rng.integers(1, 9, batch).astype(np.int32)
+        p_arr = rng.uniform(0.1, 1.0, batch).astype(np.float32)
+        init = rng.uniform(0.5, 1.0, batch).astype(np.float32)
+        decay = rng.uniform(0.5, 1.0, batch).astype(np.float32)
+        pmin = rng.uniform(0.05, 0.4, batch).astype(np.float32)
+        u = uniforms(rng, batch)
+        with_decay = case != 2
+        # the oracle, call by call
+        want = logits.copy()
+        O.add_bias_softmax(dt, want, bias, end_ids, finished, batch, Vp, V)
+        w_ids, w_fin, w_seq, w_cum, w_out = _oracle_topp(dt, want, p_arr, end_ids, u, finished.copy(), seq, skip, True)
+        reset = np.where(rng.random(batch) < 0.3, w_ids, -1).astype(np.int32)   # some rows hit their reset id
+        w_p = p_arr.copy()
+        if with_decay:
+            O.compute_topp_decay(w_p, init, w_ids, decay, pmin, reset, batch)
+        # the product, one call
+        d_x, d_bias = to_torch(logits, dt), to_torch(bias, dt)
+        d_ids = torch.full((batch,), -7, dtype=torch.int32, device="cuda")
+        d_fin, d_seq, d_skip = to_torch(finished), to_torch(seq), to_torch(skip)
+        d_cum = torch.zeros(batch, dtype=torch.float32, device="cuda")
+        d_out = torch.zeros(batch, dtype=torch.float32, device="cuda")
+        d_p, d_init, d_decay, d_pmin, d_reset = (to_torch(a) for a in (p_arr, init, decay, pmin, reset))
+        d_end, d_u = to_torch(end_ids), to_torch(u)
+        ws_size = C.c_size_t(0)
+        sizes = (dt, None, C.addressof(ws_size), None, None, V, Vp, batch) + (None,) * 8 + (1.0,) + (None,) * 7
+        ops.check(lib.ftk_fused_topp_step(*sizes))
+        ws = torch.empty(max(ws_size.value, 16), dtype=torch.uint8, device="cuda")
+        ops.check(lib.ftk_fused_topp_step(dt, ws.data_ptr(), C.addressof(ws_size), d_x.data_ptr(), ops.ptr(d_bias), V, Vp,
+                                          batch, d_end.data_ptr(), d_fin.data_ptr(), d_seq.data_ptr(),
+                                          d_ids.data_ptr(), d_cum.data_ptr(), d_out.data_ptr(), None, d_u.data_ptr(),
+                                          float(p_arr.max()), d_p.data_ptr(), d_init.data_ptr(),
+                                          d_decay.data_ptr() if with_decay else None, d_pmin.data_ptr(),
+                                          d_reset.data_ptr(), d_skip.data_ptr(), ops.current_stream()))
+        _sync(torch)
+        where = (V, Vp, batch, kind, case)
+        assert np.array_equal(np.asarray(to_numpy(d_x)).view(np.uint8), np.asarray(want).view(np.uint8)), where
+        got = (to_numpy(d_ids), to_numpy(d_fin), to_numpy(d_seq), to_numpy(d_cum), to_numpy(d_out))
+        _compare_topk(got, (w_ids, w_fin, w_seq, w_cum, w_out), dt)
+        assert np.array_equal(to_numpy(d_p).view(np.uint32), w_p.view(np.uint32)), where
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
 @pytest.mark.parametrize("max_k", [129, 512, 513, 1024])
 def test_topk_sampling_large_k_variants(env, dt, max_k):
     """Launches whose largest k exceeds 128 (and 512) take their own streaming variants: rows of several tiles,
