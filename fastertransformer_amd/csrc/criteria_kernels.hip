@@ -91,6 +91,12 @@ __global__ void test_math_kernel(int kind, const float* __restrict__ in, float* 
             case 4: y = 1.0f / (x + 1e-6f); break;             // correctly rounded division
             case 5: y = x * 1.1754944e-38f + x * 0.5f * 1.1754944e-38f; break;  // subnormal arithmetic
             case 6: y = det_expf_nonpos(x); break;
+            case 7: {
+                // pairs (numerator, denominator): the short division into the even slot, `/` into the odd one
+                const float      other = in[i ^ 1];
+                const RowDivisor div((i & 1) ? x : other);
+                y = (i & 1) ? other / x : (div.ok ? div.divide(x) : x / other);
+            } break;
             default: y = x;
         }
         out[i] = y;

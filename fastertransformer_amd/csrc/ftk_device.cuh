@@ -9,6 +9,38 @@ namespace ftk {
 
 constexpr int WAVE = 64;
 
+// Many numerators over one denominator, bit for bit the IEEE quotient. The compiler expands `n / d` into
+// v_div_scale (both operands), v_rcp, one refinement of the reciprocal, two corrections of the quotient, v_div_fmas
+// and v_div_fixup; for operands that need no scaling and no fix-up the scale and fix-up instructions pass their
+// inputs through, and what remains is the sequence below with the reciprocal's part computed once. No scaling is
+// needed when the denominator lies in [1, 2^30] and the numerator is 0 or in [2^-100, 1] (the quotient is then a
+// normal number and every remainder exact); other numerators take the ordinary division.
+struct RowDivisor {
+    float d, r;
+    bool  ok;  // the denominator allows the short sequence (same for every thread that shares it)
+
+    __device__ __forceinline__ explicit RowDivisor(float denom)
+    {
+        d              = denom;
+        ok             = denom >= 1.0f && denom <= 1073741824.0f;
+        const float r0 = __builtin_amdgcn_rcpf(denom);
+        const float e0 = __builtin_fmaf(-denom, r0, 1.0f);
+        r              = __builtin_fmaf(e0, r0, r0);
+    }
+    // requires ok; n must be +0, in (0, 1], or NaN
+    __device__ __forceinline__ float divide(float n) const
+    {
+        if (n >= 7.888609052210118e-31f || n == 0.0f) {
+            const float q0 = n * r;
+            const float m0 = __builtin_fmaf(-d, q0, n);
+            const float q1 = __builtin_fmaf(m0, r, q0);
+            const float m1 = __builtin_fmaf(-d, q1, n);
+            return __builtin_fmaf(m1, r, q1);
+        }
+        return n / d;
+    }
+};
+
 #define FTK_LAUNCH_CHECK()                                                                                             \
     do {                                                                                                               \
         hipError_t e_ = hipGetLastError();                                                                             \

@@ -93,9 +93,10 @@ FTK_HD float det_expf(float x)
 // clamp keeps -inf out of the argument reduction and lets a NaN through.
 FTK_HD float det_expf_nonpos(float x)
 {
-    x             = x < -104.0f ? -104.0f : x;
-    const float n = __builtin_rintf(x * 1.44269502162933349609375f);
-    float       r = fma_rn(n, -0.693145751953125f, x);
+    const float x0 = x;
+    x              = __builtin_fmaxf(x, -104.0f);  // one instruction on the device; a NaN leaves as -104, see below
+    const float n  = __builtin_rintf(x * 1.44269502162933349609375f);
+    float       r  = fma_rn(n, -0.693145751953125f, x);
     r             = fma_rn(n, -1.428606765330187045e-06f, r);
     float p       = 1.9875691500e-4f;
     p             = fma_rn(p, r, 1.3981999507e-3f);
@@ -105,8 +106,8 @@ FTK_HD float det_expf_nonpos(float x)
     p             = fma_rn(p, r, 5.0000001201e-1f);
     const float z = r * r;
     float       y = fma_rn(p, z, r) + 1.0f;
-    if (x != x) {
-        return x;
+    if (x0 != x0) {
+        return x0;
     }
     const int ni = (int)n;
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -299,6 +300,12 @@ FTK_HD uint32_t order_key(float f)
         u = 0u;
     }
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+// order_key for a value known to be +0, positive or NaN
+FTK_HD uint32_t order_key_nonneg(float f)
+{
+    const uint32_t u = f2u(f);
+    return u <= 0x7F800000u ? (u | 0x80000000u) : 0u;
 }
 FTK_HD float key_to_float(uint32_t k)
 {

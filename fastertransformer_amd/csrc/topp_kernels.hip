@@ -211,9 +211,17 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
             }
             return;
         }
-        transform_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) {
-            return round_t<DT>(det_expf_nonpos((x + 0.0f) - mx)) / denom;
-        });
+        const RowDivisor div(denom);
+        if (div.ok) {
+            transform_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) {
+                return div.divide(round_t<DT>(det_expf_nonpos((x + 0.0f) - mx)));
+            });
+        }
+        else {
+            transform_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) {
+                return round_t<DT>(det_expf_nonpos((x + 0.0f) - mx)) / denom;
+            });
+        }
         transform_columns<DT, SM_THREADS>(rowp, n, n_padded, [&](int, float) { return pad_e / denom; });
         return;
     }
@@ -480,12 +488,33 @@ softmax_finish_histogram_kernel(typename Storage<DT>::T* __restrict__ logits,
         }
         return p;
     };
-    typename S::T* rowp = logits + (size_t)row * n_padded;
-    if (!fin && bias == nullptr) {
-        // ordinary rows: no per-column cases in front of the arithmetic
+    typename S::T*   rowp = logits + (size_t)row * n_padded;
+    const RowDivisor div(denom);
+    if (!fin && bias == nullptr && div.ok) {
+        // Ordinary rows: no per-column cases in front of the arithmetic, the division with the row's reciprocal,
+        // and keys of values that cannot be negative (the exponential is in [0, 1] or NaN, the denominator at
+        // least 1: probabilities in [0, 1]). `x + 0.0f` is left out: it only turns -0 into +0, and the
+        // exponential of both differences is the same.
+        auto quick = [&](int v, float y) {
+            const float p = div.divide(round_t<DT>(det_expf_nonpos(y - mx)));
+            if (tally) {
+                const float    pr = round_t<DT>(p);
+                const uint32_t k  = order_key_nonneg(pr);
+                if (k > tmax) {
+                    tmax = k;
+                    tidx = v;
+                }
+                if (k > ZERO_KEY) {
+                    const int b = topp_bucket(k);
+                    atomicAdd(&cnt[b], 1u);
+                    atomicAdd(&mass[b], (uint32_t)(pr * 2147483648.0f));
+                }
+            }
+            return p;
+        };
         const int mid = min(hi, max(lo, n));
-        transform_columns<DT, TPH_THREADS>(rowp, lo, mid, [&](int v, float x) { return finish(v, x + 0.0f); });
-        transform_columns<DT, TPH_THREADS>(rowp, mid, hi, [&](int v, float) { return finish(v, -MAXT); });
+        transform_columns<DT, TPH_THREADS>(rowp, lo, mid, [&](int v, float x) { return quick(v, x); });
+        transform_columns<DT, TPH_THREADS>(rowp, mid, hi, [&](int v, float) { return quick(v, -MAXT); });
     }
     else {
         transform_columns<DT, TPH_THREADS>(rowp, lo, hi, [&](int v, float x) {

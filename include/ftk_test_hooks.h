@@ -18,7 +18,9 @@ float ftk_host_logf(float x);
 /* raw Philox-4x32-10 block for known-answer tests (host) */
 void ftk_host_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
 /* kind 0: det_expf, 1: det_logf, 2: float->half->float, 3: float->bf16->float, 4: 1/(x+1e-6), 5: subnormal
- * arithmetic, 6: det_expf_nonpos (x <= 0 or NaN); n elements on device */
+ * arithmetic, 6: det_expf_nonpos (x <= 0 or NaN), 7: `in` holds (numerator, denominator) pairs, out[2j] = the
+ * quotient by the shared-reciprocal sequence of the softmax, out[2j+1] = the ordinary division; n elements on
+ * device */
 int ftk_test_device_math(int kind, const float* in, float* out, size_t n, ftk_stream_t stream);
 /* draws `n_draws` uniforms per row into out[row*n_draws + i], advancing the states */
 int ftk_test_rng_uniform(ftk_rng_state* states, float* out, int batch_size, int n_draws, ftk_stream_t stream);

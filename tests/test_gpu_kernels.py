@@ -106,6 +106,39 @@ def test_device_exp_of_non_positive_arguments(env):
     assert np.isnan(to_numpy(out)[0])
 
 
+def test_device_division_by_a_shared_reciprocal(env):
+    """The softmax divides a row by one denominator with the reciprocal's part of the division computed once:
+    bit for bit numpy's IEEE quotient, for numerators over the whole range an exponential can take (zero,
+    subnormal, the band around the switch to the ordinary division, up to 1) and denominators from 1 to beyond
+    the range the short sequence accepts."""
+    torch, _, ops = env
+    lib = ops.ftk_hooks()
+    rng = np.random.default_rng(78)
+    n = 1 << 21
+    num = np.concatenate([
+        np.exp(-rng.uniform(0.0, 104.0, n // 2)), rng.uniform(0.0, 1.0, n // 4),
+        np.exp2(-rng.uniform(96.0, 104.0, n // 8)),                         # around 2^-100
+        rng.integers(0, 1 << 23, n // 8 - 8).view(np.int64).astype(np.uint32).view(np.float32).astype(np.float64),
+        [0.0, 1.0, 2.0 ** -100, np.nextafter(np.float32(2.0 ** -100), np.float32(0)), 2.0 ** -126, 2.0 ** -149,
+         np.nextafter(np.float32(1), np.float32(0)), 0.5]]).astype(np.float32)
+    den = np.concatenate([
+        1.0 + rng.uniform(0.0, 1.0, n // 4), np.exp(rng.uniform(0.0, 20.0, n // 2)),
+        rng.integers(1, 200000, n // 8).astype(np.float64) + 1e-6,
+        np.exp2(rng.uniform(29.0, 31.0, n // 8 - 4)), [1.0, 2.0 ** 30, np.nextafter(np.float32(2.0 ** 30), np.float32(np.inf)),
+                                                      np.nextafter(np.float32(1), np.float32(0))]]).astype(np.float32)
+    den = den[rng.permutation(den.size)]
+    pairs = np.stack([num, den], axis=1).reshape(-1).copy()
+    d_in = to_torch(pairs)
+    d_out = torch.empty_like(d_in)
+    ops.check(lib.ftk_test_device_math(7, d_in.data_ptr(), d_out.data_ptr(), pairs.size, ops.current_stream()))
+    _sync(torch)
+    out = to_numpy(d_out).reshape(-1, 2)
+    with np.errstate(under="ignore"):
+        want = (num / den).astype(np.float32)
+    assert np.array_equal(out[:, 0].view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(out[:, 1].view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
 @pytest.mark.parametrize("V,Vp", [(4, 4), (50001, 50001), (50001, 50008), (32000, 32000), (1000, 1024)])
 @pytest.mark.parametrize("with_bias", [False, True])
