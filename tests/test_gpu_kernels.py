@@ -751,19 +751,30 @@ def test_softmax_and_topp_random_shapes(env, dt, seed):
             _compare_topk(_run_topp(env, *args), _oracle_topp(*args), dt)
 
 
+@pytest.mark.parametrize("V,Vp", [(1024, 1024), (1025, 1031), (128256, 128256), (152064 - 1, 152064)])
+def test_fused_topp_step_full_vocabularies(env, V, Vp):
+    """the one-call top-p step at the reference block's width, one column beyond it, and at full vocabulary
+    sizes (several chunks per row in the dividing pass)"""
+    _fused_topp_cases(env, O.F32, np.random.default_rng(V + Vp), [(V, Vp, 3, 0), (V, Vp, 2, 1), (V, Vp, 3, 2)])
+
+
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_fused_topp_step_against_the_three_calls_of_the_oracle(env, dt, seed):
     """ftk_fused_topp_step = softmax, top-p sampler and decay in one call: the probabilities left in the logits
     buffer bit for bit, ids, flags, lengths, log-probs and the decayed top_p, on seeded random shapes with pad
     columns, finished and skipped rows, with and without an embedding bias."""
-    torch, lib, ops = env
     rng = np.random.default_rng(7000 + 100 * dt + seed)
+    shapes = []
     for case in range(5):
         V = int(rng.choice([rng.integers(9, 300), rng.integers(300, 9000), rng.integers(9000, 70000)]))
-        Vp = V + int(rng.choice([0, 0, 1, 7, 64]))
-        batch = int(rng.integers(1, 12))
-        kind = int(rng.integers(0, 3))
+        shapes.append((V, V + int(rng.choice([0, 0, 1, 7, 64])), int(rng.integers(1, 12)), int(rng.integers(0, 3))))
+    _fused_topp_cases(env, dt, rng, shapes)
+
+
+def _fused_topp_cases(env, dt, rng, shapes):
+    torch, lib, ops = env
+    for case, (V, Vp, batch, kind) in enumerate(shapes):
         if kind == 0:
             x = rng.standard_normal((batch, Vp)) * rng.uniform(0.1, 4.0)
         elif kind == 1:
