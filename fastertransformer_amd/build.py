@@ -41,6 +41,7 @@ KERNEL_UNITS = [
     ("penalty_kernels.hip", "penalty_kernels.o", []),
     ("criteria_kernels.hip", "criteria_kernels.o", []),
     ("decode_step_kernels.hip", "decode_step_kernels.o", []),
+    ("beam_kernels.hip", "beam_kernels.o", []),
 ]
 
 # -ffp-contract=off: results must match a plain IEEE evaluation operation by operation.

@@ -1,0 +1,586 @@
+// One step of beam search over [batch * beam_width, vocab] logits: log-softmax, the 2K best tokens of every beam,
+// the K best continuations of every batch entry, finished hypotheses moved to the BeamHypotheses arrays.
+//
+// Reference behaviour restated (src/fastertransformer/kernels/online_softmax_beamsearch_kernels.cu):
+//   :366-514  beam_online_softmax_topk_stage1 / stage2 - per row (max, sum of exponentials) and the 2K best
+//             elements under TopK<T, MAX_K>::insert (kernels/reduce_kernel_utils.cuh:275-322): value
+//             descending, id ascending, which no merge order changes
+//   :99-262   batch_topk_kernel - the 2 * MAX_K best of a batch entry's K * 2K candidates after length penalty
+//             and diversity term, then one thread walks them: end tokens among the first K go to the
+//             hypotheses (kernels/beam_search_topk_kernels.h:31-58), the others become the next beams
+//   :549-701  launchers and the beam-width classes
+//
+// The reference finds the best elements by inserting into per-thread sorted arrays and merging them with cub. Here
+// every selection is an exact radix select over 64-bit keys (order-preserving value bits, then the complement of
+// the position, so that keys are distinct and ties need no rule of their own): byte by byte from the top, a
+// 256-bin LDS histogram of the keys that match the bytes fixed so far; as soon as few enough match they are moved
+// to LDS and the remaining bytes are settled there.
+#include "ftk_device.cuh"
+#include "ftk_sampling.h"
+#include "ftk_transform.cuh"
+
+namespace ftk {
+
+constexpr int BM_THREADS = 256;
+constexpr int BM_WAVES   = BM_THREADS / WAVE;
+constexpr int BM_CAP     = 2048;  // keys settled in LDS
+constexpr int BM_MAX_N   = 128;   // 2 * beam_width and 2 * MAX_K are at most this
+
+struct BeamSelect {
+    unsigned long long list[BM_CAP];
+    unsigned long long out[BM_MAX_N];
+    uint32_t           hist[256];
+    uint32_t           wave_total[BM_WAVES];
+    int                n_list;
+    int                n_out;
+    int                found_bin;
+    int                found_above;
+};
+
+// The `need`-th largest of `count` keys key(i), 1 <= need <= count, distinct at least down to that one (zero keys
+// that pad a list may repeat below it): every thread of the workgroup gets it. key(i) is evaluated once per byte
+// that is settled on the caller's data (until BM_CAP or fewer keys match).
+template<class F>
+__device__ __forceinline__ unsigned long long beam_nth_key(BeamSelect& s, F&& key, int count, int need)
+{
+    const int          t      = threadIdx.x;
+    unsigned long long prefix = 0ull;
+    bool               in_lds = false;
+    int                n      = count;
+    for (int shift = 56; shift >= 0; shift -= 8) {
+        s.hist[t] = 0u;
+        __syncthreads();
+        for (int i = t; i < n; i += BM_THREADS) {
+            const unsigned long long k = in_lds ? s.list[i] : key(i);
+            if (shift == 56 || (k >> (shift + 8)) == prefix) {
+                atomicAdd(&s.hist[(uint32_t)(k >> shift) & 255u], 1u);
+            }
+        }
+        __syncthreads();
+        // thread t looks at bin 255 - t: inclusive sums from the top bin down
+        const uint32_t mine = s.hist[255 - t];
+        uint32_t       inc  = mine;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const uint32_t up = __shfl_up(inc, o, WAVE);
+            if (lane_id() >= o) {
+                inc += up;
+            }
+        }
+        if (lane_id() == WAVE - 1) {
+            s.wave_total[wave_id()] = inc;
+        }
+        __syncthreads();
+        for (int w = 0; w < wave_id(); ++w) {
+            inc += s.wave_total[w];
+        }
+        if (inc >= (uint32_t)need && inc - mine < (uint32_t)need) {
+            s.found_bin   = 255 - t;
+            s.found_above = (int)(inc - mine);
+        }
+        __syncthreads();
+        const int bin     = s.found_bin;
+        const int matched = (int)s.hist[bin];
+        need -= s.found_above;
+        prefix = (prefix << 8) | (unsigned long long)bin;
+        if (!in_lds && matched <= BM_CAP && shift > 0) {
+            // few enough keys carry the bytes fixed so far: the rest is settled on a copy in LDS
+            if (t == 0) {
+                s.n_list = 0;
+            }
+            __syncthreads();
+            for (int i = t; i < n; i += BM_THREADS) {
+                const unsigned long long k = key(i);
+                if ((k >> shift) == prefix) {
+                    s.list[atomicAdd(&s.n_list, 1)] = k;
+                }
+            }
+            __syncthreads();
+            in_lds = true;
+            n      = matched;
+        }
+        __syncthreads();
+    }
+    return prefix;
+}
+
+// Leaves the `need` largest of `count` distinct keys in s.out, largest first; need <= BM_MAX_N, need <= count.
+template<class F>
+__device__ __forceinline__ void beam_select(BeamSelect& s, F&& key, int count, int need)
+{
+    const int                t     = threadIdx.x;
+    const unsigned long long bound = beam_nth_key(s, key, count, need);
+    if (t == 0) {
+        s.n_out = 0;
+    }
+    __syncthreads();
+    for (int i = t; i < count; i += BM_THREADS) {
+        const unsigned long long k = key(i);
+        if (k >= bound) {
+            s.list[atomicAdd(&s.n_out, 1)] = k;  // exactly `need` of them
+        }
+    }
+    __syncthreads();
+    if (t < need) {
+        const unsigned long long k = s.list[t];
+        int                      r = 0;
+        for (int j = 0; j < need; ++j) {
+            r += s.list[j] > k ? 1 : 0;
+        }
+        s.out[r] = k;
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ unsigned long long beam_key(float value, uint32_t position)
+{
+    return ((unsigned long long)order_key(value) << 32) | (unsigned long long)(0xFFFFFFFFu - position);
+}
+__device__ __forceinline__ uint32_t beam_key_position(unsigned long long k)
+{
+    return 0xFFFFFFFFu - (uint32_t)k;
+}
+__device__ __forceinline__ float beam_key_value(unsigned long long k)
+{
+    return key_to_float((uint32_t)(k >> 32));
+}
+
+// element `v` of row `r` as the reference's kernels see it (:341-347, :410-416)
+template<int DT>
+__device__ __forceinline__ float beam_element(const typename Storage<DT>::T* __restrict__ x,
+                                              const typename Storage<DT>::T* __restrict__ bias, size_t row_base, int v)
+{
+    typedef Storage<DT> S;
+    const float         b = bias != nullptr ? S::ld(bias[v]) : 0.0f;
+    return round_t<DT>(S::ld(x[row_base + v]) + b);
+}
+
+struct BeamPlan {
+    int    parts;  // sections per row
+    int    section;
+    size_t off_pmax, off_psum, off_pkeys, off_cand_id, off_cand_val, bytes;
+};
+
+static inline size_t beam_align(size_t x)
+{
+    return (x + 255) & ~(size_t)255;
+}
+
+static BeamPlan beam_plan(int rows, int beam_width, int vocab)
+{
+    BeamPlan  p;
+    const int N = 2 * beam_width;
+    int       parts = (1024 + rows - 1) / (rows > 0 ? rows : 1);
+    const int by_len = vocab / 4096 > 0 ? vocab / 4096 : 1;
+    parts   = parts < by_len ? parts : by_len;
+    parts   = parts < BM_CAP / N ? parts : BM_CAP / N;  // the lists of a row are merged in LDS
+    parts   = parts < 1 ? 1 : parts;
+    while (parts > 1 && (vocab + parts - 1) / parts < N) {
+        parts--;  // every section holds at least 2K elements
+    }
+    p.parts   = parts;
+    p.section = (vocab + parts - 1) / parts;
+    const size_t r = (size_t)(rows > 0 ? rows : 1);
+    size_t       off = 0;
+    p.off_pmax = off;
+    off += beam_align(r * parts * sizeof(float));
+    p.off_psum = off;
+    off += beam_align(r * parts * sizeof(double));
+    p.off_pkeys = off;
+    off += beam_align(r * parts * N * sizeof(unsigned long long));
+    p.off_cand_id = off;
+    off += beam_align(r * N * sizeof(int));
+    p.off_cand_val = off;
+    off += beam_align(r * N * sizeof(float));
+    p.bytes = off;
+    return p;
+}
+
+// (parts x rows) workgroups: the maximum of a section
+template<int DT>
+__global__ void __launch_bounds__(BM_THREADS)
+beam_section_max_kernel(const typename Storage<DT>::T* __restrict__ x, const typename Storage<DT>::T* __restrict__ bias,
+                        const bool* __restrict__ finished, int vocab, int section, float* __restrict__ pmax)
+{
+    __shared__ float red[BM_WAVES];
+    const int        row = blockIdx.y;
+    const int        t   = threadIdx.x;
+    if (finished[row]) {
+        return;
+    }
+    const int    lo = min(vocab, (int)blockIdx.x * section);
+    const int    hi = min(vocab, lo + section);
+    const size_t rb = (size_t)row * vocab;
+    float        m  = -Storage<DT>::max_t();
+    for (int v = lo + t; v < hi; v += BM_THREADS) {
+        const float e = beam_element<DT>(x, bias, rb, v);
+        m             = e > m ? e : m;
+    }
+    m = block_max<float, BM_WAVES>(m, red, -Storage<DT>::max_t());
+    if (t == 0) {
+        pmax[(size_t)row * gridDim.x + blockIdx.x] = m;
+    }
+}
+
+// (parts x rows) workgroups: the sum of exponentials of a section against the row's maximum and its 2K best
+template<int DT>
+__global__ void __launch_bounds__(BM_THREADS)
+beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typename Storage<DT>::T* __restrict__ bias,
+                    const bool* __restrict__ finished, int vocab, int section, int N, const float* __restrict__ pmax,
+                    double* __restrict__ psum, unsigned long long* __restrict__ pkeys)
+{
+    __shared__ BeamSelect s;
+    __shared__ double     red[BM_WAVES];
+    const int             row   = blockIdx.y;
+    const int             part  = blockIdx.x;
+    const int             parts = gridDim.x;
+    const int             t     = threadIdx.x;
+    if (finished[row]) {
+        return;
+    }
+    const int    lo = min(vocab, part * section);
+    const int    hi = min(vocab, lo + section);
+    const size_t rb = (size_t)row * vocab;
+    float        m  = -Storage<DT>::max_t();
+    for (int p = 0; p < parts; ++p) {
+        const float pm = pmax[(size_t)row * parts + p];
+        m              = pm > m ? pm : m;
+    }
+    double d = 0.0;
+    for (int v = lo + t; v < hi; v += BM_THREADS) {
+        d += (double)det_expf(beam_element<DT>(x, bias, rb, v) - m);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        d += __shfl_xor(d, o, WAVE);
+    }
+    if (lane_id() == 0) {
+        red[wave_id()] = d;
+    }
+    __syncthreads();
+    if (t == 0) {
+        double tot = 0.0;
+        for (int w = 0; w < BM_WAVES; ++w) {
+            tot += red[w];
+        }
+        psum[(size_t)row * parts + part] = tot;
+    }
+    // a short last section gives fewer than N keys; the rest of its list is 0, below every key of an element
+    const int take = min(N, hi - lo);
+    if (take > 0) {
+        beam_select(s, [&](int i) { return beam_key(beam_element<DT>(x, bias, rb, lo + i), (uint32_t)(lo + i)); },
+                    hi - lo, take);
+    }
+    if (t < N) {
+        pkeys[((size_t)row * parts + part) * N + t] = t < take ? s.out[t] : 0ull;
+    }
+}
+
+// one workgroup per row: the row's 2K best from its sections' lists, val = u - m - log(d) + cum_log_probs as T
+template<int DT>
+__global__ void __launch_bounds__(BM_THREADS)
+beam_row_kernel(const bool* __restrict__ finished, const int* __restrict__ end_ids,
+                const float* __restrict__ cum_log_probs, int vocab, int K, int parts, const float* __restrict__ pmax,
+                const double* __restrict__ psum, const unsigned long long* __restrict__ pkeys,
+                int* __restrict__ cand_id, float* __restrict__ cand_val)
+{
+    typedef Storage<DT>   S;
+    __shared__ BeamSelect s;
+    const int             row  = blockIdx.x;
+    const int             t    = threadIdx.x;
+    const int             N    = 2 * K;
+    const float           MAXT = S::max_t();
+    const float           cum  = cum_log_probs[row];
+    if (finished[row]) {
+        // MAX_T at the end id, -MAX_T elsewhere (:328-336): the end id first, then the lowest ids
+        const int  end_id = end_ids[row / K];
+        const bool inside = end_id >= 0 && end_id < vocab;
+        if (t < N) {
+            int   id;
+            float u;
+            if (inside) {
+                id = t == 0 ? end_id : (t - 1 < end_id ? t - 1 : t);
+                u  = t == 0 ? MAXT : -MAXT;
+            }
+            else {
+                id = t;
+                u  = -MAXT;
+            }
+            // inside: m = MAX_T, every other exponential is 0, d = 1; otherwise m = -MAX_T and d = vocab
+            const float m    = inside ? MAXT : -MAXT;
+            const float logd = inside ? 0.0f : det_logf((float)vocab);
+            cand_id[(size_t)row * N + t]  = id + row * vocab;
+            cand_val[(size_t)row * N + t] = round_t<DT>((u - m - logd) + cum);
+        }
+        return;
+    }
+    float  m = -MAXT;
+    double d = 0.0;
+    for (int p = 0; p < parts; ++p) {
+        const float pm = pmax[(size_t)row * parts + p];
+        m              = pm > m ? pm : m;
+        d += psum[(size_t)row * parts + p];
+    }
+    const float               logd = det_logf((float)d);
+    const unsigned long long* keys = pkeys + (size_t)row * parts * N;
+    if (parts == 1) {
+        if (t < N) {
+            s.out[t] = keys[t];
+        }
+        __syncthreads();
+    }
+    else {
+        beam_select(s, [&](int i) { return keys[i]; }, parts * N, N);
+    }
+    if (t < N) {
+        const unsigned long long k    = s.out[t];
+        cand_id[(size_t)row * N + t]  = (int)beam_key_position(k) + row * vocab;
+        cand_val[(size_t)row * N + t] = round_t<DT>((beam_key_value(k) - m - logd) + cum);
+    }
+}
+
+struct BeamHypsDevice {
+    int*         output_ids_tgt;
+    int*         sequence_lengths_tgt;
+    float*       cum_log_probs;
+    float*       normed_scores;
+    float*       log_probs;
+    float*       min_normed_scores;
+    int*         num_beams;
+    bool*        is_done;
+    const int*   output_ids_src;
+    const int*   parent_ids_src;
+    const int*   end_ids;
+    const float* log_probs_src;
+    int          step;
+    int          ite;
+    int          batch_size;
+    int          local_batch_size;
+    int          max_seq_len;
+    int          early_stopping;
+};
+
+// one workgroup per batch entry (:99-262)
+template<int DT>
+__global__ void __launch_bounds__(BM_THREADS)
+beam_batch_kernel(const int* __restrict__ cand_id, const float* __restrict__ cand_val, int* __restrict__ ids,
+                  float* cum_log_probs, float* __restrict__ output_log_probs, const bool* __restrict__ finished,
+                  const int* __restrict__ sequence_lengths, BeamHypsDevice h, int K, int max_k2, int vocab,
+                  float length_penalty, float diversity_rate)
+{
+    __shared__ BeamSelect s;
+    __shared__ float      old_cum[64];
+    __shared__ float      score_of[BM_MAX_N];
+    const int             b = blockIdx.x;
+    const int             t = threadIdx.x;
+    const int             C = K * 2 * K;
+    const int*            x = cand_id + (size_t)b * C;
+    const float*          y = cand_val + (size_t)b * C;
+    if (t < K) {
+        old_cum[t] = cum_log_probs[b * K + t];
+    }
+    const bool with_hyps = h.num_beams != nullptr;
+    const int  g         = h.ite * h.local_batch_size + b;
+    if (with_hyps) {
+        const int nb = h.num_beams[g];
+        if (nb == 0 && t == 0) {
+            h.min_normed_scores[g] = 3.402823466e+38f;
+        }
+        else if (nb == K) {
+            return;
+        }
+    }
+    // (:146-156) the batch entry's own flag and length are used for all of its beams, as in the reference
+    float denom = 1.0f;
+    if (length_penalty != 0.0f) {
+        const int length = finished[b] ? sequence_lengths[b] : sequence_lengths[b] + 1;
+        if (length != 1) {
+            denom = round_t<DT>(det_expf(length_penalty * det_logf((float)length)));
+        }
+        else {
+            length_penalty = 0.0f;
+        }
+    }
+    const float div_t = round_t<DT>(diversity_rate);
+    auto        score = [&](int c) {
+        float elem = y[c];
+        if (length_penalty != 0.0f) {
+            elem = round_t<DT>(elem / denom);
+        }
+        return round_t<DT>(elem + round_t<DT>(div_t * round_t<DT>((float)(c % K))));
+    };
+    const int take = max_k2 < C ? max_k2 : C;
+    beam_select(s, [&](int c) { return beam_key(score(c), (uint32_t)c); }, C, take);
+    if (t < take) {
+        score_of[t] = score((int)beam_key_position(s.out[t]));
+    }
+    __syncthreads();
+    if (t != 0) {
+        return;
+    }
+    int*   z        = ids + (size_t)b * K;
+    float* v        = cum_log_probs + (size_t)b * K;
+    int    selected = 0;
+    for (int i = 0; i < take; ++i) {
+        const int p = (int)beam_key_position(s.out[i]);
+        if (with_hyps && x[p] % vocab == h.end_ids[b]) {
+            if (i < K) {
+                const float normed_score = score_of[i];
+                const int   num_beam     = h.num_beams[g];
+                int         beam_idx     = num_beam;
+                if (num_beam == K) {
+                    if (normed_score < h.min_normed_scores[g]) {
+                        selected = K;
+                        break;
+                    }
+                    for (int j = 0; j < K; ++j) {
+                        if (h.normed_scores[g * (K * 2) + j] == h.min_normed_scores[g]) {
+                            beam_idx = j;
+                            h.num_beams[g]--;
+                            h.min_normed_scores[g]           = 3.402823466e+38f;
+                            h.normed_scores[g * (K * 2) + j] = normed_score;
+                            for (int l = 0; l < K; ++l) {
+                                h.min_normed_scores[g] =
+                                    __builtin_fminf(h.min_normed_scores[g], h.normed_scores[g * (K * 2) + l]);
+                            }
+                            break;
+                        }
+                    }
+                }
+                const size_t tgt = ((size_t)(b + h.ite * h.local_batch_size) * (K * 2) + beam_idx) * h.max_seq_len;
+                h.output_ids_tgt[tgt + h.step] = h.end_ids[b];
+                if (h.log_probs != nullptr) {
+                    h.log_probs[tgt + h.step] = y[p] - old_cum[(x[p] / vocab) % K];
+                }
+                int prev_id = (x[p] / vocab) % K;
+                for (int j = h.step - 1; j >= 0; --j) {
+                    const size_t src =
+                        (size_t)j * h.batch_size * K + (size_t)h.ite * h.local_batch_size * K + (size_t)b * K + prev_id;
+                    h.output_ids_tgt[tgt + j] = h.output_ids_src[src];
+                    if (h.log_probs != nullptr && h.log_probs_src != nullptr) {
+                        h.log_probs[tgt + j] = h.log_probs_src[src];
+                    }
+                    prev_id = h.parent_ids_src[src];
+                }
+                const int tgt_beam              = g * (K * 2) + beam_idx;
+                h.sequence_lengths_tgt[tgt_beam] = h.step;
+                h.normed_scores[tgt_beam]        = normed_score;
+                h.min_normed_scores[g] = __builtin_fminf(h.min_normed_scores[g], h.normed_scores[tgt_beam]);
+                h.num_beams[g]++;
+                h.cum_log_probs[tgt_beam] = y[p];
+            }
+        }
+        else if ((with_hyps && i < 2 * K) || (!with_hyps && i < K)) {
+            z[selected] = x[p];
+            if (output_log_probs != nullptr) {
+                output_log_probs[b * K + selected] = y[p] - old_cum[(z[selected] / vocab) % K];
+            }
+            v[selected] = y[p];
+            selected++;
+        }
+        if (selected >= K) {
+            break;
+        }
+    }
+    if (with_hyps) {
+        if (h.num_beams[b] < K) {
+            h.is_done[b] = false;
+        }
+        else if (h.early_stopping) {
+            h.is_done[b] = true;
+        }
+    }
+}
+
+}  // namespace ftk
+
+using namespace ftk;
+
+extern "C" {
+
+int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, const bool* finished,
+                            const int* sequence_lengths, float* cum_log_probs, float* output_log_probs, int* ids,
+                            void* temp_storage, size_t* temp_storage_size, const ftk_beam_hypotheses* beam_hyps,
+                            int batch_size, int beam_width, int vocab_size, const int* end_ids, float diversity_rate,
+                            float length_penalty, ftk_stream_t stream)
+{
+    if (dtype < 0 || dtype > 2) {
+        return FTK_ERR_DTYPE;
+    }
+    if (beam_width < 2 || beam_width > 64) {
+        return FTK_ERR_ARGUMENT;  // the reference's launcher covers 1..64 (:650-688) and rejects 1 (:625)
+    }
+    if (batch_size < 0 || vocab_size < 2 * beam_width || (long long)batch_size * beam_width > 65535
+        || (long long)batch_size * beam_width * vocab_size > 0x7FFFFFFFll) {
+        return FTK_ERR_ARGUMENT;  // candidate ids are row * vocab + token in an int, as in the reference
+    }
+    const int      rows = batch_size * beam_width;
+    const BeamPlan plan = beam_plan(rows, beam_width, vocab_size);
+    if (temp_storage == nullptr) {
+        if (temp_storage_size == nullptr) {
+            return FTK_ERR_ARGUMENT;
+        }
+        *temp_storage_size = plan.bytes;
+        return 0;
+    }
+    if (temp_storage_size != nullptr && *temp_storage_size < plan.bytes) {
+        return FTK_ERR_WORKSPACE;
+    }
+    if (batch_size == 0) {
+        return 0;
+    }
+    if (length_penalty != 0.0f && sequence_lengths == nullptr) {
+        return FTK_ERR_ARGUMENT;  // (:572)
+    }
+    char*               ws       = (char*)temp_storage;
+    float*              pmax     = (float*)(ws + plan.off_pmax);
+    double*             psum     = (double*)(ws + plan.off_psum);
+    unsigned long long* pkeys    = (unsigned long long*)(ws + plan.off_pkeys);
+    int*                cand_id  = (int*)(ws + plan.off_cand_id);
+    float*              cand_val = (float*)(ws + plan.off_cand_val);
+    hipStream_t         st       = (hipStream_t)stream;
+    const int           N        = 2 * beam_width;
+    const int           max_k    = beam_width <= 4 ? 4 : beam_width <= 8 ? 8 : beam_width <= 16 ? 16 : beam_width <= 32 ? 32 : 64;
+    BeamHypsDevice      h        = {};
+    if (beam_hyps != nullptr) {
+        h.output_ids_tgt       = beam_hyps->output_ids_tgt;
+        h.sequence_lengths_tgt = beam_hyps->sequence_lengths_tgt;
+        h.cum_log_probs        = beam_hyps->cum_log_probs;
+        h.normed_scores        = beam_hyps->normed_scores;
+        h.log_probs            = beam_hyps->log_probs;
+        h.min_normed_scores    = beam_hyps->min_normed_scores;
+        h.num_beams            = beam_hyps->num_beams;
+        h.is_done              = beam_hyps->is_done;
+        h.output_ids_src       = beam_hyps->output_ids_src;
+        h.parent_ids_src       = beam_hyps->parent_ids_src;
+        h.end_ids              = beam_hyps->end_ids;
+        h.log_probs_src        = beam_hyps->log_probs_src;
+        h.step                 = beam_hyps->step;
+        h.ite                  = beam_hyps->ite;
+        h.batch_size           = beam_hyps->batch_size;
+        h.local_batch_size     = beam_hyps->local_batch_size;
+        h.max_seq_len          = beam_hyps->max_seq_len;
+        h.early_stopping       = beam_hyps->early_stopping ? 1 : 0;
+    }
+    const dim3 sections(plan.parts, rows);
+    FTK_DISPATCH_DTYPE(dtype, {
+        typedef Storage<DT>::T T;
+        beam_section_max_kernel<DT><<<sections, BM_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished,
+                                                                     vocab_size, plan.section, pmax);
+        FTK_LAUNCH_CHECK();
+        beam_section_kernel<DT><<<sections, BM_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished,
+                                                                 vocab_size, plan.section, N, pmax, psum, pkeys);
+        FTK_LAUNCH_CHECK();
+        beam_row_kernel<DT><<<rows, BM_THREADS, 0, st>>>(finished, end_ids, cum_log_probs, vocab_size, beam_width,
+                                                         plan.parts, pmax, psum, pkeys, cand_id, cand_val);
+        FTK_LAUNCH_CHECK();
+        beam_batch_kernel<DT><<<batch_size, BM_THREADS, 0, st>>>(cand_id, cand_val, ids, cum_log_probs,
+                                                                 output_log_probs, finished, sequence_lengths, h,
+                                                                 beam_width, 2 * max_k, vocab_size, length_penalty,
+                                                                 diversity_rate);
+        FTK_LAUNCH_CHECK();
+    });
+    return 0;
+}
+
+}  // extern "C"

@@ -25,6 +25,17 @@ _dec = None
 
 _vp, _i, _f, _sz, _ull, _b = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_ulonglong, C.c_bool
 
+class BeamHypotheses(C.Structure):
+    """ftk_beam_hypotheses of include/ftk_sampling.h (BeamHypotheses of the reference, field for field)"""
+    _fields_ = [("output_ids_tgt", C.c_void_p), ("sequence_lengths_tgt", C.c_void_p), ("cum_log_probs", C.c_void_p),
+                ("normed_scores", C.c_void_p), ("log_probs", C.c_void_p), ("min_normed_scores", C.c_void_p),
+                ("num_beams", C.c_void_p), ("is_done", C.c_void_p), ("output_ids_src", C.c_void_p),
+                ("parent_ids_src", C.c_void_p), ("sequence_lengths_src", C.c_void_p), ("end_ids", C.c_void_p),
+                ("log_probs_src", C.c_void_p), ("step", C.c_int), ("ite", C.c_int), ("batch_size", C.c_int),
+                ("local_batch_size", C.c_int), ("max_seq_len", C.c_int), ("length_penalty", C.c_float),
+                ("early_stopping", C.c_bool), ("is_return_normed_score", C.c_bool)]
+
+
 # name -> argtypes (restype int unless listed in _RESTYPES)
 _SIGNATURES = {
     "ftk_invoke_curand_initialize": [_vp, _sz, _ull, _vp],
@@ -57,6 +68,7 @@ _SIGNATURES = {
     "ftk_invoke_plus_scalar": [_vp, _i, _i, _vp],
     "ftk_invoke_transpose_axis01": [_vp, _vp, _vp, _i, _i, _vp],
     "ftk_invoke_finalize": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "ftk_invoke_topk_softmax": [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _f, _f, _vp],
     "ftk_error_string": [_i],
     "ftk_profile_enable": [_i],
     "ftk_profile_read": [_i, _vp, _vp],

@@ -292,6 +292,49 @@ int ftk_invoke_finalize(int* output_ids, int* sequence_lengths, float* cum_log_p
                         const float* topk_cum_log_probs, const float* topk_log_probs, const int* num_beams,
                         int beam_width, int max_seq_len, int batch_size, ftk_stream_t stream);
 
+/* BeamHypotheses, kernels/beam_search_topk_kernels.h:31-58, field for field (sequence_lengths_src,
+ * length_penalty and is_return_normed_score are carried for callers that fill the reference's struct; the kernels
+ * of this call do not read them, like the reference's). */
+typedef struct ftk_beam_hypotheses {
+    int*         output_ids_tgt;
+    int*         sequence_lengths_tgt;
+    float*       cum_log_probs;
+    float*       normed_scores;
+    float*       log_probs;
+    float*       min_normed_scores;
+    int*         num_beams;
+    bool*        is_done;
+    const int*   output_ids_src;
+    const int*   parent_ids_src;
+    const int*   sequence_lengths_src;
+    const int*   end_ids;
+    const float* log_probs_src;
+    int          step;
+    int          ite;
+    int          batch_size;
+    int          local_batch_size;
+    int          max_seq_len;
+    float        length_penalty;
+    bool         early_stopping;
+    bool         is_return_normed_score;
+} ftk_beam_hypotheses;
+
+/* invokeTopkSoftMax<T>, kernels/online_softmax_beamsearch_kernels.cu:671-701: one beam-search step over
+ * log_probs [batch_size * beam_width, vocab_size]. Per row the log-softmax and its 2 * beam_width best tokens; per
+ * batch entry the candidates ranked by cum_log_probs + log-softmax (length penalty and diversity term applied as
+ * the reference does); end tokens among the first beam_width go to the hypotheses, the others become the next beams:
+ * ids [batch_size, beam_width] receives row * vocab_size + token (the reference's absolute ids), cum_log_probs is
+ * updated in place, output_log_probs (optional) gets the step's log-probs. beam_hyps may be NULL or carry
+ * num_beams == NULL (no hypotheses kept). beam_width 2..64 and vocab_size >= 2 * beam_width, else
+ * FTK_ERR_ARGUMENT. temp_storage == NULL: size query in bytes (the reference takes a size in elements from its
+ * layer). Sums of exponentials are accumulated in double precision in no particular order, so log-probs agree with
+ * the reference's pairwise (max, sum) merges within 1e-5 relative, not bit for bit. */
+int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, const bool* finished,
+                            const int* sequence_lengths, float* cum_log_probs, float* output_log_probs, int* ids,
+                            void* temp_storage, size_t* temp_storage_size, const ftk_beam_hypotheses* beam_hyps,
+                            int batch_size, int beam_width, int vocab_size, const int* end_ids, float diversity_rate,
+                            float length_penalty, ftk_stream_t stream);
+
 /* ---- per-kernel timing of the fused step (the reference's counterpart is its CudaTimer / NVTX ranges,
  * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
  * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on

@@ -829,6 +829,232 @@ void log_prob_from_logits(float* cum_log_probs, float* log_probs, const void* lo
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Beam search step: kernels/online_softmax_beamsearch_kernels.cu:296-739 (invokeTopkSoftMax) with the
+// TopK<T, MAX_K> insert rule of kernels/reduce_kernel_utils.cuh:275-322 and BeamHypotheses of
+// kernels/beam_search_topk_kernels.h:31-58.
+//   rows:   per (batch, beam) row the 2K best of elem = T(x + bias) (a finished row: MAX_T at its end id,
+//           -MAX_T elsewhere) by (value descending, id ascending), which is what any merge order of the insert
+//           rule gives on distinct ids, and val = u - m - log(d) + cum_log_probs[row], stored as T
+//           (:336-349, :500-511);
+//   batch:  per batch entry the 2 * MAX_K best of the K * 2K candidates by (score descending, candidate index
+//           ascending), score = val with length penalty and diversity term in T arithmetic (:146-160), then the
+//           single-thread walk of :163-249 over them, literally (including its use of finished[] and
+//           sequence_lengths[] at the batch index and of num_beams / is_done at the block index).
+// Departures: m and d are the row's exact maximum and the sum of det_expf(elem - m) accumulated in double
+// precision, not the reference's chain of pairwise (m, d) merges with __expf in cub's order; powf is
+// det_expf(p * det_logf(length)); a NaN orders below every number.
+// ------------------------------------------------------------------------------------------
+struct BeamHyps {
+    int*         output_ids_tgt;
+    int*         sequence_lengths_tgt;
+    float*       cum_log_probs;
+    float*       normed_scores;
+    float*       log_probs;
+    float*       min_normed_scores;
+    int*         num_beams;
+    bool*        is_done;
+    const int*   output_ids_src;
+    const int*   parent_ids_src;
+    const int*   sequence_lengths_src;
+    const int*   end_ids;
+    const float* log_probs_src;
+    int          step;
+    int          ite;
+    int          batch_size;
+    int          local_batch_size;
+    int          max_seq_len;
+    float        length_penalty;
+    int          early_stopping;
+};
+
+static int beam_max_k(int beam_width)
+{
+    // CASE_K of :650-688
+    return beam_width <= 4 ? 4 : beam_width <= 8 ? 8 : beam_width <= 16 ? 16 : beam_width <= 32 ? 32 : 64;
+}
+
+static bool order_before(float va, int ia, float vb, int ib)
+{
+    // a NaN never wins a comparison of the insert rule; it is placed last here
+    const bool na = va != va, nb = vb != vb;
+    if (na != nb) {
+        return nb;
+    }
+    if (!na && va != vb) {
+        return va > vb;
+    }
+    return ia < ib;
+}
+
+template<int DT>
+static int topk_softmax(const typename St<DT>::T* log_probs, const typename St<DT>::T* bias, const bool* finished,
+                        const int* sequence_lengths, float* cum_log_probs, float* output_log_probs, int* ids,
+                        const BeamHyps* hyps, int batch_size, int K, int V, const int* end_ids, float diversity_rate,
+                        float length_penalty)
+{
+    typedef St<DT> S;
+    if (K < 2 || K > 64 || V < 2 * K) {
+        return -1;
+    }
+    auto        rt    = [](float f) { return S::ld(S::st(f)); };
+    const float MAXT  = S::max_t();
+    const int   N     = 2 * K;
+    const int   rows  = batch_size * K;
+    std::vector<int>   cand_id((size_t)rows * N);
+    std::vector<float> cand_val((size_t)rows * N);  // values of T
+    for (int r = 0; r < rows; ++r) {
+        std::vector<float> e(V);
+        if (finished[r]) {
+            for (int v = 0; v < V; ++v) {
+                e[v] = v == end_ids[r / K] ? MAXT : -MAXT;
+            }
+        }
+        else {
+            for (int v = 0; v < V; ++v) {
+                const float b = bias != nullptr ? S::ld(bias[v]) : 0.0f;
+                e[v]          = rt(S::ld(log_probs[(size_t)r * V + v]) + b);
+            }
+        }
+        float m = -MAXT;
+        for (int v = 0; v < V; ++v) {
+            m = e[v] > m ? e[v] : m;
+        }
+        double d = 0.0;
+        for (int v = 0; v < V; ++v) {
+            d += (double)det_expf(e[v] - m);
+        }
+        const float      logd = det_logf((float)d);
+        std::vector<int> order(V);
+        for (int v = 0; v < V; ++v) {
+            order[v] = v;
+        }
+        std::partial_sort(order.begin(), order.begin() + N, order.end(),
+                          [&](int a, int b) { return order_before(e[a], a, e[b], b); });
+        for (int i = 0; i < N; ++i) {
+            const int   v   = order[i];
+            const float val = e[v] - m - logd;
+            cand_id[(size_t)r * N + i]  = v + r * V;
+            cand_val[(size_t)r * N + i] = rt(val + cum_log_probs[r]);
+        }
+    }
+
+    const int   MAX_K2 = 2 * beam_max_k(K);
+    const int   C      = K * N;
+    const float div_t  = rt(diversity_rate);
+    for (int b = 0; b < batch_size; ++b) {
+        const int*   x = cand_id.data() + (size_t)b * C;
+        const float* y = cand_val.data() + (size_t)b * C;
+        std::vector<float> old_cum(K);
+        for (int i = 0; i < K; ++i) {
+            old_cum[i] = cum_log_probs[b * K + i];
+        }
+        const bool with_hyps = hyps != nullptr && hyps->num_beams != nullptr;
+        if (with_hyps) {
+            const int g = hyps->ite * hyps->local_batch_size + b;
+            if (hyps->num_beams[g] == 0) {
+                hyps->min_normed_scores[g] = FLT_MAX;
+            }
+            else if (hyps->num_beams[g] == K) {
+                continue;
+            }
+        }
+        std::vector<float> score(C);
+        for (int c = 0; c < C; ++c) {
+            float elem = y[c];
+            if (length_penalty != 0.0f) {
+                const int length = finished[b] ? sequence_lengths[b] : sequence_lengths[b] + 1;
+                if (length != 1) {
+                    elem = rt(elem / rt(det_expf(length_penalty * det_logf((float)length))));
+                }
+            }
+            score[c] = rt(elem + rt(div_t * rt((float)(c % K))));
+        }
+        std::vector<int> order(C);
+        for (int c = 0; c < C; ++c) {
+            order[c] = c;
+        }
+        const int take = MAX_K2 < C ? MAX_K2 : C;
+        std::partial_sort(order.begin(), order.begin() + take, order.end(),
+                          [&](int a, int c) { return order_before(score[a], a, score[c], c); });
+        int*   z        = ids + (size_t)b * K;
+        float* v        = cum_log_probs + (size_t)b * K;
+        int    selected = 0;
+        for (int i = 0; i < take; ++i) {
+            const int p = order[i];
+            if (with_hyps && x[p] % V == hyps->end_ids[b]) {
+                if (i < K) {
+                    const int   g            = hyps->ite * hyps->local_batch_size + b;
+                    const float normed_score = score[p];
+                    const int   num_beam     = hyps->num_beams[g];
+                    int         beam_idx     = num_beam;
+                    if (num_beam == K) {
+                        if (normed_score < hyps->min_normed_scores[g]) {
+                            selected = K;
+                            break;
+                        }
+                        for (int j = 0; j < K; ++j) {
+                            if (hyps->normed_scores[g * (K * 2) + j] == hyps->min_normed_scores[g]) {
+                                beam_idx = j;
+                                hyps->num_beams[g]--;
+                                hyps->min_normed_scores[g]           = FLT_MAX;
+                                hyps->normed_scores[g * (K * 2) + j] = normed_score;
+                                for (int l = 0; l < K; ++l) {
+                                    hyps->min_normed_scores[g] =
+                                        std::min(hyps->min_normed_scores[g], hyps->normed_scores[g * (K * 2) + l]);
+                                }
+                                break;
+                            }
+                        }
+                    }
+                    const size_t tgt = ((size_t)(b + hyps->ite * hyps->local_batch_size) * (K * 2) + beam_idx)
+                                       * hyps->max_seq_len;
+                    hyps->output_ids_tgt[tgt + hyps->step] = hyps->end_ids[b];
+                    if (hyps->log_probs != nullptr) {
+                        hyps->log_probs[tgt + hyps->step] = y[p] - old_cum[(x[p] / V) % K];
+                    }
+                    int prev_id = (x[p] / V) % K;
+                    for (int j = hyps->step - 1; j >= 0; --j) {
+                        const size_t src = (size_t)j * hyps->batch_size * K
+                                           + (size_t)hyps->ite * hyps->local_batch_size * K + (size_t)b * K + prev_id;
+                        hyps->output_ids_tgt[tgt + j] = hyps->output_ids_src[src];
+                        if (hyps->log_probs != nullptr && hyps->log_probs_src != nullptr) {
+                            hyps->log_probs[tgt + j] = hyps->log_probs_src[src];
+                        }
+                        prev_id = hyps->parent_ids_src[src];
+                    }
+                    const int tgt_beam                   = g * (K * 2) + beam_idx;
+                    hyps->sequence_lengths_tgt[tgt_beam] = hyps->step;
+                    hyps->normed_scores[tgt_beam]        = normed_score;
+                    hyps->min_normed_scores[g] = std::min(hyps->min_normed_scores[g], hyps->normed_scores[tgt_beam]);
+                    hyps->num_beams[g]++;
+                    hyps->cum_log_probs[tgt_beam] = y[p];
+                }
+            }
+            else if ((with_hyps && i < 2 * K) || (!with_hyps && i < K)) {
+                z[selected] = x[p];
+                if (output_log_probs != nullptr) {
+                    output_log_probs[b * K + selected] = y[p] - old_cum[(z[selected] / V) % K];
+                }
+                v[selected] = y[p];
+                selected++;
+            }
+            if (selected >= K) {
+                break;
+            }
+        }
+        if (with_hyps) {
+            if (hyps->num_beams[b] < K) {
+                hyps->is_done[b] = false;
+            }
+            else if (hyps->early_stopping) {
+                hyps->is_done[b] = true;
+            }
+        }
+    }
+    return 0;
+}
+
 }  // namespace oracle
 
 using namespace oracle;
@@ -1364,6 +1590,21 @@ void oracle_finalize(int* output_ids, int* sequence_lengths, float* cum_log_prob
             }
         }
     }
+}
+
+
+// kernels/online_softmax_beamsearch_kernels.cu:671-701; `hyps` may be NULL (the reference always passes one whose
+// num_beams may be NULL)
+int oracle_topk_softmax(int dt, const void* log_probs, const void* bias, const bool* finished,
+                        const int* sequence_lengths, float* cum_log_probs, float* output_log_probs, int* ids,
+                        const BeamHyps* hyps, int batch_size, int beam_width, int vocab_size, const int* end_ids,
+                        float diversity_rate, float length_penalty)
+{
+    int rc = -1;
+    DISPATCH(dt, rc = topk_softmax<DT>((const St<DT>::T*)log_probs, (const St<DT>::T*)bias, finished, sequence_lengths,
+                                       cum_log_probs, output_log_probs, ids, hyps, batch_size, beam_width, vocab_size,
+                                       end_ids, diversity_rate, length_penalty));
+    return rc;
 }
 
 }  // extern "C"

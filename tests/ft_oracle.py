@@ -312,3 +312,38 @@ def finalize(topk_output_ids, topk_sequence_lengths, scores, topk_cum_log_probs,
                           _p(scores), _p(topk_cum_log_probs), _p(topk_log_probs), _p(num_beams), beam_width,
                           max_seq_len, batch)
     return out_ids, seq, cum, lp
+
+
+class BeamHyps(C.Structure):
+    """BeamHyps of oracle/ft_oracle.cc"""
+    _fields_ = [("output_ids_tgt", C.c_void_p), ("sequence_lengths_tgt", C.c_void_p), ("cum_log_probs", C.c_void_p),
+                ("normed_scores", C.c_void_p), ("log_probs", C.c_void_p), ("min_normed_scores", C.c_void_p),
+                ("num_beams", C.c_void_p), ("is_done", C.c_void_p), ("output_ids_src", C.c_void_p),
+                ("parent_ids_src", C.c_void_p), ("sequence_lengths_src", C.c_void_p), ("end_ids", C.c_void_p),
+                ("log_probs_src", C.c_void_p), ("step", C.c_int), ("ite", C.c_int), ("batch_size", C.c_int),
+                ("local_batch_size", C.c_int), ("max_seq_len", C.c_int), ("length_penalty", C.c_float),
+                ("early_stopping", C.c_int)]
+
+
+def topk_softmax(dt, log_probs, bias, finished, sequence_lengths, cum_log_probs, output_log_probs, ids, hyps,
+                 batch, beam_width, vocab, end_ids, diversity_rate, length_penalty):
+    """invokeTopkSoftMax: cum_log_probs, output_log_probs, ids and the arrays `hyps` (a dict of numpy arrays and
+    ints, or None) points to are updated in place; returns the oracle's status (0 = done)"""
+    h = None
+    if hyps is not None:
+        h = BeamHyps()
+        for name, _ in BeamHyps._fields_:
+            val = hyps.get(name)
+            if isinstance(val, np.ndarray):
+                setattr(h, name, val.ctypes.data)
+            elif val is None:
+                setattr(h, name, None if name not in ("step", "ite", "batch_size", "local_batch_size", "max_seq_len",
+                                                        "length_penalty", "early_stopping") else 0)
+            else:
+                setattr(h, name, val)
+    fn = lib().oracle_topk_softmax
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_int] + [C.c_void_p] * 8 + [C.c_int] * 3 + [C.c_void_p, C.c_float, C.c_float]
+    return fn(dt, _p(log_probs), _p(bias), _p(finished), _p(sequence_lengths), _p(cum_log_probs), _p(output_log_probs),
+              _p(ids), C.addressof(h) if h is not None else None, batch, beam_width, vocab, _p(end_ids),
+              float(diversity_rate), float(length_penalty))

@@ -126,3 +126,50 @@ def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finishe
         rc = lib.ftk_fused_topk_step_static(C.addressof(a), stream)
     torch.cuda.synchronize()
     return out_ids[H].cpu().numpy(), seq.cpu().numpy(), finished.cpu().numpy(), rc, a.workspace_size
+
+
+def make_beam_case(rng, dt, batch, K, V, step=5, max_seq_len=12, with_hyps=True, finished_frac=0.2, full_frac=0.2,
+                   scale=3.0, end_spike=0.5):
+    """Seeded inputs of one beam-search step (invokeTopkSoftMax): logits [batch * K, V] in storage type `dt`, the
+    running beams' state and, optionally, the arrays of a BeamHypotheses with some entries already collected.
+    Returns a dict of numpy arrays and ints (the names of the reference's arguments and struct fields)."""
+    import ft_oracle as O
+    rows = batch * K
+    x = rng.standard_normal((rows, V)).astype(np.float32) * np.float32(scale)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    for r in range(rows):  # some beams are about to end: their end token is among their best
+        if rng.random() < end_spike:
+            x[r, end_ids[r // K]] += np.float32(rng.uniform(2.0, 5.0) * scale)
+    c = dict(log_probs=O.to_storage(x, dt), finished=rng.random(rows) < finished_frac,
+             sequence_lengths=rng.integers(1, step + 2, rows).astype(np.int32),
+             cum_log_probs=(-np.abs(rng.standard_normal(rows)) * 4).astype(np.float32), end_ids=end_ids,
+             ids=np.full((batch, K), -1, np.int32), output_log_probs=np.zeros((batch, K), np.float32))
+    if with_hyps:
+        num = np.where(rng.random(batch) < full_frac, K, rng.integers(0, K, batch)).astype(np.int32)
+        normed = (-np.abs(rng.standard_normal((batch, 2 * K))) * 3).astype(np.float32)
+        mins = np.array([normed[b, :num[b]].min() if num[b] else 0.0 for b in range(batch)], np.float32)
+        c["hyps"] = dict(
+            output_ids_tgt=np.zeros((batch, 2 * K, max_seq_len), np.int32),
+            sequence_lengths_tgt=np.zeros((batch, 2 * K), np.int32),
+            cum_log_probs=np.zeros((batch, 2 * K), np.float32), normed_scores=normed,
+            log_probs=np.zeros((batch, 2 * K, max_seq_len), np.float32), min_normed_scores=mins, num_beams=num,
+            is_done=np.zeros(batch, np.bool_),
+            output_ids_src=rng.integers(0, V, (max_seq_len, batch, K)).astype(np.int32),
+            parent_ids_src=rng.integers(0, K, (max_seq_len, batch, K)).astype(np.int32),
+            sequence_lengths_src=None, end_ids=end_ids,
+            log_probs_src=(-np.abs(rng.standard_normal((max_seq_len, batch, K)))).astype(np.float32),
+            step=step, ite=0, batch_size=batch, local_batch_size=batch, max_seq_len=max_seq_len, length_penalty=0.0,
+            early_stopping=1)
+    else:
+        c["hyps"] = None
+    return c
+
+
+def copy_beam_case(c):
+    """deep copy (the step updates its arguments in place)"""
+    out = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in c.items() if k != "hyps"}
+    out["hyps"] = None if c["hyps"] is None else {k: (v.copy() if isinstance(v, np.ndarray) else v)
+                                                  for k, v in c["hyps"].items()}
+    if out["hyps"] is not None:
+        out["hyps"]["end_ids"] = out["end_ids"]
+    return out

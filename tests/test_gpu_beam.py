@@ -1,0 +1,157 @@
+"""GPU parity of one beam-search step (ftk_invoke_topk_softmax, the reference's invokeTopkSoftMax) against the
+oracle through the C ABI: next beams' ids, parents and hypotheses bit for bit, log-probs within tolerance."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import ft_oracle as O
+from helpers import DTYPE_NAMES, DTYPES, copy_beam_case, make_beam_case, to_numpy, to_torch
+
+pytestmark = pytest.mark.gpu
+
+HYP_ARRAYS = ("output_ids_tgt", "sequence_lengths_tgt", "cum_log_probs", "normed_scores", "log_probs",
+              "min_normed_scores", "num_beams", "is_done", "output_ids_src", "parent_ids_src", "log_probs_src")
+
+
+def _lib():
+    from fastertransformer_amd import ops
+    return ops, ops.ftk()
+
+
+def _run_product(c, dt, batch, K, V, diversity, length_penalty, bias=None):
+    """the step on the GPU; returns (ids, cum_log_probs, output_log_probs, hypotheses arrays) as numpy"""
+    import torch
+    ops, lib = _lib()
+    d = {k: to_torch(c[k]) for k in ("finished", "sequence_lengths", "cum_log_probs", "end_ids", "ids",
+                                     "output_log_probs")}
+    d_x = to_torch(c["log_probs"], dt)
+    d_bias = to_torch(bias, dt) if bias is not None else None
+    hyps, d_h = None, {}
+    if c["hyps"] is not None:
+        hyps = ops.BeamHypotheses()
+        for name in HYP_ARRAYS:
+            d_h[name] = to_torch(c["hyps"][name])
+            setattr(hyps, name, d_h[name].data_ptr())
+        hyps.end_ids = d["end_ids"].data_ptr()
+        for name in ("step", "ite", "batch_size", "local_batch_size", "max_seq_len"):
+            setattr(hyps, name, int(c["hyps"][name]))
+        hyps.length_penalty = float(length_penalty)
+        hyps.early_stopping = bool(c["hyps"]["early_stopping"])
+        hyps.is_return_normed_score = True
+    size = C.c_size_t(0)
+    args = (dt, d_x.data_ptr(), ops.ptr(d_bias), d["finished"].data_ptr(), d["sequence_lengths"].data_ptr(),
+            d["cum_log_probs"].data_ptr(), d["output_log_probs"].data_ptr(), d["ids"].data_ptr())
+    tail = (C.addressof(hyps) if hyps is not None else None, batch, K, V, d["end_ids"].data_ptr(), float(diversity),
+            float(length_penalty), ops.current_stream())
+    ops.check(lib.ftk_invoke_topk_softmax(*args, None, C.addressof(size), *tail))
+    ws = torch.empty(max(size.value, 16), dtype=torch.uint8, device="cuda")
+    ops.check(lib.ftk_invoke_topk_softmax(*args, ws.data_ptr(), C.addressof(size), *tail))
+    torch.cuda.synchronize()
+    return (to_numpy(d["ids"]), to_numpy(d["cum_log_probs"]), to_numpy(d["output_log_probs"]),
+            {k: to_numpy(v) for k, v in d_h.items()})
+
+
+def _compare(c, want, got, dt):
+    ids, cum, out_lp, hyps = got
+    rtol = 2e-5 if dt == O.F32 else 4e-3
+    where = "ids"
+    assert np.array_equal(ids, want["ids"]), where
+    np.testing.assert_allclose(cum, want["cum_log_probs"], rtol=rtol, atol=1e-5)
+    np.testing.assert_allclose(out_lp, want["output_log_probs"], rtol=rtol, atol=1e-3 if dt != O.F32 else 2e-5)
+    if want["hyps"] is not None:
+        for name in ("output_ids_tgt", "sequence_lengths_tgt", "num_beams", "is_done"):
+            assert np.array_equal(hyps[name], want["hyps"][name]), name
+        for name in ("cum_log_probs", "normed_scores", "log_probs", "min_normed_scores"):
+            np.testing.assert_allclose(hyps[name], want["hyps"][name], rtol=rtol, atol=1e-3 if dt != O.F32 else 2e-5,
+                                       err_msg=name)
+
+
+def _one_case(rng, dt, batch, K, V, with_hyps, diversity, length_penalty, step=5, max_seq_len=12, **kw):
+    c = make_beam_case(rng, dt, batch, K, V, step=step, max_seq_len=max_seq_len, with_hyps=with_hyps, **kw)
+    want = copy_beam_case(c)
+    rc = O.topk_softmax(dt, want["log_probs"], None, want["finished"], want["sequence_lengths"],
+                        want["cum_log_probs"], want["output_log_probs"], want["ids"], want["hyps"], batch, K, V,
+                        want["end_ids"], diversity, length_penalty)
+    assert rc == 0
+    print("beam case", DTYPE_NAMES[dt], batch, K, V, with_hyps, diversity, length_penalty, flush=True)
+    _compare(c, want, _run_product(c, dt, batch, K, V, diversity, length_penalty), dt)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("K", [2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 64])
+def test_beam_step_every_width_class(dt, K):
+    """every beam-width class of the reference's dispatch (1-4, 5-8, 9-16, 17-32, 33-64) at its edges, with and
+    without hypotheses, penalties on and off"""
+    rng = np.random.default_rng(100 * K + dt)
+    for V in (2 * K, 2 * K + 1, 1000, 20011):
+        for with_hyps in (False, True):
+            lp = float(rng.choice([0.0, 0.6, 1.0]))
+            dv = float(rng.choice([0.0, 0.0, 0.25]))
+            _one_case(rng, dt, int(rng.integers(1, 5)), K, V, with_hyps, dv, lp)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_beam_step_full_vocabularies_and_batches(dt):
+    """vocabulary sizes of the headline configurations (several sections per row, merged per row), a batch large
+    enough for one section per row, long histories to trace"""
+    rng = np.random.default_rng(7 + dt)
+    _one_case(rng, dt, 8, 4, 50257, True, 0.0, 0.8, step=30, max_seq_len=40)
+    _one_case(rng, dt, 2, 8, 128256, True, 0.1, 0.0)
+    _one_case(rng, dt, 300, 4, 3000, True, 0.0, 1.0)
+    _one_case(rng, dt, 1, 2, 152064, False, 0.0, 0.0)
+
+
+def test_beam_step_degenerate_rows():
+    """rows of equal values (ties settled by the lower id at every stage), rows masked to -inf except a few
+    columns, every beam finished, hypotheses already complete for every entry"""
+    rng = np.random.default_rng(3)
+    batch, K, V = 3, 4, 5000
+    for kind in range(4):
+        c = make_beam_case(rng, O.F32, batch, K, V, with_hyps=True, finished_frac=0.0)
+        if kind == 0:
+            c["log_probs"][:] = np.float32(1.5)
+            c["cum_log_probs"][:] = np.float32(-1.0)
+        elif kind == 1:
+            c["log_probs"][:] = -np.inf
+            c["log_probs"][:, rng.choice(V, 3 * K, replace=False)] = rng.standard_normal(3 * K).astype(np.float32)
+        elif kind == 2:
+            c["finished"][:] = True
+        else:
+            c["hyps"]["num_beams"][:] = K
+        want = copy_beam_case(c)
+        assert O.topk_softmax(O.F32, want["log_probs"], None, want["finished"], want["sequence_lengths"],
+                              want["cum_log_probs"], want["output_log_probs"], want["ids"], want["hyps"], batch, K, V,
+                              want["end_ids"], 0.0, 0.5) == 0
+        print("degenerate kind", kind, flush=True)
+        _compare(c, want, _run_product(c, O.F32, batch, K, V, 0.0, 0.5), O.F32)
+
+
+def test_beam_step_with_bias_and_refusals():
+    import torch
+    ops, lib = _lib()
+    rng = np.random.default_rng(9)
+    batch, K, V = 2, 3, 777
+    for dt in DTYPES:
+        c = make_beam_case(rng, dt, batch, K, V, with_hyps=True)
+        bias = O.to_storage(rng.standard_normal(V).astype(np.float32), dt)
+        want = copy_beam_case(c)
+        assert O.topk_softmax(dt, want["log_probs"], bias, want["finished"], want["sequence_lengths"],
+                              want["cum_log_probs"], want["output_log_probs"], want["ids"], want["hyps"], batch, K, V,
+                              want["end_ids"], 0.0, 0.0) == 0
+        _compare(c, want, _run_product(c, dt, batch, K, V, 0.0, 0.0, bias=bias), dt)
+    size = C.c_size_t(0)
+    none = (None,) * 8
+    for K_bad in (1, 65):  # the reference's dispatch throws for these
+        assert lib.ftk_invoke_topk_softmax(O.F32, *none[:7], None, C.addressof(size), None, 2, K_bad, 1000, None, 0.0,
+                                           0.0, None) == ops.FTK_ERR_ARGUMENT
+    assert lib.ftk_invoke_topk_softmax(O.F32, *none[:7], None, C.addressof(size), None, 2, 8, 15, None, 0.0, 0.0,
+                                       None) == ops.FTK_ERR_ARGUMENT   # fewer columns than 2 * beam_width
+    assert lib.ftk_invoke_topk_softmax(7, *none[:7], None, C.addressof(size), None, 2, 8, 100, None, 0.0, 0.0,
+                                       None) == ops.FTK_ERR_DTYPE
+    ops.check(lib.ftk_invoke_topk_softmax(O.F32, *none[:7], None, C.addressof(size), None, 2, 8, 100, None, 0.0, 0.0,
+                                          None))
+    ws = torch.empty(16, dtype=torch.uint8, device="cuda")
+    small = C.c_size_t(16)
+    assert lib.ftk_invoke_topk_softmax(O.F32, *none[:7], ws.data_ptr(), C.addressof(small), None, 2, 8, 100, None,
+                                       0.0, 0.0, None) == ops.FTK_ERR_WORKSPACE

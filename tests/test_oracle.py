@@ -760,3 +760,104 @@ def test_softmax_summation_order_bit_for_bit():
             running = np.float32(running + v)
         seen_other_order_differs += int(running != total)
     assert seen_other_order_differs >= 3
+
+
+# ---- beam search step (invokeTopkSoftMax) -----------------------------------------------------------------------
+def _log_softmax64(x):
+    x = x.astype(np.float64)
+    m = x.max(axis=-1, keepdims=True)
+    return x - m - np.log(np.exp(x - m).sum(axis=-1, keepdims=True))
+
+
+def _run_oracle_beam(c, dt, batch, K, V, diversity=0.0, length_penalty=0.0):
+    rc = O.topk_softmax(dt, c["log_probs"], None, c["finished"], c["sequence_lengths"], c["cum_log_probs"],
+                        c["output_log_probs"], c["ids"], c["hyps"], batch, K, V, c["end_ids"], diversity,
+                        length_penalty)
+    assert rc == 0
+
+
+@pytest.mark.parametrize("K,V", [(2, 50), (3, 1000), (4, 50257), (8, 3000), (17, 700), (64, 2000)])
+def test_beam_step_without_hypotheses_is_the_global_top_k(K, V):
+    """No hypotheses, no penalties: the next beams are the K largest of cum_log_probs[beam] + log_softmax(row)
+    over all K * V continuations of a batch entry (a definition that knows nothing of the 2K candidates per beam),
+    in descending order, and the step's log-prob is the difference of the cumulative ones."""
+    from helpers import make_beam_case
+    rng = np.random.default_rng(K * 1000 + V)
+    batch = 3
+    c = make_beam_case(rng, O.F32, batch, K, V, with_hyps=False, finished_frac=0.0)
+    old_cum = c["cum_log_probs"].copy()
+    total = old_cum.reshape(batch, K, 1).astype(np.float64) + _log_softmax64(c["log_probs"]).reshape(batch, K, V)
+    _run_oracle_beam(c, O.F32, batch, K, V)
+    for b in range(batch):
+        flat = total[b].reshape(-1)
+        order = np.argsort(-flat, kind="stable")[:K]
+        got = c["ids"][b] - b * K * V
+        assert len(set(got.tolist())) == K and got.min() >= 0 and got.max() < K * V
+        # the same continuations in the same order, except where two of them are closer than fp32 resolves
+        np.testing.assert_allclose(flat[got], flat[order], rtol=2e-6, atol=0)
+        distinct = np.abs(np.diff(flat[np.argsort(-flat, kind="stable")[:K + 1]])) > 1e-4
+        clear = np.concatenate([[True], distinct[:-1]]) & distinct
+        assert np.array_equal(got[clear], order[clear]), b
+        np.testing.assert_allclose(c["cum_log_probs"][b * K:(b + 1) * K], flat[got], rtol=1e-5)
+        np.testing.assert_allclose(c["output_log_probs"][b], flat[got] - old_cum[b * K + got // V], rtol=1e-4,
+                                   atol=1e-5)
+
+
+def test_beam_step_finished_beams_offer_their_end_token_only():
+    """A finished beam's row is MAX_T at its end id and -MAX_T elsewhere: its only finite continuation is the end
+    token at an unchanged cumulative log-prob (no hypotheses kept here, so it stays a beam)."""
+    from helpers import make_beam_case
+    rng = np.random.default_rng(5)
+    batch, K, V = 2, 4, 300
+    c = make_beam_case(rng, O.F32, batch, K, V, with_hyps=False, finished_frac=0.0)
+    c["finished"][[1, 6]] = True
+    c["cum_log_probs"][[1, 6]] = np.float32(-0.25)   # better than anything a live beam can reach
+    _run_oracle_beam(c, O.F32, batch, K, V)
+    assert c["ids"][0, 0] == 1 * V + c["end_ids"][0] and c["cum_log_probs"][0] == np.float32(-0.25)
+    assert c["ids"][1, 0] == 6 * V + c["end_ids"][1] and c["cum_log_probs"][4] == np.float32(-0.25)
+    assert c["output_log_probs"][0, 0] == 0.0 and c["output_log_probs"][1, 0] == 0.0
+    # no other continuation of a finished beam is ever chosen
+    for b in range(batch):
+        for i in range(1, K):
+            assert c["ids"][b, i] // V not in (1, 6)
+
+
+@pytest.mark.parametrize("length_penalty", [0.0, 0.7])
+def test_beam_step_moves_end_tokens_to_the_hypotheses(length_penalty):
+    """The best continuation of entry 0 is its beam 2 ending: it becomes hypothesis number num_beams with the
+    beam's history traced back through parent_ids, the step as its length, cum / length^penalty as its score
+    (float64 here), and it is not among the next beams; entry 1 already holds K hypotheses and is left alone."""
+    from helpers import make_beam_case
+    rng = np.random.default_rng(11)
+    batch, K, V, step, L = 2, 3, 400, 4, 9
+    c = make_beam_case(rng, O.F32, batch, K, V, step=step, max_seq_len=L, finished_frac=0.0, full_frac=0.0,
+                       end_spike=0.0)
+    h = c["hyps"]
+    h["num_beams"][:] = [1, K]
+    h["min_normed_scores"][:] = [h["normed_scores"][0, 0], h["normed_scores"][1, :K].min()]
+    c["sequence_lengths"][:] = step
+    end = int(c["end_ids"][0])
+    c["log_probs"][2, end] = 40.0           # beam 2 of entry 0 ends with near certainty
+    c["cum_log_probs"][2] = np.float32(-0.5)
+    before = {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in h.items()}
+    old_ids, old_cum = c["ids"].copy(), c["cum_log_probs"].copy()
+    _run_oracle_beam(c, O.F32, batch, K, V, length_penalty=length_penalty)
+    assert h["num_beams"].tolist() == [2, K]
+    lsm = _log_softmax64(c["log_probs"][2])[end]
+    cum = -0.5 + lsm
+    np.testing.assert_allclose(h["cum_log_probs"][0, 1], cum, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(h["normed_scores"][0, 1], cum / (step + 1) ** length_penalty, rtol=1e-5, atol=1e-6)
+    assert h["sequence_lengths_tgt"][0, 1] == step and h["output_ids_tgt"][0, 1, step] == end
+    beam = 2
+    for j in range(step - 1, -1, -1):       # the path, followed independently
+        assert h["output_ids_tgt"][0, 1, j] == before["output_ids_src"][j, 0, beam]
+        assert h["log_probs"][0, 1, j] == before["log_probs_src"][j, 0, beam]
+        beam = before["parent_ids_src"][j, 0, beam]
+    np.testing.assert_allclose(h["log_probs"][0, 1, step], lsm, atol=1e-5)
+    assert h["min_normed_scores"][0] == min(before["min_normed_scores"][0], h["normed_scores"][0, 1])
+    assert all(int(t) % V != end or int(t) // V != 2 for t in c["ids"][0])
+    assert not h["is_done"][0]
+    # entry 1: K hypotheses already: nothing of it moves (the kernel returns before it selects)
+    assert np.array_equal(c["ids"][1], old_ids[1]) and np.array_equal(c["cum_log_probs"][K:], old_cum[K:])
+    assert np.array_equal(h["output_ids_tgt"][1], before["output_ids_tgt"][1])
+
