@@ -15,6 +15,7 @@
 // the position, so that keys are distinct and ties need no rule of their own): byte by byte from the top, a
 // 256-bin LDS histogram of the keys that match the bytes fixed so far; as soon as few enough match they are moved
 // to LDS and the remaining bytes are settled there.
+#include "ftk_columns.cuh"
 #include "ftk_device.cuh"
 #include "ftk_sampling.h"
 #include "ftk_transform.cuh"
@@ -28,7 +29,10 @@ constexpr int BM_MAX_N   = 128;   // 2 * beam_width and 2 * MAX_K are at most th
 
 struct BeamSelect {
     unsigned long long list[BM_CAP];
+    unsigned long long cand[BM_CAP];     // a section's elements at or above the bound from the thread maxima
+    unsigned long long slots[BM_THREADS];
     unsigned long long out[BM_MAX_N];
+    int                n_cand;
     uint32_t           hist[256];
     uint32_t           wave_total[BM_WAVES];
     int                n_list;
@@ -108,7 +112,23 @@ __device__ __forceinline__ unsigned long long beam_nth_key(BeamSelect& s, F&& ke
 template<class F>
 __device__ __forceinline__ void beam_select(BeamSelect& s, F&& key, int count, int need)
 {
-    const int                t     = threadIdx.x;
+    const int t = threadIdx.x;
+    if (count <= BM_THREADS) {
+        // one key per thread: its place is the number of larger keys
+        const unsigned long long k = t < count ? key(t) : 0ull;
+        __syncthreads();  // (the caller may still be reading what key() reads from, or s.list)
+        s.list[t] = k;
+        __syncthreads();
+        int r = 0;
+        for (int j = 0; j < count; ++j) {
+            r += s.list[j] > k ? 1 : 0;
+        }
+        if (t < count && r < need) {
+            s.out[r] = k;
+        }
+        __syncthreads();
+        return;
+    }
     const unsigned long long bound = beam_nth_key(s, key, count, need);
     if (t == 0) {
         s.n_out = 0;
@@ -153,6 +173,14 @@ __device__ __forceinline__ float beam_element(const typename Storage<DT>::T* __r
     typedef Storage<DT> S;
     const float         b = bias != nullptr ? S::ld(bias[v]) : 0.0f;
     return round_t<DT>(S::ld(x[row_base + v]) + b);
+}
+
+// the same from a value that is already loaded
+template<int DT>
+__device__ __forceinline__ float beam_element_of(float xv, const typename Storage<DT>::T* __restrict__ bias, int v)
+{
+    const float b = bias != nullptr ? Storage<DT>::ld(bias[v]) : 0.0f;
+    return round_t<DT>(xv + b);
 }
 
 struct BeamPlan {
@@ -212,10 +240,10 @@ beam_section_max_kernel(const typename Storage<DT>::T* __restrict__ x, const typ
     const int    hi = min(vocab, lo + section);
     const size_t rb = (size_t)row * vocab;
     float        m  = -Storage<DT>::max_t();
-    for (int v = lo + t; v < hi; v += BM_THREADS) {
-        const float e = beam_element<DT>(x, bias, rb, v);
+    stream_columns<DT, BM_THREADS>(x + rb, lo, hi, [&](int v, float xv) {
+        const float e = beam_element_of<DT>(xv, bias, v);
         m             = e > m ? e : m;
-    }
+    });
     m = block_max<float, BM_WAVES>(m, red, -Storage<DT>::max_t());
     if (t == 0) {
         pmax[(size_t)row * gridDim.x + blockIdx.x] = m;
@@ -246,16 +274,25 @@ beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
         const float pm = pmax[(size_t)row * parts + p];
         m              = pm > m ? pm : m;
     }
-    double d = 0.0;
-    for (int v = lo + t; v < hi; v += BM_THREADS) {
-        d += (double)det_expf(beam_element<DT>(x, bias, rb, v) - m);
-    }
+    // first pass: the sum, and every thread's largest element
+    double   d    = 0.0;
+    uint32_t kmax = 0u;
+    stream_columns<DT, BM_THREADS>(x + rb, lo, hi, [&](int v, float xv) {
+        const float e = beam_element_of<DT>(xv, bias, v);
+        d += (double)det_expf(e - m);
+        const uint32_t k = order_key(e);
+        kmax             = k > kmax ? k : kmax;
+    });
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         d += __shfl_xor(d, o, WAVE);
     }
     if (lane_id() == 0) {
         red[wave_id()] = d;
+    }
+    s.slots[t] = ((unsigned long long)kmax << 32) | (unsigned long long)(BM_THREADS - 1 - t);
+    if (t == 0) {
+        s.n_cand = 0;
     }
     __syncthreads();
     if (t == 0) {
@@ -267,9 +304,34 @@ beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     }
     // a short last section gives fewer than N keys; the rest of its list is 0, below every key of an element
     const int take = min(N, hi - lo);
+    // The N-th largest of the thread maxima is an element with at least N elements at or above it (N threads hold
+    // one each): nothing below it can be among the N best. Usually a few times N elements pass.
+    uint32_t floor_key = 0u;
+    if (hi - lo >= BM_THREADS) {
+        // (thread maxima of threads that saw no element are 0 and lower the bound at most to 0)
+        beam_select(s, [&](int i) { return s.slots[i]; }, BM_THREADS, N);
+        floor_key = (uint32_t)(s.out[N - 1] >> 32);
+    }
+    stream_columns<DT, BM_THREADS>(x + rb, lo, hi, [&](int v, float xv) {
+        const float e = beam_element_of<DT>(xv, bias, v);
+        if (order_key(e) >= floor_key) {
+            const int at = atomicAdd(&s.n_cand, 1);
+            if (at < BM_CAP) {
+                s.cand[at] = beam_key(e, (uint32_t)v);
+            }
+        }
+    });
+    __syncthreads();
+    const int passed = s.n_cand;
     if (take > 0) {
-        beam_select(s, [&](int i) { return beam_key(beam_element<DT>(x, bias, rb, lo + i), (uint32_t)(lo + i)); },
-                    hi - lo, take);
+        if (passed <= BM_CAP) {
+            beam_select(s, [&](int i) { return s.cand[i]; }, passed, take);
+        }
+        else {
+            // (rows of many equal values) the selection runs over the section itself
+            beam_select(s, [&](int i) { return beam_key(beam_element<DT>(x, bias, rb, lo + i), (uint32_t)(lo + i)); },
+                        hi - lo, take);
+        }
     }
     if (t < N) {
         pkeys[((size_t)row * parts + part) * N + t] = t < take ? s.out[t] : 0ull;
