@@ -296,4 +296,33 @@ inline void invokeFinalize(int* output_ids, int* sequence_lengths, float* cum_lo
                                   beam_width, max_seq_len, batch_size, stream));
 }
 
+// ---- beam_search_topk_kernels.h / online_softmax_beamsearch_kernels.h -----------------------------------
+typedef ftk_beam_hypotheses BeamHypotheses;  // kernels/beam_search_topk_kernels.h:31-58, the same fields
+
+// Bytes of temp_storage a call with these sizes needs (the reference's layer computes a count of floats itself,
+// layers/beam_search_layers/OnlineBeamSearchLayer.cu:201-207).
+template<typename T>
+size_t topkSoftMaxWorkspaceBytes(const int batch_size, const int beam_width, const int vocab_size)
+{
+    size_t bytes = 0;
+    check_ftk(ftk_invoke_topk_softmax(FtkDType<T>::value, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                                      nullptr, nullptr, &bytes, nullptr, batch_size, beam_width, vocab_size, nullptr,
+                                      0.0f, 0.0f, nullptr));
+    return bytes;
+}
+
+// kernels/online_softmax_beamsearch_kernels.cu:671-701; temp_storage_size counts 4-byte elements as there
+template<typename T>
+void invokeTopkSoftMax(const T* log_probs, const T* bias, const bool* finished, const int* sequence_lengths,
+                       float* cum_log_probs, float* output_log_probs, int* ids, void* temp_storage,
+                       const int temp_storage_size, BeamHypotheses* beam_hyps, const int batch_size,
+                       const int beam_width, const int vocab_size, const int* end_ids, const float diversity_rate,
+                       const float length_penalty, hipStream_t stream)
+{
+    size_t bytes = (size_t)temp_storage_size * sizeof(float);
+    check_ftk(ftk_invoke_topk_softmax(FtkDType<T>::value, log_probs, bias, finished, sequence_lengths, cum_log_probs,
+                                      output_log_probs, ids, temp_storage, &bytes, beam_hyps, batch_size, beam_width,
+                                      vocab_size, end_ids, diversity_rate, length_penalty, stream));
+}
+
 }  // namespace fastertransformer

@@ -31,11 +31,15 @@
 //    thread-by-thread float32 simulation; storage conversions against numpy and torch;
 //    det_expf / det_logf against float64;
 //  * ban_bad_words, stop words, length criterion, finalize: no reference test exists, pinned by brute
-//    force written from the source description only (finalize: a stable descending sort).
+//    force written from the source description only (finalize: a stable descending sort);
+//  * beam search step (topk_softmax): no reference test exists; pinned by the definition it must reduce to
+//    without hypotheses (the K largest of cum + log_softmax over all continuations, float64) and by
+//    scenario checks of the hypothesis bookkeeping written from the source description.
 //  PARITY UNPINNED (no reference code or no way to run it here): the rounding order of cub's
 //  BLOCK_SCAN_RAKING prefix sums in top-p (cub is not in the reference's tree), bfloat16 storage, the frequency
-//  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), and the last-ulp
-//  behaviour of __expf / logf (tolerance 1e-5 relative instead).
+//  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), the last-ulp
+//  behaviour of __expf / logf (tolerance 1e-5 relative instead), and in the beam search step the
+//  reference's pairwise (max, sum) merges in cub's order and its powf.
 //
 // Build: oracle/Makefile (g++ -O2 -ffp-contract=off).
 
