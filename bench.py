@@ -63,6 +63,10 @@ WORKLOADS = {
         dtype="bf16", batch=128, vocab=32000, vocab_padded=32000, top_k=50, top_p=0.0, temperature=1.0,
         presence_penalty=0.5, frequency_penalty=0.3, prompt=2048, zipf_history=1.2, min_length_beyond=52,
         bad_words=(64, 4), stop_words=(16, 3), end_id=2, sigma=2.0, logprobs=False),
+    # secondary line (only with --workload): one beam-search step (invokeTopkSoftMax), 32 entries x 4 beams,
+    # hypotheses kept, a few beams ending per step; the beams' state is restored outside the timed events
+    "beam_step_b32_k4_v50257_f16": dict(dtype="f16", batch=32, beam_width=4, vocab=50257, sigma=3.0),
+    "beam_step_b64_k8_v152064_f16": dict(dtype="f16", batch=64, beam_width=8, vocab=152064, sigma=3.0),
 }
 
 
@@ -345,6 +349,66 @@ def run_gpu_loop(name, w, steps, warmup, nbuf=2):
                 sampled_ids_checksum=int(output_ids[H + warmup:H + total].to(torch.int64).sum().item()))
 
 
+def run_gpu_beam(name, w, steps, warmup):
+    """Beam-search steps over one synthetic state: logits [batch * beam_width, vocab] in rotation, cumulative
+    log-probs and hypothesis counts restored before every step outside its pair of events."""
+    import ctypes as C
+    import torch
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+    from helpers import make_beam_case, to_torch
+
+    torch.cuda.set_device(0)
+    dt = {"f32": fa.F32, "f16": fa.F16, "bf16": fa.BF16}[w["dtype"]]
+    batch, K, V = w["batch"], w["beam_width"], w["vocab"]
+    rng = np.random.default_rng(1)
+    cases = [make_beam_case(rng, dt, batch, K, V, with_hyps=True, end_spike=0.05, finished_frac=0.05, full_frac=0.0,
+                            scale=w["sigma"]) for _ in range(3)]
+    c = cases[0]
+    d = {k: to_torch(c[k]) for k in ("finished", "sequence_lengths", "cum_log_probs", "end_ids", "ids",
+                                     "output_log_probs")}
+    logits = [to_torch(x["log_probs"], dt) for x in cases]
+    hyps, keep = ops.BeamHypotheses(), {}
+    for key, val in c["hyps"].items():
+        if isinstance(val, np.ndarray) and key != "end_ids":
+            keep[key] = to_torch(val)
+            setattr(hyps, key, keep[key].data_ptr())
+        elif key in ("step", "ite", "batch_size", "local_batch_size", "max_seq_len"):
+            setattr(hyps, key, int(val))
+    hyps.end_ids = d["end_ids"].data_ptr()
+    hyps.early_stopping = True
+    lib = fa.ftk()
+    size = C.c_size_t(0)
+
+    def call(x, ws):
+        ops.check(lib.ftk_invoke_topk_softmax(
+            dt, x.data_ptr(), None, d["finished"].data_ptr(), d["sequence_lengths"].data_ptr(),
+            d["cum_log_probs"].data_ptr(), d["output_log_probs"].data_ptr(), d["ids"].data_ptr(),
+            ws.data_ptr() if ws is not None else None, C.addressof(size), C.addressof(hyps), batch, K, V,
+            d["end_ids"].data_ptr(), 0.0, 0.0, ops.current_stream()))
+
+    call(logits[0], None)
+    ws = torch.empty(size.value, dtype=torch.uint8, device="cuda")
+    num0, cum0 = keep["num_beams"].clone(), d["cum_log_probs"].clone()
+    ms, checksum = [], 0
+    for i in range(steps + warmup):
+        keep["num_beams"].copy_(num0)
+        d["cum_log_probs"].copy_(cum0)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        call(logits[i % len(logits)], ws)
+        e1.record()
+        torch.cuda.synchronize()
+        if i >= warmup:
+            ms.append(e0.elapsed_time(e1))
+            checksum += int(d["ids"].to(torch.int64).sum().item())
+    ms = np.array(ms)
+    alg = batch * K * V * (4 if w["dtype"] == "f32" else 2)
+    return dict(ms_per_step=float(ms.mean()), p50_ms=float(np.percentile(ms, 50)), max_ms=float(ms.max()),
+                beams_per_s=batch * K / (ms.mean() * 1e-3), gbs=alg / (ms.mean() * 1e-3) / 1e9, bytes=alg,
+                ids_checksum=checksum)
+
+
 def _oracle_rows_per_second(w, rows, budget_s, seed):
     """the oracle's DynamicDecodeLayer on `rows`-row batches of the workload for about `budget_s` seconds of this
     thread's time; returns (rows done, seconds)"""
@@ -439,6 +503,20 @@ def main():
             "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": name, "batch": w["batch"], "vocab": w["vocab"]},
             "sampled_ids_checksum": r["sampled_ids_checksum"]}))
+        return
+    if name.startswith("beam_step"):
+        r = run_gpu_beam(name, w, a.steps, a.warmup)
+        print(json.dumps({
+            "metric": "beams extended per second, beam-search step B=%d K=%d V=%d (log-softmax, 2K best per beam, "
+                      "K best per entry, hypotheses)" % (w["batch"], w["beam_width"], w["vocab"]),
+            "value": r["beams_per_s"], "unit": "beams/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": r["ms_per_step"], "p50_ms": r["p50_ms"], "max_ms": r["max_ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+            "config": {"workload": name, "batch": w["batch"], "beam_width": w["beam_width"], "vocab": w["vocab"]},
+            "roofline": {"bound": "hbm", "achieved": r["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": r["gbs"] / HBM_PEAK_GBS, "traffic": None, "kernel": "whole step (four kernels)",
+                         "algorithmic_bytes_per_launch": r["bytes"]},
+            "ids_checksum": r["ids_checksum"]}))
         return
     if name.startswith("decode_loop"):
         r = run_gpu_loop(name, w, a.steps, a.warmup)

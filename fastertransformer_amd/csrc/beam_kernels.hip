@@ -28,7 +28,7 @@ constexpr int BM_CAP     = 2048;  // keys settled in LDS
 constexpr int BM_MAX_N   = 128;   // 2 * beam_width and 2 * MAX_K are at most this
 
 struct BeamSelect {
-    unsigned long long list[BM_CAP];
+    __attribute__((aligned(16))) unsigned long long list[BM_CAP];
     unsigned long long cand[BM_CAP];     // a section's elements at or above the bound from the thread maxima
     unsigned long long slots[BM_THREADS];
     unsigned long long out[BM_MAX_N];
@@ -117,11 +117,14 @@ __device__ __forceinline__ void beam_select(BeamSelect& s, F&& key, int count, i
         // one key per thread: its place is the number of larger keys
         const unsigned long long k = t < count ? key(t) : 0ull;
         __syncthreads();  // (the caller may still be reading what key() reads from, or s.list)
-        s.list[t] = k;
+        s.list[t] = k;  // (zeros behind the last key: they are larger than nothing)
         __syncthreads();
-        int r = 0;
-        for (int j = 0; j < count; ++j) {
-            r += s.list[j] > k ? 1 : 0;
+        const ulonglong2* pairs = reinterpret_cast<const ulonglong2*>(s.list);
+        int               r     = 0;
+        for (int j = 0; j < (count + 3) / 4; ++j) {
+            const ulonglong2 a = pairs[2 * j];
+            const ulonglong2 b = pairs[2 * j + 1];
+            r += (a.x > k ? 1 : 0) + (a.y > k ? 1 : 0) + (b.x > k ? 1 : 0) + (b.y > k ? 1 : 0);
         }
         if (t < count && r < need) {
             s.out[r] = k;
@@ -279,7 +282,7 @@ beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     uint32_t kmax = 0u;
     stream_columns<DT, BM_THREADS>(x + rb, lo, hi, [&](int v, float xv) {
         const float e = beam_element_of<DT>(xv, bias, v);
-        d += (double)det_expf(e - m);
+        d += (double)det_expf_nonpos(e - m);  // m is the row's maximum: the argument is never positive
         const uint32_t k = order_key(e);
         kmax             = k > kmax ? k : kmax;
     });
@@ -473,8 +476,14 @@ beam_batch_kernel(const int* __restrict__ cand_id, const float* __restrict__ can
     };
     const int take = max_k2 < C ? max_k2 : C;
     beam_select(s, [&](int c) { return beam_key(score(c), (uint32_t)c); }, C, take);
+    // what the walk reads about its candidates, fetched by one thread each
+    __shared__ int   cand_x[BM_MAX_N];
+    __shared__ float cand_y[BM_MAX_N];
     if (t < take) {
-        score_of[t] = score((int)beam_key_position(s.out[t]));
+        const int p = (int)beam_key_position(s.out[t]);
+        score_of[t] = score(p);
+        cand_x[t]   = x[p];
+        cand_y[t]   = y[p];
     }
     __syncthreads();
     if (t != 0) {
@@ -483,9 +492,11 @@ beam_batch_kernel(const int* __restrict__ cand_id, const float* __restrict__ can
     int*   z        = ids + (size_t)b * K;
     float* v        = cum_log_probs + (size_t)b * K;
     int    selected = 0;
+    const int end_id = with_hyps ? h.end_ids[b] : -1;
     for (int i = 0; i < take; ++i) {
-        const int p = (int)beam_key_position(s.out[i]);
-        if (with_hyps && x[p] % vocab == h.end_ids[b]) {
+        const int   xp = cand_x[i];
+        const float yp = cand_y[i];
+        if (with_hyps && xp % vocab == end_id) {
             if (i < K) {
                 const float normed_score = score_of[i];
                 const int   num_beam     = h.num_beams[g];
@@ -510,11 +521,11 @@ beam_batch_kernel(const int* __restrict__ cand_id, const float* __restrict__ can
                     }
                 }
                 const size_t tgt = ((size_t)(b + h.ite * h.local_batch_size) * (K * 2) + beam_idx) * h.max_seq_len;
-                h.output_ids_tgt[tgt + h.step] = h.end_ids[b];
+                h.output_ids_tgt[tgt + h.step] = end_id;
                 if (h.log_probs != nullptr) {
-                    h.log_probs[tgt + h.step] = y[p] - old_cum[(x[p] / vocab) % K];
+                    h.log_probs[tgt + h.step] = yp - old_cum[(xp / vocab) % K];
                 }
-                int prev_id = (x[p] / vocab) % K;
+                int prev_id = (xp / vocab) % K;
                 for (int j = h.step - 1; j >= 0; --j) {
                     const size_t src =
                         (size_t)j * h.batch_size * K + (size_t)h.ite * h.local_batch_size * K + (size_t)b * K + prev_id;
@@ -529,15 +540,15 @@ beam_batch_kernel(const int* __restrict__ cand_id, const float* __restrict__ can
                 h.normed_scores[tgt_beam]        = normed_score;
                 h.min_normed_scores[g] = __builtin_fminf(h.min_normed_scores[g], h.normed_scores[tgt_beam]);
                 h.num_beams[g]++;
-                h.cum_log_probs[tgt_beam] = y[p];
+                h.cum_log_probs[tgt_beam] = yp;
             }
         }
         else if ((with_hyps && i < 2 * K) || (!with_hyps && i < K)) {
-            z[selected] = x[p];
+            z[selected] = xp;
             if (output_log_probs != nullptr) {
-                output_log_probs[b * K + selected] = y[p] - old_cum[(z[selected] / vocab) % K];
+                output_log_probs[b * K + selected] = yp - old_cum[(z[selected] / vocab) % K];
             }
-            v[selected] = y[p];
+            v[selected] = yp;
             selected++;
         }
         if (selected >= K) {
