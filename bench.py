@@ -324,11 +324,19 @@ def run_gpu_loop(name, w, steps, warmup, nbuf=2):
     step_arr = np.zeros(1, np.int32)
     fixed = {"step": step_arr, "max_input_length": np.array([H], np.int32), "ite": np.array([0], np.uint32),
              "local_batch_size": np.array([B], np.int32), "end_id": end_id, "sequence_limit_length": limit}
-    from helpers import make_word_list
+    def word_list(n, longest):
+        # [2, L] in the reference's format: ids back to back (0 padded), then inclusive end offsets (-1 padded)
+        words = [rng.integers(1, V, int(rng.integers(1, longest + 1))) for _ in range(n)]
+        out = np.zeros((2, n * longest), np.int32)
+        out[1, :] = -1
+        flat = np.concatenate(words)
+        out[0, :flat.size] = flat
+        out[1, :n] = np.cumsum([len(x) for x in words])
+        return out
+
     for key, spec in (("bad_words_list", w.get("bad_words")), ("stop_words_list", w.get("stop_words"))):
-        if spec:  # [B, 2, L] word lists in the reference's format, random ids
-            n, longest = spec
-            lists = np.stack([make_word_list(rng, n, longest, V, L=n * longest)[0] for _ in range(B)])
+        if spec:  # [B, 2, L] word lists, random ids
+            lists = np.stack([word_list(*spec) for _ in range(B)])
             fixed[key] = torch.from_numpy(lists).to(dev)
     if "stop_words_list" in fixed:
         outs["parent_ids"] = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -356,26 +364,46 @@ def run_gpu_beam(name, w, steps, warmup):
     import torch
     import fastertransformer_amd as fa
     from fastertransformer_amd import ops
-    from helpers import make_beam_case, to_torch
 
     torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
     dt = {"f32": fa.F32, "f16": fa.F16, "bf16": fa.BF16}[w["dtype"]]
     batch, K, V = w["batch"], w["beam_width"], w["vocab"]
-    rng = np.random.default_rng(1)
-    cases = [make_beam_case(rng, dt, batch, K, V, with_hyps=True, end_spike=0.05, finished_frac=0.05, full_frac=0.0,
-                            scale=w["sigma"]) for _ in range(3)]
-    c = cases[0]
-    d = {k: to_torch(c[k]) for k in ("finished", "sequence_lengths", "cum_log_probs", "end_ids", "ids",
-                                     "output_log_probs")}
-    logits = [to_torch(x["log_probs"], dt) for x in cases]
-    hyps, keep = ops.BeamHypotheses(), {}
-    for key, val in c["hyps"].items():
-        if isinstance(val, np.ndarray) and key != "end_ids":
-            keep[key] = to_torch(val)
-            setattr(hyps, key, keep[key].data_ptr())
-        elif key in ("step", "ite", "batch_size", "local_batch_size", "max_seq_len"):
-            setattr(hyps, key, int(val))
-    hyps.end_ids = d["end_ids"].data_ptr()
+    rows, step, max_seq_len = batch * K, 5, 12
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    rnd = lambda *shape: torch.rand(*shape, generator=gen, device=dev)
+    end_ids = torch.randint(0, V, (batch,), generator=gen, device=dev, dtype=torch.int32)
+    row_end = end_ids.repeat_interleave(K).long()
+    logits = []
+    for _ in range(3):
+        x = torch.randn((rows, V), generator=gen, device=dev, dtype=torch.float32) * w["sigma"]
+        ending = rnd(rows) < 0.05                      # a few beams are about to end
+        x[torch.arange(rows, device=dev)[ending], row_end[ending]] += 4.0 * w["sigma"]
+        logits.append(x.to(fa.torch_dtype(dt)))
+    d = {"finished": rnd(rows) < 0.05,
+         "sequence_lengths": torch.randint(1, step + 2, (rows,), generator=gen, device=dev, dtype=torch.int32),
+         "cum_log_probs": -torch.randn(rows, generator=gen, device=dev).abs() * 4, "end_ids": end_ids,
+         "ids": torch.full((batch, K), -1, dtype=torch.int32, device=dev),
+         "output_log_probs": torch.zeros((batch, K), device=dev)}
+    normed = -torch.randn((batch, 2 * K), generator=gen, device=dev).abs() * 3
+    num = torch.randint(0, K, (batch,), generator=gen, device=dev, dtype=torch.int32)
+    mins = torch.stack([normed[b, :int(num[b])].min() if int(num[b]) else normed.new_zeros(()) for b in range(batch)])
+    keep = {"output_ids_tgt": torch.zeros((batch, 2 * K, max_seq_len), dtype=torch.int32, device=dev),
+            "sequence_lengths_tgt": torch.zeros((batch, 2 * K), dtype=torch.int32, device=dev),
+            "cum_log_probs": torch.zeros((batch, 2 * K), device=dev), "normed_scores": normed,
+            "log_probs": torch.zeros((batch, 2 * K, max_seq_len), device=dev), "min_normed_scores": mins,
+            "num_beams": num, "is_done": torch.zeros(batch, dtype=torch.bool, device=dev),
+            "output_ids_src": torch.randint(0, V, (max_seq_len, batch, K), generator=gen, device=dev,
+                                            dtype=torch.int32),
+            "parent_ids_src": torch.randint(0, K, (max_seq_len, batch, K), generator=gen, device=dev,
+                                            dtype=torch.int32),
+            "log_probs_src": -torch.randn((max_seq_len, batch, K), generator=gen, device=dev).abs()}
+    hyps = ops.BeamHypotheses()
+    for key, val in keep.items():
+        setattr(hyps, key, val.data_ptr())
+    hyps.end_ids = end_ids.data_ptr()
+    hyps.step, hyps.ite, hyps.batch_size, hyps.local_batch_size, hyps.max_seq_len = step, 0, batch, batch, max_seq_len
     hyps.early_stopping = True
     lib = fa.ftk()
     size = C.c_size_t(0)
@@ -388,7 +416,7 @@ def run_gpu_beam(name, w, steps, warmup):
             d["end_ids"].data_ptr(), 0.0, 0.0, ops.current_stream()))
 
     call(logits[0], None)
-    ws = torch.empty(size.value, dtype=torch.uint8, device="cuda")
+    ws = torch.empty(size.value, dtype=torch.uint8, device=dev)
     num0, cum0 = keep["num_beams"].clone(), d["cum_log_probs"].clone()
     ms, checksum = [], 0
     for i in range(steps + warmup):

@@ -605,6 +605,19 @@ int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, 
     if (length_penalty != 0.0f && sequence_lengths == nullptr) {
         return FTK_ERR_ARGUMENT;  // (:572)
     }
+    if (log_probs == nullptr || finished == nullptr || cum_log_probs == nullptr || ids == nullptr
+        || end_ids == nullptr) {
+        return FTK_ERR_ARGUMENT;  // the reference's kernels read and write all of these
+    }
+    if (beam_hyps != nullptr && beam_hyps->num_beams != nullptr
+        && (beam_hyps->output_ids_tgt == nullptr || beam_hyps->sequence_lengths_tgt == nullptr
+            || beam_hyps->cum_log_probs == nullptr || beam_hyps->normed_scores == nullptr
+            || beam_hyps->min_normed_scores == nullptr || beam_hyps->is_done == nullptr
+            || beam_hyps->end_ids == nullptr
+            || (beam_hyps->step > 0 && (beam_hyps->output_ids_src == nullptr || beam_hyps->parent_ids_src == nullptr))
+            || beam_hyps->step < 0 || beam_hyps->step >= beam_hyps->max_seq_len)) {
+        return FTK_ERR_ARGUMENT;  // a hypothesis is written at position `step` of a max_seq_len-long row
+    }
     char*               ws       = (char*)temp_storage;
     float*              pmax     = (float*)(ws + plan.off_pmax);
     double*             psum     = (double*)(ws + plan.off_psum);
