@@ -174,3 +174,17 @@ def test_tensor_map_semantics(tmp_path):
                            "-Wl,-rpath," + os.path.join(PKG, "lib"), "-Wl,-rpath,/opt/rocm/lib", "-o", exe])
     out = subprocess.run([exe], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
+
+
+def test_kernel_wrappers_instantiate_and_answer_host_queries(tmp_path):
+    """the launcher templates under the reference's header names compile for float, half and bfloat16 and their
+    host-only calls (size queries, refused arguments) answer without a device"""
+    _ensure_built()
+    exe = str(tmp_path / "test_kernel_wrappers")
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", PKG, "-I", INCLUDE,
+                           "-I", "/opt/rocm/include", os.path.join(ROOT, "tests", "cpp", "test_kernel_wrappers.cc"),
+                           "-L", os.path.join(PKG, "lib"), "-lft_decode", "-lftk_sampling",
+                           "-L", "/opt/rocm/lib", "-lamdhip64",
+                           "-Wl,-rpath," + os.path.join(PKG, "lib"), "-Wl,-rpath,/opt/rocm/lib", "-o", exe])
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
