@@ -182,8 +182,10 @@ __device__ __forceinline__ float beam_element(const typename Storage<DT>::T* __r
 template<int DT>
 __device__ __forceinline__ float beam_element_of(float xv, const typename Storage<DT>::T* __restrict__ bias, int v)
 {
-    const float b = bias != nullptr ? Storage<DT>::ld(bias[v]) : 0.0f;
-    return round_t<DT>(xv + b);
+    if (bias == nullptr) {
+        return xv;  // adding T(0) changes -0 into +0 and nothing else: same key, same exponential
+    }
+    return round_t<DT>(xv + Storage<DT>::ld(bias[v]));
 }
 
 struct BeamPlan {
@@ -278,13 +280,12 @@ beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
         m              = pm > m ? pm : m;
     }
     // first pass: the sum, and every thread's largest element
-    double   d    = 0.0;
-    uint32_t kmax = 0u;
+    double d    = 0.0;
+    float  fmax = -__builtin_inff();
     stream_columns<DT, BM_THREADS>(x + rb, lo, hi, [&](int v, float xv) {
         const float e = beam_element_of<DT>(xv, bias, v);
         d += (double)det_expf_nonpos(e - m);  // m is the row's maximum: the argument is never positive
-        const uint32_t k = order_key(e);
-        kmax             = k > kmax ? k : kmax;
+        fmax = __builtin_fmaxf(fmax, e);      // (a NaN is never the maximum, as under order_key)
     });
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
@@ -293,7 +294,19 @@ beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     if (lane_id() == 0) {
         red[wave_id()] = d;
     }
-    s.slots[t] = ((unsigned long long)kmax << 32) | (unsigned long long)(BM_THREADS - 1 - t);
+    // N <= 32 needs no more than 64 maxima to choose the N-th largest from, N <= 64 no more than 128: neighbouring
+    // threads join theirs, and the ranking below is that much shorter
+    const int group = N <= 32 ? 4 : N <= 64 ? 2 : 1;
+    if (group >= 2) {
+        fmax = __builtin_fmaxf(fmax, __shfl_xor(fmax, 1, WAVE));
+    }
+    if (group == 4) {
+        fmax = __builtin_fmaxf(fmax, __shfl_xor(fmax, 2, WAVE));
+    }
+    const int n_slots = BM_THREADS / group;
+    if (t % group == 0) {
+        s.slots[t / group] = ((unsigned long long)order_key(fmax) << 32) | (unsigned long long)(BM_THREADS - 1 - t);
+    }
     if (t == 0) {
         s.n_cand = 0;
     }
@@ -309,15 +322,14 @@ beam_section_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     const int take = min(N, hi - lo);
     // The N-th largest of the thread maxima is an element with at least N elements at or above it (N threads hold
     // one each): nothing below it can be among the N best. Usually a few times N elements pass.
-    uint32_t floor_key = 0u;
-    if (hi - lo >= BM_THREADS) {
-        // (thread maxima of threads that saw no element are 0 and lower the bound at most to 0)
-        beam_select(s, [&](int i) { return s.slots[i]; }, BM_THREADS, N);
-        floor_key = (uint32_t)(s.out[N - 1] >> 32);
-    }
+    // (a group that saw no element reports -inf, which lowers the bound at most to "every number")
+    beam_select(s, [&](int i) { return s.slots[i]; }, n_slots, N);
+    const uint32_t floor_key = (uint32_t)(s.out[N - 1] >> 32);
+    const float    floor_val = key_to_float(floor_key);
+    const bool     all_pass  = floor_key <= order_key(-__builtin_inff());  // then NaN columns are wanted too
     stream_columns<DT, BM_THREADS>(x + rb, lo, hi, [&](int v, float xv) {
         const float e = beam_element_of<DT>(xv, bias, v);
-        if (order_key(e) >= floor_key) {
+        if (e >= floor_val || all_pass) {
             const int at = atomicAdd(&s.n_cand, 1);
             if (at < BM_CAP) {
                 s.cand[at] = beam_key(e, (uint32_t)v);
