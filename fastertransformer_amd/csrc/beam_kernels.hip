@@ -577,6 +577,148 @@ beam_batch_kernel(const int* __restrict__ cand_id, const float* __restrict__ can
     }
 }
 
+// ---- the kernels around the step -----------------------------------------------------------------------------
+// kernels/beam_search_penalty_kernels.cu:24-86 (add_bias_temperature, generic and half2 forms): one workgroup per
+// (chunk, row); pad columns are masked in both forms here (the sampling layers' half2 form leaves them alone).
+template<int DT>
+__global__ void __launch_bounds__(BM_THREADS)
+beam_bias_temperature_kernel(typename Storage<DT>::T* __restrict__ logits,
+                             const typename Storage<DT>::T* __restrict__ bias, int V, int Vp, int chunk,
+                             float temperature)
+{
+    typedef Storage<DT>   S;
+    const int             row   = blockIdx.y;
+    const float           inv   = 1.0f / (temperature + 1e-6f);
+    const float           inv_t = round_t<DT>(inv);
+    const bool            pairs = DT == DT_F16 && V % 2 == 0 && Vp % 2 == 0;
+    const int             lo    = min(Vp, (int)blockIdx.x * chunk);
+    const int             hi    = min(Vp, lo + chunk);
+    typename S::T*        rowp  = logits + (size_t)row * Vp;
+    transform_columns<DT, BM_THREADS>(rowp, lo, hi, [&](int v, float x) {
+        if (v >= V) {
+            return -S::max_t();
+        }
+        if (pairs) {
+            const float y = bias != nullptr ? round_t<DT>(x + S::ld(bias[v])) : x;
+            return y * inv_t;
+        }
+        const float b = bias != nullptr ? S::ld(bias[v]) : 0.0f;
+        return round_t<DT>(x + b) * (DT == DT_F32 ? inv : inv_t);
+    });
+}
+
+// :88-154 (apply_repetition_penalty): one workgroup per beam; thread 0 follows the beam back through parent_ids and
+// computes every penalised value from the row as it is, then all threads store. Dynamic LDS: step values and ids.
+template<int DT>
+__global__ void __launch_bounds__(BM_THREADS)
+beam_repetition_kernel(typename Storage<DT>::T* __restrict__ logits, int batch_size, int K, int Vp, int step,
+                       const int* __restrict__ current_ids, const int* __restrict__ previous_ids,
+                       const int* __restrict__ parent_ids, const int* __restrict__ input_lengths,
+                       int max_input_length, float repetition_penalty, int additive)
+{
+    typedef Storage<DT>   S;
+    extern __shared__ int beam_hist[];  // [step] ids, then [step] values
+    int*                  idx  = beam_hist;
+    float*                val  = reinterpret_cast<float*>(beam_hist + step);
+    const int             t    = threadIdx.x;
+    const int             r    = blockIdx.x;
+    const int             b    = r / K;
+    typename S::T*        row  = logits + (size_t)r * Vp;
+    const int             len  = input_lengths != nullptr ? input_lengths[r] : max_input_length;
+    if (t == 0) {
+        const int   bbsize = batch_size * K;
+        const float pen    = round_t<DT>(repetition_penalty);
+        auto        penalised = [&](float x) {
+            if (additive) {
+                return round_t<DT>(x - pen);
+            }
+            return x > 0.0f ? round_t<DT>(x / pen) : round_t<DT>(x * pen);
+        };
+        int prev_id   = current_ids[r];
+        idx[step - 1] = prev_id;
+        val[step - 1] = penalised(S::ld(row[prev_id]));
+        int beam      = r % K;
+        for (int i = step - 2; i >= 0; --i) {
+            if (i >= len && i < max_input_length) {
+                continue;
+            }
+            beam    = parent_ids[(size_t)i * bbsize + b * K + beam];
+            prev_id = previous_ids[(size_t)i * bbsize + b * K + beam];
+            idx[i]  = prev_id;
+            val[i]  = penalised(S::ld(row[prev_id]));
+        }
+    }
+    __syncthreads();
+    for (int i = t; i < step; i += BM_THREADS) {
+        if (i >= len && i < max_input_length) {
+            continue;
+        }
+        row[idx[i]] = S::st(val[i]);
+    }
+}
+
+// :156-173 (apply_min_length_penalty)
+template<int DT>
+__global__ void beam_min_length_kernel(typename Storage<DT>::T* __restrict__ logits, int min_length,
+                                       const int* __restrict__ end_ids, const int* __restrict__ sequence_lengths,
+                                       int max_input_length, int K, int Vp, int rows)
+{
+    const int r = threadIdx.x + blockIdx.x * blockDim.x;
+    if (r < rows && sequence_lengths[r] + 1 - max_input_length < min_length) {
+        logits[(size_t)r * Vp + end_ids[r / K]] = Storage<DT>::st(-Storage<DT>::max_t());
+    }
+}
+
+// layers/beam_search_layers/OnlineBeamSearchLayer.cu:24-61 (update_kernel): one wave per batch entry, so that what
+// the reference leaves to the order of its threads is fixed: every row counts its token, then takes the length of
+// the beam it continues; an entry with beam_width hypotheses is finished.
+__global__ void __launch_bounds__(WAVE)
+beam_update_kernel(bool* __restrict__ finished, int* __restrict__ parent_ids, int* __restrict__ sequence_length,
+                   int* word_ids, int* output_ids, const int* __restrict__ num_beams, int ite, int hyps_local_batch,
+                   int K, int Vp, const int* __restrict__ end_ids)
+{
+    __shared__ int counted[WAVE];
+    const int      b = blockIdx.x;
+    const int      k = threadIdx.x;
+    const int      i = b * K + k;
+    int            word = 0;
+    if (k < K) {
+        counted[k] = finished[i] ? sequence_length[i] : sequence_length[i] + 1;
+        word       = word_ids[i];
+    }
+    __syncthreads();
+    if (k < K) {
+        const int  beam_id = (word / Vp) % K;
+        const int  word_id = word % Vp;
+        const bool done    = num_beams != nullptr && num_beams[ite * hyps_local_batch + b] == K;
+        sequence_length[i] = counted[beam_id];
+        finished[i]        = done || word_id == end_ids[b];
+        parent_ids[i]      = beam_id;
+        word_ids[i]        = word_id;
+        output_ids[i]      = word_id;
+    }
+}
+
+// layers/beam_search_layers/BaseBeamSearchLayer.cu:22-49 (update_indir_cache_kernel)
+__global__ void beam_indir_cache_kernel(int* __restrict__ tgt, const int* __restrict__ src,
+                                        const int* __restrict__ beam_ids, const bool* __restrict__ finished,
+                                        int start_step, int local_batch_size, int K, int max_seq_len, int step)
+{
+    int       time_step = threadIdx.x + blockIdx.x * blockDim.x;
+    const int bb        = blockIdx.y;
+    const int b         = bb / K;
+    const int beam      = bb % K;
+    if (bb >= K * local_batch_size || time_step >= min(step + 1, max_seq_len) || finished[bb]) {
+        return;
+    }
+    time_step += start_step;
+    const int    circ     = time_step % max_seq_len;
+    const int    src_beam = beam_ids[b * K + beam];
+    const size_t t_off    = (size_t)b * K * max_seq_len + (size_t)beam * max_seq_len + circ;
+    const size_t s_off    = (size_t)b * K * max_seq_len + (size_t)src_beam * max_seq_len + circ;
+    tgt[t_off]            = time_step == step ? beam : src[s_off];
+}
+
 }  // namespace ftk
 
 using namespace ftk;
@@ -678,6 +820,117 @@ int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, 
                                                                  diversity_rate);
         FTK_LAUNCH_CHECK();
     });
+    return 0;
+}
+
+
+int ftk_invoke_add_bias_apply_penalties(int dtype, int step, void* logits, const int* current_ids,
+                                        const int* previous_ids, const int* parent_ids, const int* input_lengths,
+                                        const int* sequence_lengths, const void* bias, int ite, int max_input_length,
+                                        int local_batch_size, int batch_size, int beam_width, int vocab_size,
+                                        int vocab_size_padded, const int* end_ids, float temperature,
+                                        float repetition_penalty, int repetition_penalty_type, int min_length,
+                                        ftk_stream_t stream)
+{
+    if (dtype < 0 || dtype > 2) {
+        return FTK_ERR_DTYPE;
+    }
+    if (local_batch_size < 0 || beam_width < 1 || vocab_size < 1 || vocab_size_padded < vocab_size || step < 0
+        || (long long)local_batch_size * beam_width > 65535) {
+        return FTK_ERR_ARGUMENT;
+    }
+    const int rows = local_batch_size * beam_width;
+    if (rows == 0) {
+        return 0;
+    }
+    if (logits == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (bias != nullptr || temperature != 1.0f || vocab_size != vocab_size_padded) {
+        int chunks = (1024 + rows - 1) / rows;
+        chunks     = chunks < (vocab_size_padded + 8191) / 8192 ? chunks : (vocab_size_padded + 8191) / 8192;
+        const int  chunk = ((vocab_size_padded + chunks - 1) / chunks + 7) / 8 * 8;
+        const dim3 grid((vocab_size_padded + chunk - 1) / chunk, rows);
+        FTK_DISPATCH_DTYPE(dtype, beam_bias_temperature_kernel<DT><<<grid, BM_THREADS, 0, st>>>(
+                                      (Storage<DT>::T*)logits, (const Storage<DT>::T*)bias, vocab_size,
+                                      vocab_size_padded, chunk, temperature));
+        FTK_LAUNCH_CHECK();
+    }
+    const bool  additive = repetition_penalty_type == FTK_PENALTY_ADDITIVE;
+    const float neutral  = repetition_penalty_type == FTK_PENALTY_MULTIPLICATIVE ? 1.0f : 0.0f;
+    if (repetition_penalty_type != FTK_PENALTY_NONE && step > 0 && repetition_penalty != neutral) {
+        if (current_ids == nullptr || (step > 1 && (previous_ids == nullptr || parent_ids == nullptr))) {
+            return FTK_ERR_ARGUMENT;
+        }
+        const size_t smem = (size_t)step * 2 * sizeof(int);
+        if (smem > 64 * 1024) {
+            return FTK_ERR_ARGUMENT;  // a history of more than 8192 steps does not fit the kernel's table
+        }
+        FTK_DISPATCH_DTYPE(dtype, beam_repetition_kernel<DT><<<rows, BM_THREADS, smem, st>>>(
+                                      (Storage<DT>::T*)logits, batch_size, beam_width, vocab_size_padded, step,
+                                      current_ids, previous_ids,
+                                      parent_ids != nullptr ? parent_ids + (size_t)ite * beam_width * local_batch_size :
+                                                              nullptr,
+                                      input_lengths, max_input_length, repetition_penalty, additive ? 1 : 0));
+        FTK_LAUNCH_CHECK();
+    }
+    if (step - max_input_length < min_length) {
+        if (sequence_lengths == nullptr || end_ids == nullptr) {
+            return FTK_ERR_ARGUMENT;  // the reference checks the same two
+        }
+        FTK_DISPATCH_DTYPE(dtype, beam_min_length_kernel<DT><<<(rows + 255) / 256, 256, 0, st>>>(
+                                      (Storage<DT>::T*)logits, min_length, end_ids, sequence_lengths, max_input_length,
+                                      beam_width, vocab_size_padded, rows));
+        FTK_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+int ftk_invoke_beam_update(bool* finished, int* parent_ids, int* sequence_length, int* word_ids, int* output_ids,
+                           const ftk_beam_hypotheses* beam_hyps, int local_batch_size, int beam_width,
+                           int vocab_size_padded, const int* end_ids, ftk_stream_t stream)
+{
+    if (local_batch_size < 0 || beam_width < 1 || beam_width > WAVE || vocab_size_padded < 1) {
+        return FTK_ERR_ARGUMENT;
+    }
+    if (local_batch_size == 0) {
+        return 0;
+    }
+    if (finished == nullptr || parent_ids == nullptr || sequence_length == nullptr || word_ids == nullptr
+        || output_ids == nullptr || end_ids == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    const int* num_beams = beam_hyps != nullptr ? beam_hyps->num_beams : nullptr;
+    beam_update_kernel<<<local_batch_size, WAVE, 0, (hipStream_t)stream>>>(
+        finished, parent_ids, sequence_length, word_ids, output_ids, num_beams, beam_hyps != nullptr ? beam_hyps->ite : 0,
+        beam_hyps != nullptr ? beam_hyps->local_batch_size : 0, beam_width, vocab_size_padded, end_ids);
+    FTK_LAUNCH_CHECK();
+    return 0;
+}
+
+int ftk_invoke_update_indir_cache(int* tgt_indir_cache, const int* src_indir_cache, const int* beam_ids,
+                                  const bool* finished, int batch_dim, int local_batch_size, int beam_width,
+                                  int max_seq_len, int step, ftk_stream_t stream)
+{
+    (void)batch_dim;
+    if (local_batch_size < 0 || beam_width < 1 || max_seq_len < 1 || step < 0
+        || (long long)local_batch_size * beam_width > 65535) {
+        return FTK_ERR_ARGUMENT;
+    }
+    if (local_batch_size == 0) {
+        return 0;
+    }
+    if (tgt_indir_cache == nullptr || src_indir_cache == nullptr || beam_ids == nullptr || finished == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    const int  start_step = step + 1 - max_seq_len > 0 ? step + 1 - max_seq_len : 0;
+    const int  num_steps  = step + 1 < max_seq_len ? step + 1 : max_seq_len;
+    const dim3 grid((num_steps + 63) / 64, local_batch_size * beam_width);
+    beam_indir_cache_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(tgt_indir_cache, src_indir_cache, beam_ids, finished,
+                                                                  start_step, local_batch_size, beam_width, max_seq_len,
+                                                                  step);
+    FTK_LAUNCH_CHECK();
     return 0;
 }
 

@@ -69,6 +69,10 @@ _SIGNATURES = {
     "ftk_invoke_transpose_axis01": [_vp, _vp, _vp, _i, _i, _vp],
     "ftk_invoke_finalize": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_invoke_topk_softmax": [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _f, _f, _vp],
+    "ftk_invoke_add_bias_apply_penalties": [_i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp,
+                                            _f, _f, _i, _i, _vp],
+    "ftk_invoke_beam_update": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp],
+    "ftk_invoke_update_indir_cache": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "ftk_error_string": [_i],
     "ftk_profile_enable": [_i],
     "ftk_profile_read": [_i, _vp, _vp],

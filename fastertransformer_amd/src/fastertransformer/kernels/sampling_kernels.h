@@ -325,4 +325,40 @@ void invokeTopkSoftMax(const T* log_probs, const T* bias, const bool* finished, 
                                       vocab_size, end_ids, diversity_rate, length_penalty, stream));
 }
 
+// kernels/beam_search_penalty_kernels.cu:175-267
+template<typename T>
+void invokeAddBiasApplyPenalties(int step, T* logits, const int* current_ids, const int* previous_ids,
+                                 const int* parent_ids, const int* input_lengths, const int* sequence_lengths,
+                                 const T* bias, const int ite, const int max_input_length, const int local_batch_size,
+                                 const int batch_size, const int beam_width, const int vocab_size,
+                                 const int vocab_size_padded, const int* end_ids, const float temperature,
+                                 const float repetition_penalty, const RepetitionPenaltyType repetition_penalty_type,
+                                 const int min_length, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_add_bias_apply_penalties(FtkDType<T>::value, step, logits, current_ids, previous_ids,
+                                                  parent_ids, input_lengths, sequence_lengths, bias, ite,
+                                                  max_input_length, local_batch_size, batch_size, beam_width,
+                                                  vocab_size, vocab_size_padded, end_ids, temperature,
+                                                  repetition_penalty, toFtkPenalty(repetition_penalty_type),
+                                                  min_length, stream));
+}
+
+// layers/beam_search_layers/OnlineBeamSearchLayer.cu:63-85
+inline void invokeUpdate(bool* finished, int* parent_ids, int* sequence_length, int* word_ids, int* output_ids,
+                         BeamHypotheses* beam_hyps, const int local_batch_size, const int beam_width,
+                         const int vocab_size_padded, const int* end_ids, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_beam_update(finished, parent_ids, sequence_length, word_ids, output_ids, beam_hyps,
+                                     local_batch_size, beam_width, vocab_size_padded, end_ids, stream));
+}
+
+// layers/beam_search_layers/BaseBeamSearchLayer.cu:51-77
+inline void update_indir_cache_kernelLauncher(int* tgt_indir_cache, const int* src_indir_cache, const int* beam_ids,
+                                              const bool* finished, int batch_dim, int local_batch_size,
+                                              int beam_width, int max_seq_len, int step, hipStream_t stream)
+{
+    check_ftk(ftk_invoke_update_indir_cache(tgt_indir_cache, src_indir_cache, beam_ids, finished, batch_dim,
+                                            local_batch_size, beam_width, max_seq_len, step, stream));
+}
+
 }  // namespace fastertransformer

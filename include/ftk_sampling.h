@@ -335,6 +335,42 @@ int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, 
                             int batch_size, int beam_width, int vocab_size, const int* end_ids, float diversity_rate,
                             float length_penalty, ftk_stream_t stream);
 
+/* invokeAddBiasApplyPenalties<T>, kernels/beam_search_penalty_kernels.cu:175-267: what BaseBeamSearchLayer applies
+ * to logits [local_batch_size * beam_width, vocab_size_padded] before the step above: bias and temperature with
+ * pad columns masked (when there is a bias, a temperature other than 1 or padding), the repetition
+ * (multiplicative) or presence (additive) penalty over each beam's own history, followed back through parent_ids
+ * (when step > 0 and the penalty is not the neutral value), and the min-length mask of the end id (when
+ * step - max_input_length < min_length; needs sequence_lengths and end_ids). current_ids = the ids of step - 1 of
+ * this window; previous_ids / parent_ids = the [max_seq_len, batch_size * beam_width] arrays from their start
+ * (parent_ids is offset by `ite` windows inside, previous_ids is not, as in the reference). Histories of more than
+ * 8192 steps return FTK_ERR_ARGUMENT. */
+int ftk_invoke_add_bias_apply_penalties(int dtype, int step, void* logits, const int* current_ids,
+                                        const int* previous_ids, const int* parent_ids, const int* input_lengths,
+                                        const int* sequence_lengths, const void* bias, int ite, int max_input_length,
+                                        int local_batch_size, int batch_size, int beam_width, int vocab_size,
+                                        int vocab_size_padded, const int* end_ids, float temperature,
+                                        float repetition_penalty, int repetition_penalty_type, int min_length,
+                                        ftk_stream_t stream);
+
+/* invokeUpdate, layers/beam_search_layers/OnlineBeamSearchLayer.cu:24-85: splits the absolute ids the step wrote
+ * (word_ids, [local_batch_size, beam_width]) into token (word_ids, output_ids: may be the same array) and parent
+ * beam (parent_ids), sets finished where the token is the end id, and gives every row the length of the beam it
+ * continues plus its own token. An entry whose hypotheses are complete (beam_hyps->num_beams == beam_width) gets
+ * all its beams finished. The reference's threads read and write other rows of their batch entry within one launch;
+ * here every row first counts its token, then takes the length of its parent (what a warp in lockstep does).
+ * beam_width <= 64. */
+int ftk_invoke_beam_update(bool* finished, int* parent_ids, int* sequence_length, int* word_ids, int* output_ids,
+                           const ftk_beam_hypotheses* beam_hyps, int local_batch_size, int beam_width,
+                           int vocab_size_padded, const int* end_ids, ftk_stream_t stream);
+
+/* update_indir_cache_kernelLauncher, layers/beam_search_layers/BaseBeamSearchLayer.cu:22-77: the key / value cache
+ * indirection [local_batch_size, beam_width, max_seq_len] of the beams after a step: position `step` points at
+ * the beam itself, earlier positions are copied from the parent beam (beam_ids = the step's parent_ids); rows of
+ * finished beams are left as they are. batch_dim is accepted and unused, as in the reference. */
+int ftk_invoke_update_indir_cache(int* tgt_indir_cache, const int* src_indir_cache, const int* beam_ids,
+                                  const bool* finished, int batch_dim, int local_batch_size, int beam_width,
+                                  int max_seq_len, int step, ftk_stream_t stream);
+
 /* ---- per-kernel timing of the fused step (the reference's counterpart is its CudaTimer / NVTX ranges,
  * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
  * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on

@@ -1059,6 +1059,152 @@ static int topk_softmax(const typename St<DT>::T* log_probs, const typename St<D
     return 0;
 }
 
+// ------------------------------------------------------------------------------------------
+// kernels/beam_search_penalty_kernels.cu:24-267 (invokeAddBiasApplyPenalties): bias and temperature over
+// [local_batch * beam_width, vocab_size_padded] logits with pad columns masked, the repetition / presence penalty
+// over a beam's own history (followed back through parent_ids, every token penalised from the value it had before
+// the kernel), the min-length mask. Literal, including: previous_ids is indexed with the local batch index
+// (the launcher offsets parent_ids by `ite` but not previous_ids), and the half2 kernel adds the bias only when
+// there is one while the generic kernel adds T(0) (a difference for -0 only).
+// ------------------------------------------------------------------------------------------
+template<int DT>
+static void beam_add_bias_apply_penalties(int step, typename St<DT>::T* logits, const int* current_ids,
+                                          const int* previous_ids, const int* parent_ids, const int* input_lengths,
+                                          const int* sequence_lengths, const typename St<DT>::T* bias, int ite,
+                                          int max_input_length, int local_batch_size, int batch_size, int K, int V,
+                                          int Vp, const int* end_ids, float temperature, float repetition_penalty,
+                                          int penalty_type, int min_length)
+{
+    typedef St<DT> S;
+    auto        rt   = [](float f) { return S::ld(S::st(f)); };
+    const int   rows = local_batch_size * K;
+    const float MAXT = S::max_t();
+    if (bias != nullptr || temperature != 1.0f || V != Vp) {
+        const float inv   = 1.0f / (temperature + 1e-6f);
+        const float inv_t = rt(inv);
+        const bool  pairs = DT == DT_F16 && V % 2 == 0 && Vp % 2 == 0;
+        for (int r = 0; r < rows; ++r) {
+            for (int v = 0; v < Vp; ++v) {
+                typename S::T& x = logits[(size_t)r * Vp + v];
+                if (v >= V) {
+                    x = S::st(-MAXT);
+                }
+                else if (pairs) {
+                    float y = S::ld(x);
+                    if (bias != nullptr) {
+                        y = rt(y + S::ld(bias[v]));
+                    }
+                    x = S::st(y * inv_t);
+                }
+                else {
+                    const float b = bias != nullptr ? S::ld(bias[v]) : 0.0f;
+                    x             = S::st(rt(S::ld(x) + b) * (DT == DT_F32 ? inv : inv_t));
+                }
+            }
+        }
+    }
+    const float neutral = penalty_type == PEN_MULTIPLICATIVE ? 1.0f : 0.0f;
+    if (penalty_type != PEN_NONE && step > 0 && repetition_penalty != neutral) {
+        const int*  parents = parent_ids + (size_t)ite * K * local_batch_size;
+        const int   bbsize  = batch_size * K;
+        const float pen     = rt(repetition_penalty);
+        for (int r = 0; r < rows; ++r) {
+            typename S::T*     row = logits + (size_t)r * Vp;
+            const int          b   = r / K;
+            const int          len = input_lengths != nullptr ? input_lengths[r] : max_input_length;
+            std::vector<int>   idx(step, -1);
+            std::vector<float> val(step, 0.0f);
+            auto               penalised = [&](float x) {
+                if (penalty_type == PEN_ADDITIVE) {
+                    return rt(x - pen);
+                }
+                return x > 0.0f ? rt(x / pen) : rt(x * pen);
+            };
+            int prev_id   = current_ids[r];
+            idx[step - 1] = prev_id;
+            val[step - 1] = penalised(S::ld(row[prev_id]));
+            int beam      = r % K;
+            for (int i = step - 2; i >= 0; --i) {
+                if (i >= len && i < max_input_length) {
+                    continue;
+                }
+                beam    = parents[(size_t)i * bbsize + b * K + beam];
+                prev_id = previous_ids[(size_t)i * bbsize + b * K + beam];
+                idx[i]  = prev_id;
+                val[i]  = penalised(S::ld(row[prev_id]));
+            }
+            for (int i = 0; i < step; ++i) {
+                if (i >= len && i < max_input_length) {
+                    continue;
+                }
+                row[idx[i]] = S::st(val[i]);
+            }
+        }
+    }
+    if (step - max_input_length < min_length) {
+        for (int r = 0; r < rows; ++r) {
+            if (sequence_lengths[r] + 1 - max_input_length < min_length) {
+                logits[(size_t)r * Vp + end_ids[r / K]] = S::st(-MAXT);
+            }
+        }
+    }
+}
+
+// layers/beam_search_layers/OnlineBeamSearchLayer.cu:24-61 (update_kernel). The reference's threads read
+// sequence_length and write finished of other rows of their batch entry inside one launch; the order restated here
+// is what a warp in lockstep does when an entry's rows share it: every row counts its token first, then every row
+// takes the length of the beam it continues, then an entry that has collected beam_width hypotheses is finished.
+static void beam_update(bool* finished, int* parent_ids, int* sequence_length, int* word_ids, int* output_ids,
+                        const BeamHyps* hyps, int local_batch_size, int K, int Vp, const int* end_ids)
+{
+    const int        rows = local_batch_size * K;
+    std::vector<int> counted(rows);
+    for (int i = 0; i < rows; ++i) {
+        counted[i] = finished[i] ? sequence_length[i] : sequence_length[i] + 1;
+    }
+    for (int i = 0; i < rows; ++i) {
+        const int b       = i / K;
+        const int beam_id = (word_ids[i] / Vp) % K;
+        const int word_id = word_ids[i] % Vp;
+        sequence_length[i] = counted[b * K + beam_id];
+        finished[i]        = word_id == end_ids[b];
+        parent_ids[i]      = beam_id;
+        word_ids[i]        = word_id;
+        output_ids[i]      = word_id;
+    }
+    if (hyps != nullptr && hyps->num_beams != nullptr) {
+        for (int b = 0; b < local_batch_size; ++b) {
+            if (hyps->num_beams[hyps->ite * hyps->local_batch_size + b] == K) {
+                for (int i = 0; i < K; ++i) {
+                    finished[b * K + i] = true;
+                }
+            }
+        }
+    }
+}
+
+// layers/beam_search_layers/BaseBeamSearchLayer.cu:22-77
+static void update_indir_cache(int* tgt, const int* src, const int* beam_ids, const bool* finished,
+                               int local_batch_size, int K, int max_seq_len, int step)
+{
+    const int start_step = std::max(0, step + 1 - max_seq_len);
+    const int num_steps  = std::min(step + 1, max_seq_len);
+    for (int bb = 0; bb < local_batch_size * K; ++bb) {
+        if (finished[bb]) {
+            continue;
+        }
+        const int b = bb / K, beam = bb % K;
+        const int src_beam = beam_ids[b * K + beam];
+        for (int ts = 0; ts < num_steps; ++ts) {
+            const int    time_step = ts + start_step;
+            const int    circ      = time_step % max_seq_len;
+            const size_t t_off     = (size_t)b * K * max_seq_len + (size_t)beam * max_seq_len + circ;
+            const size_t s_off     = (size_t)b * K * max_seq_len + (size_t)src_beam * max_seq_len + circ;
+            tgt[t_off]             = time_step == step ? beam : src[s_off];
+        }
+    }
+}
+
 }  // namespace oracle
 
 using namespace oracle;
@@ -1609,6 +1755,36 @@ int oracle_topk_softmax(int dt, const void* log_probs, const void* bias, const b
                                        cum_log_probs, output_log_probs, ids, hyps, batch_size, beam_width, vocab_size,
                                        end_ids, diversity_rate, length_penalty));
     return rc;
+}
+
+
+int oracle_beam_add_bias_apply_penalties(int dt, int step, void* logits, const int* current_ids,
+                                         const int* previous_ids, const int* parent_ids, const int* input_lengths,
+                                         const int* sequence_lengths, const void* bias, int ite, int max_input_length,
+                                         int local_batch_size, int batch_size, int beam_width, int vocab_size,
+                                         int vocab_size_padded, const int* end_ids, float temperature,
+                                         float repetition_penalty, int penalty_type, int min_length)
+{
+    DISPATCH(dt, beam_add_bias_apply_penalties<DT>(step, (St<DT>::T*)logits, current_ids, previous_ids, parent_ids,
+                                                   input_lengths, sequence_lengths, (const St<DT>::T*)bias, ite,
+                                                   max_input_length, local_batch_size, batch_size, beam_width,
+                                                   vocab_size, vocab_size_padded, end_ids, temperature,
+                                                   repetition_penalty, penalty_type, min_length));
+    return 0;
+}
+
+void oracle_beam_update(bool* finished, int* parent_ids, int* sequence_length, int* word_ids, int* output_ids,
+                        const BeamHyps* hyps, int local_batch_size, int beam_width, int vocab_size_padded,
+                        const int* end_ids)
+{
+    beam_update(finished, parent_ids, sequence_length, word_ids, output_ids, hyps, local_batch_size, beam_width,
+                vocab_size_padded, end_ids);
+}
+
+void oracle_update_indir_cache(int* tgt, const int* src, const int* beam_ids, const bool* finished,
+                               int local_batch_size, int beam_width, int max_seq_len, int step)
+{
+    update_indir_cache(tgt, src, beam_ids, finished, local_batch_size, beam_width, max_seq_len, step);
 }
 
 }  // extern "C"

@@ -1,6 +1,7 @@
 // Every launcher template of the reference-named headers instantiates for the three element types, and the calls
 // that need no device (size queries, argument refusals) behave: compiled and run by tests/test_cabi.py.
 #include "src/fastertransformer/kernels/ban_bad_words.h"
+#include "src/fastertransformer/kernels/beam_search_penalty_kernels.h"
 #include "src/fastertransformer/kernels/beam_search_topk_kernels.h"
 #include "src/fastertransformer/kernels/online_softmax_beamsearch_kernels.h"
 #include "src/fastertransformer/kernels/sampling_penalty_kernels.h"
@@ -34,6 +35,7 @@ static int instantiate()
         (const void*)&invokeBanBadWords<T>,
         (const void*)&invokeLogProbFromLogits<T>,
         (const void*)&invokeTopkSoftMax<T>,
+        (const void*)&invokeAddBiasApplyPenalties<T>,
         (const void*)&topkSoftMaxWorkspaceBytes<T>,
     };
     int n = 0;
@@ -45,7 +47,7 @@ static int instantiate()
 
 int main()
 {
-    if (instantiate<float>() != 18 || instantiate<half>() != 18 || instantiate<bfloat16>() != 18) {
+    if (instantiate<float>() != 19 || instantiate<half>() != 19 || instantiate<bfloat16>() != 19) {
         return 1;
     }
     // size queries run on the host

@@ -347,3 +347,38 @@ def topk_softmax(dt, log_probs, bias, finished, sequence_lengths, cum_log_probs,
     return fn(dt, _p(log_probs), _p(bias), _p(finished), _p(sequence_lengths), _p(cum_log_probs), _p(output_log_probs),
               _p(ids), C.addressof(h) if h is not None else None, batch, beam_width, vocab, _p(end_ids),
               float(diversity_rate), float(length_penalty))
+
+
+def beam_add_bias_apply_penalties(dt, step, logits, current_ids, previous_ids, parent_ids, input_lengths,
+                                  sequence_lengths, bias, ite, max_input_length, local_batch, batch, beam_width, V, Vp,
+                                  end_ids, temperature, repetition_penalty, penalty_type, min_length):
+    """invokeAddBiasApplyPenalties: logits [local_batch * beam_width, Vp] are updated in place"""
+    fn = lib().oracle_beam_add_bias_apply_penalties
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_int, C.c_int] + [C.c_void_p] * 7 + [C.c_int] * 7 + [C.c_void_p, C.c_float, C.c_float, C.c_int,
+                                                                          C.c_int]
+    return fn(dt, step, _p(logits), _p(current_ids), _p(previous_ids), _p(parent_ids), _p(input_lengths),
+              _p(sequence_lengths), _p(bias), ite, max_input_length, local_batch, batch, beam_width, V, Vp,
+              _p(end_ids), float(temperature), float(repetition_penalty), penalty_type, min_length)
+
+
+def beam_update(finished, parent_ids, sequence_length, word_ids, output_ids, num_beams, ite, local_batch, beam_width,
+                Vp, end_ids):
+    """invokeUpdate; num_beams (or None) stands for the BeamHypotheses argument"""
+    h = None
+    if num_beams is not None:
+        h = BeamHyps()
+        h.num_beams, h.ite, h.local_batch_size = num_beams.ctypes.data, ite, local_batch
+    fn = lib().oracle_beam_update
+    fn.restype = None
+    fn.argtypes = [C.c_void_p] * 6 + [C.c_int] * 3 + [C.c_void_p]
+    fn(_p(finished), _p(parent_ids), _p(sequence_length), _p(word_ids), _p(output_ids),
+       C.addressof(h) if h is not None else None, local_batch, beam_width, Vp, _p(end_ids))
+
+
+def update_indir_cache(tgt, src, beam_ids, finished, local_batch, beam_width, max_seq_len, step):
+    fn = lib().oracle_update_indir_cache
+    fn.restype = None
+    fn.argtypes = [C.c_void_p] * 4 + [C.c_int] * 4
+    fn(_p(tgt), _p(src), _p(beam_ids), _p(finished), local_batch, beam_width, max_seq_len, step)
+

@@ -173,3 +173,13 @@ def copy_beam_case(c):
     if out["hyps"] is not None:
         out["hyps"]["end_ids"] = out["end_ids"]
     return out
+
+
+def make_beam_history(rng, batch, K, V, step, max_seq_len, max_input_length):
+    """ids and parent beams of `step` earlier steps ([max_seq_len, batch * K]) and per-beam input lengths"""
+    out_ids = np.zeros((max_seq_len, batch * K), np.int32)
+    parents = np.zeros((max_seq_len, batch * K), np.int32)
+    out_ids[:step] = rng.integers(0, V, (step, batch * K))
+    parents[:step] = rng.integers(0, K, (step, batch * K))
+    input_lengths = rng.integers(1, max_input_length + 1, batch * K).astype(np.int32)
+    return out_ids, parents, input_lengths

@@ -155,3 +155,84 @@ def test_beam_step_with_bias_and_refusals():
     small = C.c_size_t(16)
     assert lib.ftk_invoke_topk_softmax(O.F32, *none[:7], ws.data_ptr(), C.addressof(small), None, 2, 8, 100, None,
                                        0.0, 0.0, None) == ops.FTK_ERR_WORKSPACE
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("penalty_type", [0, 1, 2], ids=["presence", "repetition", "none"])
+def test_beam_penalties(dt, penalty_type):
+    """ftk_invoke_add_bias_apply_penalties against the oracle, bit for bit: even and odd vocabularies (the half2
+    form and the generic one), pad columns, with and without bias, windows of a larger batch, long histories"""
+    import torch
+    from helpers import make_beam_history
+    ops, lib = _lib()
+    rng = np.random.default_rng(40 + dt + 10 * penalty_type)
+    for V, Vp, batch, local, ite, K, step, max_input in ((300, 300, 3, 3, 0, 4, 7, 4), (301, 304, 4, 2, 1, 3, 5, 5),
+                                                         (50257, 50264, 2, 2, 0, 2, 1, 1), (32000, 32000, 5, 5, 0, 8, 40, 8),
+                                                         (1000, 1024, 2, 1, 1, 64, 12, 3)):
+        L = step + 3
+        out_ids, parents, input_lengths = make_beam_history(rng, batch, K, V, step, L, max_input)
+        rows = local * K
+        for with_bias, temperature in ((False, 1.0), (True, 0.7), (False, 1.6)):
+            x = O.to_storage((rng.standard_normal((rows, Vp)) * 3).astype(np.float32), dt)
+            bias = O.to_storage(rng.standard_normal(Vp).astype(np.float32), dt) if with_bias else None
+            seq = rng.integers(max_input, max_input + 6, rows).astype(np.int32)
+            end_ids = rng.integers(0, V, local).astype(np.int32)
+            current = out_ids[step - 1, ite * rows:(ite + 1) * rows].copy()
+            lens = input_lengths[:rows].copy()
+            penalty = 1.0 if penalty_type == 2 else float(rng.choice([0.5, 1.3, 2.0]))
+            min_length = int(rng.integers(0, 8))
+            want = x.copy()
+            O.beam_add_bias_apply_penalties(dt, step, want, current, out_ids, parents, lens, seq, bias, ite, max_input,
+                                            local, batch, K, V, Vp, end_ids, temperature, penalty, penalty_type,
+                                            min_length)
+            d = [to_torch(a) for a in (current, out_ids, parents, lens, seq, end_ids)]
+            d_x, d_bias = to_torch(x, dt), (to_torch(bias, dt) if with_bias else None)
+            print("penalties", DTYPE_NAMES[dt], V, Vp, batch, local, ite, K, step, with_bias, temperature, flush=True)
+            ops.check(lib.ftk_invoke_add_bias_apply_penalties(
+                dt, step, d_x.data_ptr(), d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                d[4].data_ptr(), ops.ptr(d_bias), ite, max_input, local, batch, K, V, Vp, d[5].data_ptr(),
+                temperature, penalty, penalty_type, min_length, ops.current_stream()))
+            torch.cuda.synchronize()
+            got = to_numpy(d_x)
+            assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))
+
+
+def test_beam_update_and_cache_indirection():
+    import torch
+    ops, lib = _lib()
+    rng = np.random.default_rng(61)
+    for batch, K, Vp, L, step in ((4, 3, 500, 9, 5), (70, 64, 32000, 20, 25), (1, 2, 50264, 6, 0), (300, 4, 1000, 64, 63)):
+        word = (rng.integers(0, K, (batch, K)) + np.arange(batch)[:, None] * K) * Vp + rng.integers(0, Vp, (batch, K))
+        word = word.astype(np.int32).reshape(-1)
+        end_ids = rng.integers(0, Vp, batch).astype(np.int32)
+        ends = rng.random(batch * K) < 0.2
+        word[ends] = word[ends] // Vp * Vp + np.repeat(end_ids, K)[ends]
+        finished = rng.random(batch * K) < 0.3
+        seq = rng.integers(3, 9, batch * K).astype(np.int32)
+        num_beams = np.where(rng.random(batch) < 0.3, K, rng.integers(0, K, batch)).astype(np.int32)
+        for hyps_on in (True, False):
+            f, s_, w = finished.copy(), seq.copy(), word.copy()
+            parent, out = np.full(batch * K, -1, np.int32), np.full(batch * K, -1, np.int32)
+            O.beam_update(f, parent, s_, w, out, num_beams if hyps_on else None, 0, batch, K, Vp, end_ids)
+            d_f, d_s, d_w, d_end, d_num = (to_torch(a) for a in (finished, seq, word, end_ids, num_beams))
+            d_parent = torch.full((batch * K,), -1, dtype=torch.int32, device="cuda")
+            hyps = ops.BeamHypotheses()
+            hyps.num_beams, hyps.ite, hyps.local_batch_size = d_num.data_ptr(), 0, batch
+            # output_ids and word_ids are the same array in the layer's call
+            ops.check(lib.ftk_invoke_beam_update(d_f.data_ptr(), d_parent.data_ptr(), d_s.data_ptr(), d_w.data_ptr(),
+                                                 d_w.data_ptr(), C.addressof(hyps) if hyps_on else None, batch, K, Vp,
+                                                 d_end.data_ptr(), ops.current_stream()))
+            torch.cuda.synchronize()
+            for got, want in ((d_f, f), (d_parent, parent), (d_s, s_), (d_w, w)):
+                assert np.array_equal(to_numpy(got), want)
+            src = rng.integers(0, K, (batch, K, L)).astype(np.int32)
+            tgt = np.full((batch, K, L), -7, np.int32)
+            want_tgt = tgt.copy()
+            O.update_indir_cache(want_tgt, src, parent, f, batch, K, L, step)
+            d_tgt, d_src = to_torch(tgt), to_torch(src)
+            ops.check(lib.ftk_invoke_update_indir_cache(d_tgt.data_ptr(), d_src.data_ptr(), d_parent.data_ptr(),
+                                                        d_f.data_ptr(), batch, batch, K, L, step,
+                                                        ops.current_stream()))
+            torch.cuda.synchronize()
+            assert np.array_equal(to_numpy(d_tgt), want_tgt)
+

@@ -861,3 +861,104 @@ def test_beam_step_moves_end_tokens_to_the_hypotheses(length_penalty):
     assert np.array_equal(c["ids"][1], old_ids[1]) and np.array_equal(c["cum_log_probs"][K:], old_cum[K:])
     assert np.array_equal(h["output_ids_tgt"][1], before["output_ids_tgt"][1])
 
+
+# ---- the kernels around the beam search step ---------------------------------------------------------------------
+def _beam_penalties_by_numpy(x, bias, V, Vp, K, step, out_ids, parents, input_lengths, seq, end_ids, max_input,
+                             temperature, penalty, multiplicative, min_length):
+    """the description, independently: (x + bias) * 1/(T + 1e-6) with pads masked, every token of a beam's own
+    history (followed back through the parent beams, prompt padding skipped) penalised once from its value before
+    the penalty, the end id masked while the sequence is shorter than min_length; fp32 operation by operation"""
+    f = np.float32
+    rows = x.shape[0]
+    y = x.astype(f).copy()
+    if bias is not None or temperature != 1.0 or V != Vp:
+        inv = f(1.0) / (f(temperature) + f(1e-6))
+        b = bias.astype(f) if bias is not None else np.zeros(Vp, f)
+        y[:, :V] = (y[:, :V] + b[:V]) * inv
+        y[:, V:] = -np.finfo(f).max
+    if penalty is not None and step > 0:
+        before = y.copy()
+        for r in range(rows):
+            b_, beam = r // K, r % K
+            tokens = [out_ids[step - 1, r]]
+            for i in range(step - 2, -1, -1):
+                if input_lengths[r] <= i < max_input:
+                    continue
+                beam = parents[i, b_ * K + beam]
+                tokens.append(out_ids[i, b_ * K + beam])
+            for tok in set(int(t) for t in tokens):
+                v = before[r, tok]
+                y[r, tok] = (v / f(penalty) if v > 0 else v * f(penalty)) if multiplicative else v - f(penalty)
+    if step - max_input < min_length:
+        for r in range(rows):
+            if seq[r] + 1 - max_input < min_length:
+                y[r, end_ids[r // K]] = -np.finfo(f).max
+    return y
+
+
+@pytest.mark.parametrize("multiplicative", [True, False])
+@pytest.mark.parametrize("with_bias,temperature,V,Vp", [(False, 1.0, 300, 300), (True, 0.7, 300, 300),
+                                                        (False, 1.3, 301, 304), (True, 1.0, 1000, 1024)])
+def test_beam_penalties_against_the_description(multiplicative, with_bias, temperature, V, Vp):
+    from helpers import make_beam_history
+    rng = np.random.default_rng(V + Vp + int(multiplicative))
+    batch, K, step, L, max_input = 3, 4, 7, 12, 4
+    out_ids, parents, input_lengths = make_beam_history(rng, batch, K, V, step, L, max_input)
+    x = (rng.standard_normal((batch * K, Vp)) * 3).astype(np.float32)
+    bias = rng.standard_normal(Vp).astype(np.float32) if with_bias else None
+    seq = rng.integers(max_input, max_input + 5, batch * K).astype(np.int32)
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    penalty, min_length = (1.3 if multiplicative else 0.6), 5
+    want = _beam_penalties_by_numpy(x, bias, V, Vp, K, step, out_ids, parents, input_lengths, seq, end_ids, max_input,
+                                    temperature, penalty, multiplicative, min_length)
+    got = x.copy()
+    O.beam_add_bias_apply_penalties(O.F32, step, got, out_ids[step - 1].copy(), out_ids, parents, input_lengths, seq,
+                                    bias, 0, max_input, batch, batch, K, V, Vp, end_ids, temperature, penalty,
+                                    1 if multiplicative else 0, min_length)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the neutral penalty and a step past min_length leave the row alone
+    same = x.copy()
+    O.beam_add_bias_apply_penalties(O.F32, 50, same, out_ids[step - 1].copy(),
+                                    out_ids, parents, input_lengths, seq, None, 0, max_input, batch, batch, K, Vp, Vp,
+                                    end_ids, 1.0, 1.0 if multiplicative else 0.0, 1 if multiplicative else 0, 0)
+    assert np.array_equal(same, x)
+
+
+def test_beam_update_and_cache_indirection_against_the_description():
+    rng = np.random.default_rng(21)
+    batch, K, Vp, L, step = 4, 3, 500, 9, 5
+    word = (rng.integers(0, K, (batch, K)) + np.arange(batch)[:, None] * K) * Vp + rng.integers(0, Vp, (batch, K))
+    word = word.astype(np.int32).reshape(-1)
+    end_ids = rng.integers(0, Vp, batch).astype(np.int32)
+    word[2] = (2 // K * K + 1) * Vp + end_ids[0]     # row 2 continues beam 1 of entry 0 with the end token
+    finished = rng.random(batch * K) < 0.3
+    seq = rng.integers(3, 9, batch * K).astype(np.int32)
+    num_beams = np.array([0, K, 1, 2], np.int32)
+    f, s_, w = finished.copy(), seq.copy(), word.copy()
+    parent, out = np.full(batch * K, -1, np.int32), np.full(batch * K, -1, np.int32)
+    O.beam_update(f, parent, s_, w, out, num_beams, 0, batch, K, Vp, end_ids)
+    counted = np.where(finished, seq, seq + 1)
+    for i in range(batch * K):
+        b = i // K
+        beam, tok = (word[i] // Vp) % K, word[i] % Vp
+        assert parent[i] == beam and w[i] == tok and out[i] == tok
+        assert s_[i] == counted[b * K + beam]
+        assert f[i] == (tok == end_ids[b] or num_beams[b] == K)
+    assert f[2] and f[K:2 * K].all()
+    # cache indirection: position `step` names the beam itself, earlier ones come from the parent beam's row
+    src = rng.integers(0, K, (batch, K, L)).astype(np.int32)
+    tgt = np.full((batch, K, L), -7, np.int32)
+    O.update_indir_cache(tgt, src, parent, f, batch, K, L, step)
+    for b in range(batch):
+        for k in range(K):
+            if f[b * K + k]:
+                assert (tgt[b, k] == -7).all()
+                continue
+            assert tgt[b, k, step] == k
+            assert np.array_equal(tgt[b, k, :step], src[b, parent[b * K + k], :step])
+            assert (tgt[b, k, step + 1:] == -7).all()
+    # a step beyond the window wraps around: every position of the window is rewritten
+    tgt2 = np.full((batch, K, L), -7, np.int32)
+    O.update_indir_cache(tgt2, src, parent, np.zeros(batch * K, bool), batch, K, L, L + 3)
+    assert (tgt2 != -7).all() and all(tgt2[b, k, (L + 3) % L] == k for b in range(batch) for k in range(K))
+
