@@ -34,7 +34,8 @@
 //    force written from the source description only (finalize: a stable descending sort);
 //  * beam search step (topk_softmax): no reference test exists; pinned by the definition it must reduce to
 //    without hypotheses (the K largest of cum + log_softmax over all continuations, float64) and by
-//    scenario checks of the hypothesis bookkeeping written from the source description.
+//    scenario checks of the hypothesis bookkeeping written from the source description; the penalties,
+//    update and cache-indirection kernels around it by independent numpy restatements of the description.
 //  PARITY UNPINNED (no reference code or no way to run it here): the rounding order of cub's
 //  BLOCK_SCAN_RAKING prefix sums in top-p (cub is not in the reference's tree), bfloat16 storage, the frequency
 //  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), the last-ulp
