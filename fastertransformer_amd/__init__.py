@@ -5,8 +5,8 @@ include/ftk_sampling.h) and fastertransformer_amd/lib/libft_decode.so (host C++ 
 include/ft_decode_c.h). This package only loads them and passes device pointers of torch tensors
 through; there is no Python or CPU fallback, and loading fails loudly when the libraries are missing.
 """
-from .ops import (F32, F16, BF16, PENALTY_ADDITIVE, PENALTY_MULTIPLICATIVE, PENALTY_NONE, DynamicDecodeLayer,
-                  FtkError, decode_lib, ftk, lib_dir, torch_dtype)
+from .ops import (F32, F16, BF16, PENALTY_ADDITIVE, PENALTY_MULTIPLICATIVE, PENALTY_NONE, BeamHypotheses,
+                  DynamicDecodeLayer, FtkError, OnlineBeamSearchLayer, decode_lib, ftk, lib_dir, torch_dtype)
 
-__all__ = ["F32", "F16", "BF16", "PENALTY_ADDITIVE", "PENALTY_MULTIPLICATIVE", "PENALTY_NONE", "DynamicDecodeLayer",
-           "FtkError", "decode_lib", "ftk", "lib_dir", "torch_dtype"]
+__all__ = ["F32", "F16", "BF16", "PENALTY_ADDITIVE", "PENALTY_MULTIPLICATIVE", "PENALTY_NONE", "BeamHypotheses",
+           "DynamicDecodeLayer", "FtkError", "OnlineBeamSearchLayer", "decode_lib", "ftk", "lib_dir", "torch_dtype"]

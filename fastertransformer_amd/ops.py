@@ -170,6 +170,12 @@ def decode_lib():
         lib.ft_dynamic_decode_setup.argtypes = [_vp, _sz, _sz, _i, C.POINTER(C.c_char_p), C.POINTER(FtTensor)]
         lib.ft_dynamic_decode_forward.argtypes = [_vp, _i, C.POINTER(C.c_char_p), C.POINTER(FtTensor), _i,
                                                   C.POINTER(C.c_char_p), C.POINTER(FtTensor)]
+        lib.ft_online_beam_search_create.restype = _vp
+        lib.ft_online_beam_search_create.argtypes = [_i, _sz, _sz, _vp]
+        lib.ft_online_beam_search_destroy.argtypes = [_vp]
+        lib.ft_online_beam_search_destroy.restype = None
+        lib.ft_online_beam_search_forward.argtypes = [_vp, _i, C.POINTER(C.c_char_p), C.POINTER(FtTensor), _i,
+                                                      C.POINTER(C.c_char_p), C.POINTER(FtTensor)]
         _dec = lib
     return _dec
 
@@ -342,3 +348,36 @@ class DynamicDecodeLayer:
                                                  pout.names, pout.descs)
         if rc != 0:
             self._raise(rc, "forward")
+
+
+class OnlineBeamSearchLayer:
+    """fastertransformer::OnlineBeamSearchLayer<T>: forward(outputs, inputs) is one beam-search step over a window
+    of the batch. Tensor names and shapes are those of the reference layer (include/ft_decode_c.h); the optional
+    output "beam_hyps" is a BeamHypotheses structure of this module."""
+
+    def __init__(self, dtype, vocab_size, vocab_size_padded, stream=None):
+        self._lib = decode_lib()
+        s = current_stream() if stream is None else stream
+        self._h = self._lib.ft_online_beam_search_create(dtype, vocab_size, vocab_size_padded, s)
+        if not self._h:
+            raise FtkError("ft_online_beam_search_create: " + self._lib.ft_decode_last_error().decode())
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.ft_online_beam_search_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def forward(self, output_tensors, input_tensors):
+        outs = dict(output_tensors)
+        if isinstance(outs.get("beam_hyps"), BeamHypotheses):
+            # the layer reads the structure through a host pointer, as the reference's does
+            outs["beam_hyps"] = np.frombuffer(outs["beam_hyps"], dtype=np.uint8)
+        n_in, d_in, keep_in = _pack(input_tensors)
+        n_out, d_out, keep_out = _pack(outs)
+        rc = self._lib.ft_online_beam_search_forward(self._h, len(keep_in), n_in, d_in, len(keep_out), n_out, d_out)
+        if rc != 0:
+            raise FtkError("forward: " + self._lib.ft_decode_last_error().decode())
+

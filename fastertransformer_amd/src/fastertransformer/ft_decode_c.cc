@@ -4,6 +4,7 @@
 #include <string>
 
 #include "src/fastertransformer/layers/DynamicDecodeLayer.h"
+#include "src/fastertransformer/layers/beam_search_layers/OnlineBeamSearchLayer.h"
 
 namespace ft = fastertransformer;
 
@@ -17,6 +18,11 @@ struct DecodeHandle {
     std::unique_ptr<ft::DynamicDecodeLayer<float>>         f32;
     std::unique_ptr<ft::DynamicDecodeLayer<ft::half>>      f16;
     std::unique_ptr<ft::DynamicDecodeLayer<ft::bfloat16>>  bf16;
+};
+
+struct BeamHandle {
+    std::unique_ptr<ft::Allocator<ft::AllocatorType::HIP>> allocator;
+    std::unique_ptr<ft::DynamicDecodeBaseLayer>            layer;
 };
 
 ft::TensorMap toMap(int n, const char* const* names, const ft_tensor* tensors)
@@ -158,6 +164,58 @@ int ft_dynamic_decode_forward(void* handle, int n_in, const char* const* in_name
         else {
             h->bf16->forward(&out, &in);
         }
+    });
+}
+
+void* ft_online_beam_search_create(int dtype, size_t vocab_size, size_t vocab_size_padded, void* stream)
+{
+    BeamHandle* h  = nullptr;
+    const int   rc = guarded([&]() {
+        int device = 0;
+        check_hip_error(hipGetDevice(&device));
+        std::unique_ptr<BeamHandle> p(new BeamHandle());
+        p->allocator.reset(new ft::Allocator<ft::AllocatorType::HIP>(device));
+        p->allocator->setStream((hipStream_t)stream);
+        hipStream_t st = (hipStream_t)stream;
+        if (dtype == FTK_DTYPE_F32) {
+            p->layer.reset(new ft::OnlineBeamSearchLayer<float>(0, 0, 0, 0, vocab_size, vocab_size_padded, 0, 0.0f, 1.0f,
+                                                                0.0f, 1.0f, st, nullptr, p->allocator.get(), false));
+        }
+        else if (dtype == FTK_DTYPE_F16) {
+            p->layer.reset(new ft::OnlineBeamSearchLayer<ft::half>(0, 0, 0, 0, vocab_size, vocab_size_padded, 0, 0.0f,
+                                                                   1.0f, 0.0f, 1.0f, st, nullptr, p->allocator.get(),
+                                                                   false));
+        }
+        else if (dtype == FTK_DTYPE_BF16) {
+            p->layer.reset(new ft::OnlineBeamSearchLayer<ft::bfloat16>(0, 0, 0, 0, vocab_size, vocab_size_padded, 0,
+                                                                       0.0f, 1.0f, 0.0f, 1.0f, st, nullptr,
+                                                                       p->allocator.get(), false));
+        }
+        else {
+            throw std::runtime_error("unsupported dtype");
+        }
+        h = p.release();
+    });
+    return rc == FT_OK ? h : nullptr;
+}
+
+void ft_online_beam_search_destroy(void* handle)
+{
+    BeamHandle* h = (BeamHandle*)handle;
+    if (h != nullptr) {
+        h->layer.reset();  // frees its workspace through the allocator
+        delete h;
+    }
+}
+
+int ft_online_beam_search_forward(void* handle, int n_in, const char* const* in_names, const ft_tensor* in_tensors,
+                                  int n_out, const char* const* out_names, const ft_tensor* out_tensors)
+{
+    BeamHandle* h = (BeamHandle*)handle;
+    return guarded([&]() {
+        ft::TensorMap in  = toMap(n_in, in_names, in_tensors);
+        ft::TensorMap out = toMap(n_out, out_names, out_tensors);
+        h->layer->forward(&out, &in);
     });
 }
 

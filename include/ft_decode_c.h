@@ -48,6 +48,18 @@ int ft_dynamic_decode_setup(void* handle, size_t batch_size, size_t beam_width, 
 int ft_dynamic_decode_forward(void* handle, int n_in, const char* const* in_names, const ft_tensor* in_tensors,
                               int n_out, const char* const* out_names, const ft_tensor* out_tensors);
 
+/* fastertransformer::OnlineBeamSearchLayer<T> (reference: layers/beam_search_layers/OnlineBeamSearchLayer.h:24-64,
+ * BaseBeamSearchLayer.h:27-71): one beam-search step per forward call, tensors by name as the reference's layer
+ * documents them (inputs: logits, step, ite, max_input_length, end_id, src_cache_indirection, optional
+ * embedding_bias, input_lengths, temperature, len_penalty, beam_search_diversity_rate, repetition_penalty or
+ * presence_penalty, min_length; outputs: output_ids, finished, cum_log_probs, parent_ids, sequence_length,
+ * tgt_cache_indirection, optional output_log_probs and beam_hyps = a host pointer to an ftk_beam_hypotheses).
+ * The layer keeps no state between steps apart from its workspace. */
+void* ft_online_beam_search_create(int dtype, size_t vocab_size, size_t vocab_size_padded, void* stream);
+void  ft_online_beam_search_destroy(void* handle);
+int   ft_online_beam_search_forward(void* handle, int n_in, const char* const* in_names, const ft_tensor* in_tensors,
+                                    int n_out, const char* const* out_names, const ft_tensor* out_tensors);
+
 #ifdef __cplusplus
 }
 #endif

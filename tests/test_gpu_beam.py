@@ -236,3 +236,97 @@ def test_beam_update_and_cache_indirection():
             torch.cuda.synchronize()
             assert np.array_equal(to_numpy(d_tgt), want_tgt)
 
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+@pytest.mark.parametrize("penalty", ["repetition_penalty", "presence_penalty", None])
+def test_online_beam_search_layer_decode_loop(dt, penalty):
+    """OnlineBeamSearchLayer::forward step after step (penalties over beam histories, the step, the update of the
+    beams, the cache indirection, hypotheses collected on the way) against the same sequence of oracle calls: ids,
+    parents, flags, lengths, hypotheses and cache indirection bit for bit, log-probs within tolerance."""
+    import torch
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+    rng = np.random.default_rng(200 + dt + (0 if penalty is None else len(penalty)))
+    batch, K, V, Vp, max_input, L, steps = 3, 4, 997, 1000, 3, 12, 7
+    rows = batch * K
+    temperature, diversity, len_pen, min_length = 0.8, 0.1, 0.7, 2
+    pen_val = {"repetition_penalty": 1.2, "presence_penalty": 0.4, None: None}[penalty]
+    ptype = {"repetition_penalty": 1, "presence_penalty": 0, None: 2}[penalty]
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    # host state of the oracle run
+    out_ids = np.zeros((L, rows), np.int32)
+    out_ids[:max_input] = rng.integers(0, V, (max_input, rows))
+    parents = np.zeros((L, rows), np.int32)
+    parents[:max_input] = np.arange(rows) % K
+    out_lp = np.zeros((L, rows), np.float32)
+    finished = np.zeros(rows, np.bool_)
+    seq = np.full(rows, max_input - 1, np.int32)
+    cum = np.tile(np.array([0.0] + [-1e20] * (K - 1), np.float32), batch)   # only beam 0 counts at the first step
+    input_lengths = rng.integers(1, max_input + 1, rows).astype(np.int32)
+    hyps = dict(output_ids_tgt=np.zeros((batch, 2 * K, L), np.int32), sequence_lengths_tgt=np.zeros((batch, 2 * K), np.int32),
+                cum_log_probs=np.zeros((batch, 2 * K), np.float32), normed_scores=np.zeros((batch, 2 * K), np.float32),
+                log_probs=np.zeros((batch, 2 * K, L), np.float32), min_normed_scores=np.zeros(batch, np.float32),
+                num_beams=np.zeros(batch, np.int32), is_done=np.zeros(batch, np.bool_))
+    cache = [rng.integers(0, K, (batch, K, L)).astype(np.int32), np.zeros((batch, K, L), np.int32)]
+    # the same state on the device
+    d = {k: to_torch(v) for k, v in dict(out_ids=out_ids.reshape(L, batch, K), parents=parents, out_lp=out_lp.reshape(L, batch, K),
+                                         finished=finished, seq=seq, cum=cum, input_lengths=input_lengths,
+                                         end_ids=end_ids).items()}
+    d_h = {k: to_torch(v) for k, v in hyps.items()}
+    d_cache = [to_torch(c) for c in cache]
+    dh = ops.BeamHypotheses()
+    for k, v in d_h.items():
+        setattr(dh, k, v.data_ptr())
+    dh.early_stopping, dh.is_return_normed_score = True, True
+    layer = fa.OnlineBeamSearchLayer(dt, V, Vp)
+    for i in range(steps):
+        step = max_input + i
+        x = (rng.standard_normal((rows, Vp)) * 3).astype(np.float32)
+        for r in range(rows):       # end tokens show up often enough to fill the hypotheses
+            if rng.random() < 0.25:
+                x[r, end_ids[r // K]] += 9.0
+        logits = O.to_storage(x, dt)
+        # ---- oracle
+        want = logits.copy()
+        O.beam_add_bias_apply_penalties(dt, step, want, out_ids[step - 1], out_ids, parents, input_lengths, seq, None, 0,
+                                        max_input, batch, batch, K, V, Vp, end_ids, temperature,
+                                        pen_val if pen_val is not None else 1.0, ptype, min_length)
+        h = dict(hyps, output_ids_src=out_ids, parent_ids_src=parents, sequence_lengths_src=None, end_ids=end_ids,
+                 log_probs_src=out_lp, step=step, ite=0, batch_size=batch, local_batch_size=batch, max_seq_len=L,
+                 length_penalty=len_pen, early_stopping=1)
+        assert O.topk_softmax(dt, want, None, finished, seq, cum, out_lp[step], out_ids[step], h, batch, K, Vp, end_ids,
+                              diversity, len_pen) == 0
+        O.beam_update(finished, parents[step], seq, out_ids[step], out_ids[step], hyps["num_beams"], 0, batch, K, Vp,
+                      end_ids)
+        O.update_indir_cache(cache[1], cache[0], parents[step], finished, batch, K, L, step)
+        # ---- the layer
+        ins = {"logits": to_torch(logits, dt).reshape(batch, K, Vp), "step": np.array([step], np.int32),
+               "ite": np.array([0], np.int32), "max_input_length": np.array([max_input], np.int32),
+               "end_id": d["end_ids"], "src_cache_indirection": d_cache[0], "input_lengths": d["input_lengths"],
+               "temperature": np.array([temperature], np.float32), "len_penalty": np.array([len_pen], np.float32),
+               "beam_search_diversity_rate": np.array([diversity], np.float32),
+               "min_length": np.array([min_length], np.int32)}
+        if penalty is not None:
+            ins[penalty] = np.array([pen_val], np.float32)
+        outs = {"output_ids": d["out_ids"], "finished": d["finished"], "cum_log_probs": d["cum"],
+                "parent_ids": d["parents"], "sequence_length": d["seq"], "tgt_cache_indirection": d_cache[1],
+                "output_log_probs": d["out_lp"], "beam_hyps": dh}
+        print("layer step", DTYPE_NAMES[dt], penalty, step, flush=True)
+        layer.forward(outs, ins)
+        torch.cuda.synchronize()
+        rtol, atol = (2e-5, 2e-5) if dt == O.F32 else (4e-3, 1e-3)
+        assert np.array_equal(to_numpy(d["out_ids"]).reshape(L, rows)[step], out_ids[step]), step
+        assert np.array_equal(to_numpy(d["parents"])[step], parents[step])
+        assert np.array_equal(to_numpy(d["finished"]), finished) and np.array_equal(to_numpy(d["seq"]), seq)
+        np.testing.assert_allclose(to_numpy(d["cum"]), cum, rtol=rtol, atol=atol)
+        np.testing.assert_allclose(to_numpy(d["out_lp"]).reshape(L, rows)[step], out_lp[step], rtol=rtol, atol=atol)
+        assert np.array_equal(to_numpy(d_cache[1]), cache[1])
+        for name in ("output_ids_tgt", "sequence_lengths_tgt", "num_beams", "is_done"):
+            assert np.array_equal(to_numpy(d_h[name]), hyps[name]), name
+        for name in ("cum_log_probs", "normed_scores", "log_probs", "min_normed_scores"):
+            np.testing.assert_allclose(to_numpy(d_h[name]), hyps[name], rtol=rtol, atol=atol, err_msg=name)
+        cache.reverse()
+        d_cache.reverse()
+    assert hyps["num_beams"].sum() > 0   # the loop did collect hypotheses
+    layer.close()
+
