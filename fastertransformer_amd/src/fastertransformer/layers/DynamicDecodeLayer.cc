@@ -1,5 +1,7 @@
 #include "src/fastertransformer/layers/DynamicDecodeLayer.h"
 
+#include <cstring>
+
 namespace fastertransformer {
 
 template<typename T>
@@ -24,6 +26,9 @@ void DynamicDecodeLayer<T>::initialize()
                                             cublas_wrapper_, allocator_, false);
     topp_decode_ = new TopPSamplingLayer<T>(0, vocab_size_, vocab_size_padded_, 0, 0.0f, 0, 1.0f, 0.0f, 1.0f, stream_,
                                             cublas_wrapper_, allocator_, false, cuda_device_prop_);
+    online_beamsearch_decode_ =
+        new OnlineBeamSearchLayer<T>(0, 0, 0, 0, vocab_size_, vocab_size_padded_, 0, 0.0f, 1.0f, 0.0f, 1.0f, stream_,
+                                     cublas_wrapper_, allocator_, is_free_buffer_after_forward_);
     allocateBuffer();
 }
 
@@ -44,6 +49,7 @@ DynamicDecodeLayer<T>::DynamicDecodeLayer(size_t vocab_size, size_t vocab_size_p
 template<typename T>
 DynamicDecodeLayer<T>::~DynamicDecodeLayer()
 {
+    delete online_beamsearch_decode_;
     delete topk_decode_;
     delete topp_decode_;
     freeBuffer();
@@ -62,15 +68,35 @@ void DynamicDecodeLayer<T>::setStream(hipStream_t stream)
     BaseLayer::setStream(stream);
     topk_decode_->setStream(stream);
     topp_decode_->setStream(stream);
+    online_beamsearch_decode_->setStream(stream);
 }
 
 // reference: DynamicDecodeLayer<T>::setup, layers/DynamicDecodeLayer.cc:153-178
 template<typename T>
 void DynamicDecodeLayer<T>::setup(const size_t batch_size, const size_t beam_width, TensorMap* runtime_args)
 {
-    FT_CHECK_WITH_INFO(beam_width == 1, "this engine implements the sampling path only (beam_width must be 1)");
-    topk_decode_->setup(batch_size, beam_width, runtime_args);
-    topp_decode_->setup(batch_size, beam_width, runtime_args);
+    // reference: hasDiffRuntimeArgs, layers/DynamicDecodeLayer.cc:476-514
+    has_diff_runtime_args_ = false;
+    for (const char* key : {"beam_search_diversity_rate", "temperature", "len_penalty", "repetition_penalty",
+                            "presence_penalty", "min_length"}) {
+        if (!runtime_args->isExist(key)) {
+            continue;
+        }
+        const Tensor& t = runtime_args->at(key);
+        FT_CHECK(t.shape.size() == 1);
+        FT_CHECK_WITH_INFO(t.type == TYPE_FP32 || t.type == TYPE_INT32 || t.type == TYPE_UINT32
+                               || t.type == TYPE_UINT64,
+                           std::string(key) + ": " + t.toString() + " is invalid.");
+        const size_t width = Tensor::getTypeSize(t.type);
+        const char*  data  = (const char*)t.data;
+        for (size_t j = 1; j < t.shape[0]; ++j) {
+            has_diff_runtime_args_ = has_diff_runtime_args_ || memcmp(data, data + j * width, width) != 0;
+        }
+    }
+    if (beam_width == 1) {
+        topk_decode_->setup(batch_size, beam_width, runtime_args);
+        topp_decode_->setup(batch_size, beam_width, runtime_args);
+    }
 }
 
 template<typename T>
@@ -112,13 +138,24 @@ void DynamicDecodeLayer<T>::forward(TensorMap* output_tensors, TensorMap* input_
 {
     const Tensor& logits = input_tensors->at("logits");
     FT_CHECK(logits.shape.size() == 3);
-    FT_CHECK_WITH_INFO(logits.shape[1] == 1, "this engine implements the sampling path only (beam_width must be 1)");
     const int    ite   = (int)input_tensors->at("ite").getVal<uint>();
     const int    step  = input_tensors->at("step").getVal<int>();
     const size_t batch = logits.shape[0];
     const size_t rows  = (size_t)input_tensors->at("local_batch_size").getVal<int>();
     const size_t first = (size_t)ite * rows;  // the window: rows [first, first + rows) of the batch
     FT_CHECK_WITH_INFO(first + rows <= batch, "ite / local_batch_size window exceeds the batch");
+    if (logits.shape[1] > 1) {
+        FT_CHECK_WITH_INFO(!input_tensors->isExist("bad_words_list") && !input_tensors->isExist("stop_words_list"),
+                           "bad_words_list / stop_words_list are not supported with beam search in this engine");
+        forwardBeams(output_tensors, input_tensors, ite, rows);
+        if (input_tensors->isExist("sequence_limit_length")) {
+            invokeLengthCriterion(output_tensors->at("finished").getPtr<bool>(),
+                                  output_tensors->at("should_stop").getPtr<bool>(), h_pinned_finished_sum_,
+                                  input_tensors->at("sequence_limit_length").getPtr<const uint32_t>(), (int)batch,
+                                  (int)logits.shape[1], step, stream_);
+        }
+        return;
+    }
 
     banBadWords(output_tensors, input_tensors, first, rows, step);
 
@@ -152,6 +189,49 @@ void DynamicDecodeLayer<T>::forward(TensorMap* output_tensors, TensorMap* input_
     topp_decode_->forward(&window_out, &window_in);
 
     stopCriteria(output_tensors, input_tensors, first, rows, step);
+}
+
+// reference: the beam_width > 1 branch of DynamicDecodeLayer<T>::forward, layers/DynamicDecodeLayer.cc:286-385. The
+// entries of the window go to the beam-search layer together, or one by one when setup() saw per-entry runtime
+// values that differ; per-beam state is cut to the sub-window, everything else is handed over whole (including
+// the cache indirections, which the layer indexes from the sub-window's first entry, as the reference's does).
+template<typename T>
+void DynamicDecodeLayer<T>::forwardBeams(TensorMap* output_tensors, TensorMap* input_tensors, int ite, size_t rows)
+{
+    const Tensor& logits = input_tensors->at("logits");
+    const size_t  beams  = logits.shape[1];
+    const size_t  group  = has_diff_runtime_args_ ? 1 : rows;  // entries per call of the layer
+    const size_t  calls  = rows / group;
+    FT_CHECK_WITH_INFO(output_tensors->isExist("cum_log_probs"), "cum_log_probs should be provided in beam search.");
+    for (uint sub = (uint)(ite * calls); sub < (uint)((ite + 1) * calls); ++sub) {
+        const size_t first_entry = (size_t)sub * group;
+        const size_t first_beam  = first_entry * beams;
+        TensorMap    in({{"logits", rowWindow(logits, first_entry, group)},
+                         {"end_id", rowWindow(input_tensors->at("end_id"), first_entry, group)},
+                         {"ite", Tensor{MEMORY_CPU, TYPE_UINT32, {1}, &sub}}});
+        if (input_tensors->isExist("input_lengths")) {
+            in.insert({"input_lengths", rowWindow(input_tensors->at("input_lengths"), first_entry, group)});
+        }
+        for (auto it = input_tensors->begin(); it != input_tensors->end(); ++it) {
+            // step, max_input_length, embedding_bias, src_cache_indirection and the runtime values of the step
+            if (!in.isExist(it->first) && it->first.find("random_seed") == std::string::npos) {
+                in.insert({it->first, it->second});
+            }
+        }
+        TensorMap out;
+        for (const char* key : {"output_ids", "parent_ids", "tgt_cache_indirection", "output_log_probs", "beam_hyps"}) {
+            if (output_tensors->isExist(key)) {
+                out.insert({key, output_tensors->at(key)});
+            }
+        }
+        for (const char* key : kRowOutputs) {
+            if (output_tensors->isExist(key)) {
+                const Tensor& t = output_tensors->at(key);  // [batch * beam_width]
+                out.insert({key, Tensor{t.where, t.type, {group * beams}, t.getPtrWithOffset(first_beam)}});
+            }
+        }
+        online_beamsearch_decode_->forward(&out, &in);
+    }
 }
 
 // Bad words are masked on the caller's logits before either layer looks at them (layers/DynamicDecodeLayer.cc:

@@ -1,10 +1,12 @@
-// Per-step decode orchestrator: bad words -> top-k / top-p sampling -> stop words -> length criterion.
+// Per-step decode orchestrator: bad words -> top-k / top-p sampling -> stop words -> length criterion, or, for
+// logits with more than one beam per entry, the beam-search layer and the length criterion.
 // Public surface of the reference's src/fastertransformer/layers/DynamicDecodeLayer.h:29-75.
-// Beam search (beam_width > 1) is outside this engine and raises an error.
+// Bad-word and stop-word lists are not supported together with beam search and raise an error.
 #pragma once
 #include <string>
 #include <unordered_map>
 
+#include "src/fastertransformer/layers/beam_search_layers/OnlineBeamSearchLayer.h"
 #include "src/fastertransformer/layers/sampling_layers/TopKSamplingLayer.h"
 #include "src/fastertransformer/layers/sampling_layers/TopPSamplingLayer.h"
 
@@ -19,9 +21,14 @@ protected:
     // the two parts of a step around the sampling layers; `first` / `rows`: the micro-batch window
     void banBadWords(TensorMap* output_tensors, TensorMap* input_tensors, size_t first, size_t rows, int step);
     void stopCriteria(TensorMap* output_tensors, TensorMap* input_tensors, size_t first, size_t rows, int step);
+    // the step for logits [batch, beam_width > 1, vocab_padded]
+    void forwardBeams(TensorMap* output_tensors, TensorMap* input_tensors, int ite, size_t rows);
 
     TopKSamplingLayer<T>* topk_decode_ = nullptr;
     TopPSamplingLayer<T>* topp_decode_ = nullptr;
+    OnlineBeamSearchLayer<T>* online_beamsearch_decode_ = nullptr;
+    // setup() saw per-entry values that differ: beam search then takes the entries of a window one by one
+    bool has_diff_runtime_args_ = false;
 
     size_t vocab_size_;
     size_t vocab_size_padded_;

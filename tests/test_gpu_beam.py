@@ -330,3 +330,74 @@ def test_online_beam_search_layer_decode_loop(dt, penalty):
     assert hyps["num_beams"].sum() > 0   # the loop did collect hypotheses
     layer.close()
 
+
+@pytest.mark.parametrize("windows", [1, 2], ids=["one_window", "two_windows"])
+def test_dynamic_decode_layer_with_beams(windows):
+    """DynamicDecodeLayer::forward on logits [batch, beam_width > 1, vocab]: the beam-search layer per window of the
+    batch and the length criterion, against the same oracle calls; bad-word lists are refused with beams."""
+    import torch
+    import fastertransformer_amd as fa
+    from fastertransformer_amd import ops
+    dt = O.F32
+    rng = np.random.default_rng(300 + windows)
+    batch, K, V, Vp, max_input, L, steps = 4, 3, 500, 504, 2, 10, 5
+    local = batch // windows
+    rows = batch * K
+    end_ids = rng.integers(0, V, batch).astype(np.int32)
+    out_ids = np.zeros((L, rows), np.int32)
+    out_ids[:max_input] = rng.integers(0, V, (max_input, rows))
+    parents = np.zeros((L, rows), np.int32)
+    parents[:max_input] = np.arange(rows) % K
+    finished = np.zeros(rows, np.bool_)
+    seq = np.full(rows, max_input - 1, np.int32)
+    cum = np.tile(np.array([0.0] + [-1e20] * (K - 1), np.float32), batch)
+    limit = np.full(batch, max_input + 3, np.uint32)     # the length criterion ends every beam at that step
+    d = {k: to_torch(v) for k, v in dict(out_ids=out_ids.reshape(L, batch, K), parents=parents, finished=finished,
+                                         seq=seq, cum=cum, end_ids=end_ids, limit=limit).items()}
+    src = [rng.integers(0, K, (local, K, L)).astype(np.int32), np.zeros((local, K, L), np.int32)]
+    d_src = [to_torch(c) for c in src]
+    layer = fa.DynamicDecodeLayer(dt, V, Vp)
+    layer.setup(batch, K, {"temperature": np.array([0.9], np.float32)})
+    should_stop = np.zeros(1, np.bool_)
+    for i in range(steps):
+        step = max_input + i
+        x = (rng.standard_normal((rows, Vp)) * 3).astype(np.float32)
+        d_x = to_torch(x).reshape(batch, K, Vp)
+        for ite in range(windows):
+            lo, hi = ite * local * K, (ite + 1) * local * K
+            want = x[lo:hi].copy()
+            O.beam_add_bias_apply_penalties(dt, step, want, out_ids[step - 1, lo:hi].copy(), out_ids, parents, None,
+                                            seq[lo:hi], None, ite, max_input, local, batch, K, V, Vp,
+                                            end_ids[ite * local:(ite + 1) * local], 0.9, 1.0, 2, 0)
+            ids_w, cum_w, fin_w, seq_w = out_ids[step, lo:hi].copy(), cum[lo:hi].copy(), finished[lo:hi].copy(), seq[lo:hi].copy()
+            assert O.topk_softmax(dt, want, None, fin_w, seq_w, cum_w, None, ids_w, None, local, K, Vp,
+                                  end_ids[ite * local:(ite + 1) * local], 0.0, 0.0) == 0
+            par_w = np.zeros(local * K, np.int32)
+            O.beam_update(fin_w, par_w, seq_w, ids_w, ids_w, None, ite, local, K, Vp, end_ids[ite * local:(ite + 1) * local])
+            O.update_indir_cache(src[1], src[0], par_w, fin_w, local, K, L, step)
+            out_ids[step, lo:hi], parents[step, lo:hi] = ids_w, par_w
+            cum[lo:hi], finished[lo:hi], seq[lo:hi] = cum_w, fin_w, seq_w
+            ins = {"logits": d_x, "step": np.array([step], np.int32), "max_input_length": np.array([max_input], np.int32),
+                   "ite": np.array([ite], np.uint32), "local_batch_size": np.array([local], np.int32),
+                   "end_id": d["end_ids"], "src_cache_indirection": d_src[0],
+                   "temperature": np.array([0.9], np.float32), "sequence_limit_length": d["limit"]}
+            outs = {"output_ids": d["out_ids"], "finished": d["finished"], "cum_log_probs": d["cum"],
+                    "parent_ids": d["parents"], "sequence_length": d["seq"], "tgt_cache_indirection": d_src[1],
+                    "should_stop": should_stop}
+            print("dynamic decode with beams", windows, step, ite, flush=True)
+            layer.forward(outs, ins)
+            torch.cuda.synchronize()
+            # the length criterion runs over the whole batch after every window
+            finished |= step >= np.repeat(limit, K)
+            assert np.array_equal(to_numpy(d_src[1]), src[1])
+        assert np.array_equal(to_numpy(d["out_ids"]).reshape(L, rows)[step], out_ids[step]), step
+        assert np.array_equal(to_numpy(d["parents"])[step], parents[step])
+        assert np.array_equal(to_numpy(d["finished"]), finished) and np.array_equal(to_numpy(d["seq"]), seq)
+        np.testing.assert_allclose(to_numpy(d["cum"]), cum, rtol=2e-5, atol=2e-5)
+        assert bool(should_stop[0]) == bool(finished.all())
+        src.reverse()
+        d_src.reverse()
+    assert finished.all() and should_stop[0]
+    with pytest.raises(fa.FtkError):
+        layer.forward(outs, dict(ins, bad_words_list=torch.zeros((2, 4), dtype=torch.int32, device="cuda")))
+

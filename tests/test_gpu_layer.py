@@ -304,8 +304,9 @@ def test_error_behaviour():
         layer.setup(4, 1, {"runtime_top_k": np.array([1, 2, 3], np.uint32)})
     with pytest.raises(fa.FtkError):  # wrong seed array size: BaseSamplingLayer.cc:135-139
         layer.setup(4, 1, {"random_seed": np.array([1, 2, 3], np.uint64)})
-    with pytest.raises(fa.FtkError):  # beam search is not part of this engine
-        layer.setup(4, 2, {})
+    layer.setup(4, 2, {})             # beam search: nothing to set up, the step reads its values from its inputs
+    with pytest.raises(fa.FtkError):  # per-entry runtime values must be one-dimensional (DynamicDecodeLayer.cc:482)
+        layer.setup(4, 2, {"temperature": np.ones((2, 2), np.float32)})
     layer.setup(2, 1, {"runtime_top_k": np.array([2], np.uint32)})
     logits = torch.zeros((2, 1, V), device="cuda")
     out_ids = torch.zeros((3, 2), dtype=torch.int32, device="cuda")

@@ -169,8 +169,7 @@ def test_argument_placement_is_checked(th):
         fwd(th.zeros((batch, 1, VOCAB - 8), device="cuda"))
     with pytest.raises(RuntimeError):   # device tensors on the device
         fwd(th.zeros((batch, 1, VOCAB), device="cuda"), end_id=eos.cpu())
-    with pytest.raises(RuntimeError):   # beam search is not part of this library
-        op.setup(batch, 2, k_cpu, None, None, None, None, None, None, None, None, None, None, None)
+    op.setup(batch, 2, k_cpu, None, None, None, None, None, None, None, None, None, None, None)  # beams: no state
     op.setup(batch, 1, k_cpu, None, None, None, None, None, None, None, None, None, None, None)
     assert not bool(fwd(th.zeros((batch, 1, VOCAB), device="cuda")))
     op.broadcast_from_last_pipeline([ids])
