@@ -48,6 +48,62 @@ __global__ void stop_words_kernel(const int* __restrict__ output_ids, const int*
     }
 }
 
+// The two kernels above for beam search: grid (ceil(L/block), rows * beams); the history is followed through
+// parent_ids (ftk_words.cuh). `id_offset` is added to the column index as given, like the reference does.
+template<int DT>
+__global__ void ban_bad_words_beams_kernel(typename Storage<DT>::T* __restrict__ logits,
+                                           const int* __restrict__ output_ids, const int* __restrict__ parent_ids,
+                                           int batch_size, int beams, const int* __restrict__ bad_words,
+                                           int bad_words_len, bool share_words, int id_offset, int vocab_size_padded,
+                                           int step)
+{
+    typedef Storage<DT> S;
+    const int           w     = blockIdx.x * blockDim.x + threadIdx.x;
+    const int           row   = blockIdx.y;
+    const int           entry = row / beams;
+    if (w >= bad_words_len) {
+        return;
+    }
+    const WordList words =
+        word_list(share_words ? bad_words : bad_words + (size_t)entry * 2 * bad_words_len, bad_words_len);
+    const int* first;
+    int        count;
+    if (!words.ngram(w, &first, &count) || count < 1) {
+        return;
+    }
+    const size_t base = (size_t)id_offset + (size_t)entry * beams;
+    const bool   ban  = count == 1
+                     || beam_history_ends_with(first, count - 1, output_ids + base, parent_ids + base,
+                                               (size_t)batch_size * beams, row % beams, beams, step - 1);
+    const int tok = first[count - 1];
+    if (ban && 0 < tok && tok < vocab_size_padded) {
+        logits[(size_t)row * vocab_size_padded + tok] = S::st(-__builtin_inff());
+    }
+}
+
+__global__ void stop_words_beams_kernel(const int* __restrict__ output_ids, const int* __restrict__ parent_ids,
+                                        const int* __restrict__ stop_words, bool* __restrict__ finished, int id_offset,
+                                        int stop_words_len, int batch_size, int beams, int step)
+{
+    const int w     = blockIdx.x * blockDim.x + threadIdx.x;
+    const int row   = blockIdx.y;
+    const int entry = row / beams;
+    if (w >= stop_words_len) {
+        return;
+    }
+    const WordList words = word_list(stop_words + (size_t)entry * 2 * stop_words_len, stop_words_len);
+    const int*     first;
+    int            count;
+    if (!words.ngram(w, &first, &count)) {
+        return;
+    }
+    const size_t base = (size_t)id_offset + (size_t)entry * beams;
+    if (beam_history_ends_with(first, count, output_ids + base, parent_ids + base, (size_t)batch_size * beams,
+                               row % beams, beams, step)) {
+        finished[row] = true;
+    }
+}
+
 // src/fastertransformer/kernels/stop_criteria_kernels.cu:106-133: one workgroup; the count goes to
 // pinned host memory with a system-scope release so the waiting host thread sees it.
 __global__ void __launch_bounds__(512)
@@ -173,11 +229,20 @@ int ftk_invoke_ban_bad_words(int dtype, void* logits, const int* output_ids_buf,
     if (bad_words_len == 0 || local_batch_size <= 0) {
         return 0;
     }
-    (void)parent_ids_buf;
-    if (beam_width != 1) {
-        return FTK_ERR_ARGUMENT;  // sampling only: one hypothesis per row
+    if (beam_width < 1 || (beam_width > 1 && parent_ids_buf == nullptr)
+        || (long long)local_batch_size * beam_width > 65535) {
+        return FTK_ERR_ARGUMENT;
     }
     const int block = (int)min((size_t)256, ((bad_words_len + 63) / 64) * 64);
+    if (beam_width > 1) {
+        dim3 beams_grid((unsigned)((bad_words_len + block - 1) / block), (unsigned)(local_batch_size * beam_width));
+        FTK_DISPATCH_DTYPE(dtype, ban_bad_words_beams_kernel<DT><<<beams_grid, block, 0, (hipStream_t)stream>>>(
+                                      (Storage<DT>::T*)logits, output_ids_buf, parent_ids_buf, batch_size, beam_width,
+                                      bad_words, (int)bad_words_len, share_words, id_offset, vocab_size_padded,
+                                      (int)step));
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
     dim3      grid((unsigned)((bad_words_len + block - 1) / block), (unsigned)local_batch_size);
     FTK_DISPATCH_DTYPE(dtype, ban_bad_words_kernel<DT><<<grid, block, 0, (hipStream_t)stream>>>(
                                   (Storage<DT>::T*)logits, output_ids_buf, batch_size, bad_words, (int)bad_words_len,
@@ -193,11 +258,18 @@ int ftk_invoke_stop_words_criterion_rows(const int* output_ids, const int* paren
     if (stop_words_len == 0 || num_rows <= 0) {
         return 0;
     }
-    (void)parent_ids;
-    if (beam_width != 1) {
-        return FTK_ERR_ARGUMENT;  // sampling only: one hypothesis per row
+    if (beam_width < 1 || (beam_width > 1 && parent_ids == nullptr) || (long long)num_rows * beam_width > 65535) {
+        return FTK_ERR_ARGUMENT;
     }
     const int block = (int)min((size_t)256, ((stop_words_len + 63) / 64) * 64);
+    if (beam_width > 1) {
+        dim3 beams_grid((unsigned)((stop_words_len + block - 1) / block), (unsigned)(num_rows * beam_width));
+        stop_words_beams_kernel<<<beams_grid, block, 0, (hipStream_t)stream>>>(
+            output_ids, parent_ids, stop_words, finished, (int)id_offset, (int)stop_words_len, batch_size, beam_width,
+            step);
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
     dim3      grid((unsigned)((stop_words_len + block - 1) / block), (unsigned)num_rows);
     stop_words_kernel<<<grid, block, 0, (hipStream_t)stream>>>(output_ids, stop_words, finished, (int)id_offset,
                                                                (int)stop_words_len, batch_size, step);

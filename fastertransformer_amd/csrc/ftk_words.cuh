@@ -2,8 +2,8 @@
 //
 // Layout (examples/pytorch/gpt/utils/word_list.py:36-67): a list is [2, L] ints; row 0 holds the token ids of
 // all n-grams back to back (0-padded), row 1 the inclusive end offset of each n-gram (-1-padded): n-gram w
-// spans ids [end[w-1] (or 0), end[w]). The history of a row is a column of output_ids [max_seq, batch].
-// Sampling only: one hypothesis per row, so there is no parent-id chain to follow.
+// spans ids [end[w-1] (or 0), end[w]). The history of a row is a column of output_ids [max_seq, batch]; with beams
+// ([max_seq, batch, beam_width]) it is followed backwards through parent_ids, one beam index per time.
 #pragma once
 #include "ftk_device.cuh"
 
@@ -42,6 +42,30 @@ __device__ __forceinline__ bool history_ends_with(const int* __restrict__ tokens
     }
     for (int t = count - 1; t >= 0; --t) {
         if (column[(size_t)(last - (count - 1) + t) * stride] != tokens[t]) {
+            return false;
+        }
+    }
+    return true;
+}
+
+// The same with beams (ban_bad_words.cu:55-74, stop_criteria_kernels.cu:52-72): `entry` points at the batch entry's
+// first beam in row 0 of output_ids / parent_ids ([max_seq, stride] each), the walk starts in beam `beam`; after a
+// token matches, that time's parent becomes the beam of the time before, and a parent outside [0, beams) ends the
+// match.
+__device__ __forceinline__ bool beam_history_ends_with(const int* __restrict__ tokens, int count,
+                                                       const int* __restrict__ ids, const int* __restrict__ parents,
+                                                       size_t stride, int beam, int beams, int last)
+{
+    if (count > last + 1) {
+        return false;
+    }
+    for (int t = count - 1; t >= 0; --t) {
+        const size_t at = (size_t)(last - (count - 1) + t) * stride;
+        if (ids[at + beam] != tokens[t]) {
+            return false;
+        }
+        beam = parents[at + beam];
+        if (beam < 0 || beam >= beams) {
             return false;
         }
     }

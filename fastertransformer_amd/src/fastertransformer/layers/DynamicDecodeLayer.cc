@@ -145,15 +145,9 @@ void DynamicDecodeLayer<T>::forward(TensorMap* output_tensors, TensorMap* input_
     const size_t first = (size_t)ite * rows;  // the window: rows [first, first + rows) of the batch
     FT_CHECK_WITH_INFO(first + rows <= batch, "ite / local_batch_size window exceeds the batch");
     if (logits.shape[1] > 1) {
-        FT_CHECK_WITH_INFO(!input_tensors->isExist("bad_words_list") && !input_tensors->isExist("stop_words_list"),
-                           "bad_words_list / stop_words_list are not supported with beam search in this engine");
+        banBadWords(output_tensors, input_tensors, first, rows, step);
         forwardBeams(output_tensors, input_tensors, ite, rows);
-        if (input_tensors->isExist("sequence_limit_length")) {
-            invokeLengthCriterion(output_tensors->at("finished").getPtr<bool>(),
-                                  output_tensors->at("should_stop").getPtr<bool>(), h_pinned_finished_sum_,
-                                  input_tensors->at("sequence_limit_length").getPtr<const uint32_t>(), (int)batch,
-                                  (int)logits.shape[1], step, stream_);
-        }
+        stopCriteria(output_tensors, input_tensors, first, rows, step);
         return;
     }
 
@@ -254,9 +248,14 @@ void DynamicDecodeLayer<T>::banBadWords(TensorMap* output_tensors, TensorMap* in
     const bool   one_list = rank == 2 || words.shape[0] == 1;
     const size_t length   = words.shape[rank - 1];
     const int*   lists    = one_list ? words.getPtr<const int>() : words.getPtrWithOffset<const int>(first * 2 * length);
+    // (the reference offsets the logits by `first` rows of the vocabulary and the history columns by `first`, whatever
+    // the beam width: layers/DynamicDecodeLayer.cc:261-280)
+    const size_t beams = input_tensors->at("logits").shape[1];
     invokeBanBadWords((T*)input_tensors->at("logits").getPtrWithOffset(first * vocab_size_padded_),
-                      output_tensors->at("output_ids").getPtr<const int>(), (const int*)nullptr, (int)batch, (int)rows,
-                      1, lists, one_list, length, (int)first, (int)vocab_size_padded_, (size_t)step, stream_);
+                      output_tensors->at("output_ids").getPtr<const int>(),
+                      beams > 1 ? output_tensors->at("parent_ids").getPtr<const int>() : (const int*)nullptr,
+                      (int)batch, (int)rows, (int)beams, lists, one_list, length, (int)first, (int)vocab_size_padded_,
+                      (size_t)step, stream_);
 }
 
 // After sampling: stop words on the rows of this window (layers/DynamicDecodeLayer.cc:449-462; the reference
@@ -267,22 +266,24 @@ void DynamicDecodeLayer<T>::stopCriteria(TensorMap* output_tensors, TensorMap* i
                                          size_t rows, int step)
 {
     const size_t batch = input_tensors->at("logits").shape[0];
+    const size_t beams = input_tensors->at("logits").shape[1];
     if (input_tensors->isExist("stop_words_list")) {
         const Tensor& words  = input_tensors->at("stop_words_list");
         const size_t  length = words.shape[2];
         FT_CHECK_WITH_INFO(output_tensors->at("finished", Tensor()).getPtr<bool>() != nullptr,
                            "stop_words_list needs the finished output");
         check_ftk(ftk_invoke_stop_words_criterion_rows(
-            output_tensors->at("output_ids").getPtr<const int>(), nullptr,
+            output_tensors->at("output_ids").getPtr<const int>(),
+            beams > 1 ? output_tensors->at("parent_ids").getPtr<const int>() : nullptr,
             words.getPtrWithOffset<const int>(first * 2 * length),
-            output_tensors->at("finished").getPtrWithOffset<bool>(first), first, length, (int)batch, (int)rows, 1, step,
-            stream_));
+            output_tensors->at("finished").getPtrWithOffset<bool>(first * beams), first * beams, length, (int)batch,
+            (int)rows, (int)beams, step, stream_));
     }
     if (input_tensors->isExist("sequence_limit_length")) {
         invokeLengthCriterion(output_tensors->at("finished").getPtr<bool>(),
                               output_tensors->at("should_stop").getPtr<bool>(), h_pinned_finished_sum_,
-                              input_tensors->at("sequence_limit_length").getPtr<const uint32_t>(), (int)batch, 1, step,
-                              stream_);
+                              input_tensors->at("sequence_limit_length").getPtr<const uint32_t>(), (int)batch,
+                              (int)beams, step, stream_);
     }
 }
 

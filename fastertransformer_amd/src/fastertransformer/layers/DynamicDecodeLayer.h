@@ -1,7 +1,6 @@
 // Per-step decode orchestrator: bad words -> top-k / top-p sampling -> stop words -> length criterion, or, for
 // logits with more than one beam per entry, the beam-search layer and the length criterion.
 // Public surface of the reference's src/fastertransformer/layers/DynamicDecodeLayer.h:29-75.
-// Bad-word and stop-word lists are not supported together with beam search and raise an error.
 #pragma once
 #include <string>
 #include <unordered_map>

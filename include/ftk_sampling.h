@@ -157,13 +157,16 @@ int ftk_invoke_min_length_penalty(int dtype, void* logits, const int* min_length
 
 /* ---- kernels/ban_bad_words.h, kernels/stop_criteria_kernels.h ------------------------------ */
 
-/* invokeBanBadWords<T>, kernels/ban_bad_words.cu:88-120 */
+/* invokeBanBadWords<T>, kernels/ban_bad_words.cu:88-120. With beam_width > 1 the logits are
+ * [local_batch_size * beam_width, vocab_size_padded], a word list belongs to a batch entry, and a beam's history is
+ * followed back through parent_ids_buf ([max_seq_len, batch_size * beam_width], required then). */
 int ftk_invoke_ban_bad_words(int dtype, void* logits, const int* output_ids_buf, const int* parent_ids_buf,
                              int batch_size, int local_batch_size, int beam_width, const int* bad_words,
                              bool share_words, size_t bad_words_len, int id_offset, int vocab_size_padded,
                              size_t step, ftk_stream_t stream);
 
-/* invokeStopWordsCriterion, kernels/stop_criteria_kernels.cu:83-104 */
+/* invokeStopWordsCriterion, kernels/stop_criteria_kernels.cu:83-104 (with beam_width > 1: finished
+ * [batch_size * beam_width], histories followed back through parent_ids) */
 int ftk_invoke_stop_words_criterion(const int* output_ids, const int* parent_ids, const int* stop_words,
                                     bool* finished, size_t id_offset, size_t stop_words_len, int batch_size,
                                     int beam_width, int step, ftk_stream_t stream);

@@ -35,7 +35,8 @@
 //  * beam search step (topk_softmax): no reference test exists; pinned by the definition it must reduce to
 //    without hypotheses (the K largest of cum + log_softmax over all continuations, float64) and by
 //    scenario checks of the hypothesis bookkeeping written from the source description; the penalties,
-//    update and cache-indirection kernels around it by independent numpy restatements of the description.
+//    update and cache-indirection kernels around it, and the word lists with beams, by independent numpy
+//    restatements of the description.
 //  PARITY UNPINNED (no reference code or no way to run it here): the rounding order of cub's
 //  BLOCK_SCAN_RAKING prefix sums in top-p (cub is not in the reference's tree), bfloat16 storage, the frequency
 //  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), the last-ulp
@@ -706,6 +707,81 @@ static void stop_words_criterion(const int* output_ids, const int* stop_words, b
                 }
             }
             if (should) {
+                finished[row] = true;
+            }
+        }
+    }
+}
+
+// The two word-list kernels with beams (kernels/ban_bad_words.cu:22-86, kernels/stop_criteria_kernels.cu:24-81 with
+// beam_width > 1): the history of a beam is read backwards, the token of a time from the beam reached so far, then
+// that time's parent; a parent outside [0, beam_width) ends the match. `id_offset` is added as given (the layer
+// passes ite * local_batch_size, without the beam width). with_last: the n-gram includes the token written at
+// `step` (stop words) or ends one before it and bans its last token (bad words).
+static bool beam_history_matches(const int* output_ids, const int* parent_ids, const int* tokens, int count, int last,
+                                 size_t stride, size_t base, int beam, int K)
+{
+    for (int t = count - 1; t >= 0; --t) {
+        const size_t at = (size_t)(last - (count - 1) + t) * stride + base;
+        if (output_ids[at + beam] != tokens[t]) {
+            return false;
+        }
+        if (K > 1) {
+            beam = parent_ids[at + beam];
+            if (beam < 0 || beam >= K) {
+                return false;
+            }
+        }
+    }
+    return true;
+}
+
+template<int DT>
+static void ban_bad_words_beams(typename St<DT>::T* logits, const int* output_ids, const int* parent_ids,
+                                int batch_size, int local_batch_size, int K, const int* bad_words, bool share_words,
+                                int bad_words_len, int id_offset, int vocab_size_padded, int step)
+{
+    typedef St<DT> S;
+    for (int row = 0; row < local_batch_size * K; ++row) {
+        const int  b       = row / K;
+        const int* base    = share_words ? bad_words : bad_words + (size_t)b * 2 * bad_words_len;
+        const int* offsets = base + bad_words_len;
+        for (int id = 0; id < bad_words_len; ++id) {
+            if (offsets[id] < 0) {
+                continue;
+            }
+            const int start = id > 0 ? offsets[id - 1] : 0;
+            const int size  = offsets[id] - start;
+            bool      ban   = size == 1;
+            if (size > 1 && step >= size - 1) {
+                ban = beam_history_matches(output_ids, parent_ids, base + start, size - 1, step - 1,
+                                           (size_t)batch_size * K, (size_t)id_offset + (size_t)b * K, row % K, K);
+            }
+            const int tok = size >= 1 ? base[offsets[id] - 1] : 0;
+            if (ban && 0 < tok && tok < vocab_size_padded) {
+                logits[(size_t)row * vocab_size_padded + tok] = S::st(-INFINITY);
+            }
+        }
+    }
+}
+
+static void stop_words_criterion_beams(const int* output_ids, const int* parent_ids, const int* stop_words,
+                                       bool* finished, int id_offset, int stop_words_len, int batch_size, int rows,
+                                       int K, int step)
+{
+    for (int row = 0; row < rows * K; ++row) {
+        const int  b       = row / K;
+        const int* base    = stop_words + (size_t)b * 2 * stop_words_len;
+        const int* offsets = base + stop_words_len;
+        for (int id = 0; id < stop_words_len; ++id) {
+            if (offsets[id] < 0) {
+                continue;
+            }
+            const int start = id > 0 ? offsets[id - 1] : 0;
+            const int size  = offsets[id] - start;
+            if (step + 1 >= size
+                && beam_history_matches(output_ids, parent_ids, base + start, size, step, (size_t)batch_size * K,
+                                        (size_t)id_offset + (size_t)b * K, row % K, K)) {
                 finished[row] = true;
             }
         }
@@ -1786,6 +1862,25 @@ void oracle_update_indir_cache(int* tgt, const int* src, const int* beam_ids, co
                                int local_batch_size, int beam_width, int max_seq_len, int step)
 {
     update_indir_cache(tgt, src, beam_ids, finished, local_batch_size, beam_width, max_seq_len, step);
+}
+
+
+int oracle_ban_bad_words_beams(int dtype, void* logits, const int* output_ids, const int* parent_ids, int batch_size,
+                               int local_batch_size, int beam_width, const int* bad_words, int share_words,
+                               int bad_words_len, int id_offset, int vocab_size_padded, int step)
+{
+    DISPATCH(dtype, ban_bad_words_beams<DT>((St<DT>::T*)logits, output_ids, parent_ids, batch_size, local_batch_size,
+                                            beam_width, bad_words, share_words != 0, bad_words_len, id_offset,
+                                            vocab_size_padded, step));
+    return 0;
+}
+
+void oracle_stop_words_criterion_beams(const int* output_ids, const int* parent_ids, const int* stop_words,
+                                       bool* finished, int id_offset, int stop_words_len, int batch_size, int rows,
+                                       int beam_width, int step)
+{
+    stop_words_criterion_beams(output_ids, parent_ids, stop_words, finished, id_offset, stop_words_len, batch_size,
+                               rows, beam_width, step);
 }
 
 }  // extern "C"

@@ -382,3 +382,21 @@ def update_indir_cache(tgt, src, beam_ids, finished, local_batch, beam_width, ma
     fn.argtypes = [C.c_void_p] * 4 + [C.c_int] * 4
     fn(_p(tgt), _p(src), _p(beam_ids), _p(finished), local_batch, beam_width, max_seq_len, step)
 
+
+def ban_bad_words_beams(dt, logits, output_ids, parent_ids, batch, local_batch, beam_width, bad_words, share_words,
+                        bad_words_len, id_offset, Vp, step):
+    fn = lib().oracle_ban_bad_words_beams
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_int] + [C.c_void_p] * 3 + [C.c_int] * 3 + [C.c_void_p] + [C.c_int] * 5
+    return fn(dt, _p(logits), _p(output_ids), _p(parent_ids), batch, local_batch, beam_width, _p(bad_words),
+              int(share_words), bad_words_len, id_offset, Vp, step)
+
+
+def stop_words_criterion_beams(output_ids, parent_ids, stop_words, finished, id_offset, stop_words_len, batch, rows,
+                               beam_width, step):
+    fn = lib().oracle_stop_words_criterion_beams
+    fn.restype = None
+    fn.argtypes = [C.c_void_p] * 4 + [C.c_int] * 6
+    fn(_p(output_ids), _p(parent_ids), _p(stop_words), _p(finished), id_offset, stop_words_len, batch, rows,
+       beam_width, step)
+

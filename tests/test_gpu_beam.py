@@ -363,6 +363,12 @@ def test_dynamic_decode_layer_with_beams(windows):
         step = max_input + i
         x = (rng.standard_normal((rows, Vp)) * 3).astype(np.float32)
         d_x = to_torch(x).reshape(batch, K, Vp)
+        # word lists ride along in the one-window variant (with several windows the reference offsets the bad-word
+        # launch by entries, not by beams)
+        bad = stop = None
+        if windows == 1 and step >= 2:
+            bad = _beam_word_lists(rng, batch, K, V, 6, 3, 24, out_ids, parents, step, with_last=False)
+            O.ban_bad_words_beams(dt, x, out_ids, parents, batch, batch, K, bad, False, 24, 0, Vp, step)
         for ite in range(windows):
             lo, hi = ite * local * K, (ite + 1) * local * K
             want = x[lo:hi].copy()
@@ -384,6 +390,11 @@ def test_dynamic_decode_layer_with_beams(windows):
             outs = {"output_ids": d["out_ids"], "finished": d["finished"], "cum_log_probs": d["cum"],
                     "parent_ids": d["parents"], "sequence_length": d["seq"], "tgt_cache_indirection": d_src[1],
                     "should_stop": should_stop}
+            if bad is not None:
+                # stop words: some of them end with what a beam has just chosen (known from the oracle's step)
+                stop = _beam_word_lists(rng, batch, K, V, 4, 2, 16, out_ids, parents, step, with_last=True)
+                O.stop_words_criterion_beams(out_ids, parents, stop, finished, 0, 16, batch, batch, K, step)
+                ins["bad_words_list"], ins["stop_words_list"] = to_torch(bad), to_torch(stop)
             print("dynamic decode with beams", windows, step, ite, flush=True)
             layer.forward(outs, ins)
             torch.cuda.synchronize()
@@ -398,6 +409,68 @@ def test_dynamic_decode_layer_with_beams(windows):
         src.reverse()
         d_src.reverse()
     assert finished.all() and should_stop[0]
-    with pytest.raises(fa.FtkError):
-        layer.forward(outs, dict(ins, bad_words_list=torch.zeros((2, 4), dtype=torch.int32, device="cuda")))
+
+
+def _beam_word_lists(rng, batch, K, V, n_words, max_len, L, out_ids, parents, step, with_last):
+    """[batch, 2, L] word lists; about half of the words are copied from the history of a beam of their entry,
+    followed back through the parent beams (ending at `step` when with_last, one before it otherwise, where a random
+    last token is appended), so that they match"""
+    lists = np.zeros((batch, 2, L), np.int32)
+    lists[:, 1, :] = -1
+    for b in range(batch):
+        flat, ends = [], []
+        for w in range(n_words):
+            n = int(rng.integers(1, max_len + 1))
+            take = n if with_last else n - 1
+            last = step if with_last else step - 1
+            if rng.random() < 0.5 and take <= last + 1:
+                beam, toks = int(rng.integers(0, K)), []
+                for t in range(last, last - take, -1):
+                    toks.append(int(out_ids[t, b * K + beam]))
+                    beam = int(parents[t, b * K + beam])
+                word = toks[::-1] + ([] if with_last else [int(rng.integers(1, V))])
+            else:
+                word = [int(x) for x in rng.integers(1, V, n)]
+            flat += word
+            ends.append(len(flat))
+        lists[b, 0, :len(flat)] = flat
+        lists[b, 1, :len(ends)] = ends
+    return lists
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_word_lists_with_beams(dt):
+    """ftk_invoke_ban_bad_words and ftk_invoke_stop_words_criterion with beam_width > 1 against the oracle: words
+    that match a beam's history through its parent beams, words that do not, shared and per-entry lists, a parent
+    outside the beam range (ends the match)"""
+    import torch
+    ops, lib = _lib()
+    rng = np.random.default_rng(77 + dt)
+    for batch, K, V, step, L in ((3, 4, 300, 6, 40), (2, 8, 1000, 3, 24), (5, 2, 50, 9, 64)):
+        rows = batch * K
+        out_ids = rng.integers(1, V, (step + 2, rows)).astype(np.int32)
+        parents = rng.integers(0, K, (step + 2, rows)).astype(np.int32)
+        parents[step - 1, 0] = K + 3     # a broken chain for whoever walks through it
+        for share in (False, True):
+            bad = _beam_word_lists(rng, batch, K, V, 8, 4, L, out_ids, parents, step, with_last=False)
+            words = bad[0] if share else bad
+            x = O.to_storage(rng.standard_normal((rows, V)).astype(np.float32), dt)
+            want = x.copy()
+            O.ban_bad_words_beams(dt, want, out_ids, parents, batch, batch, K, np.ascontiguousarray(words), share, L, 0, V,
+                                  step)
+            d_x, d_ids, d_par, d_w = to_torch(x, dt), to_torch(out_ids), to_torch(parents), to_torch(np.ascontiguousarray(words))
+            ops.check(lib.ftk_invoke_ban_bad_words(dt, d_x.data_ptr(), d_ids.data_ptr(), d_par.data_ptr(), batch, batch,
+                                                   K, d_w.data_ptr(), share, L, 0, V, step, ops.current_stream()))
+            torch.cuda.synchronize()
+            got = np.asarray(to_numpy(d_x))
+            assert np.array_equal(got.view(np.uint8), np.asarray(want).view(np.uint8))
+            assert np.isinf(O.to_f32(want, dt)).sum() > 0          # something was banned
+        stop = _beam_word_lists(rng, batch, K, V, 6, 3, L, out_ids, parents, step, with_last=True)
+        fin = np.zeros(rows, np.bool_)
+        O.stop_words_criterion_beams(out_ids, parents, stop, fin, 0, L, batch, batch, K, step)
+        d_fin, d_stop = to_torch(np.zeros(rows, np.bool_)), to_torch(stop)
+        ops.check(lib.ftk_invoke_stop_words_criterion(d_ids.data_ptr(), d_par.data_ptr(), d_stop.data_ptr(),
+                                                      d_fin.data_ptr(), 0, L, batch, K, step, ops.current_stream()))
+        torch.cuda.synchronize()
+        assert np.array_equal(to_numpy(d_fin), fin) and fin.any()
 

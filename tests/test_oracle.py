@@ -962,3 +962,61 @@ def test_beam_update_and_cache_indirection_against_the_description():
     O.update_indir_cache(tgt2, src, parent, np.zeros(batch * K, bool), batch, K, L, L + 3)
     assert (tgt2 != -7).all() and all(tgt2[b, k, (L + 3) % L] == k for b in range(batch) for k in range(K))
 
+
+def test_word_lists_with_beams_against_the_description():
+    """bad words and stop words with beam_width > 1: a word matches a beam when the beam's own history, read backwards
+    through the parent beams, ends with it (bad words: with all but its last token, one step earlier); restated here
+    by building every beam's history first and comparing lists"""
+    rng = np.random.default_rng(31)
+    batch, K, V, step, L = 3, 4, 30, 6, 48
+    rows = batch * K
+    out_ids = rng.integers(1, V, (step + 1, rows)).astype(np.int32)
+    parents = rng.integers(0, K, (step + 1, rows)).astype(np.int32)
+
+    def history(row, last, n):
+        """the n tokens ending at time `last` of the beam `row`, oldest first; None if the chain leaves the beams"""
+        b, beam, toks = row // K, row % K, []
+        for t in range(last, last - n, -1):
+            toks.append(int(out_ids[t, b * K + beam]))
+            beam = int(parents[t, b * K + beam])
+            if not 0 <= beam < K:
+                return None
+        return toks[::-1]
+
+    lists = np.zeros((batch, 2, L), np.int32)
+    lists[:, 1, :] = -1
+    words = {}
+    for b in range(batch):
+        flat, ends, words[b] = [], [], []
+        for w in range(10):
+            n = int(rng.integers(1, 4))
+            if rng.random() < 0.6:
+                word = history(b * K + int(rng.integers(0, K)), step - 1, n - 1) + [int(rng.integers(1, V))]
+            else:
+                word = [int(x) for x in rng.integers(1, V, n)]
+            words[b].append(word)
+            flat += word
+            ends.append(len(flat))
+        lists[b, 0, :len(flat)], lists[b, 1, :len(ends)] = flat, ends
+    x = np.zeros((rows, V), np.float32)
+    O.ban_bad_words_beams(O.F32, x, out_ids, parents, batch, batch, K, lists, False, L, 0, V, step)
+    for r in range(rows):
+        banned = {w[-1] for w in words[r // K] if len(w) == 1 or history(r, step - 1, len(w) - 1) == w[:-1]}
+        assert set(np.nonzero(np.isinf(x[r]))[0].tolist()) == banned, r
+    # stop words: the same lists, now matched including the token of `step`
+    fin = np.zeros(rows, np.bool_)
+    stop = lists.copy()
+    for b in range(batch):      # make some of them end with what a beam just wrote
+        w0 = history(b * K + 1, step, 2)
+        stop[b, 0, :2], stop[b, 1, 0] = w0, 2
+        words[b][0] = w0
+        rest = [w for w in words[b][1:]]
+        flat = w0 + [t for w in rest for t in w]
+        stop[b, 0, :len(flat)] = flat
+        stop[b, 1, :len(words[b])] = np.cumsum([len(w) for w in words[b]])
+    O.stop_words_criterion_beams(out_ids, parents, stop, fin, 0, L, batch, batch, K, step)
+    for r in range(rows):
+        want = any(history(r, step, len(w)) == w for w in words[r // K])
+        assert fin[r] == want, r
+    assert fin.any()
+
