@@ -258,7 +258,23 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     typedef typename S::T T;
     // a thread's load: LP_CHAINS neighbouring columns
     typedef typename std::conditional<sizeof(T) == 4, uint4, uint2>::type Chunk;
-    __shared__ TopkShared s;
+    // The row's history bitmap lives in LDS that nothing else uses while the row streams: the ordered-list area
+    // of the select phase holds its first words, an array behind the select state the rest (four workgroups then
+    // fit a compute unit even with the window of the largest vocabularies). Both are addressed as words of one
+    // object, so that the choice between them is a choice between two uniform offsets.
+    constexpr int LP_BM_OVERLAY = (int)(sizeof(TopkShared::sel) / sizeof(uint32_t));
+    constexpr int LP_BM_TAIL    = BMW > LP_BM_OVERLAY ? BMW - LP_BM_OVERLAY : 1;
+    struct LpShared {
+        TopkShared s;
+        uint32_t   bitmap_tail[LP_BM_TAIL];
+    };
+    static_assert(sizeof(TopkShared) % sizeof(uint32_t) == 0 && offsetof(LpShared, bitmap_tail) == sizeof(TopkShared),
+                  "the tail follows the select state word for word");
+    static_assert(LP_BM_OVERLAY % (LP_BLOCK / 32) == 0, "a round's bitmap words lie on one side of the seam");
+    constexpr int LP_BM_HEAD_AT = (int)(offsetof(TopkShared, sel) / sizeof(uint32_t));
+    constexpr int LP_BM_TAIL_AT = (int)(sizeof(TopkShared) / sizeof(uint32_t)) - LP_BM_OVERLAY;
+    __shared__ LpShared   sh;
+    TopkShared&           s = sh.s;
     __shared__ uint32_t   slot_key[2][LP_THREADS];
     __shared__ float      warp_sum[32];
     const int             t   = threadIdx.x;
@@ -277,12 +293,19 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
             hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
         }
     }
-    Chunk raw[LP_RING];
-    auto  load = [&](int slot, int n) {
-        // the last round may reach past the row: such a thread reads its chunk of the round before (never used).
-        // Rows are 16-byte aligned, so a chunk that starts inside the padded row lies inside it.
-        const int col = n * LP_BLOCK + t * LP_CHAINS;
-        raw[slot]     = base[(col < p.Vp ? col : col - LP_BLOCK) / LP_CHAINS];
+    Chunk        raw[LP_RING];
+    const int    tcol  = t * LP_CHAINS;  // the thread's first column within a round
+    const Chunk* tbase = base + t;
+    // the last round may reach past the row: such a thread reads its chunk of the round before (never used).
+    // Rows are 16-byte aligned, so a chunk that starts inside the padded row lies inside it.
+    const bool last_inside = (rounds - 1) * LP_BLOCK + tcol < p.Vp;
+    auto       load        = [&](int slot, int n) {
+        if (n + 1 < rounds) {  // uniform: the round's offset stays in scalar registers
+            raw[slot] = tbase[(size_t)n * LP_THREADS];
+        }
+        else {
+            raw[slot] = tbase[(size_t)(last_inside ? n : n - 1) * LP_THREADS];
+        }
     };
 #pragma unroll
     for (int r = 0; r < LP_RING; ++r) {
@@ -323,20 +346,18 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
         s.n_cand  = 0;
         s.misc[0] = draw_bits;
     }
-    constexpr int LP_BM_OVERLAY = (int)(sizeof(s.sel) / sizeof(uint32_t));
-    constexpr int LP_BM_TAIL    = BMW > LP_BM_OVERLAY ? BMW - LP_BM_OVERLAY : 1;
-    __shared__ uint32_t bitmap_tail[LP_BM_TAIL];
+    uint32_t* const lds_words = reinterpret_cast<uint32_t*>(&sh);
+    auto            bitmap_at = [&](int w) { return (w < LP_BM_OVERLAY ? LP_BM_HEAD_AT : LP_BM_TAIL_AT) + w; };
     if (hist) {
-        uint32_t* head_words = reinterpret_cast<uint32_t*>(&s.sel);
-        const int words      = min(BMW, (p.V + 31) / 32 + 1);
+        const int words = min(BMW, (p.V + 31) / 32 + 1);
         for (int i = t; i < words; i += LP_THREADS) {
-            (i < LP_BM_OVERLAY ? head_words[i] : bitmap_tail[i - LP_BM_OVERLAY]) = 0u;
+            lds_words[bitmap_at(i)] = 0u;
         }
         lds_barrier();
         auto mark = [&](int pos, int id) {
             if (id >= 0 && id < p.V && rowctx.history_position_counts(pos)) {
                 const int w = id >> 5;
-                atomicOr(w < LP_BM_OVERLAY ? &head_words[w] : &bitmap_tail[w - LP_BM_OVERLAY], 1u << (id & 31));
+                atomicOr(&lds_words[bitmap_at(w)], 1u << (id & 31));
             }
         };
 #pragma unroll
@@ -352,23 +373,16 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     const bool  bitsv = hist || rowctx.has_vector_bits();
     const uint32_t KMIN = min_valid_key<DT>();
 
-    // The row's history bitmap lives in LDS that nothing else uses while the row streams: the ordered-list area
-    // of the select phase holds its first words, a small array of its own the rest (four workgroups then fit a
-    // compute unit even with the window of the largest vocabularies).
-    auto bitmap_word = [&](int w) -> uint32_t {
-        if constexpr (BMW > 0) {
-            return w < LP_BM_OVERLAY ? reinterpret_cast<const uint32_t*>(&s.sel)[w] : bitmap_tail[w - LP_BM_OVERLAY];
-        }
-        else {
-            return rowctx.bm_word(w);
-        }
-    };
-    // e values of the LP_CHAINS columns a chunk holds (first column `col`); columns >= V give 0
-    auto e_values = [&](const Chunk& v, int col, float* e) {
-        uint32_t bits = 0u;
+    // e values of the LP_CHAINS columns of round n that a chunk holds; columns >= V give 0. What depends on the
+    // round alone (the side of the bitmap seam, whether the round holds the masked end id or the end of the
+    // vocabulary) is decided in scalar registers.
+    auto e_values = [&](const Chunk& v, int n, float* e) {
+        const int col  = n * LP_BLOCK + tcol;
+        uint32_t  bits = 0u;
         if (bitsv) {
-            if (BMW > 0) {
-                bits = (bitmap_word(col >> 5) >> (col & 31)) & ((1u << LP_CHAINS) - 1u);
+            if constexpr (BMW > 0) {
+                const int at = (n < LP_BM_OVERLAY / (LP_BLOCK / 32) ? LP_BM_HEAD_AT : LP_BM_TAIL_AT) + n * (LP_BLOCK / 32);
+                bits         = (lds_words[at + (tcol >> 5)] >> (tcol & 31)) & ((1u << LP_CHAINS) - 1u);
             }
             else {
                 bits = rowctx.vector_bits(col, LP_CHAINS);
@@ -380,8 +394,14 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
             y[c] = rowctx.fast(lp_chunk_element<DT>(v, c));
         }
         // rare: a column of the history, the masked end id, the end of the vocabulary
-        const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - col);
-        if (bits != 0u || rel_end < (uint32_t)LP_CHAINS || col + LP_CHAINS > p.V) {
+        const bool     tail_round = (n + 1) * LP_BLOCK > p.V;
+        const bool     end_round  = (uint32_t)(rowctx.masked_end_id - n * LP_BLOCK) < (uint32_t)LP_BLOCK;
+        const uint32_t rel_end    = (uint32_t)(rowctx.masked_end_id - col);
+        bool           rare       = bits != 0u;
+        if (tail_round || end_round) {
+            rare = rare || rel_end < (uint32_t)LP_CHAINS || col + LP_CHAINS > p.V;
+        }
+        if (rare) {
 #pragma unroll
             for (int c = 0; c < LP_CHAINS; ++c) {
                 if ((bits >> c) & 1u) {
@@ -392,11 +412,25 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                 }
             }
         }
+        float d[LP_CHAINS];
 #pragma unroll
         for (int c = 0; c < LP_CHAINS; ++c) {
-            e[c] = round_t<DT>(det_expf_nonpos(y[c] - row_max));
+            d[c] = y[c] - row_max;
         }
-        if (col + LP_CHAINS > p.V) {
+        // one look for a NaN per chunk instead of one per column
+        if (__builtin_isunordered(d[0], d[1]) || __builtin_isunordered(d[2], d[3])) {
+#pragma unroll
+            for (int c = 0; c < LP_CHAINS; ++c) {
+                e[c] = round_t<DT>(det_expf_nonpos(d[c]));
+            }
+        }
+        else {
+#pragma unroll
+            for (int c = 0; c < LP_CHAINS; ++c) {
+                e[c] = round_t<DT>(det_expf_nonpos_number(d[c]));
+            }
+        }
+        if (tail_round && col + LP_CHAINS > p.V) {
 #pragma unroll
             for (int c = 0; c < LP_CHAINS; ++c) {
                 e[c] = col + c < p.V ? e[c] : 0.0f;  // (what lies behind the vocabulary adds nothing)
@@ -443,7 +477,7 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
 #pragma unroll
         for (int n = 0; n < LP_HEAD; ++n) {
             if (n < head) {
-                e_values(raw[n], n * LP_BLOCK + t * LP_CHAINS, head_e[n]);
+                e_values(raw[n], n, head_e[n]);
 #pragma unroll
                 for (int c = 0; c < LP_CHAINS; ++c) {
                     acc[c] = acc[c] + head_e[n][c];
@@ -479,12 +513,18 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                 const int slot = (LP_HEAD + r) % LP_RING;
                 float     e[LP_CHAINS];
                 const int col0 = n * LP_BLOCK + t * LP_CHAINS;
-                e_values(raw[slot], col0, e);
+                e_values(raw[slot], n, e);
 #pragma unroll
                 for (int c = 0; c < LP_CHAINS; ++c) {
                     acc[c] = acc[c] + e[c];
-                    if (e[c] >= thr_low && col0 + c < p.V) {
-                        push(e[c], col0 + c);
+                }
+                // one look per chunk for a candidate (a NaN is none, with or without the maximum)
+                if (__builtin_fmaxf(__builtin_fmaxf(e[0], e[1]), __builtin_fmaxf(e[2], e[3])) >= thr_low) {
+#pragma unroll
+                    for (int c = 0; c < LP_CHAINS; ++c) {
+                        if (e[c] >= thr_low && col0 + c < p.V) {
+                            push(e[c], col0 + c);
+                        }
                     }
                 }
                 if (n + LP_RING < rounds) {

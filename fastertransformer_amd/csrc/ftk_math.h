@@ -90,13 +90,12 @@ FTK_HD float det_expf(float x)
 // det_expf for arguments that are never positive (x <= 0 or NaN), as in exp(y - max): the same value bit for
 // bit, without the range checks. Below -104 the scaled result is under half of the smallest subnormal and rounds
 // to zero like det_expf's cut-off at -103.97 (between the two, 2^-150 times a factor below one does too); the
-// clamp keeps -inf out of the argument reduction and lets a NaN through.
-FTK_HD float det_expf_nonpos(float x)
+// clamp keeps -inf out of the argument reduction; it would also turn a NaN into a number, hence the two forms.
+FTK_HD float det_expf_nonpos_number(float x)  // x is not a NaN (a NaN would come out as a number)
 {
-    const float x0 = x;
-    x              = __builtin_fmaxf(x, -104.0f);  // one instruction on the device; a NaN leaves as -104, see below
-    const float n  = __builtin_rintf(x * 1.44269502162933349609375f);
-    float       r  = fma_rn(n, -0.693145751953125f, x);
+    x             = __builtin_fmaxf(x, -104.0f);  // one instruction on the device
+    const float n = __builtin_rintf(x * 1.44269502162933349609375f);
+    float       r = fma_rn(n, -0.693145751953125f, x);
     r             = fma_rn(n, -1.428606765330187045e-06f, r);
     float p       = 1.9875691500e-4f;
     p             = fma_rn(p, r, 1.3981999507e-3f);
@@ -106,10 +105,7 @@ FTK_HD float det_expf_nonpos(float x)
     p             = fma_rn(p, r, 5.0000001201e-1f);
     const float z = r * r;
     float       y = fma_rn(p, z, r) + 1.0f;
-    if (x0 != x0) {
-        return x0;
-    }
-    const int ni = (int)n;
+    const int   ni = (int)n;
 #if defined(__HIP_DEVICE_COMPILE__)
     return __builtin_ldexpf(y, ni);
 #else
@@ -119,6 +115,11 @@ FTK_HD float det_expf_nonpos(float x)
     y            = y * u2f((uint32_t)(n2 + 127) << 23);
     return y;
 #endif
+}
+FTK_HD float det_expf_nonpos(float x)
+{
+    const float y = det_expf_nonpos_number(x);  // the clamp inside drops a NaN: it is put back here
+    return x != x ? x : y;
 }
 
 // Cephes logf: x = m 2^e, m in [sqrt(1/2), sqrt 2), f = m - 1, log x = f - f^2/2 + f^3 P(f) + e ln2.
