@@ -204,7 +204,9 @@ void DynamicDecodeLayer<T>::forwardBeams(TensorMap* output_tensors, TensorMap* i
                          {"end_id", rowWindow(input_tensors->at("end_id"), first_entry, group)},
                          {"ite", Tensor{MEMORY_CPU, TYPE_UINT32, {1}, &sub}}});
         if (input_tensors->isExist("input_lengths")) {
-            in.insert({"input_lengths", rowWindow(input_tensors->at("input_lengths"), first_entry, group)});
+            // [batch, beam_width], or the same values as one flat list: one length per beam either way
+            const Tensor& t = input_tensors->at("input_lengths");
+            in.insert({"input_lengths", Tensor{t.where, t.type, {group, beams}, t.getPtrWithOffset(first_beam)}});
         }
         for (auto it = input_tensors->begin(); it != input_tensors->end(); ++it) {
             // step, max_input_length, embedding_bias, src_cache_indirection and the runtime values of the step

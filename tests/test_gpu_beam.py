@@ -243,13 +243,32 @@ def test_online_beam_search_layer_decode_loop(dt, penalty):
     """OnlineBeamSearchLayer::forward step after step (penalties over beam histories, the step, the update of the
     beams, the cache indirection, hypotheses collected on the way) against the same sequence of oracle calls: ids,
     parents, flags, lengths, hypotheses and cache indirection bit for bit, log-probs within tolerance."""
+    rng = np.random.default_rng(200 + dt + (0 if penalty is None else len(penalty)))
+    collected = _decode_loop_case(rng, dt, penalty, batch=3, K=4, V=997, Vp=1000, max_input=3, L=12, steps=7,
+                                  temperature=0.8, diversity=0.1, len_pen=0.7, min_length=2)
+    assert collected > 0   # the loop did collect hypotheses
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 64, 64, 1, 6, 5), (2, 8, 2051, 2056, 4, 16, 9), (5, 3, 333, 336, 2, 9, 6),
+                                   (2, 16, 4099, 4104, 2, 8, 5)], ids=lambda s: "b%d_k%d_v%d" % s[:3])
+def test_online_beam_search_layer_decode_loop_shapes(shape):
+    """The same loop at other batch sizes, beam widths and vocabularies, with and without length penalty and
+    diversity rate."""
+    batch, K, V, Vp, max_input, L, steps = shape
+    rng = np.random.default_rng(260 + K)
+    for dt, penalty, diversity, len_pen in ((O.F32, "repetition_penalty", 0.0, 0.0), (O.F16, None, 0.3, 1.0),
+                                            (O.BF16, "presence_penalty", 0.05, 0.4)):
+        _decode_loop_case(rng, dt, penalty, batch=batch, K=K, V=V, Vp=Vp, max_input=max_input, L=L, steps=steps,
+                          temperature=float(rng.choice([1.0, 0.7, 1.3])), diversity=diversity, len_pen=len_pen,
+                          min_length=int(rng.integers(0, 4)))
+
+
+def _decode_loop_case(rng, dt, penalty, batch, K, V, Vp, max_input, L, steps, temperature, diversity, len_pen,
+                      min_length):
     import torch
     import fastertransformer_amd as fa
     from fastertransformer_amd import ops
-    rng = np.random.default_rng(200 + dt + (0 if penalty is None else len(penalty)))
-    batch, K, V, Vp, max_input, L, steps = 3, 4, 997, 1000, 3, 12, 7
     rows = batch * K
-    temperature, diversity, len_pen, min_length = 0.8, 0.1, 0.7, 2
     pen_val = {"repetition_penalty": 1.2, "presence_penalty": 0.4, None: None}[penalty]
     ptype = {"repetition_penalty": 1, "presence_penalty": 0, None: 2}[penalty]
     end_ids = rng.integers(0, V, batch).astype(np.int32)
@@ -327,14 +346,17 @@ def test_online_beam_search_layer_decode_loop(dt, penalty):
             np.testing.assert_allclose(to_numpy(d_h[name]), hyps[name], rtol=rtol, atol=atol, err_msg=name)
         cache.reverse()
         d_cache.reverse()
-    assert hyps["num_beams"].sum() > 0   # the loop did collect hypotheses
     layer.close()
+    return int(hyps["num_beams"].sum())
 
 
+@pytest.mark.parametrize("differing", [False, True], ids=["same_runtime_values", "differing_runtime_values"])
 @pytest.mark.parametrize("windows", [1, 2], ids=["one_window", "two_windows"])
-def test_dynamic_decode_layer_with_beams(windows):
+def test_dynamic_decode_layer_with_beams(windows, differing):
     """DynamicDecodeLayer::forward on logits [batch, beam_width > 1, vocab]: the beam-search layer per window of the
-    batch and the length criterion, against the same oracle calls; bad-word lists are refused with beams."""
+    batch and the length criterion, against the same oracle calls, with word lists in the one-window variant. When
+    setup() saw per-entry runtime values that differ, the entries go to the beam-search layer one by one, each call
+    reading the first value of every list (layers/DynamicDecodeLayer.cc:289-294, BaseBeamSearchLayer.cu:220)."""
     import torch
     import fastertransformer_amd as fa
     from fastertransformer_amd import ops
@@ -357,7 +379,9 @@ def test_dynamic_decode_layer_with_beams(windows):
     src = [rng.integers(0, K, (local, K, L)).astype(np.int32), np.zeros((local, K, L), np.int32)]
     d_src = [to_torch(c) for c in src]
     layer = fa.DynamicDecodeLayer(dt, V, Vp)
-    layer.setup(batch, K, {"temperature": np.array([0.9], np.float32)})
+    temperatures = np.array([0.9, 1.3, 0.9, 0.6] if differing else [0.9], np.float32)
+    layer.setup(batch, K, {"temperature": temperatures})
+    group = 1 if differing else local     # entries per call of the beam-search layer
     should_stop = np.zeros(1, np.bool_)
     for i in range(steps):
         step = max_input + i
@@ -370,23 +394,26 @@ def test_dynamic_decode_layer_with_beams(windows):
             bad = _beam_word_lists(rng, batch, K, V, 6, 3, 24, out_ids, parents, step, with_last=False)
             O.ban_bad_words_beams(dt, x, out_ids, parents, batch, batch, K, bad, False, 24, 0, Vp, step)
         for ite in range(windows):
-            lo, hi = ite * local * K, (ite + 1) * local * K
-            want = x[lo:hi].copy()
-            O.beam_add_bias_apply_penalties(dt, step, want, out_ids[step - 1, lo:hi].copy(), out_ids, parents, None,
-                                            seq[lo:hi], None, ite, max_input, local, batch, K, V, Vp,
-                                            end_ids[ite * local:(ite + 1) * local], 0.9, 1.0, 2, 0)
-            ids_w, cum_w, fin_w, seq_w = out_ids[step, lo:hi].copy(), cum[lo:hi].copy(), finished[lo:hi].copy(), seq[lo:hi].copy()
-            assert O.topk_softmax(dt, want, None, fin_w, seq_w, cum_w, None, ids_w, None, local, K, Vp,
-                                  end_ids[ite * local:(ite + 1) * local], 0.0, 0.0) == 0
-            par_w = np.zeros(local * K, np.int32)
-            O.beam_update(fin_w, par_w, seq_w, ids_w, ids_w, None, ite, local, K, Vp, end_ids[ite * local:(ite + 1) * local])
-            O.update_indir_cache(src[1], src[0], par_w, fin_w, local, K, L, step)
-            out_ids[step, lo:hi], parents[step, lo:hi] = ids_w, par_w
-            cum[lo:hi], finished[lo:hi], seq[lo:hi] = cum_w, fin_w, seq_w
+            for sub in range(ite * local // group, (ite + 1) * local // group):
+                lo, hi = sub * group * K, (sub + 1) * group * K
+                ends = end_ids[sub * group:(sub + 1) * group]
+                want = x[lo:hi].copy()
+                O.beam_add_bias_apply_penalties(dt, step, want, out_ids[step - 1, lo:hi].copy(), out_ids, parents, None,
+                                                seq[lo:hi], None, sub, max_input, group, batch, K, V, Vp, ends, 0.9, 1.0,
+                                                2, 0)
+                ids_w, cum_w, fin_w, seq_w = (out_ids[step, lo:hi].copy(), cum[lo:hi].copy(), finished[lo:hi].copy(),
+                                              seq[lo:hi].copy())
+                assert O.topk_softmax(dt, want, None, fin_w, seq_w, cum_w, None, ids_w, None, group, K, Vp, ends, 0.0,
+                                      0.0) == 0
+                par_w = np.zeros(group * K, np.int32)
+                O.beam_update(fin_w, par_w, seq_w, ids_w, ids_w, None, sub, group, K, Vp, ends)
+                O.update_indir_cache(src[1], src[0], par_w, fin_w, group, K, L, step)
+                out_ids[step, lo:hi], parents[step, lo:hi] = ids_w, par_w
+                cum[lo:hi], finished[lo:hi], seq[lo:hi] = cum_w, fin_w, seq_w
             ins = {"logits": d_x, "step": np.array([step], np.int32), "max_input_length": np.array([max_input], np.int32),
                    "ite": np.array([ite], np.uint32), "local_batch_size": np.array([local], np.int32),
                    "end_id": d["end_ids"], "src_cache_indirection": d_src[0],
-                   "temperature": np.array([0.9], np.float32), "sequence_limit_length": d["limit"]}
+                   "temperature": temperatures, "sequence_limit_length": d["limit"]}
             outs = {"output_ids": d["out_ids"], "finished": d["finished"], "cum_log_probs": d["cum"],
                     "parent_ids": d["parents"], "sequence_length": d["seq"], "tgt_cache_indirection": d_src[1],
                     "should_stop": should_stop}
