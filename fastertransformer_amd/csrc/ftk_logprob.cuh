@@ -57,10 +57,15 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
     const int             t     = threadIdx.x;
     const int             row   = blockIdx.y;
     const int             chunk = blockIdx.x;
-    const T*              rowp  = (const T*)p.logits + (size_t)row * p.Vp;  // 16-byte aligned (host check)
-    const uint4*          base  = reinterpret_cast<const uint4*>(rowp);
-    const int             vhi   = p.V / EPV;  // whole vectors below column V
-    const int             vb    = min(vhi, chunk * l.subs_per_wg * LG_SUB_VECS);
+    // Rows may start anywhere: the 16-byte vectors are those of the memory, `a` columns of the first one lie in
+    // front of the row. Vectors [vlo, vhi) lie inside columns [0, V); the first and the last workgroup of a row
+    // look at the few columns in front of and behind them one by one.
+    const T*              rowp  = (const T*)p.logits + (size_t)row * p.Vp;
+    const int             a     = (int)(((uintptr_t)rowp & 15u) / sizeof(T));
+    const uint4*          base  = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(rowp) - a * sizeof(T));
+    const int             vlo   = (a + EPV - 1) / EPV;
+    const int             vhi   = max(vlo, (a + p.V) / EPV);
+    const int             vb    = min(vhi, vlo + chunk * l.subs_per_wg * LG_SUB_VECS);
     const int             ve    = min(vhi, vb + l.subs_per_wg * LG_SUB_VECS);
     const int             nvec  = ve - vb;
     const int             nsub  = (nvec + LG_SUB_VECS - 1) / LG_SUB_VECS;
@@ -94,9 +99,10 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
     if (skip || fin) {
         return;
     }
-    const bool last_wg = chunk == (int)gridDim.x - 1;
-    const int  lo_col  = vb * EPV;
-    const int  hi_col  = last_wg ? p.V : ve * EPV;
+    const bool first_wg = chunk == 0;
+    const bool last_wg  = chunk == (int)gridDim.x - 1;
+    const int  lo_col   = first_wg ? 0 : vb * EPV - a;
+    const int  hi_col   = last_wg ? p.V : ve * EPV - a;
     if (hist) {
         uint32_t* window = fused_lds_bitmap<FusedRow<DT, BMW>::LDS_WORDS>();
         const int origin = lo_col & ~31;
@@ -131,7 +137,7 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
     auto vector_max = [&](const uint4& v, int first) -> float {
         uint32_t bits = 0u;
         if (bitsv) {
-            if (BMW > 0) {
+            if (BMW > 0 && a == 0) {  // the flags of a vector never straddle a word of the bitmap
                 const int rel = first - rowctx.bm_origin;
                 bits          = (rowctx.bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
             }
@@ -165,7 +171,7 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
 #pragma unroll
                 for (int j = 0; j < LG_NV; ++j) {
                     const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
-                    const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV);
+                    const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV - a);
                     m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
                 }
                 if (q + R < nsub) {
@@ -174,9 +180,15 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
             }
         }
     }
+    if (first_wg) {
+        // the columns in front of the first whole vector
+        for (int v = t; v < min(p.V, vlo * EPV - a); v += LG_THREADS) {
+            m = __builtin_fmaxf(m, topk_value_at<DT>(rowctx, v));
+        }
+    }
     if (last_wg) {
         // the columns behind the last whole vector
-        for (int v = vhi * EPV + t; v < p.V; v += LG_THREADS) {
+        for (int v = vhi * EPV - a + t; v < p.V; v += LG_THREADS) {
             m = __builtin_fmaxf(m, topk_value_at<DT>(rowctx, v));
         }
     }
@@ -279,9 +291,14 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     __shared__ float      warp_sum[32];
     const int             t   = threadIdx.x;
     const int             row = blockIdx.x;
+    // Rows may start anywhere: the chunks are those of the memory, `a` columns of the first one lie in front of
+    // the row. Slot c of thread t then holds column n * LP_BLOCK + 4 t + c - a in round n, always of the same
+    // summation chain (4 t + c - a modulo LP_BLOCK) and in ascending order; the chains are put back in their
+    // places before they are added up.
     const T*              rowp = (const T*)p.logits + (size_t)row * p.Vp;
-    const Chunk*          base = reinterpret_cast<const Chunk*>(rowp);
-    const int             rounds = (p.V + LP_BLOCK - 1) / LP_BLOCK;  // columns >= V are masked: e = 0 exactly
+    const int             a    = (int)(((uintptr_t)rowp % sizeof(Chunk)) / sizeof(T));
+    const Chunk*          base = reinterpret_cast<const Chunk*>(reinterpret_cast<const char*>(rowp) - a * sizeof(T));
+    const int             rounds = (p.V + a + LP_BLOCK - 1) / LP_BLOCK;  // columns outside [0, V) are masked: e = 0 exactly
 
     // history first, then the first loads of the row, then the arguments
     const bool hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
@@ -297,8 +314,8 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     const int    tcol  = t * LP_CHAINS;  // the thread's first column within a round
     const Chunk* tbase = base + t;
     // the last round may reach past the row: such a thread reads its chunk of the round before (never used).
-    // Rows are 16-byte aligned, so a chunk that starts inside the padded row lies inside it.
-    const bool last_inside = (rounds - 1) * LP_BLOCK + tcol < p.Vp;
+    // A chunk of the memory that starts in front of the padded row's end holds at least one of its elements.
+    const bool last_inside = (rounds - 1) * LP_BLOCK + tcol < a + p.Vp;
     auto       load        = [&](int slot, int n) {
         if (n + 1 < rounds) {  // uniform: the round's offset stays in scalar registers
             raw[slot] = tbase[(size_t)n * LP_THREADS];
@@ -377,12 +394,26 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     // round alone (the side of the bitmap seam, whether the round holds the masked end id or the end of the
     // vocabulary) is decided in scalar registers.
     auto e_values = [&](const Chunk& v, int n, float* e) {
-        const int col  = n * LP_BLOCK + tcol;
+        const int col  = n * LP_BLOCK + tcol - a;
         uint32_t  bits = 0u;
         if (bitsv) {
             if constexpr (BMW > 0) {
-                const int at = (n < LP_BM_OVERLAY / (LP_BLOCK / 32) ? LP_BM_HEAD_AT : LP_BM_TAIL_AT) + n * (LP_BLOCK / 32);
-                bits         = (lds_words[at + (tcol >> 5)] >> (tcol & 31)) & ((1u << LP_CHAINS) - 1u);
+                if (a == 0) {
+                    const int at = (n < LP_BM_OVERLAY / (LP_BLOCK / 32) ? LP_BM_HEAD_AT : LP_BM_TAIL_AT) + n * (LP_BLOCK / 32);
+                    bits         = (lds_words[at + (tcol >> 5)] >> (tcol & 31)) & ((1u << LP_CHAINS) - 1u);
+                }
+                else if (col >= 0) {
+                    // the four flags may straddle two words (the bitmap carries one word of slack)
+                    const int sh = col & 31;
+                    bits         = lds_words[bitmap_at(col >> 5)] >> sh;
+                    if (sh + LP_CHAINS > 32) {
+                        bits |= lds_words[bitmap_at((col >> 5) + 1)] << (32 - sh);
+                    }
+                    bits &= (1u << LP_CHAINS) - 1u;
+                }
+                else {
+                    bits = (lds_words[bitmap_at(0)] << (-col)) & ((1u << LP_CHAINS) - 1u);  // columns 0 .. at slots -col ..
+                }
             }
             else {
                 bits = rowctx.vector_bits(col, LP_CHAINS);
@@ -394,12 +425,12 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
             y[c] = rowctx.fast(lp_chunk_element<DT>(v, c));
         }
         // rare: a column of the history, the masked end id, the end of the vocabulary
-        const bool     tail_round = (n + 1) * LP_BLOCK > p.V;
-        const bool     end_round  = (uint32_t)(rowctx.masked_end_id - n * LP_BLOCK) < (uint32_t)LP_BLOCK;
+        const bool     edge_round = (n + 1) * LP_BLOCK - a > p.V || (a != 0 && n == 0);
+        const bool     end_round  = (uint32_t)(rowctx.masked_end_id - (n * LP_BLOCK - a)) < (uint32_t)LP_BLOCK;
         const uint32_t rel_end    = (uint32_t)(rowctx.masked_end_id - col);
         bool           rare       = bits != 0u;
-        if (tail_round || end_round) {
-            rare = rare || rel_end < (uint32_t)LP_CHAINS || col + LP_CHAINS > p.V;
+        if (edge_round || end_round) {
+            rare = rare || rel_end < (uint32_t)LP_CHAINS || col + LP_CHAINS > p.V || col < 0;
         }
         if (rare) {
 #pragma unroll
@@ -407,7 +438,7 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                 if ((bits >> c) & 1u) {
                     y[c] = rowctx.flagged(y[c]);
                 }
-                if ((uint32_t)c == rel_end || col + c >= p.V) {
+                if ((uint32_t)c == rel_end || (uint32_t)(col + c) >= (uint32_t)p.V) {
                     y[c] = -S::max_t();
                 }
             }
@@ -430,10 +461,10 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                 e[c] = round_t<DT>(det_expf_nonpos_number(d[c]));
             }
         }
-        if (tail_round && col + LP_CHAINS > p.V) {
+        if (edge_round && (col + LP_CHAINS > p.V || col < 0)) {
 #pragma unroll
             for (int c = 0; c < LP_CHAINS; ++c) {
-                e[c] = col + c < p.V ? e[c] : 0.0f;  // (what lies behind the vocabulary adds nothing)
+                e[c] = (uint32_t)(col + c) < (uint32_t)p.V ? e[c] : 0.0f;  // (what lies outside the row adds nothing)
             }
         }
     };
@@ -494,8 +525,8 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
             if (n < head) {
 #pragma unroll
                 for (int c = 0; c < LP_CHAINS; ++c) {
-                    const int col = n * LP_BLOCK + t * LP_CHAINS + c;
-                    if (head_e[n][c] >= thr_low && col < p.V) {
+                    const int col = n * LP_BLOCK + tcol + c - a;
+                    if (head_e[n][c] >= thr_low && (uint32_t)col < (uint32_t)p.V) {
                         push(head_e[n][c], col);
                     }
                 }
@@ -512,7 +543,7 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
             if (n < rounds) {
                 const int slot = (LP_HEAD + r) % LP_RING;
                 float     e[LP_CHAINS];
-                const int col0 = n * LP_BLOCK + t * LP_CHAINS;
+                const int col0 = n * LP_BLOCK + tcol - a;
                 e_values(raw[slot], n, e);
 #pragma unroll
                 for (int c = 0; c < LP_CHAINS; ++c) {
@@ -522,7 +553,7 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                 if (__builtin_fmaxf(__builtin_fmaxf(e[0], e[1]), __builtin_fmaxf(e[2], e[3])) >= thr_low) {
 #pragma unroll
                     for (int c = 0; c < LP_CHAINS; ++c) {
-                        if (e[c] >= thr_low && col0 + c < p.V) {
+                        if (e[c] >= thr_low && (uint32_t)(col0 + c) < (uint32_t)p.V) {
                             push(e[c], col0 + c);
                         }
                     }
@@ -535,6 +566,21 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                     rebound(dmax);
                 }
             }
+        }
+    }
+    if (a != 0) {
+        // chain 4 t + c - a (modulo LP_BLOCK) back to slot c of thread t; the bitmap's first words are done with
+        float* chain = reinterpret_cast<float*>(lds_words + LP_BM_HEAD_AT);
+        static_assert(sizeof(TopkShared::sel) >= LP_BLOCK * sizeof(float), "one float per chain");
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < LP_CHAINS; ++c) {
+            chain[(tcol + c - a) & (LP_BLOCK - 1)] = acc[c];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < LP_CHAINS; ++c) {
+            acc[c] = chain[tcol + c];
         }
     }
     // ---- the sum, in the reference's order: chain t = 4 * thread + c; butterflies with masks 16, 8, 4 run

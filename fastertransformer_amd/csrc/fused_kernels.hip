@@ -211,11 +211,11 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
                            && (size_t)a->vocab_size / (16 / elem) >= (size_t)lplan.splits * slot_u * LG_THREADS;
     const int      lean_mode  = one_read ? 1 : (two_reads ? 2 : 0);
     // Log-prob outputs: the two-read step covers what the lean gather covers, for vocabularies of at least 1024
-    // columns (the reference's softmax block) in rows that start on 16-byte boundaries.
+    // columns (the reference's softmax block); rows may start anywhere an element may.
     const bool want_log_probs = a->cum_log_probs != nullptr || a->output_log_probs != nullptr;
     if (want_log_probs
-        && (lean_mode != 1 || a->embedding_bias != nullptr || a->max_top_k > TK_STAGE || a->vocab_size < LP_BLOCK || ((size_t)a->vocab_size_padded * elem) % 16 != 0
-            || ((uintptr_t)a->logits & 15u) != 0)) {
+        && (lean_mode != 1 || a->embedding_bias != nullptr || a->max_top_k > TK_STAGE || a->vocab_size < LP_BLOCK
+            || ((uintptr_t)a->logits % (uintptr_t)elem) != 0)) {
         return FTK_ERR_UNSUPPORTED;
     }
     const size_t   slot_bytes = lean_mode == 2 ? (size_t)lplan.splits * slot_u * LG_THREADS * sizeof(uint32_t) : 0;

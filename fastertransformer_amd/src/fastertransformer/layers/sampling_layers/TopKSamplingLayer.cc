@@ -139,9 +139,20 @@ static bool fusedDisabled()
     return env != nullptr && env[0] == '1';
 }
 
+// With log-prob outputs the fused step gives every row to one workgroup, which pays once the rows outnumber the
+// compute units (256): measured on MI355X it passes the kernel sequence between 256 and 512 rows at vocabularies
+// from 32000 to 152064 columns. FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS overrides the smallest window that takes it
+// (read at every step).
+static int fusedLogProbsMinRows()
+{
+    const char* env = std::getenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS");
+    return env != nullptr && env[0] != '\0' ? std::atoi(env) : 384;
+}
+
 // One streaming pass over the logits for the whole penalty + mask + top-k pipeline - two passes when log-prob
 // outputs are requested, which need the probabilities of the whole row. Not taken with the frequency-penalty
-// extension, nor for the configurations the fused step reports as unsupported with log-probs.
+// extension, nor for the configurations the fused step reports as unsupported with log-probs, nor for log-probs
+// on small windows.
 template<typename T>
 bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_tensors)
 {
@@ -156,6 +167,9 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
     const int step             = input_tensors->at("step").template getVal<int>();
     const int max_input_length = input_tensors->at("max_input_length").template getVal<int>();
     const int off              = ite * local_batch_size;
+    if ((cum_log_probs != nullptr || output_log_probs != nullptr) && local_batch_size < fusedLogProbsMinRows()) {
+        return false;
+    }
 
     ftk_fused_topk_args a{};
     a.dtype             = FtkDType<T>::value;
@@ -208,7 +222,7 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
     a.workspace = nullptr;
     const int query = ftk_fused_topk_step(&a, stream_);
     if (query == FTK_ERR_UNSUPPORTED) {
-        return false;  // log-probs with a bias, a large k, a tiny vocabulary or unaligned rows: the kernel sequence
+        return false;  // log-probs with a bias, a large k or a tiny vocabulary: the kernel sequence
     }
     check_ftk(query);
     if (a.workspace_size > sampling_workspace_size_) {

@@ -224,8 +224,9 @@ typedef struct ftk_fused_topk_args {
     /* Log-prob outputs (both NULL: none). With either one the step takes the probabilities of the whole row as
      * the reference does (softmax after the penalties, top-k on probabilities): cum_log_probs[b] += log p,
      * output_log_probs[b] = log p - log(sum of the k probabilities). Covered for launches without embedding
-     * bias, largest k <= 128, vocab_size >= 1024 and 16-byte aligned rows; anything else returns
-     * FTK_ERR_UNSUPPORTED (also for the size query) and launches nothing: run the kernel sequence instead. */
+     * bias, largest k <= 128 and vocab_size >= 1024 (rows of any pitch, starting on any element boundary);
+     * anything else returns FTK_ERR_UNSUPPORTED (also for the size query) and launches nothing: run the kernel
+     * sequence instead. Every row goes to one workgroup here, which pays from a few hundred rows on. */
     float* cum_log_probs;    /* [local] or NULL */
     float* output_log_probs; /* [local] or NULL: the row of this step */
     void*  workspace;

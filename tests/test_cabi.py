@@ -100,6 +100,19 @@ def test_workspace_queries_and_argument_errors():
     a.dtype, a.vocab_size, a.vocab_size_padded, a.batch_size, a.local_batch_size, a.max_top_k = fa.F16, 50257, 51200, 256, 256, 64
     a.workspace = None
     assert lib.ftk_fused_topk_step(C.addressof(a), None) == 0 and a.workspace_size > 0
+    # with log-prob outputs the fused step takes rows of any pitch and start (GPT-2's 50257 fp32 columns unpadded,
+    # a buffer that starts on an odd element), but no vocabulary under 1024 columns
+    keep = C.create_string_buffer(64)
+    a.cum_log_probs = C.addressof(keep)
+    a.dtype, a.vocab_size, a.vocab_size_padded, a.logits = fa.F32, 50257, 50257, 0x1000 + 4
+    assert lib.ftk_fused_topk_step(C.addressof(a), None) == 0 and a.workspace_size > 0
+    a.dtype, a.logits = fa.F16, 0x1000 + 6
+    assert lib.ftk_fused_topk_step(C.addressof(a), None) == 0
+    a.logits = 0x1000 + 1      # not even an element boundary
+    assert lib.ftk_fused_topk_step(C.addressof(a), None) == fa.ops.FTK_ERR_UNSUPPORTED
+    a.logits, a.vocab_size, a.vocab_size_padded = 0x1000, 1000, 1000
+    assert lib.ftk_fused_topk_step(C.addressof(a), None) == fa.ops.FTK_ERR_UNSUPPORTED
+    a.cum_log_probs, a.logits, a.vocab_size, a.vocab_size_padded = None, None, 50257, 51200
     a.max_top_k = 2000
     assert lib.ftk_fused_topk_step(C.addressof(a), None) == fa.ops.FTK_ERR_TOPK_DOMAIN
     assert lib.ftk_fused_topk_step(None, None) == fa.ops.FTK_ERR_ARGUMENT

@@ -90,7 +90,9 @@ def test_config1_cpu_reference_step(logprobs):
     c = Case(O.F32, B, V, V, max_input_length=64, gen_len=3, runtime_top_k=[40], runtime_top_p=[0.0],
              temperature=[1.0], repetition_penalty=[1.2], end_ids=np.full(B, 50256, np.int32),
              prompt=_history(rng, 64, B, V), with_cum=logprobs, with_out_lp=logprobs)
-    _run_case(c, rng, 3, lambda i: make_logits(rng, O.F32, B, V, V, 2.0), check_logits=logprobs)
+    # (rows of 50257 fp32 columns start off 16-byte boundaries; both variants take a fused step, which leaves the
+    # caller's logits alone)
+    _run_case(c, rng, 3, lambda i: make_logits(rng, O.F32, B, V, V, 2.0), check_logits=False)
 
 
 @pytest.mark.parametrize("logprobs", [False, True], ids=["fused", "logprobs"])
@@ -427,6 +429,63 @@ def test_fused_step_with_log_probs_random_scenarios(dt, seed):
             x = O.to_f32(make_logits(rng, dt, B, V, Vp, scale), dt)
             rows = rng.random(B) < 0.2
             x[rows, end[rows]] = 40.0  # these rows finish
+            return O.to_storage(x, dt)
+
+        _run_case(c, rng, 3, logits_fn, check_logits=False)
+
+
+def test_log_probs_on_small_windows_take_the_kernel_sequence(monkeypatch):
+    """Without the override of the test session, log-prob outputs send windows of fewer than 384 rows through the
+    kernel sequence (which writes the penalised logits and the probabilities back like the reference) and larger
+    ones through the fused step (which leaves the logits alone); the results are the reference's either way."""
+    monkeypatch.delenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS")
+    rng = np.random.default_rng(7200)
+    V = 2051
+    for B, mutated in ((8, True), (400, False)):
+        c = Case(O.F32, B, V, V, max_input_length=4, gen_len=2, runtime_top_k=[8], runtime_top_p=[0.9],
+                 temperature=[0.7], repetition_penalty=[1.3], prompt=_history(rng, 4, B, V), with_cum=True,
+                 with_out_lp=True)
+        fed = []
+
+        def logits_fn(i):
+            fed.append(make_logits(rng, O.F32, B, V, V, 2.0))
+            return fed[-1]
+
+        snap = _run_case(c, rng, 2, logits_fn, check_logits=mutated)
+        assert np.array_equal(np.asarray(snap["logits"]).reshape(B, V), fed[-1].reshape(B, V)) == (not mutated)
+
+
+@pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
+def test_fused_step_with_log_probs_rows_off_vector_boundaries(dt):
+    """Log-probs on rows whose pitch is not a multiple of 16 bytes (GPT-2's 50257 columns unpadded, odd paddings): the
+    rows of a batch then start at every offset inside a 16-byte vector, the summation chains of the reference's
+    softmax are rotated against the loads, and history flags straddle bitmap words. Ids, flags and lengths bit
+    for bit, log-probs to tolerance; long histories use the bitmap in memory, short ones the one in LDS."""
+    rng = np.random.default_rng(7100 + dt)
+    for V, Vp, B, H, max_k in ((50257, 50257, 9, 64, 40), (1024, 1027, 13, 5, 8), (4999, 5001, 6, 700, 64),
+                               (33001, 33003, 17, 30, 128), (152063, 152065, 5, 12, 64), (1029, 1029, 3, 0, 1)):
+        ks = rng.integers(1, max_k + 1, B).astype(np.uint32)
+        ks[0] = max_k
+        ps = np.where(rng.random(B) < 0.5, 1.0, rng.uniform(0.2, 0.99, B)).astype(np.float32)
+        kw = {"temperature": rng.uniform(0.5, 1.6, B)}
+        if H > 0:
+            if rng.random() < 0.5:
+                kw["repetition_penalty"] = rng.uniform(1.0, 1.6, B)
+            else:
+                kw["presence_penalty"] = rng.uniform(0.0, 1.5, B)
+            kw["prompt"] = _history(rng, H, B, V, zipf=1.3 if rng.random() < 0.5 else None)
+            kw["input_lengths"] = rng.integers(1, H + 1, B)
+        kw["min_length"] = rng.integers(0, 4, B)
+        end = rng.integers(0, V, B).astype(np.int32)
+        end[0], end[-1] = 0, V - 1            # the masked end id in the first and in the last chunk of a row
+        c = Case(dt, B, V, Vp, max_input_length=H, gen_len=3, runtime_top_k=ks, runtime_top_p=ps, end_ids=end,
+                 with_cum=True, with_out_lp=True, **kw)
+        scale = float(rng.uniform(0.5, 4.0))
+
+        def logits_fn(i):
+            x = O.to_f32(make_logits(rng, dt, B, V, Vp, scale), dt)
+            x[:, 0] += 2.0 * scale            # the row's edges matter
+            x[:, V - 1] += 2.0 * scale
             return O.to_storage(x, dt)
 
         _run_case(c, rng, 3, logits_fn, check_logits=False)
