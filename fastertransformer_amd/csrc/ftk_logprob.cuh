@@ -83,15 +83,15 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
     auto  load = [&](int slot, int q) {
 #pragma unroll
         for (int j = 0; j < LG_NV; ++j) {
-            const int vi = min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1);
+            // past the end: a harmless vector (the last one; the one that holds the row's start if there is none)
+            const int vi = max(min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1), 0);
             raw[slot][j] = lean_stream_load(base + vi);
         }
     };
+    // every load is issued whatever the sub-tile, so that a wait can name the oldest load in flight
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        if (r < nsub) {
-            load(r, r);
-        }
+        load(r, r);
     }
     const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
     const bool        fin  = row_flag_or(p.finished_in, row, p.end_ids + row, false);
@@ -163,21 +163,26 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
         }
         return vm;
     };
-    for (int q0 = 0; q0 < nsub; q0 += R) {
+    auto sub_tile = [&](int r, int q) {
+#pragma unroll
+        for (int j = 0; j < LG_NV; ++j) {
+            const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
+            const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV - a);
+            m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
+        }
+    };
+    int q0 = 0;
+    for (; q0 + R <= nsub; q0 += R) {  // whole groups: no guards, every slot is loaded again
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const int q = q0 + r;
-            if (q < nsub) {
+            sub_tile(r, q0 + r);
+            load(r, q0 + r + R);
+        }
+    }
 #pragma unroll
-                for (int j = 0; j < LG_NV; ++j) {
-                    const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
-                    const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV - a);
-                    m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
-                }
-                if (q + R < nsub) {
-                    load(r, q + R);
-                }
-            }
+    for (int r = 0; r < R - 1; ++r) {  // the last sub-tiles: their vectors are on their way or here
+        if (q0 + r < nsub) {
+            sub_tile(r, q0 + r);
         }
     }
     if (first_wg) {
@@ -316,19 +321,15 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     // the last round may reach past the row: such a thread reads its chunk of the round before (never used).
     // A chunk of the memory that starts in front of the padded row's end holds at least one of its elements.
     const bool last_inside = (rounds - 1) * LP_BLOCK + tcol < a + p.Vp;
-    auto       load        = [&](int slot, int n) {
-        if (n + 1 < rounds) {  // uniform: the round's offset stays in scalar registers
-            raw[slot] = tbase[(size_t)n * LP_THREADS];
-        }
-        else {
-            raw[slot] = tbase[(size_t)(last_inside ? n : n - 1) * LP_THREADS];
-        }
+    // Every load is issued whatever the round (one past the row's end fetches the last round's chunk again, unused):
+    // with the same number of loads on every path the waits can name the oldest load instead of all of them.
+    auto load = [&](int slot, int n) {
+        const int m = min(n, rounds - 1);
+        raw[slot]   = tbase[(size_t)((m + 1 < rounds || last_inside) ? m : m - 1) * LP_THREADS];
     };
 #pragma unroll
     for (int r = 0; r < LP_RING; ++r) {
-        if (r < rounds) {
-            load(r, r);
-        }
+        load(r, r);
     }
     const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
     const bool        fin  = row_flag_or(l.finished, row, p.end_ids + row, false);
@@ -514,10 +515,8 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
                     acc[c] = acc[c] + head_e[n][c];
                     tmax   = __builtin_fmaxf(tmax, head_e[n][c]);
                 }
-                if (n + LP_RING < rounds) {
-                    load(n, n + LP_RING);
-                }
             }
+            load(n, n + LP_RING);
         }
         rebound(order_key(tmax));
 #pragma unroll
@@ -535,37 +534,48 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     }
     // ---- the rest of the row; the bound is raised again after 8, 16, 32, ... rounds
     static_assert(LP_RING % LP_HEAD == 0 && LP_RING > LP_HEAD, "the ring continues where the head stopped");
-    int next_tighten = 2 * LP_HEAD;
-    for (int n0 = LP_HEAD; n0 < rounds; n0 += LP_RING) {
+    int  next_tighten = 2 * LP_HEAD;
+    auto one_round    = [&](int slot, int n) {
+        float     e[LP_CHAINS];
+        const int col0 = n * LP_BLOCK + tcol - a;
+        e_values(raw[slot], n, e);
 #pragma unroll
-        for (int r = 0; r < LP_RING; ++r) {
-            const int n = n0 + r;
-            if (n < rounds) {
-                const int slot = (LP_HEAD + r) % LP_RING;
-                float     e[LP_CHAINS];
-                const int col0 = n * LP_BLOCK + tcol - a;
-                e_values(raw[slot], n, e);
+        for (int c = 0; c < LP_CHAINS; ++c) {
+            acc[c] = acc[c] + e[c];
+        }
+        // one look per chunk for a candidate (a NaN is none, with or without the maximum)
+        if (__builtin_fmaxf(__builtin_fmaxf(e[0], e[1]), __builtin_fmaxf(e[2], e[3])) >= thr_low) {
 #pragma unroll
-                for (int c = 0; c < LP_CHAINS; ++c) {
-                    acc[c] = acc[c] + e[c];
-                }
-                // one look per chunk for a candidate (a NaN is none, with or without the maximum)
-                if (__builtin_fmaxf(__builtin_fmaxf(e[0], e[1]), __builtin_fmaxf(e[2], e[3])) >= thr_low) {
-#pragma unroll
-                    for (int c = 0; c < LP_CHAINS; ++c) {
-                        if (e[c] >= thr_low && (uint32_t)(col0 + c) < (uint32_t)p.V) {
-                            push(e[c], col0 + c);
-                        }
-                    }
-                }
-                if (n + LP_RING < rounds) {
-                    load(slot, n + LP_RING);
-                }
-                if (n + 1 == next_tighten && n + 1 < rounds) {
-                    next_tighten *= 2;
-                    rebound(dmax);
+            for (int c = 0; c < LP_CHAINS; ++c) {
+                if (e[c] >= thr_low && (uint32_t)(col0 + c) < (uint32_t)p.V) {
+                    push(e[c], col0 + c);
                 }
             }
+        }
+    };
+    auto tighten = [&](int n) {
+        if (n + 1 == next_tighten && n + 1 < rounds) {
+            next_tighten *= 2;
+            rebound(dmax);
+        }
+    };
+    int n0 = LP_HEAD;
+    // whole groups of LP_RING rounds: no guards, every slot is loaded again
+    for (; n0 + LP_RING <= rounds; n0 += LP_RING) {
+#pragma unroll
+        for (int r = 0; r < LP_RING; ++r) {
+            const int slot = (LP_HEAD + r) % LP_RING;
+            one_round(slot, n0 + r);
+            load(slot, n0 + r + LP_RING);
+            tighten(n0 + r);
+        }
+    }
+    // the last rounds (fewer than LP_RING): their chunks are on their way or here
+#pragma unroll
+    for (int r = 0; r < LP_RING - 1; ++r) {
+        if (n0 + r < rounds) {
+            one_round((LP_HEAD + r) % LP_RING, n0 + r);
+            tighten(n0 + r);
         }
     }
     if (a != 0) {

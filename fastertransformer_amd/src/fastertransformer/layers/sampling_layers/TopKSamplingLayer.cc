@@ -139,14 +139,14 @@ static bool fusedDisabled()
     return env != nullptr && env[0] == '1';
 }
 
-// With log-prob outputs the fused step gives every row to one workgroup, which pays once the rows outnumber the
-// compute units (256): measured on MI355X it passes the kernel sequence between 256 and 512 rows at vocabularies
-// from 32000 to 152064 columns. FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS overrides the smallest window that takes it
-// (read at every step).
+// With log-prob outputs the fused step gives every row to one workgroup, which pays once there are enough rows to
+// keep the compute units busy: measured on MI355X it draws level with the kernel sequence between 128 and 192
+// rows at vocabularies from 32000 to 152064 columns and wins from there on.
+// FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS overrides the smallest window that takes it (read at every step).
 static int fusedLogProbsMinRows()
 {
     const char* env = std::getenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS");
-    return env != nullptr && env[0] != '\0' ? std::atoi(env) : 384;
+    return env != nullptr && env[0] != '\0' ? std::atoi(env) : 192;
 }
 
 // One streaming pass over the logits for the whole penalty + mask + top-k pipeline - two passes when log-prob

@@ -435,7 +435,7 @@ def test_fused_step_with_log_probs_random_scenarios(dt, seed):
 
 
 def test_log_probs_on_small_windows_take_the_kernel_sequence(monkeypatch):
-    """Without the override of the test session, log-prob outputs send windows of fewer than 384 rows through the
+    """Without the override of the test session, log-prob outputs send windows of fewer than 192 rows through the
     kernel sequence (which writes the penalised logits and the probabilities back like the reference) and larger
     ones through the fused step (which leaves the logits alone); the results are the reference's either way."""
     monkeypatch.delenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS")
