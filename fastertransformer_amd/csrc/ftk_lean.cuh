@@ -237,8 +237,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
     auto         load = [&](int slot, int q) {
 #pragma unroll
         for (int j = 0; j < LG_NV; ++j) {
-            // past the end: a harmless vector (the last one; the one that holds the row's start if there is none)
-            const int vi = max(min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1), 0);
+            const int vi = min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1);  // past the end: a harmless vector
             raw[slot][j] = lean_stream_load(base + vi);
             if constexpr (BIAS) {
                 rawb[slot][j] = bias_base[vi];
@@ -263,11 +262,11 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
         const float x = vector_element<DT>(v, e);
         return has_bias ? round_t<DT>(x + vector_element<DT>(b, e)) : x;
     };
-    // Every load is issued whatever the sub-tile: with the same number of loads on every path a wait can name the
-    // oldest load in flight instead of all of them.
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        load(r, r);
+        if (r < nsub) {
+            load(r, r);
+        }
     }
 
     // PRESET: the row's maxima from the SLOTS launch, thread t looks at slot t of every group
@@ -610,46 +609,37 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 
     // ---- the stream. The bound is raised again after 4, 8, 16, ... sub-tiles: the k-th largest of the lanes'
     // largest candidates bounds the k-th largest of everything seen so far.
-    int  next_tighten = 4;
-    auto sub_tile     = [&](int r, int q, bool reload) {
-#pragma unroll
-        for (int j = 0; j < LG_NV; ++j) {
-            const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
-            const float m   = vector_max(raw[r][j], rawb[BIAS ? r : 0][j]) * mul;
-            park((all_hit || m >= thr_hot) && rel < nvec, raw[r][j], (vb + rel) * EPV - a);
-        }
-        if (reload) {
-            load(r, q + R);
-        }
-        const bool tighten = MODE == LG_MODE_STREAM && q + 1 == next_tighten && q + 1 < nsub;
-        if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
-            drain();
-        }
-        if (tighten) {
-            next_tighten *= 2;
-            s.slot_key[par][t] = dmax;
-            lds_barrier();
-            const uint32_t P = lean_kth_of_slots(s.slot_key[par], k);
-            par ^= 1;
-            if (P > thr) {
-                set_threshold(P);
-                valid = true;
-            }
-        }
-    };
-    int q0 = 0;
-    // whole groups of R sub-tiles: no guards, every slot is loaded again (past the end: a harmless vector)
-    for (; q0 + R <= nsub; q0 += R) {
+    int next_tighten = 4;
+    for (int q0 = 0; q0 < nsub; q0 += R) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            sub_tile(r, q0 + r, true);
-        }
-    }
-    // the last sub-tiles (fewer than R): their vectors are on their way or here
+            const int q = q0 + r;
+            if (q < nsub) {
 #pragma unroll
-    for (int r = 0; r < R - 1; ++r) {
-        if (q0 + r < nsub) {
-            sub_tile(r, q0 + r, false);
+                for (int j = 0; j < LG_NV; ++j) {
+                    const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
+                    const float m   = vector_max(raw[r][j], rawb[BIAS ? r : 0][j]) * mul;
+                    park((all_hit || m >= thr_hot) && rel < nvec, raw[r][j], (vb + rel) * EPV - a);
+                }
+                if (q + R < nsub) {
+                    load(r, q + R);
+                }
+                const bool tighten = MODE == LG_MODE_STREAM && q + 1 == next_tighten && q + 1 < nsub;
+                if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
+                    drain();
+                }
+                if (tighten) {
+                    next_tighten *= 2;
+                    s.slot_key[par][t] = dmax;
+                    lds_barrier();
+                    const uint32_t P = lean_kth_of_slots(s.slot_key[par], k);
+                    par ^= 1;
+                    if (P > thr) {
+                        set_threshold(P);
+                        valid = true;
+                    }
+                }
+            }
         }
     }
 

@@ -83,15 +83,15 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
     auto  load = [&](int slot, int q) {
 #pragma unroll
         for (int j = 0; j < LG_NV; ++j) {
-            // past the end: a harmless vector (the last one; the one that holds the row's start if there is none)
-            const int vi = max(min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1), 0);
+            const int vi = min(vb + q * LG_SUB_VECS + j * LG_THREADS + t, ve - 1);
             raw[slot][j] = lean_stream_load(base + vi);
         }
     };
-    // every load is issued whatever the sub-tile, so that a wait can name the oldest load in flight
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        load(r, r);
+        if (r < nsub) {
+            load(r, r);
+        }
     }
     const bool        skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
     const bool        fin  = row_flag_or(p.finished_in, row, p.end_ids + row, false);
@@ -163,26 +163,21 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
         }
         return vm;
     };
-    auto sub_tile = [&](int r, int q) {
-#pragma unroll
-        for (int j = 0; j < LG_NV; ++j) {
-            const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
-            const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV - a);
-            m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
-        }
-    };
-    int q0 = 0;
-    for (; q0 + R <= nsub; q0 += R) {  // whole groups: no guards, every slot is loaded again
+    for (int q0 = 0; q0 < nsub; q0 += R) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            sub_tile(r, q0 + r);
-            load(r, q0 + r + R);
-        }
-    }
+            const int q = q0 + r;
+            if (q < nsub) {
 #pragma unroll
-    for (int r = 0; r < R - 1; ++r) {  // the last sub-tiles: their vectors are on their way or here
-        if (q0 + r < nsub) {
-            sub_tile(r, q0 + r);
+                for (int j = 0; j < LG_NV; ++j) {
+                    const int   rel = q * LG_SUB_VECS + j * LG_THREADS + t;
+                    const float vm  = vector_max(raw[r][j], (vb + min(rel, nvec - 1)) * EPV - a);
+                    m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
+                }
+                if (q + R < nsub) {
+                    load(r, q + R);
+                }
+            }
         }
     }
     if (first_wg) {
