@@ -23,7 +23,8 @@
 // Rows it cannot bound take the literal replay on probabilities computed on the fly.
 // Preconditions (checked by the host, which otherwise reports FTK_ERR_UNSUPPORTED and the layer runs the kernel
 // sequence): no embedding bias, largest k <= 128, vocabulary >= 1024 (the reference's block is min(V, 1024)
-// threads), rows aligned to 16 bytes.
+// threads). Rows may have any pitch and start on any element boundary: the loads are the aligned vectors of the
+// memory, and the few columns of the first one that lie in front of the row are masked.
 #pragma once
 #include <type_traits>
 
