@@ -28,8 +28,13 @@
 //    top-k set against numpy on distinct values; inverse CDF and log-probs against float64;
 //  * temperature, repetition / presence, min-length, end mask, softmax, top-p walk and decay:
 //    closed forms in float64 / exact binary cases; the softmax's summation order bit for bit against a
-//    thread-by-thread float32 simulation; storage conversions against numpy and torch;
-//    det_expf / det_logf against float64;
+//    thread-by-thread float32 simulation; the rounding order of top-p's prefix sums
+//    (cub::BlockScan<float, 256>::InclusiveSum with the running prefix, BLOCK_SCAN_RAKING) against a
+//    thread-by-thread float32 simulation written from the vendored sources
+//    (3rdparty/cub/block/specializations/block_scan_raking.cuh:601-655,
+//    3rdparty/cub/warp/specializations/warp_scan_shfl.cuh:199-232, :465-487, :543-609), position for position, on
+//    draws that a running sum or another raking split of the same terms would cross elsewhere
+//    (tests/cub_block_scan.py); storage conversions against numpy and torch; det_expf / det_logf against float64;
 //  * ban_bad_words, stop words, length criterion, finalize: no reference test exists, pinned by brute
 //    force written from the source description only (finalize: a stable descending sort);
 //  * beam search step (topk_softmax): no reference test exists; pinned by the definition it must reduce to
@@ -37,8 +42,7 @@
 //    scenario checks of the hypothesis bookkeeping written from the source description; the penalties,
 //    update and cache-indirection kernels around it, and the word lists with beams, by independent numpy
 //    restatements of the description.
-//  PARITY UNPINNED (no reference code or no way to run it here): the rounding order of cub's
-//  BLOCK_SCAN_RAKING prefix sums in top-p (cub is not in the reference's tree), bfloat16 storage, the frequency
+//  PARITY UNPINNED (no reference code or no way to run it here): bfloat16 storage, the frequency
 //  penalty, the random stream (cuRAND XORWOW is replaced; draws are injected), the last-ulp
 //  behaviour of __expf / logf (tolerance 1e-5 relative instead), and in the beam search step the
 //  reference's pairwise (max, sum) merges in cub's order and its powf.

@@ -509,6 +509,34 @@ def test_topp_sampling_flat_and_tied_rows(env, dt):
         _compare_topk(_run_topp(env, *args), _oracle_topp(*args), dt)
 
 
+@pytest.mark.parametrize("force_deep", [False, True])
+def test_topp_pick_follows_the_reference_scan_order(env, force_deep):
+    """Draws that lie within a bit of a prefix sum: the position depends on the rounding order of the reference's
+    block scan (cub BLOCK_SCAN_RAKING with a running prefix, simulated thread by thread from the vendored sources in
+    tests/cub_block_scan.py). Every draw of the set is crossed at another position by a plain running sum, a 64 x 4
+    or a 16 x 16 raking of the same terms; the expected ids come from the simulation, not from the oracle."""
+    import cub_block_scan as S
+    from test_oracle import _topp_rows_for_scan_order
+    cases = []
+    for probs in _topp_rows_for_scan_order():
+        order = np.argsort(-probs, kind="stable")
+        for r, pos, alt_pos in S.discriminating_draws(probs[order]):
+            cases.append((probs, r, int(order[pos])))
+    assert len(cases) >= 60
+    V = max(len(c[0]) for c in cases)
+    batch = len(cases)
+    probs = np.zeros((batch, V), np.float32)          # shorter rows end in zeros: they trail the order
+    for b, (row, _, _) in enumerate(cases):
+        probs[b, :len(row)] = row
+    u = np.array([c[1] for c in cases], np.float32)
+    want = np.array([c[2] for c in cases], np.int32)
+    p_arr = np.ones(batch, np.float32)                # r = u * 1.0f exactly
+    end_ids = np.zeros(batch, np.int32)
+    got = _run_topp(env, O.F32, probs, p_arr, end_ids, u, force_deep=force_deep)
+    assert np.array_equal(got[0], want), np.nonzero(got[0] != want)[0]
+    assert np.array_equal(_oracle_topp(O.F32, probs, p_arr, end_ids, u)[0], want)
+
+
 def test_topp_decay_and_initialize(env):
     torch, lib, ops = env
     rng = np.random.default_rng(3)

@@ -478,6 +478,61 @@ def test_topp_nucleus_property_random_rows():
         np.testing.assert_allclose(cum[b], np.log(pr[ids[b]]), rtol=1e-5, atol=1e-6)
 
 
+def _topp_rows_for_scan_order():
+    """sorted-descending rows whose prefix sums round differently under different summation orders"""
+    rng = np.random.default_rng(2024)
+    rows = []
+    for V, scale in ((2000, 2.5), (3000, 1.0), (1500, 0.3), (5000, 4.0), (6000, 0.05)):
+        x = rng.standard_normal(V) * scale
+        e = np.exp(x - x.max())
+        rows.append((e / e.sum()).astype(np.float32))
+    ranks = rng.permutation(4000) + 1.0                     # Zipf(1.1) over a permutation, with noise
+    z = np.exp(-1.1 * np.log(ranks) + rng.standard_normal(4000) * 0.5)
+    rows.append((z / z.sum()).astype(np.float32))
+    return rows
+
+
+def test_topp_prefix_sum_order_bit_for_bit():
+    """The position top-p emits is the first one whose fp32 prefix sum reaches the draw, so the rounding order of
+    those sums (cub's BLOCK_SCAN_RAKING with a running prefix over tiles of 256) decides ids whenever a draw
+    lies within a bit of a prefix sum. tests/cub_block_scan.py simulates that scan thread by thread from the
+    vendored cub sources; on draws chosen so that a plain running sum, a 64 x 4 and a 16 x 16 raking of the same
+    terms cross at another position, the oracle must emit exactly the simulated position."""
+    import cub_block_scan as C
+    disagree = {"running": 0, "raking64x4": 0, "raking16x16": 0}
+    checked = deepest = 0
+    for probs in _topp_rows_for_scan_order():
+        order = np.argsort(-probs, kind="stable")           # the stable descending sort of :1106-1119
+        draws = C.discriminating_draws(probs[order])
+        assert draws
+        for r, pos, alt_pos in draws:
+            ids, seq, fin, cum, out = _oracle_topp(probs.reshape(1, -1), [r], [1.0])
+            assert ids[0] == order[pos], (len(probs), float(r), pos, alt_pos)
+            np.testing.assert_allclose(cum[0], np.log(np.float64(probs[order[pos]])), rtol=1e-5, atol=1e-6)
+            checked += 1
+            deepest = max(deepest, pos)                     # running totals of many tiles take part
+            for name, other in alt_pos.items():
+                disagree[name] += int(other != pos)
+    # the draw set separates the reference's order from each of the three other orders
+    assert checked >= 60 and deepest >= 8 * 256 and all(n >= 15 for n in disagree.values()), (checked, disagree)
+
+
+def test_topp_prefix_sums_whole_rows_bit_for_bit():
+    """every prefix sum of a row, not only the crossing: a draw equal to the simulated c_i must be crossed at the
+    first position whose simulated sum reaches it, for a spread of positions along the row (tile seams, segment
+    seams of the raking grid, positions inside a segment)"""
+    import cub_block_scan as C
+    probs = _topp_rows_for_scan_order()[0]
+    order = np.argsort(-probs, kind="stable")
+    c = C.prefix_sums(probs[order])
+    positions = [0, 1, 7, 8, 9, 31, 32, 33, 63, 64, 255, 256, 257, 263, 264, 511, 512, 700, 1023, 1024, 1500]
+    rows = np.repeat(probs.reshape(1, -1), len(positions), axis=0)
+    u = np.array([c[i] for i in positions], np.float32)
+    ids, _, _, _, _ = _oracle_topp(rows, u, np.ones(len(positions), np.float32))
+    for b, i in enumerate(positions):
+        assert ids[b] == order[C.pick_position(c, c[i])], i
+
+
 def test_topp_decay_closed_form():
     n = 7
     initial = np.linspace(0.5, 0.95, n).astype(np.float32)
