@@ -464,6 +464,35 @@ __device__ __forceinline__ float rng_next_uniform(RngState* st)
     return (float)o[0] * 2.3283064365386963e-10f + 1.16415321826934814453125e-10f;
 }
 
+// What a row's draw is made from, requested ahead of time without control flow (`safe`: any valid 4-byte aligned
+// address, read when an array is absent): the injected draw, or the row's generator state.
+struct RowDrawSource {
+    float    injected;
+    uint32_t seed_lo, seed_hi, off_lo, off_hi;
+};
+__device__ __forceinline__ RowDrawSource row_draw_source(const RngState* rng, const float* injected, int b,
+                                                         const void* safe)
+{
+    const uint32_t* st   = rng != nullptr ? reinterpret_cast<const uint32_t*>(rng + b) : nullptr;
+    const uint32_t* from = reinterpret_cast<const uint32_t*>(safe);
+    RowDrawSource   d;
+    d.injected = *(injected != nullptr ? injected + b : reinterpret_cast<const float*>(safe));
+    d.seed_lo  = *(st != nullptr ? st + 0 : from);
+    d.seed_hi  = *(st != nullptr ? st + 1 : from);
+    d.off_lo   = *(st != nullptr ? st + 2 : from);
+    d.off_hi   = *(st != nullptr ? st + 3 : from);
+    return d;
+}
+// One thread per row: the generated draw (same values as rng_next_uniform) and the counter the row's state goes on
+// with, which the caller stores.
+__device__ __forceinline__ float row_draw_generate(const RowDrawSource& d, uint64_t* next_offset)
+{
+    uint32_t o[4];
+    philox4x32_10(d.off_lo, d.off_hi, 0u, 0u, d.seed_lo, d.seed_hi, o);
+    *next_offset = (((uint64_t)d.off_hi << 32) | d.off_lo) + 1;
+    return (float)o[0] * 2.3283064365386963e-10f + 1.16415321826934814453125e-10f;
+}
+
 // The draw of row `b`: injected when the caller supplied one, generated otherwise.
 __device__ __forceinline__ float row_uniform(RngState* rng, const float* injected, int b)
 {

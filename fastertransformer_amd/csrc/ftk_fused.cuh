@@ -85,6 +85,25 @@ __device__ __forceinline__ float uniform_f(float x)
     return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x)));
 }
 
+// A row's per-row arguments, requested in one block without control flow so that they share one trip to memory
+// (the arithmetic on them, which waits for the values, comes afterwards).
+struct FusedRowArgs {
+    float temperature, penalty;
+    int   input_length, min_length, sequence_length, end_id;
+};
+__device__ __forceinline__ FusedRowArgs fused_row_args(const FusedParams& p, int row)
+{
+    const void*  safe = p.end_ids + row;
+    FusedRowArgs a;
+    a.temperature     = row_arg_or(p.temperatures, row, safe, 1.0f);
+    a.penalty         = row_arg_or(p.penalties, row, safe, 0.0f);
+    a.input_length    = row_arg_or(p.input_lengths, row, safe, p.max_input_length);
+    a.min_length      = row_arg_or(p.min_lengths, row, safe, 0);
+    a.sequence_length = row_arg_or(p.min_lengths != nullptr ? p.sequence_length_in : nullptr, row, safe, 0);
+    a.end_id          = p.end_ids[row];
+    return a;
+}
+
 template<int DT, int BMW>
 struct FusedRow {
     static constexpr int  LDS_WORDS = BMW > 0 ? BMW : 1;
@@ -109,20 +128,20 @@ struct FusedRow {
     const int*      history;  // output_ids + row, stride batch_size
     int             batch_size, step, input_length, max_input_length;
 
-    __device__ __forceinline__ FusedRow(const FusedParams& p, int row)
+    __device__ __forceinline__ FusedRow(const FusedParams& p, int row): FusedRow(p, row, fused_row_args(p, row)) {}
+    __device__ __forceinline__ FusedRow(const FusedParams& p, int row, const FusedRowArgs& args)
     {
         rowp        = (const T*)p.logits + (size_t)row * p.Vp;
         bias        = (const T*)p.bias;
         V           = p.V;
         Vp          = p.Vp;
         temp_active = p.temperatures != nullptr;
-        const void*              safe = p.end_ids + row;
-        const TemperatureCtx<DT> tc(row_arg_or(p.temperatures, row, safe, 1.0f), V, Vp, false);
+        const TemperatureCtx<DT> tc(args.temperature, V, Vp, false);
         inv           = tc.inv;
         fast_mul      = temp_active ? tc.inv : 1.0f;
         keep_pads     = tc.keep_pads;
         penalty_type  = p.penalties != nullptr ? p.penalty_type : 2;
-        penalty       = row_arg_or(p.penalties, row, safe, 0.0f);
+        penalty       = args.penalty;
         if (penalty_type == 0) {  // additive
             up_mul_neg = 1.0f;
             up_mul_pos = 1.0f;
@@ -143,7 +162,7 @@ struct FusedRow {
         batch_size    = p.batch_size;
         step          = p.step;
         max_input_length = p.max_input_length;
-        input_length  = row_arg_or(p.input_lengths, row, safe, p.max_input_length);
+        input_length  = args.input_length;
         // values that are the same for every lane of the workgroup but come out of floating-point
         // arithmetic: move them to scalar registers, they stay live for the whole kernel
         inv        = uniform_f(inv);
@@ -152,11 +171,10 @@ struct FusedRow {
         up_mul_neg = uniform_f(up_mul_neg);
         up_mul_pos = uniform_f(up_mul_pos);
         up_add     = uniform_f(up_add);
-        const int min_length = row_arg_or(p.min_lengths, row, safe, 0);
-        const int seq_length = row_arg_or(p.min_lengths != nullptr ? p.sequence_length_in : nullptr, row, safe, 0);
-        const int end_id     = p.end_ids[row];
-        masked_end_id =
-            (p.min_lengths != nullptr && min_length_masks(seq_length, p.max_input_length, min_length)) ? end_id : -1;
+        masked_end_id = (p.min_lengths != nullptr
+                         && min_length_masks(args.sequence_length, p.max_input_length, args.min_length)) ?
+                            args.end_id :
+                            -1;
     }
     __device__ __forceinline__ const T* data() const
     {

@@ -1,0 +1,631 @@
+// The fused decode step in one launch for batches of about one row per compute unit: a 1024-thread workgroup owns
+// a whole row. It streams the row once like the lean gather of ftk_lean.cuh (same ring of sub-tiles, same
+// parking of vectors that may hold a candidate, same exact evaluation), but
+//   - the bound is one per row instead of one per share of a row: far fewer candidates (about 3 k instead of
+//     4 x 3 k at k = 64 over 128 Ki columns),
+//   - candidates go to a list in LDS, never to memory: no list headers, no second launch, no trip to memory between
+//     the read of the row and its selection,
+//   - the replay of the reference's tie orders (topk_stage1 / topk_stage2_sampling of
+//     src/fastertransformer/kernels/sampling_topk_kernels.cu:130-312) ranks the candidates with all sixteen waves.
+// Sixteen waves per compute unit are in flight, as with four 256-thread workgroups, and the same bytes per thread.
+// Rows the kernel cannot bound (a list that outgrows LDS) are walked again by the first four waves with the general
+// stream of ftk_topk.cuh, as the merging kernel of the lean gather does.
+#pragma once
+#include "ftk_lean.cuh"
+
+namespace ftk {
+
+constexpr int RW_THREADS    = 1024;
+constexpr int RW_WAVES      = RW_THREADS / WAVE;
+constexpr int RW_NV         = 4;                    // 16-byte vectors per thread and sub-tile
+constexpr int RW_SUB_VECS   = RW_THREADS * RW_NV;   // a sub-tile: 64 KB
+#ifndef FTK_RW_RING
+#define FTK_RW_RING 2
+#endif
+constexpr int RW_RING       = FTK_RW_RING;          // sub-tiles in flight per thread
+constexpr int RW_PARK_GROUP = 2;                    // vectors a wave parks between two looks at its list's fill
+constexpr int RW_STAGE      = LG_DRAIN_AT + RW_PARK_GROUP * WAVE;
+constexpr int RW_HIST_U     = 4;                    // history ids a thread requests before the logits: the longest
+                                                    // history the kernel takes is RW_HIST_U * RW_THREADS positions
+constexpr int RW_MIN_SUBS   = 4;                    // shortest row the launcher sends here, in sub-tiles
+
+struct RowwideShared {
+    uint4    stage_raw[RW_WAVES][RW_STAGE];
+    int      stage_first[RW_WAVES][RW_STAGE];
+    uint32_t slot_key[RW_THREADS];
+    uint32_t bound;
+    int      n_out;
+};
+
+// The largest value P, to within its low sixteen bits, such that at least k of 256 keys are >= P (0 when fewer
+// than k are non-zero); slot i of the 256 is the largest of keys i, i + 256, i + 512, i + 768 of the workgroup, all
+// of them keys of distinct elements. The first wave finds it, every thread gets it. Two barriers.
+__device__ __forceinline__ uint32_t rowwide_bound(RowwideShared& s, uint32_t my_key, int k)
+{
+    s.slot_key[threadIdx.x] = my_key;
+    lds_barrier();
+    if (wave_id() == 0) {
+        uint32_t kk[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int i = lane_id() + g * WAVE;
+            kk[g]       = max(max(s.slot_key[i], s.slot_key[i + 256]), max(s.slot_key[i + 512], s.slot_key[i + 768]));
+        }
+        uint32_t P = 0u;
+#pragma unroll
+        for (int bit = 31; bit >= 16; --bit) {
+            const uint32_t cand = P | (1u << bit);
+            int            c    = 0;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                c += (int)__builtin_popcountll(__ballot(kk[g] >= cand));
+            }
+            P = c >= k ? cand : P;
+        }
+        if (lane_id() == 0) {
+            s.bound = P;
+        }
+    }
+    lds_barrier();
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)s.bound);
+}
+
+// Both tie orders of the reference by counting, for a list of at most 256 candidates, by the first TK_THREADS threads
+// of the workgroup (the others have left): the composite keys and the counting of the small case of topk_select_lds.
+// Candidates are in s.cand; on return the ordered list is in s.sel (values in w, columns in idx); returns its length.
+__device__ __forceinline__ int rowwide_rank(TopkShared& s, int n, int k, int max_top_k)
+{
+    const int t       = threadIdx.x;
+    const int bs1_log = max_top_k <= 16 ? 7 : 8;
+    const int BS1     = 1 << bs1_log;
+    const int BS2     = max_top_k <= 32 ? 128 : 256;
+    constexpr int CAP = 256;
+    const uint32_t      my_key = t < n ? s.cand.key[t] : 0u;
+    const uint32_t      my_idx = t < n ? s.cand.idx[t] : 0u;
+    unsigned long long* A      = s.keys;                                    // stage-1 keys  [0, 256)
+    unsigned long long* B      = s.keys + CAP;                              // stage-2 keys  [256, 512)
+    int*                cnt    = reinterpret_cast<int*>(s.keys + 2 * CAP);  // 3 x 256 counts
+    const int           n2     = (n + 1) & ~1;
+    int                 CP     = 2;
+    while (CP < n) {
+        CP <<= 1;
+    }
+    const int parts = TK_THREADS / CP;  // CP <= 256
+    const int c     = t & (CP - 1);
+    const int part  = t / CP;
+    const int pairs = n2 >> 1;
+    const int per   = (pairs + parts - 1) / parts;
+    const int jlo   = min(pairs, part * per) * 2;
+    const int jhi   = min(pairs, part * per + per) * 2;
+    lds_barrier();  // every candidate is in registers: the list's memory can be reused
+    unsigned long long mine = ~0ull;
+    if (t < n) {
+        const int blk   = (int)(my_idx >> bs1_log);
+        const int tt    = (int)(my_idx & (uint32_t)(BS1 - 1));
+        const int slice = blk & 7;
+        mine = ((unsigned long long)slice << 61) | ((unsigned long long)(~my_key) << 29)
+               | ((unsigned long long)(BS1 - 1 - tt) << 21) | (unsigned long long)(blk >> 3);
+    }
+    if (t < n2) {
+        A[t] = mine;  // (an odd list is padded with a key that never counts)
+    }
+    cnt[t]           = 0;
+    cnt[CAP + t]     = 0;
+    cnt[2 * CAP + t] = 0;
+    if (t == 0) {
+        s.misc[1] = 0;
+    }
+    lds_barrier();
+    {
+        const unsigned long long key  = c < n ? A[c] : ~0ull;
+        const unsigned long long base = key & (7ull << 61);  // below it: the keys of lower slices
+        int                      q = 0, qs = 0;
+#pragma unroll 4
+        for (int j = jlo; j < jhi; j += 2) {
+            const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&A[j]);
+            q += kk.x < key ? 1 : 0;
+            q += kk.y < key ? 1 : 0;
+            qs += kk.x < base ? 1 : 0;
+            qs += kk.y < base ? 1 : 0;
+        }
+        if (c < n && jhi > jlo) {
+            atomicAdd(&cnt[c], q);
+            atomicAdd(&cnt[CAP + c], qs);
+        }
+    }
+    lds_barrier();
+    unsigned long long k2 = ~0ull;
+    if (t < n) {
+        const int slice = (int)(mine >> 61);
+        const int r     = cnt[t] - cnt[CAP + t];  // rank inside the slice
+        if (r < k) {
+            const int pos = slice * k + r;
+            k2 = ((unsigned long long)(uint32_t)(mine >> 29) << 32) | ((unsigned long long)(BS2 - 1 - pos % BS2) << 24)
+                 | ((unsigned long long)(pos / BS2) << 12);
+        }
+    }
+    if (t < n2) {
+        B[t] = k2;
+    }
+    lds_barrier();
+    {
+        const unsigned long long key = c < n ? B[c] : ~0ull;
+        int                      q = 0, kept = 0;
+#pragma unroll 4
+        for (int j = jlo; j < jhi; j += 2) {
+            const ulonglong2 kk = *reinterpret_cast<const ulonglong2*>(&B[j]);
+            q += kk.x < key ? 1 : 0;
+            q += kk.y < key ? 1 : 0;
+            kept += kk.x != ~0ull ? 1 : 0;
+            kept += kk.y != ~0ull ? 1 : 0;
+        }
+        if (c < n && jhi > jlo) {
+            atomicAdd(&cnt[2 * CAP + c], q);
+        }
+        if (c == 0 && jhi > jlo) {
+            atomicAdd(&s.misc[1], kept);  // entries that stage 1 kept, over all parts
+        }
+    }
+    lds_barrier();
+    const int n_list = min(k, s.misc[1]);
+    if (t < n && k2 != ~0ull) {
+        const int q2 = cnt[2 * CAP + t];
+        if (q2 < n_list) {
+            s.sel.w[q2]   = key_to_float(~(uint32_t)(k2 >> 32));
+            s.sel.idx[q2] = (int)my_idx;
+        }
+    }
+    lds_barrier();
+    return n_list;
+}
+
+// What is left to the first four waves when a row's list is still longer than 256 entries after the cut (the
+// selection of topk_select_lds for long lists) or outgrew LDS (the whole row is walked again with the stream that
+// recovers from overfull tiles; rows it cannot bound either take the literal replay). Not inlined, so that the
+// kernel's registers are planned for its stream; the launch arguments are passed by value (a reference would move
+// the kernel's own copy from scalar registers to scratch memory).
+template<int DT>
+__device__ __noinline__ void rowwide_rare(TopkShared& ts, const FusedParams p, const FusedLaunch l,
+                                          const FusedRowArgs args, int row, int n, uint32_t thr, int k, float tp,
+                                          float u, const TopkOutputs out)
+{
+    TopkEntry*      row_entries = l.entries + (size_t)row * l.row_entries;
+    FusedRow<DT, 0> r0(p, row, args);
+    if (n > TK_CCAP) {
+        r0.prepare_whole_row();
+        __syncthreads();
+        n = topk_stream<DT, FusedRow<DT, 0>, 0>(r0, ts, p.Vp, k, 0, topk_row_tiles<DT>(r0.rowp, p.Vp), &thr);
+    }
+    topk_select_lds<DT, FusedRow<DT, 0>, true>(r0, ts, n, thr, row, p.Vp, k, tp, p.max_top_k, row_entries, false, u,
+                                               p.end_ids, out);
+}
+
+// Requirements the launcher checks: rows start on 16-byte boundaries (so a vector never straddles a word of the
+// history bitmap and there are no columns in front of the first vector), no embedding bias, the largest k at most
+// LG_MAX_K, at least RW_MIN_SUBS sub-tiles per row, the row's history bitmap fits BMW words, and a history of at most
+// RW_HIST_U * RW_THREADS positions.
+// Keeps a launch argument in a scalar register of its own from here on. Without it the compiler, short of scalar
+// registers, reads arguments again from the kernel-argument segment wherever they are used, and every such read
+// issued after the bulk of the row has been requested queues behind it.
+template<typename V>
+__device__ __forceinline__ void rowwide_pin(V& v)
+{
+    asm("" : "+s"(v));  // (not volatile: a volatile statement counts as a store to any address, and loads behind
+                        // such a store are no longer scalar loads)
+}
+
+template<int DT, int BMW>
+__global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedParams p_in, const FusedLaunch l_in)
+{
+    FusedParams p = p_in;
+    FusedLaunch l = l_in;
+    rowwide_pin(p.V);
+    rowwide_pin(p.Vp);
+    rowwide_pin(p.step);
+    rowwide_pin(p.max_input_length);
+    rowwide_pin(p.max_top_k);
+    rowwide_pin(p.penalty_type);
+    // (pointers that are only stored through, at the end: a pinned pointer is a generic one to the compiler)
+    rowwide_pin(l.ids);
+    rowwide_pin(l.sequence_length);
+    rowwide_pin(l.finished);
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         EPV = (int)(16 / sizeof(T));
+    constexpr int         R   = RW_RING;
+    static_assert(BMW > 0, "the history bitmap of the whole row lives in LDS");
+    __shared__ RowwideShared s;
+    __shared__ TopkShared    ts;
+    const int                t    = threadIdx.x;
+    const int                row  = blockIdx.x;
+    const int                lane = lane_id();
+    const int                wv   = wave_id();
+#ifdef FTK_RW_STAMPS
+    unsigned long long* stamps = reinterpret_cast<unsigned long long*>(l.entries + (size_t)blockIdx.x * l.row_entries);
+#define RW_STAMP(i) if (threadIdx.x == 0) { stamps[i] = wall_clock64(); }
+#else
+#define RW_STAMP(i)
+#endif
+    RW_STAMP(0)
+
+    // the row's address, pinned as a number and used as a pointer to global memory
+    typedef unsigned int                                  u4 __attribute__((ext_vector_type(4)));
+    typedef const __attribute__((address_space(1))) u4*   GlobalVec;
+    unsigned long long base_addr = (unsigned long long)((const T*)p.logits + (size_t)row * p.Vp);
+    rowwide_pin(base_addr);
+    const int nvec = p.V / EPV;  // whole vectors inside columns [0, V)
+    const int    nsub = (nvec + RW_SUB_VECS - 1) / RW_SUB_VECS;
+
+    // ---- everything the row needs from memory is requested at once, in one block without control flow: the
+    // per-row arguments (scalar loads), the token history (time-major: every id is a cache line of its own; positions
+    // past the step re-read the last one), then the first sub-tiles of the row
+    const void*         safe   = p.end_ids + row;
+    const bool          skip   = row_flag_or(p.skip_decode, row, safe, false);
+    const bool          fin    = row_flag_or(p.finished_in, row, safe, false);
+    const int           k      = row_arg_or(p.top_ks, row, safe, p.max_top_k);
+    const float         tp     = row_arg_or(p.top_ps, row, safe, 1.0f);
+    const FusedRowArgs  args   = fused_row_args(p, row);
+    const int           seq_in = row_arg_or((const int*)l_in.sequence_length, row, safe, 0);  // (the unpinned copy: a
+                                                                    // load through a pointer known to be global)
+    const RowDrawSource draw   = row_draw_source(l.rng, l.uniforms, row, safe);
+    const bool         injected     = l.uniforms != nullptr;
+    unsigned long long counter_addr = (unsigned long long)(l.rng != nullptr ? &l.rng[row].offset : nullptr);
+    rowwide_pin(counter_addr);
+    const bool         hist = p.bitmaps != nullptr && p.penalties != nullptr;
+    int                hist_ids[RW_HIST_U];
+    {
+        const int* column = hist ? p.output_ids + row : p.end_ids;  // (without a history: any valid address)
+        const int  last   = hist ? p.step - 1 : 0;
+        const int  stride = hist ? p.batch_size : 0;
+#pragma unroll
+        for (int u = 0; u < RW_HIST_U; ++u) {
+            hist_ids[u] = column[(size_t)min(t + u * RW_THREADS, last) * stride];
+        }
+    }
+    uint4 raw[R][RW_NV];
+    auto  load = [&](int slot, int q) {
+#pragma unroll
+        for (int j = 0; j < RW_NV; ++j) {
+            const int vi = min(q * RW_SUB_VECS + j * RW_THREADS + t, nvec - 1);  // past the end: a harmless vector
+            const u4  v  = __builtin_nontemporal_load((GlobalVec)(base_addr + (unsigned long long)vi * 16ull));
+            raw[slot][j] = make_uint4(v.x, v.y, v.z, v.w);
+        }
+    };
+    // Only the first sub-tile for now: a compute unit holds about that much in flight, further loads would wait at
+    // issue until data returns and hold up the barriers of the set-up below. The rest of the ring follows once the
+    // bitmap is built.
+    load(0, 0);
+    // while all that is on its way: an empty bitmap of the row's history
+    uint32_t* window = fused_lds_bitmap<BMW>();
+    if (hist) {
+        const int words = min(BMW, (p.V + 31) / 32 + 1);
+        for (int i = t; i < words; i += RW_THREADS) {
+            window[i] = 0u;
+        }
+    }
+    if (t == 0) {
+        s.n_out = 0;
+    }
+    lds_barrier();
+
+    FusedRow<DT, BMW> rowctx(p, row, args);
+    if (skip || fin) {
+        if (fin && !skip && t == 0) {
+            l.ids[row] = args.end_id;
+        }
+        return;
+    }
+    // the row's draw: taken once, by the rows that take part (like the reference's curand_uniform)
+    if (t == 0) {
+        float u = draw.injected;
+        if (!injected) {
+            uint64_t next;
+            u = row_draw_generate(draw, &next);
+            *(__attribute__((address_space(1))) uint64_t*)counter_addr = next;
+        }
+        ts.misc[0] = __float_as_int(u);
+    }
+    if (hist) {
+#pragma unroll
+        for (int u = 0; u < RW_HIST_U; ++u) {
+            const int pos = t + u * RW_THREADS;
+            const int id  = hist_ids[u];
+            if (pos < p.step && id >= 0 && id < p.V && rowctx.history_position_counts(pos)) {
+                atomicOr(&window[id >> 5], 1u << (id & 31));
+            }
+        }
+        rowctx.bm_mode   = 1;
+        rowctx.bm_origin = 0;
+    }
+    lds_barrier();
+#pragma unroll
+    for (int r = 1; r < R; ++r) {
+        load(r, r);  // (rows have at least RW_MIN_SUBS >= R sub-tiles)
+    }
+    RW_STAMP(1)
+    const bool     bitsv   = hist;
+    const uint32_t KMIN    = min_valid_key<DT>();
+    const float    NEG_INF = -__builtin_inff();
+    const float    mul     = rowctx.fast_mul;
+    // a multiplier that is not positive and finite does not keep the order: every vector is evaluated exactly
+    const bool all_hit = !(mul > 0.0f && mul < __builtin_inff());
+
+    uint32_t thr     = KMIN;  // candidates are the elements with key >= thr
+    float    thr_f   = key_to_float(thr);
+    float    thr_hot = NEG_INF;  // (without a bound every vector is looked at exactly)
+    auto     set_threshold = [&](uint32_t key) {
+        thr     = key;
+        thr_f   = key_to_float(key);
+        // What the unrounded, unpenalised product of an element must reach for its final value to reach thr_f:
+        // rounding to T can lift a product by half a unit of T, and a history penalty that raises values
+        // (a multiplicative one below 1, a negative additive one) can lift it further.
+        float h = lean_below_rounding<DT>(thr_f);
+        if (bitsv) {
+            const float pen = rowctx.penalty;
+            float       g   = h;
+            bool        raises;
+            if (rowctx.penalty_type == 0) {
+                raises = !(pen >= 0.0f);
+                g      = h + pen;
+            }
+            else {
+                raises = !(pen >= 1.0f);
+                g      = (pen > 0.0f && pen < 1.0f) ? (h > 0.0f ? h * pen : h / pen) : NEG_INF;
+            }
+            if (raises) {
+                g = g - (__builtin_fabsf(g) * 9.5367431640625e-07f + 1.0e-37f);
+                g = lean_below_rounding<DT>(g);
+                h = __builtin_fminf(h, g);
+            }
+        }
+        if (!(h == h) || !(__builtin_fabsf(thr_f) < __builtin_inff())) {
+            h = NEG_INF;
+        }
+        thr_hot = uniform_f(h);
+    };
+
+    // flags of the vector that starts at column `first` (a multiple of EPV): one bit per column of the history
+    auto vector_flags = [&](int first) -> uint32_t {
+        return bitsv ? (window[first >> 5] >> (first & 31)) & ((1u << EPV) - 1u) : 0u;
+    };
+
+    // ---- first bound: the k-th largest of 256 maxima over the first sub-tile (the first of the row to arrive).
+    // Only vectors whose elements all take the plain transform count (no history column in the 32-column word of
+    // the bitmap around them, not the masked end id), so that every maximum is the final value of an element.
+    {
+        uint32_t word[RW_NV];
+#pragma unroll
+        for (int j = 0; j < RW_NV; ++j) {
+            word[j] = bitsv ? window[((j * RW_THREADS + t) * EPV) >> 5] : 0u;  // (inside the row: nsub >= 2)
+        }
+        float tmax = NEG_INF;
+#pragma unroll
+        for (int j = 0; j < RW_NV; ++j) {
+            const int   first = (j * RW_THREADS + t) * EPV;
+            const bool  clean = word[j] == 0u && rowctx.interior_vector(first, EPV);
+            const float vm    = lean_raw_max<DT>(raw[0][j]);
+            tmax              = __builtin_fmaxf(tmax, clean ? vm : NEG_INF);
+        }
+        tmax = all_hit ? NEG_INF : rowctx.fast(tmax);  // (the transform keeps the order)
+        const uint32_t P = rowwide_bound(s, order_key(tmax), k);
+        if (P >= KMIN) {
+            set_threshold(P);
+        }
+    }
+
+    RW_STAMP(2)
+    // ---- parking and exact evaluation
+    int      wcount = 0;   // vectors parked by this wave (wave-uniform)
+    int      rot    = 0;   // spreads the evaluated vectors over the lanes from one evaluation to the next
+    uint32_t dmax   = 0u;  // largest key this lane has put on the list
+    // Evaluate what the wave has parked: one vector per lane and round. The elements that reach the bound get
+    // their slots on the row's list with one LDS atomic per round.
+    auto drain = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        const int staged = wcount;
+        for (int e0 = 0; e0 < staged; e0 += WAVE) {
+            const int  e    = e0 + ((lane - rot) & (WAVE - 1));
+            const bool have = e < staged;
+            float      x[EPV];
+            uint32_t   mask  = 0u;
+            int        first = 0;
+            if (have) {
+                const uint4 v       = s.stage_raw[wv][e];
+                first               = s.stage_first[wv][e];
+                const uint32_t bits = vector_flags(first);
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    x[c] = rowctx.fast(vector_element<DT>(v, c));
+                }
+                if (bits != 0u) {  // rare: a column of the history
+#pragma unroll
+                    for (int c = 0; c < EPV; ++c) {
+                        if ((bits >> c) & 1u) {
+                            x[c] = rowctx.flagged(x[c]);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    mask |= x[c] >= thr_f ? (1u << c) : 0u;
+                }
+                const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - first);  // the masked end id is no candidate
+                mask &= rel_end < (uint32_t)EPV ? ~(1u << rel_end) : ~0u;
+            }
+            const int cnt = __builtin_popcount(mask);
+            int       pre = 0, total = 0;
+#pragma unroll
+            for (int bit = 0; (1 << bit) <= EPV; ++bit) {
+                const unsigned long long bm = __ballot((cnt >> bit) & 1);
+                pre += (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(bm >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)bm, 0u))
+                       << bit;
+                total += (int)__builtin_popcountll(bm) << bit;
+            }
+            if (total > 0) {
+                int base_slot = 0;
+                if (lane == 0) {
+                    base_slot = atomicAdd(&s.n_out, total);
+                }
+                int slot = __builtin_amdgcn_readfirstlane(base_slot) + pre;
+#pragma unroll
+                for (int c = 0; c < EPV; ++c) {
+                    if ((mask >> c) & 1u) {
+                        const uint32_t key = order_key(x[c]);
+                        if (slot < TK_CCAP) {
+                            ts.cand.key[slot] = key;
+                            ts.cand.idx[slot] = (uint32_t)(first + c);
+                        }
+                        dmax = key > dmax ? key : dmax;
+                        ++slot;
+                    }
+                }
+            }
+        }
+        rot    = (rot + staged) & (WAVE - 1);
+        wcount = 0;
+    };
+    static_assert(RW_STAGE >= LG_DRAIN_AT - 1 + RW_PARK_GROUP * WAVE, "a group of vectors always fits the parking list");
+    static_assert(RW_NV % RW_PARK_GROUP == 0, "whole groups per sub-tile");
+    auto park = [&](bool hit, const uint4& v, int first) {
+        const unsigned long long m = __ballot(hit);
+        if (m != 0ull) {
+            if (hit) {
+                const int slot = wcount
+                                 + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                                  __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                s.stage_raw[wv][slot]   = v;
+                s.stage_first[wv][slot] = first;
+            }
+            wcount += (int)__builtin_popcountll(m);
+        }
+    };
+
+    // ---- the stream. The bound is raised again after 2, 4, 8, ... sub-tiles: the k-th largest of the largest
+    // candidates of disjoint groups of lanes bounds the k-th largest of everything seen so far. (The ring holds
+    // several microseconds of the compute unit's share of the bandwidth: memory does not wait for these pauses.)
+    int next_tighten = 2;
+    for (int q0 = 0; q0 < nsub; q0 += R) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int q = q0 + r;
+            if (q < nsub) {
+#pragma unroll
+                for (int j = 0; j < RW_NV; ++j) {
+                    const int   rel = q * RW_SUB_VECS + j * RW_THREADS + t;
+                    const float m   = lean_raw_max<DT>(raw[r][j]) * mul;
+                    park((all_hit || m >= thr_hot) && rel < nvec, raw[r][j], rel * EPV);
+                    if ((j + 1) % RW_PARK_GROUP == 0 && j + 1 < RW_NV && wcount >= LG_DRAIN_AT) {
+                        drain();
+                    }
+                }
+                if (q + R < nsub) {
+                    load(r, q + R);
+                }
+                const bool tighten = q + 1 == next_tighten && q + 1 < nsub;
+                if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
+                    drain();
+                }
+                if (tighten) {
+                    next_tighten *= 2;
+                    const uint32_t P = rowwide_bound(s, dmax, k);
+                    if (P > thr) {
+                        set_threshold(P);
+                    }
+                }
+            }
+        }
+    }
+
+    RW_STAMP(3)
+    // ---- the columns behind the last whole vector, one by one (fewer than a vector's worth)
+    {
+        const int v = nvec * EPV + t;
+        if (v < p.V && !rowctx.never_selected(v)) {
+            const float xv = topk_value_at<DT>(rowctx, v);
+            if (xv >= thr_f) {
+                const int slot = atomicAdd(&s.n_out, 1);
+                if (slot < TK_CCAP) {
+                    ts.cand.key[slot] = order_key(xv);
+                    ts.cand.idx[slot] = (uint32_t)v;
+                }
+            }
+        }
+    }
+    lds_barrier();
+    RW_STAMP(4)
+    if (wv >= TK_WAVES) {
+        return;  // the first four waves, one per SIMD, select
+    }
+    TopkOutputs out;
+    out.ids                = l.ids;
+    out.sequence_length    = l.sequence_length;
+    out.finished           = l.finished;
+    out.cum_log_probs      = nullptr;
+    out.output_log_probs   = nullptr;
+    out.sequence_length_in = seq_in;
+    out.cum_log_prob_in    = 0.0f;
+    out.end_id_in          = args.end_id;
+    int         n = s.n_out;
+    const float u = __int_as_float(ts.misc[0]);
+    if (n > k + k / 2 && n > 96 && n <= 4 * TK_THREADS) {
+        // Far more candidates than needed: raise the bound once more, to the k-th largest of 256 disjoint groups of
+        // the list's own entries (at least k entries reach it), and keep what reaches it. The ranking compares every
+        // candidate with every other one; this keeps it short.
+        uint32_t ck[4], ci[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int i = t + r * TK_THREADS;
+            ck[r]       = i < n ? ts.cand.key[i] : 0u;
+            ci[r]       = i < n ? ts.cand.idx[i] : 0u;
+        }
+        s.slot_key[t] = max(max(ck[0], ck[1]), max(ck[2], ck[3]));
+        if (t == 0) {
+            ts.n_cand = 0;
+        }
+        lds_barrier();
+        const uint32_t P = lean_kth_of_slots(s.slot_key, k);
+        if (P > thr) {
+            thr = P;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool               keep = ck[r] >= P;  // (the slots past the list hold 0 < P)
+                const unsigned long long m    = __ballot(keep);
+                int                      at   = 0;
+                if (lane == 0 && m != 0ull) {
+                    at = atomicAdd(&ts.n_cand, (int)__builtin_popcountll(m));
+                }
+                at = __builtin_amdgcn_readfirstlane(at);
+                if (keep) {
+                    const int slot = at
+                                     + (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                    ts.cand.key[slot] = ck[r];
+                    ts.cand.idx[slot] = ci[r];
+                }
+            }
+            lds_barrier();
+            n = ts.n_cand;
+        }
+    }
+    if (n <= 256) {
+        const int n_list = rowwide_rank(ts, n, k, p.max_top_k);
+        topk_finish_list<DT>(ts, n_list, row, p.Vp, tp, false, u, p.end_ids, out);
+    }
+    else {
+        rowwide_rare<DT>(ts, p, l, args, row, n, thr, k, tp, u, out);
+    }
+    RW_STAMP(6)
+}
+
+// Launchers, one per element type (lean_kernels.hip). window: 1 = the row's bitmap fits the small LDS window,
+// 2 = the large one. start / stop: optional events carried by the launch.
+int rowwide_launch_f32(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+                       hipEvent_t stop);
+int rowwide_launch_f16(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start,
+                       hipEvent_t stop);
+int rowwide_launch_bf16(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                        hipEvent_t start, hipEvent_t stop);
+
+}  // namespace ftk

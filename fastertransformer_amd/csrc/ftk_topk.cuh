@@ -1157,6 +1157,34 @@ __device__ __forceinline__ void topk_emit(const TopkOutputs& o, int row, int id,
     }
 }
 
+// The end of the selection, by the TK_THREADS threads that are left of a workgroup: the ordered list (values in
+// s.sel.w, columns in s.sel.idx, n_list entries) -> weights (sampling_topk_kernels.cu:264-279: exp(x - max) on
+// logits, the value itself on probabilities), the sequential sum and walk of the reference by thread 0, the row's
+// outputs. The list is padded with zero weights to a multiple of 32 for the walk, which reads 32 at a time.
+template<int DT>
+__device__ __forceinline__ void topk_finish_list(TopkShared& s, int n_list, int row, int vocab, float p, bool probs_in,
+                                                 float u, const int* end_ids, const TopkOutputs& out)
+{
+    const int   t  = threadIdx.x;
+    const float x0 = n_list > 0 ? s.sel.w[0] : 0.0f;
+    __syncthreads();
+    for (int i = t; i < ((n_list + 31) & ~31); i += TK_THREADS) {
+        const float x = i < n_list ? s.sel.w[i] : 0.0f;
+        s.sel.w[i]    = i < n_list ? (probs_in ? x : det_expf(x - x0)) : 0.0f;
+    }
+    __syncthreads();
+    if (t == 0) {
+        if (n_list == 0) {
+            topk_emit(out, row, 0, probs_in, 0.0f, 0.0f, end_ids, false);
+        }
+        else {
+            float     s_sum;
+            const int pick = topk_sample_walk(s.sel.w, n_list, u, p, &s_sum);
+            topk_emit(out, row, s.sel.idx[pick] % vocab, probs_in, s.sel.w[pick], s_sum, end_ids, true);
+        }
+    }
+}
+
 // Literal replay for rows the gather could not bound. `Row::key_at(v)` re-reads the row.
 // Every pick is the smallest composite key strictly greater than the previous pick, where the
 // composite encodes the reference's order; picks of stage 1 go to `picks` (8k entries, global).
@@ -1681,25 +1709,7 @@ __device__ __forceinline__ void topk_select_lds(Row& rowctx, TopkShared& s, int 
         __syncthreads();
     }
 
-    // ---- weights (sampling_topk_kernels.cu:264-279): exp(x - max) on logits, the value itself on
-    // probabilities; the list is padded with zero weights to a multiple of 32 for the walk, which reads 32 at a time
-    const float x0 = n_list > 0 ? s.sel.w[0] : 0.0f;
-    __syncthreads();
-    for (int i = t; i < ((n_list + 31) & ~31); i += TK_THREADS) {
-        const float x = i < n_list ? s.sel.w[i] : 0.0f;
-        s.sel.w[i]        = i < n_list ? (probs_in ? x : det_expf(x - x0)) : 0.0f;
-    }
-    __syncthreads();
-    if (t == 0) {
-        if (n_list == 0) {
-            topk_emit(out, row, 0, probs_in, 0.0f, 0.0f, end_ids, false);
-        }
-        else {
-            float     s_sum;
-            const int pick = topk_sample_walk(s.sel.w, n_list, u, p, &s_sum);
-            topk_emit(out, row, s.sel.idx[pick] % vocab, probs_in, s.sel.w[pick], s_sum, end_ids, true);
-        }
-    }
+    topk_finish_list<DT>(s, n_list, row, vocab, p, probs_in, u, end_ids, out);
 }
 
 // What a select workgroup asks for before it knows anything about its row: wave w takes the first

@@ -24,6 +24,7 @@
 #include "ftk_fused.cuh"
 #include "ftk_lean.cuh"
 #include "ftk_logprob.cuh"
+#include "ftk_rowwide.cuh"
 
 namespace ftk {
 
@@ -173,9 +174,18 @@ extern "C" void ftk_test_set_fused_two_launches(int v)
 {
     g_fused_two_launches = v;
 }
+// Test hook: which kernels the last fused step launched. 0: general stream, 1: lean gather + select, 2: lean gather
+// that also selects (one 256-thread workgroup per row), 3: one 1024-thread workgroup per row, 4: log-prob step.
+static int g_fused_last_path = -1;
+extern "C" int ftk_test_last_fused_path(void)
+{
+    return g_fused_last_path;
+}
+#define FTK_NOTE_PATH(v) (g_fused_last_path = (v))
 #else
 static constexpr int g_fused_force_general = 0;
 static constexpr int g_fused_two_launches  = 0;
+#define FTK_NOTE_PATH(v) ((void)0)
 #endif
 
 extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
@@ -218,6 +228,17 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             || ((uintptr_t)a->logits % (uintptr_t)elem) != 0)) {
         return FTK_ERR_UNSUPPORTED;
     }
+    // About one row per compute unit (or a few rounds of that), a small k, long rows, no bias: a 1024-thread
+    // workgroup per row does the whole step in one launch (ftk_rowwide.cuh). It pays when the rounds of 256
+    // workgroups are nearly full and the row's history bitmap fits its LDS window.
+    const int  rw_rounds = (rows + 255) / 256;
+    const bool rowwide   = lean_mode == 1 && !want_log_probs && a->embedding_bias == nullptr && lplan.splits > 1
+                         && g_fused_two_launches == 0 && rows * 5 >= rw_rounds * 256 * 4
+                         && (size_t)a->vocab_size / (16 / elem) >= (size_t)RW_MIN_SUBS * RW_SUB_VECS
+                         && (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_LARGE
+                         && ((uintptr_t)a->logits & 15u) == 0 && ((size_t)a->vocab_size_padded * elem) % 16 == 0
+                         && (a->penalty_type == FTK_PENALTY_NONE || a->penalties == nullptr
+                             || a->step <= RW_HIST_U * RW_THREADS);
     const size_t   slot_bytes = lean_mode == 2 ? (size_t)lplan.splits * slot_u * LG_THREADS * sizeof(uint32_t) : 0;
     const size_t   lean_bytes =
         (size_t)(rows > 0 ? rows : 0)
@@ -279,7 +300,10 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && (many == 0 || lean_mode != 0)
                            && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1 && !want_log_probs
                                || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
-        if (local) {
+        if (rowwide) {
+            p.lds_window = (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
+        }
+        else if (local) {
             p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
         }
         else {
@@ -338,6 +362,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         l.entries      = (TopkEntry*)(l.headers + (size_t)rows * lplan.splits);
         const dim3 lgrid(lplan.splits, rows);
         if (want_log_probs) {
+            FTK_NOTE_PATH(4);
             LogProbLaunch lp;
             lp.cum_log_probs    = a->cum_log_probs;
             lp.output_log_probs = a->output_log_probs;
@@ -369,9 +394,19 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             }
             return rc;
         }
+        if (rowwide) {
+            FTK_NOTE_PATH(3);
+            hipEvent_t e0, e1;
+            take_events(1, &e0, &e1);
+            const int w = p.lds_window == 2 ? 2 : 1;
+            return a->dtype == FTK_DTYPE_F32 ? rowwide_launch_f32(w, rows, st, p, l, e0, e1) :
+                   a->dtype == FTK_DTYPE_F16 ? rowwide_launch_f16(w, rows, st, p, l, e0, e1) :
+                                               rowwide_launch_bf16(w, rows, st, p, l, e0, e1);
+        }
         // one workgroup per row: it also orders and samples, the step is one launch
         const bool row_select =
             lean_mode == 1 && lplan.splits == 1 && a->embedding_bias == nullptr && g_fused_two_launches == 0;
+        FTK_NOTE_PATH(row_select ? 2 : 1);
         auto launch_lean = [&](int mode, int timer) -> int {
             hipEvent_t e0, e1;
             take_events(timer, &e0, &e1);
@@ -405,6 +440,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         }
         return lean_select_launch_bf16(rows, st, p, l, e0, e1);
     }
+    FTK_NOTE_PATH(0);
     if (plan.splits == 1) {
         return launch_general(FUSED_KIND_ROW, window, dim3(rows));
     }

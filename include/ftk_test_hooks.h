@@ -31,6 +31,10 @@ void ftk_test_set_fused_force_general(int enable);
 /* non-zero: the fused step keeps gather and selection in two launches also where one workgroup per row could do
    both in one; process-wide */
 void ftk_test_set_fused_two_launches(int enable);
+/* which kernels the last fused step of this process launched: 0 general stream, 1 lean gather + select, 2 lean gather
+   that also selects (one 256-thread workgroup per row), 3 one 1024-thread workgroup per row, 4 log-prob step;
+   -1 before the first step */
+int ftk_test_last_fused_path(void);
 
 #ifdef __cplusplus
 }
