@@ -27,6 +27,14 @@ constexpr int RW_PARK_GROUP = 2;                    // vectors a wave parks betw
 constexpr int RW_STAGE      = LG_DRAIN_AT + RW_PARK_GROUP * WAVE;
 constexpr int RW_HIST_U     = 4;                    // history ids a thread requests before the logits: the longest
                                                     // history the kernel takes is RW_HIST_U * RW_THREADS positions
+#ifndef FTK_RW_T1
+#define FTK_RW_T1 6
+#endif
+#ifndef FTK_RW_GAP
+#define FTK_RW_GAP 2
+#endif
+constexpr int RW_FIRST_TIGHTEN = FTK_RW_T1;
+constexpr int RW_TAIL_GAP      = FTK_RW_GAP;
 constexpr int RW_MIN_SUBS   = 4;                    // shortest row the launcher sends here, in sub-tiles
 
 struct RowwideShared {
@@ -34,7 +42,7 @@ struct RowwideShared {
     int      stage_first[RW_WAVES][RW_STAGE];
     uint32_t slot_key[RW_THREADS];
     uint32_t bound;
-    int      n_out;
+    int      n_list[2];  // length of the row's list; the second counter takes over when the list is pruned
 };
 
 // The largest value P, to within its low sixteen bits, such that at least k of 256 keys are >= P (0 when fewer
@@ -179,6 +187,75 @@ __device__ __forceinline__ int rowwide_rank(TopkShared& s, int n, int k, int max
     return n_list;
 }
 
+// The usual case of rowwide_rank in one counting pass over 32-bit keys: when the candidates' keys are all different
+// and no stage-1 slice holds more than k of them, stage 1 drops none of them and both tie rules are idle, so the
+// reference's list is the candidates in descending order of value, cut at k. Returns the length of the list (in
+// s.sel, like rowwide_rank), or -1 when one of the two conditions fails (s.cand is left as it was). Called by the
+// first TK_THREADS threads; n <= 256.
+__device__ __forceinline__ int rowwide_rank_distinct(TopkShared& s, int n, int k, int max_top_k)
+{
+    const int      t       = threadIdx.x;
+    const int      bs1_log = max_top_k <= 16 ? 7 : 8;
+    const uint32_t my_key  = t < n ? s.cand.key[t] : 0u;
+    const uint32_t my_idx  = t < n ? s.cand.idx[t] : 0u;
+    int*           cnt     = s.sel.idx + 1024;  // 2 x 256 counts, clear of the list this function writes
+    int            CP      = 4;
+    while (CP < n) {
+        CP <<= 1;
+    }
+    const int parts = TK_THREADS / CP;
+    const int c     = t & (CP - 1);
+    const int part  = t / CP;
+    const int quads = (n + 3) >> 2;
+    const int per   = (quads + parts - 1) / parts;
+    const int jlo   = min(quads, part * per) * 4;
+    const int jhi   = min(quads, part * per + per) * 4;
+    if (t < 4) {
+        s.cand.key[n + t] = 0u;  // the last four keys read may lie past the list: a key that is above nothing
+    }
+    if (t < 8) {
+        s.slice_count[t] = 0;
+    }
+    cnt[t]              = 0;
+    cnt[TK_THREADS + t] = 0;
+    if (t == 0) {
+        s.misc[1] = 0;
+    }
+    lds_barrier();
+    if (t < n) {
+        atomicAdd(&s.slice_count[(my_idx >> bs1_log) & 7u], 1);
+    }
+    {
+        const uint32_t key = c < n ? s.cand.key[c] : 0xFFFFFFFFu;
+        int            above = 0, equal = 0;
+#pragma unroll 2
+        for (int j = jlo; j < jhi; j += 4) {
+            const uint4 kk = *reinterpret_cast<const uint4*>(&s.cand.key[j]);
+            above += (kk.x > key ? 1 : 0) + (kk.y > key ? 1 : 0) + (kk.z > key ? 1 : 0) + (kk.w > key ? 1 : 0);
+            equal += (kk.x == key ? 1 : 0) + (kk.y == key ? 1 : 0) + (kk.z == key ? 1 : 0) + (kk.w == key ? 1 : 0);
+        }
+        if (c < n && jhi > jlo) {
+            atomicAdd(&cnt[c], above);
+            atomicAdd(&cnt[TK_THREADS + c], equal);
+        }
+    }
+    lds_barrier();
+    if (t < n && (cnt[TK_THREADS + t] != 1 || s.slice_count[(my_idx >> bs1_log) & 7u] > k)) {
+        s.misc[1] = 1;
+    }
+    lds_barrier();
+    if (s.misc[1] != 0) {
+        return -1;
+    }
+    const int n_list = min(k, n);
+    if (t < n && cnt[t] < n_list) {
+        s.sel.w[cnt[t]]   = key_to_float(my_key);
+        s.sel.idx[cnt[t]] = (int)my_idx;
+    }
+    lds_barrier();
+    return n_list;
+}
+
 // What is left to the first four waves when a row's list is still longer than 256 entries after the cut (the
 // selection of topk_select_lds for long lists) or outgrew LDS (the whole row is walked again with the stream that
 // recovers from overfull tiles; rows it cannot bound either take the literal replay). Not inlined, so that the
@@ -304,7 +381,8 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         }
     }
     if (t == 0) {
-        s.n_out = 0;
+        s.n_list[0] = 0;
+        s.n_list[1] = 0;
     }
     lds_barrier();
 
@@ -415,6 +493,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
 
     RW_STAMP(2)
     // ---- parking and exact evaluation
+    int      cur    = 0;   // which counter holds the length of the list
     int      wcount = 0;   // vectors parked by this wave (wave-uniform)
     int      rot    = 0;   // spreads the evaluated vectors over the lanes from one evaluation to the next
     uint32_t dmax   = 0u;  // largest key this lane has put on the list
@@ -466,7 +545,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
             if (total > 0) {
                 int base_slot = 0;
                 if (lane == 0) {
-                    base_slot = atomicAdd(&s.n_out, total);
+                    base_slot = atomicAdd(&s.n_list[cur], total);
                 }
                 int slot = __builtin_amdgcn_readfirstlane(base_slot) + pre;
 #pragma unroll
@@ -502,10 +581,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         }
     };
 
-    // ---- the stream. The bound is raised again after 2, 4, 8, ... sub-tiles: the k-th largest of the largest
+    // ---- the stream. The bound is raised again after 2, 4, 6, 8, 16, ... sub-tiles: the k-th largest of the largest
     // candidates of disjoint groups of lanes bounds the k-th largest of everything seen so far. (The ring holds
     // several microseconds of the compute unit's share of the bandwidth: memory does not wait for these pauses.)
-    int next_tighten = 2;
+    int next_tighten = RW_FIRST_TIGHTEN;  // then twice that plus two, ...
     for (int q0 = 0; q0 < nsub; q0 += R) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -523,15 +602,51 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
                 if (q + R < nsub) {
                     load(r, q + R);
                 }
-                const bool tighten = q + 1 == next_tighten && q + 1 < nsub;
-                if (wcount >= LG_DRAIN_AT || tighten || q + 1 == nsub) {
+                // Once or twice per row the bound is raised and the list pruned (after 6, 14, 30, ... sub-tiles while
+                // more than four remain, and two sub-tiles before the end, so that the selection at the end starts
+                // from little more than k candidates). Every pause of the whole workgroup costs about a
+                // microsecond of the stream, which is why there are so few.
+                const int  done    = q + 1;
+                const bool tighten = (done == next_tighten && done + RW_TAIL_GAP + 2 <= nsub) || (done + RW_TAIL_GAP == nsub && nsub >= 4);
+                if (wcount >= LG_DRAIN_AT || tighten || done == nsub) {
                     drain();
                 }
                 if (tighten) {
-                    next_tighten *= 2;
-                    const uint32_t P = rowwide_bound(s, dmax, k);
+                    if (done == next_tighten) {
+                        next_tighten = 2 * next_tighten + 2;
+                    }
+                    lds_barrier();  // every wave has evaluated what it had parked: the list is complete so far
+                    const int      n_now   = s.n_list[cur];
+                    const bool     listed  = n_now <= RW_THREADS;  // one entry per thread
+                    const uint32_t key     = t < n_now ? ts.cand.key[t] : 0u;
+                    const uint32_t idx     = t < n_now ? ts.cand.idx[t] : 0u;
+                    // the k-th largest of 256 disjoint groups of the list's entries; of the lanes' largest entries when
+                    // the list is longer than the workgroup
+                    const uint32_t P = rowwide_bound(s, listed ? key : dmax, k);
                     if (P > thr) {
                         set_threshold(P);
+                        if (listed) {
+                            // entries below the new bound (collected under an older one) leave the list
+                            const bool               keep = key >= P;  // (P > 0: the slots past the list drop out)
+                            const unsigned long long m    = __ballot(keep);
+                            int                      at   = 0;
+                            if (lane == 0 && m != 0ull) {
+                                at = atomicAdd(&s.n_list[cur ^ 1], (int)__builtin_popcountll(m));
+                            }
+                            at = __builtin_amdgcn_readfirstlane(at);
+                            if (keep) {
+                                const int slot = at
+                                                 + (int)__builtin_amdgcn_mbcnt_hi(
+                                                     (uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+                                ts.cand.key[slot] = key;
+                                ts.cand.idx[slot] = idx;
+                            }
+                            lds_barrier();
+                            if (t == 0) {
+                                s.n_list[cur] = 0;  // (not looked at before the next pruning, several barriers away)
+                            }
+                            cur ^= 1;
+                        }
                     }
                 }
             }
@@ -545,7 +660,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         if (v < p.V && !rowctx.never_selected(v)) {
             const float xv = topk_value_at<DT>(rowctx, v);
             if (xv >= thr_f) {
-                const int slot = atomicAdd(&s.n_out, 1);
+                const int slot = atomicAdd(&s.n_list[cur], 1);
                 if (slot < TK_CCAP) {
                     ts.cand.key[slot] = order_key(xv);
                     ts.cand.idx[slot] = (uint32_t)v;
@@ -567,7 +682,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
     out.sequence_length_in = seq_in;
     out.cum_log_prob_in    = 0.0f;
     out.end_id_in          = args.end_id;
-    int         n = s.n_out;
+    int         n = s.n_list[cur];
     const float u = __int_as_float(ts.misc[0]);
     if (n > k + k / 2 && n > 96 && n <= 4 * TK_THREADS) {
         // Far more candidates than needed: raise the bound once more, to the k-th largest of 256 disjoint groups of
@@ -610,7 +725,15 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         }
     }
     if (n <= 256) {
-        const int n_list = rowwide_rank(ts, n, k, p.max_top_k);
+        RW_STAMP(5)
+        int n_list = rowwide_rank_distinct(ts, n, k, p.max_top_k);
+        if (n_list < 0) {
+            n_list = rowwide_rank(ts, n, k, p.max_top_k);
+        }
+        RW_STAMP(7)
+#ifdef FTK_RW_STAMPS
+        if (threadIdx.x == 0) { stamps[9] = (unsigned long long)n; }
+#endif
         topk_finish_list<DT>(ts, n_list, row, p.Vp, tp, false, u, p.end_ids, out);
     }
     else {
