@@ -165,8 +165,13 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     alg = algorithmic_bytes(w, mid_step)
     gather_ms = kernel_ms[1]
     achieved = alg / (gather_ms * 1e-3) / 1e9 if gather_ms > 0 else 0.0
-    # launches without a bias stream with the lean gather (largest k beyond 128: twice, maxima first)
-    dominant = "lean_gather_kernel"
+    # Which kernel streams the logits: one 1024-thread workgroup per row does the whole step in one launch where the
+    # batch fills the chip in nearly full rounds of 256 rows (rowwide_step_kernel); otherwise the lean gather
+    # (largest k beyond 192: twice, maxima first) followed by a selection launch. Timer 1 carries either.
+    rounds = (B + 255) // 256
+    rowwide = (not isinstance(w["top_k"], tuple) and w["top_k"] <= 192 and B < 1024 and B * 5 >= rounds * 256 * 4
+               and V // (16 // (4 if w["dtype"] == "f32" else 2)) >= 4 * 4096)
+    dominant = "rowwide_step_kernel" if rowwide else "lean_gather_kernel"
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
         kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2], maxima=kernel_ms[3]),
@@ -437,6 +442,129 @@ def run_gpu_beam(name, w, steps, warmup):
                 ids_checksum=checksum)
 
 
+# ---- the other BASELINE configurations: short timed runs and a one-step oracle check each -------------------------
+
+SECONDARY = [
+    "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9",
+    "decode_step_b256_v51200_f16_topk1-1024_topp0.9_temp0.8_rep1.1",
+    "decode_loop_b1024_v152064_f16_topk64_topp0.9_logprobs",
+    "decode_loop_b128_v32000_bf16_hist2048_presence0.5_freq0.3_minlen_badwords_stopwords_topk50",
+]
+
+
+def _secondary_case(name, w, rng):
+    """the workload as one decode step of the test harness: (Case arguments, logits [B, Vp] as numpy storage, step)"""
+    import ft_oracle as O
+    from helpers import make_word_list
+    dt = {"f32": O.F32, "f16": O.F16, "bf16": O.BF16}[w["dtype"]]
+    B, V, Vp, H = w["batch"], w["vocab"], w["vocab_padded"], w["prompt"]
+    kw = dict(max_input_length=H, gen_len=1)
+    if name.startswith("topp_step"):
+        base = -w["zipf_s"] * np.log(np.arange(1, V + 1, dtype=np.float64))
+        base = (base - np.log(np.exp(base).sum())).astype(np.float32)
+        x = rng.standard_normal((B, V), dtype=np.float32) * np.float32(w["noise"])
+        for b in range(B):
+            x[b] += base[rng.permutation(V)]
+        lo, hi = w["top_p"]
+        kw.update(runtime_top_k=[0], runtime_top_p=rng.uniform(lo, hi, B), top_p_decay=np.full(B, w["top_p_decay"]),
+                  top_p_min=np.full(B, w["top_p_min"]), top_p_reset_ids=np.full(B, w["top_p_reset_id"]))
+        return dt, kw, x, 0
+    x = O.to_storage(rng.standard_normal((B, Vp), dtype=np.float32) * np.float32(w["sigma"]), dt)
+    if "zipf_history" in w:
+        prompt = np.minimum(rng.zipf(w["zipf_history"], (H, B)), V - 1).astype(np.int32)
+    else:
+        prompt = rng.integers(0, V, (H, B)).astype(np.int32)
+    if isinstance(w["top_k"], tuple):
+        top_ks = np.random.default_rng(0).choice(np.array(w["top_k"], np.uint32), B).astype(np.uint32)
+    else:
+        top_ks = [w["top_k"]]
+    kw.update(runtime_top_k=top_ks, runtime_top_p=[w["top_p"]], temperature=[w["temperature"]], prompt=prompt,
+              end_ids=np.full(B, w.get("end_id", V - 1), np.int32))
+    for key in ("repetition_penalty", "presence_penalty", "frequency_penalty"):
+        if w.get(key) is not None:
+            kw[key] = [w[key]]
+    if "min_length_beyond" in w:
+        kw["min_length"] = [H + w["min_length_beyond"]]
+    if name.startswith("decode_loop"):
+        kw["sequence_limit_length"] = np.full(B, H + 8, np.uint32)
+        if w.get("logprobs", True):
+            kw.update(with_cum=True, with_out_lp=True)
+    if w.get("bad_words"):
+        n, longest = w["bad_words"]
+        kw["bad_words"] = np.stack([make_word_list(rng, n, longest, V, L=n * longest)[0] for _ in range(B)])
+    if w.get("stop_words"):
+        n, longest = w["stop_words"]
+        kw["stop_words"] = np.stack([make_word_list(rng, n, longest, V, L=n * longest)[0] for _ in range(B)])
+    return dt, kw, x, H
+
+
+def secondary_oracle_check(name, w, rows_checked=None):
+    """One step of the workload at its full batch through the product's DynamicDecodeLayer, and the same step on the
+    CPU oracle for the first `rows_checked` rows (rows are independent): ids, flags and lengths must be identical,
+    log-probs within the tolerance of the type. Outside every timed region."""
+    import ft_oracle as O
+    from decode_harness import Case, OracleRunner, ProductRunner
+    from helpers import uniforms
+    rng = np.random.default_rng(2025)
+    dt, kw, x, step = _secondary_case(name, w, rng)
+    B, V, Vp = w["batch"], w["vocab"], w["vocab_padded"]
+    n = B if rows_checked is None else min(B, rows_checked)
+    u = uniforms(rng, B)
+    full = Case(dt, B, V, Vp, **kw)
+    product = ProductRunner(full)
+    product.step(step, x, u)
+    got = product.snapshot()
+
+    def cut(key, v):
+        if v is None or np.ndim(v) == 0 or key in ("max_input_length", "gen_len"):
+            return v
+        v = np.asarray(v)
+        if key == "prompt":
+            return v[:, :n]
+        return v[:n] if v.shape[0] == B else v
+    sub = Case(dt, n, V, Vp, **{k: cut(k, v) for k, v in kw.items()})
+    oracle = OracleRunner(sub)
+    oracle.step(step, x[:n].copy(), u[:n])
+    ref = oracle.snapshot()
+    ok = np.array_equal(got["output_ids"][:, :n], ref["output_ids"])
+    for key in ("finished", "sequence_length"):
+        if ref[key] is not None:
+            ok = ok and np.array_equal(got[key][:n], ref[key])
+    rtol = 1e-5 if dt == O.F32 else 2e-3
+    for key in ("cum_log_probs", "output_log_probs"):
+        if ref[key] is not None:
+            a = got[key][..., :n] if key == "output_log_probs" else got[key][:n]
+            ok = ok and bool(np.allclose(a, ref[key], rtol=rtol, atol=1e-6))
+    return dict(rows=n, of=B, step=int(step), ids_checksum=int(ref["output_ids"][step].astype(np.int64).sum()),
+                identical=bool(ok))
+
+
+def run_secondary(steps, warmup):
+    """the other configurations of the benchmark set, a few steps each: per-step time, algorithmic bytes per step,
+    their share of the HBM peak, and the one-step oracle check"""
+    out = []
+    for name in SECONDARY:
+        w = WORKLOADS[name]
+        elem = 4 if w["dtype"] == "f32" else 2
+        if name.startswith("topp_step"):
+            r = run_gpu_topp(name, w, steps, warmup)
+            ms, extra, hist = r["ms_per_step"], dict(p50_ms=r["p50_ms"], max_ms=r["max_ms"]), 0
+        elif name.startswith("decode_loop"):
+            r = run_gpu_loop(name, w, steps, warmup)
+            ms, extra = r["ms_per_step"], dict(p50_ms=r["p50_ms"], p99_ms=r["p99_ms"], max_ms=r["max_ms"])
+            hist = w["prompt"] + warmup + steps // 2
+        else:
+            r = run_gpu(name, w, steps, warmup)
+            ms, extra, hist = r["gpu_ms_per_step"], dict(kernel_ms=r["kernel_ms"]), w["prompt"] + warmup + steps // 2
+        alg = w["batch"] * w["vocab_padded"] * elem + w["batch"] * hist * 4 + w["batch"] * 32
+        check = secondary_oracle_check(name, w, rows_checked=64 if w["batch"] > 256 else None)
+        out.append(dict(workload=name, dtype=w["dtype"], batch=w["batch"], vocab=w["vocab"], steps=steps, warmup=warmup,
+                        ms_per_step=ms, tokens_per_s=w["batch"] / (ms * 1e-3), algorithmic_bytes_per_step=alg,
+                        hbm_gbs=alg / (ms * 1e-3) / 1e9, frac=alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        oracle_check=check, **extra))
+    return out
+
+
 def _oracle_rows_per_second(w, rows, budget_s, seed):
     """the oracle's DynamicDecodeLayer on `rows`-row batches of the workload for about `budget_s` seconds of this
     thread's time; returns (rows done, seconds)"""
@@ -499,6 +627,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the short runs of the other configurations that the default line carries under `configs`")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run five plain device copies of 128 MiB, the known-size kernel that FETCH_SIZE / "
                          "WRITE_SIZE counter readings are scaled by")
@@ -596,6 +726,8 @@ def main():
         "step_hbm_frac": r["step_gbs"] / HBM_PEAK_GBS, "sampled_ids_checksum": r["sampled_ids_checksum"],
         "oracle_check": r["oracle_check"],
     }
+    if not a.no_secondary:
+        line["configs"] = run_secondary(min(a.steps, 20), min(a.warmup, 3))
     if not a.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline(w)
     print(json.dumps(line))
