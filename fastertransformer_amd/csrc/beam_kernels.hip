@@ -688,8 +688,13 @@ beam_update_kernel(bool* __restrict__ finished, int* __restrict__ parent_ids, in
     }
     __syncthreads();
     if (k < K) {
-        const int  beam_id = (word / Vp) % K;
-        const int  word_id = word % Vp;
+        // A slot the step left untouched (an entry that is complete, or one with fewer than K continuations) holds
+        // whatever the caller's buffer held: a negative value counts as "this beam, its end token", so that no index
+        // below leaves its range (the reference reads other rows' memory there; ids are absolute over the batch,
+        // (entry * K + beam) * Vp + token, and any non-negative one is brought into range by the modulo).
+        const bool valid   = word >= 0;
+        const int  beam_id = valid ? (word / Vp) % K : k;
+        const int  word_id = valid ? word % Vp : end_ids[b];
         const bool done    = num_beams != nullptr && num_beams[ite * hyps_local_batch + b] == K;
         sequence_length[i] = counted[beam_id];
         finished[i]        = done || word_id == end_ids[b];

@@ -549,7 +549,14 @@ extern "C" int ftk_measure_plain_read(const void* data, size_t bytes, float* sin
 // Same step, with the workspace taken from a fixed array in device memory instead of the caller. Every GPU
 // the library runs on holds its own copy of the array from the moment the code object is loaded until the
 // process ends; its address on a device is looked up once, with that device current.
-static __device__ __align__(256) unsigned char scratch[FTK_FUSED_STATIC_WORKSPACE_BYTES];
+// (The test build of the library, which a test process loads next to the product library, keeps a token array and
+// refuses every step: one 32 MiB array per GPU and process is enough.)
+#ifdef FTK_TEST_HOOKS
+constexpr size_t FTK_STATIC_BYTES = 256;
+#else
+constexpr size_t FTK_STATIC_BYTES = FTK_FUSED_STATIC_WORKSPACE_BYTES;
+#endif
+static __device__ __align__(256) unsigned char scratch[FTK_STATIC_BYTES];
 
 namespace {
 constexpr int FTK_MAX_DEVICES = 64;
@@ -592,13 +599,13 @@ extern "C" int ftk_fused_topk_step_static(ftk_fused_topk_args* a, ftk_stream_t s
         return rc;
     }
     a->workspace_size = q.workspace_size;  // reported back, so that the caller sees what was needed
-    if (q.workspace_size > (size_t)FTK_FUSED_STATIC_WORKSPACE_BYTES) {
+    if (q.workspace_size > FTK_STATIC_BYTES) {
         return FTK_ERR_STATIC_WORKSPACE;
     }
     // Nothing in the workspace has to start at zero: list headers are written by every streaming workgroup
     // before the merging kernel reads them, lists are read up to the count in their header, and the history
     // bitmaps are cleared by the kernel that fills them.
     q.workspace      = ptr;
-    q.workspace_size = (size_t)FTK_FUSED_STATIC_WORKSPACE_BYTES;
+    q.workspace_size = FTK_STATIC_BYTES;
     return ftk_fused_topk_step(&q, stream);
 }

@@ -250,14 +250,16 @@ void DynamicDecodeLayer<T>::banBadWords(TensorMap* output_tensors, TensorMap* in
     const bool   one_list = rank == 2 || words.shape[0] == 1;
     const size_t length   = words.shape[rank - 1];
     const int*   lists    = one_list ? words.getPtr<const int>() : words.getPtrWithOffset<const int>(first * 2 * length);
-    // (the reference offsets the logits by `first` rows of the vocabulary and the history columns by `first`, whatever
-    // the beam width: layers/DynamicDecodeLayer.cc:261-280)
+    // The window starts `first` entries, that is first * beams rows of logits and columns of the history, into the
+    // batch. (The reference offsets both by `first` whatever the beam width, layers/DynamicDecodeLayer.cc:261-280:
+    // with beams, a later window's bans then land on other beams' rows and follow other beams' histories. Not
+    // reproduced; the stop-word launch of the reference, :449-462, already counts in beams.)
     const size_t beams = input_tensors->at("logits").shape[1];
-    invokeBanBadWords((T*)input_tensors->at("logits").getPtrWithOffset(first * vocab_size_padded_),
+    invokeBanBadWords((T*)input_tensors->at("logits").getPtrWithOffset(first * beams * vocab_size_padded_),
                       output_tensors->at("output_ids").getPtr<const int>(),
                       beams > 1 ? output_tensors->at("parent_ids").getPtr<const int>() : (const int*)nullptr,
-                      (int)batch, (int)rows, (int)beams, lists, one_list, length, (int)first, (int)vocab_size_padded_,
-                      (size_t)step, stream_);
+                      (int)batch, (int)rows, (int)beams, lists, one_list, length, (int)(first * beams),
+                      (int)vocab_size_padded_, (size_t)step, stream_);
 }
 
 // After sampling: stop words on the rows of this window (layers/DynamicDecodeLayer.cc:449-462; the reference

@@ -71,11 +71,32 @@ void TopKSamplingLayer<T>::freeBuffer()
     BaseSamplingLayer<T>::freeBuffer();
 }
 
+// Two environment switches, read once per setup() (not per step: getenv is neither free nor safe against a
+// concurrent setenv in a serving process).
+// FT_SAMPLING_DISABLE_FUSED=1 forces the kernel-by-kernel sequence of the reference.
+static bool fusedDisabledByEnvironment()
+{
+    const char* env = std::getenv("FT_SAMPLING_DISABLE_FUSED");
+    return env != nullptr && env[0] == '1';
+}
+
+// With log-prob outputs the fused step gives every row to one workgroup, which pays once there are enough rows to
+// keep the compute units busy: measured on MI355X it draws level with the kernel sequence between 128 and 192
+// rows at vocabularies from 32000 to 152064 columns and wins from there on.
+// FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS overrides the smallest window that takes it.
+static int fusedLogProbsMinRowsFromEnvironment()
+{
+    const char* env = std::getenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS");
+    return env != nullptr && env[0] != '\0' ? std::atoi(env) : 192;
+}
+
 // reference: TopKSamplingLayer<T>::setup, layers/sampling_layers/TopKSamplingLayer.cu:134-186
 template<typename T>
 void TopKSamplingLayer<T>::setup(const size_t batch_size, const size_t beam_width, TensorMap* runtime_args)
 {
     BaseSamplingLayer<T>::setup(batch_size, beam_width, runtime_args);
+    fused_disabled_           = fusedDisabledByEnvironment();
+    fused_log_probs_min_rows_ = fusedLogProbsMinRowsFromEnvironment();
 
     uint         tmp_top_k     = 0;
     const Tensor runtime_top_k = runtime_args->isExist("runtime_top_k") ?
@@ -131,24 +152,6 @@ void TopKSamplingLayer<T>::ensureWorkspace(int local_batch_size)
     }
 }
 
-// FT_SAMPLING_DISABLE_FUSED=1 forces the kernel-by-kernel sequence of the reference (read at every step, so
-// that one process can run both).
-static bool fusedDisabled()
-{
-    const char* env = std::getenv("FT_SAMPLING_DISABLE_FUSED");
-    return env != nullptr && env[0] == '1';
-}
-
-// With log-prob outputs the fused step gives every row to one workgroup, which pays once there are enough rows to
-// keep the compute units busy: measured on MI355X it draws level with the kernel sequence between 128 and 192
-// rows at vocabularies from 32000 to 152064 columns and wins from there on.
-// FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS overrides the smallest window that takes it (read at every step).
-static int fusedLogProbsMinRows()
-{
-    const char* env = std::getenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS");
-    return env != nullptr && env[0] != '\0' ? std::atoi(env) : 192;
-}
-
 // One streaming pass over the logits for the whole penalty + mask + top-k pipeline - two passes when log-prob
 // outputs are requested, which need the probabilities of the whole row. Not taken with the frequency-penalty
 // extension, nor for the configurations the fused step reports as unsupported with log-probs, nor for log-probs
@@ -158,7 +161,7 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
 {
     float* cum_log_probs    = output_tensors->at("cum_log_probs", Tensor()).template getPtr<float>();
     float* output_log_probs = output_tensors->at("output_log_probs", Tensor()).template getPtr<float>();
-    if (fusedDisabled() || this->has_frequency_penalty_) {
+    if (fused_disabled_ || this->has_frequency_penalty_) {
         return false;
     }
     const int batch_size       = output_tensors->at("output_ids").shape[1];
@@ -167,7 +170,7 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
     const int step             = input_tensors->at("step").template getVal<int>();
     const int max_input_length = input_tensors->at("max_input_length").template getVal<int>();
     const int off              = ite * local_batch_size;
-    if ((cum_log_probs != nullptr || output_log_probs != nullptr) && local_batch_size < fusedLogProbsMinRows()) {
+    if ((cum_log_probs != nullptr || output_log_probs != nullptr) && local_batch_size < fused_log_probs_min_rows_) {
         return false;
     }
 

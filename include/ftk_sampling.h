@@ -244,7 +244,10 @@ int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
  * a step that needs more than the array returns FTK_ERR_STATIC_WORKSPACE and launches nothing (the headline
  * step, 256 rows x 128256 fp32 with a history penalty, needs about 21 MB). All calls on one GPU share that
  * GPU's array: calls that overlap in time on one GPU (different streams or threads) race; calls on one stream
- * are safe back to back. */
+ * are safe back to back. The array is the current device's (make the stream's device current, as for any launch),
+ * and its address is looked up on the first call on a device (hipGetDevice + hipGetSymbolAddress): make that first
+ * call outside any graph capture. Every process that loads the library holds the 32 MiB on every GPU it touches,
+ * whether or not it calls this entry point. */
 #define FTK_FUSED_STATIC_WORKSPACE_BYTES (32u << 20)
 int ftk_fused_topk_step_static(ftk_fused_topk_args* args, ftk_stream_t stream);
 

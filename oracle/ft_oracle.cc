@@ -1244,9 +1244,12 @@ static void beam_update(bool* finished, int* parent_ids, int* sequence_length, i
         counted[i] = finished[i] ? sequence_length[i] : sequence_length[i] + 1;
     }
     for (int i = 0; i < rows; ++i) {
-        const int b       = i / K;
-        const int beam_id = (word_ids[i] / Vp) % K;
-        const int word_id = word_ids[i] % Vp;
+        const int b = i / K;
+        // a slot the step left untouched holds the caller's old contents: a negative value counts as "this beam,
+        // its end token" (the reference indexes other rows' memory with it)
+        const bool valid   = word_ids[i] >= 0;
+        const int  beam_id = valid ? (word_ids[i] / Vp) % K : i % K;
+        const int  word_id = valid ? word_ids[i] % Vp : end_ids[b];
         sequence_length[i] = counted[b * K + beam_id];
         finished[i]        = word_id == end_ids[b];
         parent_ids[i]      = beam_id;

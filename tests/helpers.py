@@ -87,7 +87,8 @@ def uniforms(rng, n):
 def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=None):
     """One fused decode step straight through the C ABI (temperature 0.8, repetition penalty 1.1 over `history`,
     top-k `k`, top-p 0.9, injected draws). entry: "caller" = ftk_fused_topk_step with a workspace of the queried
-    size, "static" = ftk_fused_topk_step_static. Returns (ids, sequence_length, finished, rc, needed bytes)."""
+    size, "static" = ftk_fused_topk_step_static. Returns (ids, sequence_length, finished, rc, needed bytes, change of
+    the device's free memory across the static call)."""
     import ctypes as C
     import fastertransformer_amd as fa
     from fastertransformer_amd import ops
@@ -121,11 +122,16 @@ def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finishe
         ws = torch.empty(a.workspace_size, dtype=torch.uint8, device=dev)
         a.workspace = ws.data_ptr()
         rc = lib.ftk_fused_topk_step(C.addressof(a), stream)
+        torch.cuda.synchronize()
+        freed = 0
     else:
         a.workspace, a.workspace_size = None, 0
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]  # (the driver's figure: torch's own pool does not hide anything)
         rc = lib.ftk_fused_topk_step_static(C.addressof(a), stream)
-    torch.cuda.synchronize()
-    return out_ids[H].cpu().numpy(), seq.cpu().numpy(), finished.cpu().numpy(), rc, a.workspace_size
+        torch.cuda.synchronize()
+        freed = torch.cuda.mem_get_info()[0] - free_before
+    return out_ids[H].cpu().numpy(), seq.cpu().numpy(), finished.cpu().numpy(), rc, a.workspace_size, freed
 
 
 def make_beam_case(rng, dt, batch, K, V, step=5, max_seq_len=12, with_hyps=True, finished_frac=0.2, full_frac=0.2,

@@ -207,6 +207,7 @@ def test_beam_update_and_cache_indirection():
         end_ids = rng.integers(0, Vp, batch).astype(np.int32)
         ends = rng.random(batch * K) < 0.2
         word[ends] = word[ends] // Vp * Vp + np.repeat(end_ids, K)[ends]
+        word[rng.random(batch * K) < 0.1] = -7   # slots the step never wrote: the caller's old contents
         finished = rng.random(batch * K) < 0.3
         seq = rng.integers(3, 9, batch * K).astype(np.int32)
         num_beams = np.where(rng.random(batch) < 0.3, K, rng.integers(0, K, batch)).astype(np.int32)
@@ -387,10 +388,12 @@ def test_dynamic_decode_layer_with_beams(windows, differing):
         step = max_input + i
         x = (rng.standard_normal((rows, Vp)) * 3).astype(np.float32)
         d_x = to_torch(x).reshape(batch, K, Vp)
-        # word lists ride along in the one-window variant (with several windows the reference offsets the bad-word
-        # launch by entries, not by beams)
+        # Bad-word lists ride along in every variant: each beam is banned from its own entry's list over its own
+        # history, whichever window it belongs to (with several windows the reference offsets the launch of a later
+        # window by entries instead of by beams, so that the bans land on other beams' rows; that defect is not
+        # reproduced). Stop-word lists in the one-window variant.
         bad = stop = None
-        if windows == 1 and step >= 2:
+        if step >= 2:
             bad = _beam_word_lists(rng, batch, K, V, 6, 3, 24, out_ids, parents, step, with_last=False)
             O.ban_bad_words_beams(dt, x, out_ids, parents, batch, batch, K, bad, False, 24, 0, Vp, step)
         for ite in range(windows):
@@ -418,10 +421,12 @@ def test_dynamic_decode_layer_with_beams(windows, differing):
                     "parent_ids": d["parents"], "sequence_length": d["seq"], "tgt_cache_indirection": d_src[1],
                     "should_stop": should_stop}
             if bad is not None:
+                ins["bad_words_list"] = to_torch(bad)
+            if bad is not None and windows == 1:
                 # stop words: some of them end with what a beam has just chosen (known from the oracle's step)
                 stop = _beam_word_lists(rng, batch, K, V, 4, 2, 16, out_ids, parents, step, with_last=True)
                 O.stop_words_criterion_beams(out_ids, parents, stop, finished, 0, 16, batch, batch, K, step)
-                ins["bad_words_list"], ins["stop_words_list"] = to_torch(bad), to_torch(stop)
+                ins["stop_words_list"] = to_torch(stop)
             print("dynamic decode with beams", windows, step, ite, flush=True)
             layer.forward(outs, ins)
             torch.cuda.synchronize()

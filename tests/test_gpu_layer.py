@@ -441,7 +441,7 @@ def test_log_probs_on_small_windows_take_the_kernel_sequence(monkeypatch):
     monkeypatch.delenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS")
     rng = np.random.default_rng(7200)
     V = 2051
-    for B, mutated in ((8, True), (400, False)):
+    for B, mutated in ((8, True), (191, True), (192, False), (400, False)):
         c = Case(O.F32, B, V, V, max_input_length=4, gen_len=2, runtime_top_k=[8], runtime_top_p=[0.9],
                  temperature=[0.7], repetition_penalty=[1.3], prompt=_history(rng, 4, B, V), with_cum=True,
                  with_out_lp=True)

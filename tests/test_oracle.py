@@ -986,6 +986,7 @@ def test_beam_update_and_cache_indirection_against_the_description():
     word = word.astype(np.int32).reshape(-1)
     end_ids = rng.integers(0, Vp, batch).astype(np.int32)
     word[2] = (2 // K * K + 1) * Vp + end_ids[0]     # row 2 continues beam 1 of entry 0 with the end token
+    word[7] = -7                                      # a slot the step never wrote: the caller's old contents
     finished = rng.random(batch * K) < 0.3
     seq = rng.integers(3, 9, batch * K).astype(np.int32)
     num_beams = np.array([0, K, 1, 2], np.int32)
@@ -995,7 +996,7 @@ def test_beam_update_and_cache_indirection_against_the_description():
     counted = np.where(finished, seq, seq + 1)
     for i in range(batch * K):
         b = i // K
-        beam, tok = (word[i] // Vp) % K, word[i] % Vp
+        beam, tok = ((word[i] // Vp) % K, word[i] % Vp) if word[i] >= 0 else (i % K, end_ids[b])
         assert parent[i] == beam and w[i] == tok and out[i] == tok
         assert s_[i] == counted[b * K + beam]
         assert f[i] == (tok == end_ids[b] or num_beams[b] == K)
