@@ -27,6 +27,10 @@ struct FusedParams {
     int          bitmap_words;
     int          bitmaps_ready;  // history_bitmap_kernel filled `bitmaps`
     int          lds_window;        // 0: none, 1: small LDS bitmap window, 2: large
+    // A launch over a vocabulary shard (a producer hands over columns [col_offset, col_offset + V) of every row:
+    // `logits` points at the shard's first column, Vp is the pitch of its rows): token ids in the history and the
+    // end ids are global, and so are the column numbers the launch reports. 0 for whole rows.
+    int          col_offset;
 };
 
 // History bitmaps: bit v set <=> token v occurs in the row's (non-padding) history, i.e. column v gets
@@ -127,6 +131,7 @@ struct FusedRow {
     bool            global_ready;
     const int*      history;  // output_ids + row, stride batch_size
     int             batch_size, step, input_length, max_input_length;
+    int             col_offset;  // global number of column 0 (a vocabulary shard), see FusedParams
 
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row): FusedRow(p, row, fused_row_args(p, row)) {}
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row, const FusedRowArgs& args)
@@ -171,9 +176,11 @@ struct FusedRow {
         up_mul_neg = uniform_f(up_mul_neg);
         up_mul_pos = uniform_f(up_mul_pos);
         up_add     = uniform_f(up_add);
+        col_offset    = p.col_offset;
         masked_end_id = (p.min_lengths != nullptr
-                         && min_length_masks(args.sequence_length, p.max_input_length, args.min_length)) ?
-                            args.end_id :
+                         && min_length_masks(args.sequence_length, p.max_input_length, args.min_length)
+                         && args.end_id >= p.col_offset) ?
+                            args.end_id - p.col_offset :  // (beyond the shard: no column of it matches)
                             -1;
     }
     __device__ __forceinline__ const T* data() const
@@ -205,7 +212,7 @@ struct FusedRow {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int t = t0 + u * blockDim.x;
-                ids[u]      = (t < step && history_position_counts(t)) ? history[(size_t)t * batch_size] : -1;
+                ids[u] = (t < step && history_position_counts(t)) ? history[(size_t)t * batch_size] - col_offset : -1;
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {

@@ -225,7 +225,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 #pragma unroll
         for (int u = 0; u < LG_HIST_U; ++u) {
             const int pos = t + u * LG_THREADS;
-            hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
+            hist_ids[u]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] - p.col_offset : -1;
         }
     }
     // An embedding bias (rows and bias on 16-byte boundaries: the launcher checks) is read alongside: the same
@@ -321,7 +321,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
             mark(t + u * LG_THREADS, hist_ids[u]);
         }
         for (int pos = t + LG_HIST_U * LG_THREADS; pos < p.step; pos += LG_THREADS) {
-            mark(pos, p.output_ids[(size_t)pos * p.batch_size + row]);
+            mark(pos, p.output_ids[(size_t)pos * p.batch_size + row] - p.col_offset);
         }
         rowctx.bm_mode   = 1;
         rowctx.bm_origin = origin;
@@ -579,7 +579,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                     if ((mask >> c) & 1u) {
                         const uint32_t key = order_key(x[c]);
                         if (slot < TK_CCAP) {
-                            out[slot] = TopkEntry{key, (uint32_t)(first + c)};
+                            out[slot] = TopkEntry{key, (uint32_t)(first + c + p.col_offset)};
                         }
                         dmax = key > dmax ? key : dmax;
                         ++slot;
@@ -651,7 +651,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
                 if (xv >= thr_f) {
                     const int slot = atomicAdd(&s.n_out, 1);
                     if (slot < TK_CCAP) {
-                        out[slot] = TopkEntry{order_key(xv), (uint32_t)v};
+                        out[slot] = TopkEntry{order_key(xv), (uint32_t)(v + p.col_offset)};
                     }
                 }
             }
@@ -883,6 +883,13 @@ __device__ __forceinline__ void lean_select_row(TopkShared& s, const FusedParams
     if (n < 0) {
         // A workgroup of the gather could not hold its candidates. Walk the whole row again, here, with the
         // stream that recovers from overfull tiles; only rows it cannot bound either take the literal replay.
+        if (p.logits == nullptr) {
+            // (lists merged from vocabulary shards without the rows at hand: the row is reported as not sampled)
+            if (threadIdx.x == 0) {
+                l.ids[row] = -1;
+            }
+            return;
+        }
         r.prepare_whole_row();
         __syncthreads();
         n = topk_stream<DT, FusedRow<DT, BMW>, 0>(r, s, p.Vp, k, 0, topk_row_tiles<DT>(r.rowp, p.Vp), &thr);

@@ -451,6 +451,310 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     return launch_general(FUSED_KIND_SELECT, 0, dim3(rows));
 }
 
+// ---- producer hand-over: the step over vocabulary shards ------------------------------------------------------
+// The reference writes the logits of a step from the last GEMM (under tensor parallelism one vocabulary shard per
+// rank, gathered afterwards: src/fastertransformer/models/multi_gpu_gpt/ParallelGpt.cc:1374-1433) and reads them
+// back in DynamicDecodeLayer::forward (:1436-1501). Here a producer - a GEMM epilogue, or a rank that holds one
+// shard - can hand over columns [col_offset, col_offset + cols) of every row on their own: the gather below leaves,
+// per row and shard, the bounded candidate lists of the lean gather (every element at or above a lower bound of the
+// k-th largest value of the shard's own columns) and, on request, the shard's (maximum, sum of exp(x - maximum)) of
+// the final values; the merge runs the selection over the lists of all shards, which is the same deterministic
+// computation wherever it runs. What crosses between the two is at most lists_per_shard * (16 + 8 * 2048) bytes
+// per row and shard, typically a few hundred entries, instead of the row.
+namespace ftk {
+
+struct ShardLayout {
+    LeanPlan plan;   // how a shard of the widest kind is cut into workgroups
+    int      total;  // lists per row over all shards
+    size_t   bitmap_bytes, bytes;
+};
+
+static ShardLayout shard_layout(const ftk_fused_topk_args* a, const ftk_topk_shards* sh, int elem, int global_vp)
+{
+    ShardLayout y;
+    const int   rows = a->local_batch_size > 0 ? a->local_batch_size : 1;
+    y.plan           = lean_plan(sh->shard_width, rows, elem, 256 * LG_OCCUPANCY);
+    const int most   = TK_MAXSPLIT / (sh->n_shards > 0 ? sh->n_shards : 1);
+    if (y.plan.splits > most) {
+        const int epv  = 16 / elem;
+        const int nsub = (sh->shard_width / epv + 1 + LG_SUB_VECS - 1) / LG_SUB_VECS;
+        y.plan.subs_per_wg = (nsub + most - 1) / most;
+        y.plan.splits      = (nsub + y.plan.subs_per_wg - 1) / y.plan.subs_per_wg;
+    }
+    y.total        = y.plan.splits * sh->n_shards;
+    const int words = (global_vp + 31) / 32 + 1;
+    y.bitmap_bytes = ((size_t)rows * words * sizeof(uint32_t) + 255) / 256 * 256;  // the merge's recovery path
+    y.bytes = y.bitmap_bytes + (size_t)rows * y.total * (sizeof(TopkChunkHeader) + (size_t)TK_CCAP * sizeof(TopkEntry));
+    return y;
+}
+
+// (maximum, sum of exp(x - maximum)) over the final values of a shard's columns, one workgroup per row. The final
+// value of a column is what top-k sees: temperature, history penalty, min-length and pad masks applied.
+template<int DT>
+__global__ void __launch_bounds__(256) shard_stats_kernel(FusedParams p, float* __restrict__ partials, int n_shards,
+                                                          int shard)
+{
+    __shared__ float sh_m[4], sh_s[4];
+    const int        row = blockIdx.x;
+    if (row_flag_or(p.skip_decode, row, p.end_ids + row, false)
+        || row_flag_or(p.finished_in, row, p.end_ids + row, false)) {
+        if (threadIdx.x == 0) {  // rows that do not take part: an empty shard
+            partials[((size_t)row * n_shards + shard) * 2 + 0] = -__builtin_inff();
+            partials[((size_t)row * n_shards + shard) * 2 + 1] = 0.0f;
+        }
+        return;
+    }
+    FusedRow<DT, FUSED_BITMAP_WORDS_LARGE> r(p, row);
+    r.prepare(0, p.V);
+    __syncthreads();
+    float m = -__builtin_inff(), sum = 0.0f;
+    for (int v = threadIdx.x; v < p.V; v += 256) {
+        if (r.never_selected(v)) {
+            continue;
+        }
+        const float x = topk_value_at<DT>(r, v);
+        if (x > m) {
+            sum = sum * det_expf(m - x) + 1.0f;  // (exp(-inf) = 0 on the first element)
+            m   = x;
+        }
+        else if (x > -__builtin_inff()) {
+            sum += det_expf(x - m);
+        }
+    }
+    auto merge = [](float& m0, float& s0, float m1, float s1) {
+        const float mm = __builtin_fmaxf(m0, m1);
+        if (mm > -__builtin_inff()) {
+            s0 = s0 * det_expf(m0 - mm) + s1 * det_expf(m1 - mm);
+        }
+        m0 = mm;
+    };
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        merge(m, sum, __shfl_xor(m, o, WAVE), __shfl_xor(sum, o, WAVE));
+    }
+    if (lane_id() == 0) {
+        sh_m[wave_id()] = m;
+        sh_s[wave_id()] = sum;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w) {
+            merge(m, sum, sh_m[w], sh_s[w]);
+        }
+        partials[((size_t)row * n_shards + shard) * 2 + 0] = m;
+        partials[((size_t)row * n_shards + shard) * 2 + 1] = sum;
+    }
+}
+
+__global__ void shard_stats_combine_kernel(const float* __restrict__ partials, float* __restrict__ row_stats, int rows,
+                                           int n_shards)
+{
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows) {
+        return;
+    }
+    float m = -__builtin_inff();
+    for (int i = 0; i < n_shards; ++i) {
+        m = __builtin_fmaxf(m, partials[((size_t)row * n_shards + i) * 2]);
+    }
+    float sum = 0.0f;
+    for (int i = 0; i < n_shards; ++i) {
+        const float mi = partials[((size_t)row * n_shards + i) * 2];
+        if (mi > -__builtin_inff()) {
+            sum += partials[((size_t)row * n_shards + i) * 2 + 1] * det_expf(mi - m);
+        }
+    }
+    row_stats[2 * row]     = m;
+    row_stats[2 * row + 1] = sum;
+}
+
+}  // namespace ftk
+
+static int shard_common_checks(const ftk_fused_topk_args* a, const ftk_topk_shards* sh)
+{
+    if (a == nullptr || sh == nullptr) {
+        return FTK_ERR_ARGUMENT;
+    }
+    if (a->dtype < 0 || a->dtype > 2) {
+        return FTK_ERR_DTYPE;
+    }
+    if (a->max_top_k < 1 || a->max_top_k > 1024) {
+        return FTK_ERR_TOPK_DOMAIN;
+    }
+    if (sh->n_shards < 1 || sh->n_shards > 16 || sh->shard_width < 1) {
+        return FTK_ERR_ARGUMENT;
+    }
+    if (a->max_top_k > LG_MAX_K || a->embedding_bias != nullptr || a->cum_log_probs != nullptr
+        || a->output_log_probs != nullptr) {
+        return FTK_ERR_UNSUPPORTED;  // one read of the shard, no bias, no log-prob outputs (see row_stats)
+    }
+    return 0;
+}
+
+extern "C" int ftk_fused_topk_shard_gather(ftk_fused_topk_args* a, const ftk_topk_shards* sh, ftk_stream_t stream)
+{
+    int rc = shard_common_checks(a, sh);
+    if (rc != 0) {
+        return rc;
+    }
+    const int elem = a->dtype == FTK_DTYPE_F32 ? 4 : 2;
+    const int rows = a->local_batch_size;
+    if (sh->shard < 0 || sh->shard >= sh->n_shards || sh->col_offset < 0 || a->vocab_size > sh->shard_width
+        || a->vocab_size > a->vocab_size_padded) {
+        return FTK_ERR_ARGUMENT;
+    }
+    const ShardLayout y = shard_layout(a, sh, elem, sh->global_vocab_size_padded);
+    if (a->workspace == nullptr) {
+        a->workspace_size = y.bytes;
+        return 0;
+    }
+    if (a->workspace_size < y.bytes) {
+        return FTK_ERR_WORKSPACE;
+    }
+    if (rows <= 0) {
+        return 0;
+    }
+    if (a->logits == nullptr || a->end_ids == nullptr || a->top_ks == nullptr
+        || (a->min_lengths != nullptr && a->sequence_length == nullptr)) {
+        return FTK_ERR_ARGUMENT;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    FusedParams p{};
+    p.logits             = a->logits;
+    p.V                  = a->vocab_size;
+    p.Vp                 = a->vocab_size_padded;
+    p.batch_size         = a->batch_size;
+    p.step               = a->step;
+    p.max_input_length   = a->max_input_length;
+    p.temperatures       = a->temperatures;
+    p.penalties          = a->penalty_type != FTK_PENALTY_NONE ? a->penalties : nullptr;
+    p.penalty_type       = a->penalty_type;
+    p.min_lengths        = a->min_lengths;
+    p.end_ids            = a->end_ids;
+    p.input_lengths      = a->input_lengths;
+    p.output_ids         = a->output_ids;
+    p.sequence_length_in = a->sequence_length;
+    p.top_ks             = a->top_ks;
+    p.top_ps             = a->top_ps;
+    p.max_top_k          = a->max_top_k;
+    p.skip_decode        = a->skip_decode;
+    p.finished_in        = a->finished;
+    p.bitmap_words       = (sh->global_vocab_size_padded + 31) / 32 + 1;
+    p.col_offset         = sh->col_offset;
+    int window           = 1;
+    if (p.penalties != nullptr && a->step > 0) {
+        if (a->output_ids == nullptr) {
+            return FTK_ERR_ARGUMENT;
+        }
+        // the history bitmap of a workgroup's columns lives in LDS (no whole-row bitmaps in this mode)
+        const int    epv   = 16 / elem;
+        const size_t words = ((size_t)y.plan.subs_per_wg * LG_SUB_VECS * epv + 2 * epv) / 32 + 4;
+        if (words > (size_t)FUSED_BITMAP_WORDS_LARGE || a->step > FUSED_SPLIT_BITMAP_MAX_STEP) {
+            return FTK_ERR_UNSUPPORTED;
+        }
+        p.bitmaps    = (uint32_t*)a->workspace;  // (marks "a history penalty applies"; the memory is not touched)
+        p.lds_window = words <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
+        window       = p.lds_window;
+    }
+    else {
+        p.penalties = nullptr;
+    }
+    char*       ws = (char*)a->workspace;
+    FusedLaunch l{};
+    l.splits      = y.total;
+    l.subs_per_wg = y.plan.subs_per_wg;
+    l.row_entries = (size_t)y.total * TK_CCAP;
+    // this shard's lists sit at [shard * lists_per_shard, ...) of every row's lists
+    l.headers = (TopkChunkHeader*)(ws + y.bitmap_bytes) + (size_t)sh->shard * y.plan.splits;
+    l.entries = (TopkEntry*)((TopkChunkHeader*)(ws + y.bitmap_bytes) + (size_t)rows * y.total)
+                + (size_t)sh->shard * y.plan.splits * TK_CCAP;
+    if (sh->partials != nullptr && p.penalties != nullptr
+        && (size_t)a->vocab_size / 32 + 4 > (size_t)FUSED_BITMAP_WORDS_LARGE) {
+        return FTK_ERR_UNSUPPORTED;  // (the statistics kernel keeps the bitmap of the shard's columns in LDS)
+    }
+    const dim3 grid(y.plan.splits, rows);  // (workgroups past a narrow shard's columns leave empty lists)
+    rc = a->dtype == FTK_DTYPE_F32 ? lean_gather_launch_f32(LG_MODE_STREAM, false, window, grid, st, p, l, nullptr, nullptr) :
+         a->dtype == FTK_DTYPE_F16 ? lean_gather_launch_f16(LG_MODE_STREAM, false, window, grid, st, p, l, nullptr, nullptr) :
+                                     lean_gather_launch_bf16(LG_MODE_STREAM, false, window, grid, st, p, l, nullptr, nullptr);
+    if (rc != 0 || sh->partials == nullptr) {
+        return rc;
+    }
+    FTK_DISPATCH_DTYPE(a->dtype, hipLaunchKernelGGL((shard_stats_kernel<DT>), dim3(rows), dim3(256), 0, st, p,
+                                                    sh->partials, sh->n_shards, sh->shard));
+    FTK_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int ftk_fused_topk_shard_merge(ftk_fused_topk_args* a, const ftk_topk_shards* sh, ftk_stream_t stream)
+{
+    int rc = shard_common_checks(a, sh);
+    if (rc != 0) {
+        return rc;
+    }
+    const int         elem = a->dtype == FTK_DTYPE_F32 ? 4 : 2;
+    const int         rows = a->local_batch_size;
+    const ShardLayout y    = shard_layout(a, sh, elem, a->vocab_size_padded);
+    if (a->workspace == nullptr) {
+        a->workspace_size = y.bytes;
+        return 0;
+    }
+    if (a->workspace_size < y.bytes || sh->global_vocab_size_padded != a->vocab_size_padded) {
+        return a->workspace_size < y.bytes ? FTK_ERR_WORKSPACE : FTK_ERR_ARGUMENT;
+    }
+    if (rows <= 0) {
+        return 0;
+    }
+    if (a->ids == nullptr || a->end_ids == nullptr || a->top_ks == nullptr
+        || (a->rng_state == nullptr && a->uniform_draws == nullptr)
+        || (sh->row_stats != nullptr && sh->partials == nullptr)) {
+        return FTK_ERR_ARGUMENT;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    FusedParams p{};
+    p.logits             = a->logits;  // whole rows for the recovery of rows whose lists overflowed, or null
+    p.V                  = a->vocab_size;
+    p.Vp                 = a->vocab_size_padded;
+    p.batch_size         = a->batch_size;
+    p.step               = a->step;
+    p.max_input_length   = a->max_input_length;
+    p.temperatures       = a->temperatures;
+    p.penalties          = (a->penalty_type != FTK_PENALTY_NONE && a->step > 0) ? a->penalties : nullptr;
+    p.penalty_type       = a->penalty_type;
+    p.min_lengths        = a->min_lengths;
+    p.end_ids            = a->end_ids;
+    p.input_lengths      = a->input_lengths;
+    p.output_ids         = a->output_ids;
+    p.sequence_length_in = a->sequence_length;
+    p.top_ks             = a->top_ks;
+    p.top_ps             = a->top_ps;
+    p.max_top_k          = a->max_top_k;
+    p.skip_decode        = a->skip_decode;
+    p.finished_in        = a->finished;
+    p.bitmaps            = p.penalties != nullptr ? (uint32_t*)a->workspace : nullptr;
+    p.bitmap_words       = (a->vocab_size_padded + 31) / 32 + 1;
+    char*       ws = (char*)a->workspace;
+    FusedLaunch l{};
+    l.ids             = a->ids;
+    l.sequence_length = a->sequence_length;
+    l.finished        = a->finished;
+    l.rng             = (RngState*)a->rng_state;
+    l.uniforms        = a->uniform_draws;
+    l.splits          = y.total;
+    l.row_entries     = (size_t)y.total * TK_CCAP;
+    l.headers         = (TopkChunkHeader*)(ws + y.bitmap_bytes);
+    l.entries         = (TopkEntry*)(l.headers + (size_t)rows * y.total);
+    rc = a->dtype == FTK_DTYPE_F32 ? lean_select_launch_f32(rows, st, p, l, nullptr, nullptr) :
+         a->dtype == FTK_DTYPE_F16 ? lean_select_launch_f16(rows, st, p, l, nullptr, nullptr) :
+                                     lean_select_launch_bf16(rows, st, p, l, nullptr, nullptr);
+    if (rc != 0 || sh->row_stats == nullptr) {
+        return rc;
+    }
+    hipLaunchKernelGGL(shard_stats_combine_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, sh->partials,
+                       sh->row_stats, rows, sh->n_shards);
+    FTK_LAUNCH_CHECK();
+    return 0;
+}
+
 // ---- plain read of a buffer: the yardstick of the streaming kernels ------------------------------------
 // What the gather would cost if it did nothing but fetch: the same launch shape (256-thread workgroups, four
 // per compute unit, each walking a contiguous share in sub-tiles of four 16-byte vectors per thread with two

@@ -73,6 +73,8 @@ _SIGNATURES = {
                                             _f, _f, _i, _i, _vp],
     "ftk_invoke_beam_update": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp],
     "ftk_invoke_update_indir_cache": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "ftk_fused_topk_shard_gather": [_vp, _vp, _vp],
+    "ftk_fused_topk_shard_merge": [_vp, _vp, _vp],
     "ftk_error_string": [_i],
     "ftk_profile_enable": [_i],
     "ftk_profile_read": [_i, _vp, _vp],
@@ -220,6 +222,12 @@ class FusedTopkArgs(C.Structure):
         ("finished", _vp), ("cum_log_probs", _vp), ("output_log_probs", _vp), ("workspace", _vp),
         ("workspace_size", _sz),
     ]
+
+
+class TopkShards(C.Structure):
+    """struct ftk_topk_shards"""
+    _fields_ = [("n_shards", _i), ("shard_width", _i), ("global_vocab_size_padded", _i), ("shard", _i),
+                ("col_offset", _i), ("partials", _vp), ("row_stats", _vp)]
 
 
 # ---- DynamicDecodeLayer over the C handle API ------------------------------------------------------

@@ -236,6 +236,41 @@ typedef struct ftk_fused_topk_args {
 /* workspace == NULL in args: writes the required size into args->workspace_size, launches nothing. */
 int ftk_fused_topk_step(ftk_fused_topk_args* args, ftk_stream_t stream);
 
+/* ---- the fused step over vocabulary shards (producer hand-over) --------------------------------------
+ * The reference writes a step's logits from its last GEMM - one vocabulary shard per rank under tensor parallelism,
+ * gathered afterwards - and reads them back in DynamicDecodeLayer::forward
+ * (src/fastertransformer/models/multi_gpu_gpt/ParallelGpt.cc:1374-1433, :1436-1501). These two entry points let a
+ * producer (a GEMM epilogue working through column tiles, or a rank that holds one shard) hand over columns
+ * [col_offset, col_offset + args->vocab_size) of every row on their own:
+ *   gather: args->logits points at the shard's first column of the first row, args->vocab_size is the number of the
+ *           shard's columns that lie inside the vocabulary, args->vocab_size_padded the pitch of its rows in
+ *           elements; token ids (history, end ids) are global. Leaves, per row and shard, candidate lists that hold
+ *           every element at or above a lower bound of the k-th largest value of the shard's columns (column numbers
+ *           global), and in `partials`, when given, the shard's (maximum, sum of exp(x - maximum)) over the final
+ *           values (after temperature, penalties and masks). Samples nothing.
+ *   merge:  after every shard's gather: the selection of ftk_fused_topk_step over the lists of all shards. ids, lengths
+ *           and flags are those of ftk_fused_topk_step on the whole rows, bit for bit. args->vocab_size /
+ *           vocab_size_padded are the whole vocabulary's; args->logits are the whole rows, or NULL when nobody holds
+ *           them (a row whose lists overflowed - thousands of candidates tied around the k-th value - then gets id -1).
+ *           `row_stats`, when given (with `partials`), receives the rows' (maximum, sum of exp(x - maximum)) combined
+ *           over the shards: log p of the sampled token = x - maximum - log(sum), within 1e-5 of the reference's
+ *           softmax but not in its summation order.
+ * Both calls take the same workspace (size query: workspace == NULL, from either call with the same n_shards,
+ * shard_width and batch) and the same per-row arguments. Largest k <= 192, no embedding bias, no log-prob outputs
+ * (FTK_ERR_UNSUPPORTED otherwise); with a history penalty the step must not exceed 8192. What a rank would send
+ * instead of its shard of the row is its lists: typically a few hundred entries of 8 bytes per row. */
+typedef struct ftk_topk_shards {
+    int    n_shards;                 /* shards a row is cut into, 1 .. 16 */
+    int    shard_width;              /* columns of the widest shard: fixes the workspace layout for every call */
+    int    global_vocab_size_padded; /* of the whole rows (sizes the merge's recovery bitmaps) */
+    int    shard;                    /* gather: which shard this call reads */
+    int    col_offset;               /* gather: global number of the shard's first column */
+    float* partials;                 /* [local_batch][n_shards][2] or NULL */
+    float* row_stats;                /* merge: [local_batch][2] or NULL */
+} ftk_topk_shards;
+int ftk_fused_topk_shard_gather(ftk_fused_topk_args* args, const ftk_topk_shards* shards, ftk_stream_t stream);
+int ftk_fused_topk_shard_merge(ftk_fused_topk_args* args, const ftk_topk_shards* shards, ftk_stream_t stream);
+
 /* The fused step for callers that cannot allocate device memory (code under HIP graph capture, serving loops
  * and harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arguments and results as
  * ftk_fused_topk_step, except that args->workspace is ignored: the workspace is a fixed array of
