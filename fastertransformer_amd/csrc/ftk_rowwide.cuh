@@ -35,7 +35,9 @@ constexpr int RW_HIST_U     = 4;                    // history ids a thread requ
 #endif
 constexpr int RW_FIRST_TIGHTEN = FTK_RW_T1;
 constexpr int RW_TAIL_GAP      = FTK_RW_GAP;
-constexpr int RW_MIN_SUBS   = 4;                    // shortest row the launcher sends here, in sub-tiles
+constexpr int RW_MIN_SUBS   = 4;                    // shortest row that a batch of full rounds sends here, in sub-tiles
+constexpr int RW_SMALL_BYTES = 32 << 20;            // a launch that reads less than this takes the kernel at any
+                                                    // batch up to 256 rows: it is bound by latency, not bandwidth
 
 struct RowwideShared {
     uint4    stage_raw[RW_WAVES][RW_STAGE];
@@ -198,7 +200,7 @@ __device__ __forceinline__ int rowwide_rank_distinct(TopkShared& s, int n, int k
     const int      bs1_log = max_top_k <= 16 ? 7 : 8;
     const uint32_t my_key  = t < n ? s.cand.key[t] : 0u;
     const uint32_t my_idx  = t < n ? s.cand.idx[t] : 0u;
-    int*           cnt     = s.sel.idx + 1024;  // 2 x 256 counts, clear of the list this function writes
+    int*           cnt     = s.sel.idx + 1024;  // 256 counts and 256 marks, clear of the list this function writes
     int            CP      = 4;
     while (CP < n) {
         CP <<= 1;
@@ -226,31 +228,34 @@ __device__ __forceinline__ int rowwide_rank_distinct(TopkShared& s, int n, int k
         atomicAdd(&s.slice_count[(my_idx >> bs1_log) & 7u], 1);
     }
     {
-        const uint32_t key = c < n ? s.cand.key[c] : 0xFFFFFFFFu;
-        int            above = 0, equal = 0;
+        const uint32_t key   = c < n ? s.cand.key[c] : 0xFFFFFFFFu;
+        int            above = 0;
 #pragma unroll 2
         for (int j = jlo; j < jhi; j += 4) {
             const uint4 kk = *reinterpret_cast<const uint4*>(&s.cand.key[j]);
             above += (kk.x > key ? 1 : 0) + (kk.y > key ? 1 : 0) + (kk.z > key ? 1 : 0) + (kk.w > key ? 1 : 0);
-            equal += (kk.x == key ? 1 : 0) + (kk.y == key ? 1 : 0) + (kk.z == key ? 1 : 0) + (kk.w == key ? 1 : 0);
         }
         if (c < n && jhi > jlo) {
             atomicAdd(&cnt[c], above);
-            atomicAdd(&cnt[TK_THREADS + c], equal);
         }
     }
     lds_barrier();
-    if (t < n && (cnt[TK_THREADS + t] != 1 || s.slice_count[(my_idx >> bs1_log) & 7u] > k)) {
-        s.misc[1] = 1;
+    // Keys that are all different give n different counts: two candidates with the same count have the same key.
+    int rank = 0;
+    if (t < n) {
+        rank = cnt[t];
+        if (atomicAdd(&cnt[TK_THREADS + rank], 1) != 0 || s.slice_count[(my_idx >> bs1_log) & 7u] > k) {
+            s.misc[1] = 1;
+        }
     }
     lds_barrier();
     if (s.misc[1] != 0) {
         return -1;
     }
     const int n_list = min(k, n);
-    if (t < n && cnt[t] < n_list) {
-        s.sel.w[cnt[t]]   = key_to_float(my_key);
-        s.sel.idx[cnt[t]] = (int)my_idx;
+    if (t < n && rank < n_list) {
+        s.sel.w[rank]   = key_to_float(my_key);
+        s.sel.idx[rank] = (int)my_idx;
     }
     lds_barrier();
     return n_list;
@@ -279,7 +284,7 @@ __device__ __noinline__ void rowwide_rare(TopkShared& ts, const FusedParams p, c
 
 // Requirements the launcher checks: rows start on 16-byte boundaries (so a vector never straddles a word of the
 // history bitmap and there are no columns in front of the first vector), no embedding bias, the largest k at most
-// LG_MAX_K, at least RW_MIN_SUBS sub-tiles per row, the row's history bitmap fits BMW words, and a history of at most
+// LG_MAX_K, at least one whole vector per row, the row's history bitmap fits BMW words, and a history of at most
 // RW_HIST_U * RW_THREADS positions.
 // Keeps a launch argument in a scalar register of its own from here on. Without it the compiler, short of scalar
 // registers, reads arguments again from the kernel-argument segment wherever they are used, and every such read
@@ -418,7 +423,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
     lds_barrier();
 #pragma unroll
     for (int r = 1; r < R; ++r) {
-        load(r, r);  // (rows have at least RW_MIN_SUBS >= R sub-tiles)
+        load(r, r);  // (past the row's end: the last vector again, never looked at)
     }
     RW_STAMP(1)
     const bool     bitsv   = hist;
@@ -474,13 +479,13 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         uint32_t word[RW_NV];
 #pragma unroll
         for (int j = 0; j < RW_NV; ++j) {
-            word[j] = bitsv ? window[((j * RW_THREADS + t) * EPV) >> 5] : 0u;  // (inside the row: nsub >= 2)
+            word[j] = bitsv ? window[(min(j * RW_THREADS + t, nvec - 1) * EPV) >> 5] : 0u;
         }
         float tmax = NEG_INF;
 #pragma unroll
         for (int j = 0; j < RW_NV; ++j) {
             const int   first = (j * RW_THREADS + t) * EPV;
-            const bool  clean = word[j] == 0u && rowctx.interior_vector(first, EPV);
+            const bool  clean = j * RW_THREADS + t < nvec && word[j] == 0u && rowctx.interior_vector(first, EPV);
             const float vm    = lean_raw_max<DT>(raw[0][j]);
             tmax              = __builtin_fmaxf(tmax, clean ? vm : NEG_INF);
         }

@@ -231,10 +231,15 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     // About one row per compute unit (or a few rounds of that), a small k, long rows, no bias: a 1024-thread
     // workgroup per row does the whole step in one launch (ftk_rowwide.cuh). It pays when the rounds of 256
     // workgroups are nearly full and the row's history bitmap fits its LDS window.
+    // Small launches (a few megabytes of logits) are bound by latency: they take the same kernel at any batch up to
+    // 256 rows, one launch instead of two with lists through memory in between.
     const int  rw_rounds = (rows + 255) / 256;
+    const bool rw_full   = rows * 5 >= rw_rounds * 256 * 4
+                         && (size_t)a->vocab_size / (16 / elem) >= (size_t)RW_MIN_SUBS * RW_SUB_VECS;
+    const bool rw_small  = rows <= 256 && (size_t)rows * a->vocab_size_padded * elem <= (size_t)RW_SMALL_BYTES
+                          && a->vocab_size >= 1024;
     const bool rowwide   = lean_mode == 1 && !want_log_probs && a->embedding_bias == nullptr && lplan.splits > 1
-                         && g_fused_two_launches == 0 && rows * 5 >= rw_rounds * 256 * 4
-                         && (size_t)a->vocab_size / (16 / elem) >= (size_t)RW_MIN_SUBS * RW_SUB_VECS
+                         && g_fused_two_launches == 0 && (rw_full || rw_small)
                          && (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_LARGE
                          && ((uintptr_t)a->logits & 15u) == 0 && ((size_t)a->vocab_size_padded * elem) % 16 == 0
                          && (a->penalty_type == FTK_PENALTY_NONE || a->penalties == nullptr

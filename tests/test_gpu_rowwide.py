@@ -109,15 +109,16 @@ def test_rowwide_generated_draws_are_reproducible():
 
 def test_rowwide_kernel_is_what_these_shapes_take():
     """the test build of the library reports the path of its last fused step: 3 = one 1024-thread workgroup per row;
-    the same rows in two launches (hook) and a batch of 100 rows do not take it, and all agree on the ids"""
+    the same rows in two launches (hook) and a batch of 100 long rows do not take it, 100 short rows do (a launch
+    of a few megabytes is bound by latency), and all agree on the ids"""
     import torch
     from fastertransformer_amd import ops
     from helpers import run_fused_step
     hooks = ops.ftk_hooks()
     gen = torch.Generator(device="cuda")
     gen.manual_seed(9)
-    V, H, k = 65600, 16, 64
-    for B, want in ((256, 3), (100, 1)):
+    H, k = 16, 64
+    for B, V, want in ((256, 65600, 3), (100, 128256, 1), (100, 32000, 3)):  # (small launches take it at any batch)
         logits = torch.randn((B, V), generator=gen, device="cuda") * 2.0
         history = torch.randint(0, V, (H, B), generator=gen, device="cuda", dtype=torch.int32)
         draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
