@@ -31,6 +31,9 @@ struct FusedParams {
     // `logits` points at the shard's first column, Vp is the pitch of its rows): token ids in the history and the
     // end ids are global, and so are the column numbers the launch reports. 0 for whole rows.
     int          col_offset;
+    // Frequency penalty (an extension of the additive rule): a column that occurs `count` times in the row's history
+    // gets x - penalty - frequency * count. Null: none. Only the kernels that keep a table of the counts in LDS take it.
+    const float* frequencies;
 };
 
 // History bitmaps: bit v set <=> token v occurs in the row's (non-padding) history, i.e. column v gets
@@ -92,7 +95,7 @@ __device__ __forceinline__ float uniform_f(float x)
 // A row's per-row arguments, requested in one block without control flow so that they share one trip to memory
 // (the arithmetic on them, which waits for the values, comes afterwards).
 struct FusedRowArgs {
-    float temperature, penalty;
+    float temperature, penalty, frequency;
     int   input_length, min_length, sequence_length, end_id;
 };
 __device__ __forceinline__ FusedRowArgs fused_row_args(const FusedParams& p, int row)
@@ -101,11 +104,54 @@ __device__ __forceinline__ FusedRowArgs fused_row_args(const FusedParams& p, int
     FusedRowArgs a;
     a.temperature     = row_arg_or(p.temperatures, row, safe, 1.0f);
     a.penalty         = row_arg_or(p.penalties, row, safe, 0.0f);
+    a.frequency       = row_arg_or(p.frequencies, row, safe, 0.0f);
     a.input_length    = row_arg_or(p.input_lengths, row, safe, p.max_input_length);
     a.min_length      = row_arg_or(p.min_lengths, row, safe, 0);
     a.sequence_length = row_arg_or(p.min_lengths != nullptr ? p.sequence_length_in : nullptr, row, safe, 0);
     a.end_id          = p.end_ids[row];
     return a;
+}
+
+// How often each token id occurs in a row's history: an open-addressing table in LDS, one 32-bit word per distinct
+// id, (id + 1) << 13 | count. Ids below 2^18 and at most 4096 history positions (half the slots), which the
+// launcher checks.
+constexpr int      FUSED_COUNT_SLOTS = 8192;
+constexpr int      FUSED_COUNT_BITS  = 13;
+constexpr int      FUSED_COUNT_MAX_VOCAB = 1 << 18;
+__device__ __forceinline__ uint32_t fused_count_hash(int id)
+{
+    return ((uint32_t)id * 2654435761u) >> (32 - FUSED_COUNT_BITS);
+}
+__device__ __forceinline__ void fused_count_insert(uint32_t* table, int id)
+{
+    const uint32_t tag = (uint32_t)(id + 1) << FUSED_COUNT_BITS;
+    uint32_t       h   = fused_count_hash(id);
+    for (int probe = 0; probe < FUSED_COUNT_SLOTS; ++probe) {
+        const uint32_t old = atomicCAS(&table[h], 0u, tag | 1u);
+        if (old == 0u) {
+            return;
+        }
+        if ((old >> FUSED_COUNT_BITS) == (uint32_t)(id + 1)) {
+            atomicAdd(&table[h], 1u);
+            return;
+        }
+        h = (h + 1) & (FUSED_COUNT_SLOTS - 1);
+    }
+}
+__device__ __forceinline__ int fused_count_lookup(const uint32_t* table, int id)
+{
+    uint32_t h = fused_count_hash(id);
+    for (int probe = 0; probe < FUSED_COUNT_SLOTS; ++probe) {
+        const uint32_t e = table[h];
+        if (e == 0u) {
+            return 0;
+        }
+        if ((e >> FUSED_COUNT_BITS) == (uint32_t)(id + 1)) {
+            return (int)(e & ((1u << FUSED_COUNT_BITS) - 1u));
+        }
+        h = (h + 1) & (FUSED_COUNT_SLOTS - 1);
+    }
+    return 0;
 }
 
 template<int DT, int BMW>
@@ -132,6 +178,10 @@ struct FusedRow {
     const int*      history;  // output_ids + row, stride batch_size
     int             batch_size, step, input_length, max_input_length;
     int             col_offset;  // global number of column 0 (a vocabulary shard), see FusedParams
+    int             team;        // threads that call prepare() / prepare_whole_row() together (the whole workgroup
+                                 // unless the caller says otherwise: some of a workgroup's waves may have left)
+    float           frequency;   // frequency penalty of the row (with count_table), see FusedParams
+    const uint32_t* count_table; // null: no frequency penalty
 
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row): FusedRow(p, row, fused_row_args(p, row)) {}
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row, const FusedRowArgs& args)
@@ -177,6 +227,9 @@ struct FusedRow {
         up_mul_pos = uniform_f(up_mul_pos);
         up_add     = uniform_f(up_add);
         col_offset    = p.col_offset;
+        team          = (int)blockDim.x;
+        frequency     = uniform_f(args.frequency);
+        count_table   = nullptr;  // (the kernel that keeps the table sets it)
         masked_end_id = (p.min_lengths != nullptr
                          && min_length_masks(args.sequence_length, p.max_input_length, args.min_length)
                          && args.end_id >= p.col_offset) ?
@@ -200,18 +253,18 @@ struct FusedRow {
         uint32_t* window = fused_lds_bitmap<LDS_WORDS>();
         const int origin = lo & ~31;
         const int words  = min(LDS_WORDS, (hi - origin + 31) / 32 + 1);
-        for (int i = threadIdx.x; i < words; i += blockDim.x) {
+        for (int i = threadIdx.x; i < words; i += team) {
             window[i] = 0u;
         }
         __syncthreads();
         // the history is time-major: every id is a cache line of its own, so the reads are issued eight
         // deep before the first one is used
         constexpr int U = 8;
-        for (int t0 = threadIdx.x; t0 < step; t0 += U * blockDim.x) {
+        for (int t0 = threadIdx.x; t0 < step; t0 += U * team) {
             int ids[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int t = t0 + u * blockDim.x;
+                const int t = t0 + u * team;
                 ids[u] = (t < step && history_position_counts(t)) ? history[(size_t)t * batch_size] - col_offset : -1;
             }
 #pragma unroll
@@ -239,12 +292,12 @@ struct FusedRow {
             return;  // (a workgroup with an LDS window owns the whole row: the window already covers it)
         }
         const int words = (Vp + 31) / 32 + 1;
-        for (int i = threadIdx.x; i < words; i += blockDim.x) {
+        for (int i = threadIdx.x; i < words; i += team) {
             global_bm[i] = 0u;
         }
         __threadfence_block();
         __syncthreads();
-        for (int t = threadIdx.x; t < step; t += blockDim.x) {
+        for (int t = threadIdx.x; t < step; t += team) {
             if (history_position_counts(t)) {
                 const int id = history[(size_t)t * batch_size];
                 if (id >= 0 && id < Vp) {
@@ -308,10 +361,20 @@ struct FusedRow {
     {
         return round_t<DT>(x * fast_mul);  // fast_mul is 1 without a temperature: exact, and x is a T already
     }
-    // the same column when it is in the history
-    __device__ __forceinline__ float flagged(float xf) const
+    // the same column (number v) when it is in the history
+    __device__ __forceinline__ float flagged(float xf, int v) const
     {
+        if (count_table != nullptr) {
+            return round_t<DT>(frequency_value(xf, penalty, frequency, fused_count_lookup(count_table, v + col_offset)));
+        }
         return round_t<DT>(repetition_value(xf, penalty, penalty_type));
+    }
+    // the kernel's table of counts is in place: columns of the history take the frequency rule from here on
+    __device__ __forceinline__ void use_count_table(const uint32_t* table)
+    {
+        count_table = table;
+        // (the cheap upper bound of flagged_upper holds while neither term raises a value)
+        up_ok = up_ok && penalty >= 0.0f && frequency >= 0.0f;
     }
     // Never below flagged(xf), without the division and without branches: for the multiplicative rule
     // x * RN(1/p) * (1 + 2^-20) >= x / p for x >= 0 and a positive finite p (as real numbers, so also after
@@ -355,7 +418,7 @@ struct FusedRow {
             }
         }
         if (in_history) {
-            x = round_t<DT>(repetition_value(x, penalty, penalty_type));
+            x = flagged(x, v);
         }
         if (v == masked_end_id) {
             x = -S::max_t();

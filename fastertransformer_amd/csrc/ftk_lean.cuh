@@ -548,7 +548,7 @@ __global__ void __launch_bounds__(LG_THREADS, OCC) lean_gather_kernel(FusedParam
 #pragma unroll
                     for (int c = 0; c < EPV; ++c) {
                         if ((bits >> c) & 1u) {
-                            x[c] = rowctx.flagged(x[c]);
+                            x[c] = rowctx.flagged(x[c], first + c);
                         }
                     }
                 }

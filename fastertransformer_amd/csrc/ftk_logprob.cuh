@@ -155,7 +155,7 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
         for (int c = 0; c < EPV; ++c) {
             float x = rowctx.fast(vector_element<DT>(v, c));
             if ((bits >> c) & 1u) {
-                x = rowctx.flagged(x);
+                x = rowctx.flagged(x, first + c);
             }
             if ((uint32_t)c == rel_end) {
                 x = -S::max_t();
@@ -433,7 +433,7 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
 #pragma unroll
             for (int c = 0; c < LP_CHAINS; ++c) {
                 if ((bits >> c) & 1u) {
-                    y[c] = rowctx.flagged(y[c]);
+                    y[c] = rowctx.flagged(y[c], col + c);
                 }
                 if ((uint32_t)c == rel_end || (uint32_t)(col + c) >= (uint32_t)p.V) {
                     y[c] = -S::max_t();

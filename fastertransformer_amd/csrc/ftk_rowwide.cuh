@@ -40,6 +40,7 @@ constexpr int RW_SMALL_BYTES = 32 << 20;            // a launch that reads less 
                                                     // batch up to 256 rows: it is bound by latency, not bandwidth
 
 struct RowwideShared {
+    uint32_t count_table[FUSED_COUNT_SLOTS];  // occurrences of the history's ids (rows with a frequency penalty)
     uint4    stage_raw[RW_WAVES][RW_STAGE];
     int      stage_first[RW_WAVES][RW_STAGE];
     uint32_t slot_key[RW_THREADS];
@@ -269,10 +270,14 @@ __device__ __forceinline__ int rowwide_rank_distinct(TopkShared& s, int n, int k
 template<int DT>
 __device__ __noinline__ void rowwide_rare(TopkShared& ts, const FusedParams p, const FusedLaunch l,
                                           const FusedRowArgs args, int row, int n, uint32_t thr, int k, float tp,
-                                          float u, const TopkOutputs out)
+                                          float u, const TopkOutputs out, const uint32_t* count_table)
 {
     TopkEntry*      row_entries = l.entries + (size_t)row * l.row_entries;
     FusedRow<DT, 0> r0(p, row, args);
+    r0.team = TK_THREADS;  // (the other waves of the workgroup have left)
+    if (count_table != nullptr) {
+        r0.use_count_table(count_table);
+    }
     if (n > TK_CCAP) {
         r0.prepare_whole_row();
         __syncthreads();
@@ -379,10 +384,17 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
     load(0, 0);
     // while all that is on its way: an empty bitmap of the row's history
     uint32_t* window = fused_lds_bitmap<BMW>();
+    const bool counting = hist && p.frequencies != nullptr;  // a frequency penalty: the history's ids are counted too
     if (hist) {
         const int words = min(BMW, (p.V + 31) / 32 + 1);
         for (int i = t; i < words; i += RW_THREADS) {
             window[i] = 0u;
+        }
+        if (counting) {
+#pragma unroll
+            for (int i = 0; i < FUSED_COUNT_SLOTS / RW_THREADS; ++i) {
+                s.count_table[t + i * RW_THREADS] = 0u;
+            }
         }
     }
     if (t == 0) {
@@ -415,10 +427,16 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
             const int id  = hist_ids[u];
             if (pos < p.step && id >= 0 && id < p.V && rowctx.history_position_counts(pos)) {
                 atomicOr(&window[id >> 5], 1u << (id & 31));
+                if (counting) {
+                    fused_count_insert(s.count_table, id);
+                }
             }
         }
         rowctx.bm_mode   = 1;
         rowctx.bm_origin = 0;
+        if (counting) {
+            rowctx.use_count_table(s.count_table);  // (read after the barrier below)
+        }
     }
     lds_barrier();
 #pragma unroll
@@ -448,8 +466,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
             float       g   = h;
             bool        raises;
             if (rowctx.penalty_type == 0) {
-                raises = !(pen >= 0.0f);
-                g      = h + pen;
+                // (with a frequency penalty a column loses pen + frequency * count, count between 1 and the step)
+                const float per_count = counting ? __builtin_fminf(rowctx.frequency, rowctx.frequency * (float)p.step) : 0.0f;
+                g                     = h + (pen + per_count);
+                raises                = !(g >= h);
             }
             else {
                 raises = !(pen >= 1.0f);
@@ -527,7 +547,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
 #pragma unroll
                     for (int c = 0; c < EPV; ++c) {
                         if ((bits >> c) & 1u) {
-                            x[c] = rowctx.flagged(x[c]);
+                            x[c] = rowctx.flagged(x[c], first + c);
                         }
                     }
                 }
@@ -742,7 +762,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         topk_finish_list<DT>(ts, n_list, row, p.Vp, tp, false, u, p.end_ids, out);
     }
     else {
-        rowwide_rare<DT>(ts, p, l, args, row, n, thr, k, tp, u, out);
+        rowwide_rare<DT>(ts, p, l, args, row, n, thr, k, tp, u, out, counting ? s.count_table : nullptr);
     }
     RW_STAMP(6)
 }

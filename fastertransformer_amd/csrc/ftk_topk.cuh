@@ -122,7 +122,7 @@ __device__ __forceinline__ void lds_barrier()
 //   vector_bits(first, n)  - one bit per flagged column of a 16-byte vector
 //   plain_vector(first, n) - true when no column of the span needs an index-dependent rule
 //   fast(x)                - index-independent transform of an interior column
-//   flagged(xf)            - fast(x) -> value of a flagged interior column
+//   flagged(xf, v)         - fast(x) -> value of the flagged interior column v
 //   flagged_upper(xf)      - a cheap value that is never below flagged(xf): decides which vectors are
 //                            looked at again, the exact value is computed for those only
 //   tile_bits(...)         - the flags of a whole tile of an aligned row, EPV bits per vector, packed
@@ -163,7 +163,7 @@ struct PlainRow {
     {
         return x;
     }
-    __device__ __forceinline__ float flagged(float xf) const
+    __device__ __forceinline__ float flagged(float xf, int) const
     {
         return xf;
     }
@@ -818,7 +818,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
 #pragma unroll
                 for (int j = 0; j < EPV; ++j) {
                     if ((bits >> j) & 1u) {
-                        x[j] = rowctx.flagged(x[j]);
+                        x[j] = rowctx.flagged(x[j], first + j);
                     }
                 }
             }
@@ -936,7 +936,7 @@ __device__ __forceinline__ int topk_stream(Row& rowctx, TopkShared& s, int vocab
 #pragma unroll
                         for (int j = 0; j < EPV; ++j) {
                             if ((bits >> j) & 1u) {
-                                x[j] = rowctx.flagged(x[j]);
+                                x[j] = rowctx.flagged(x[j], first + j);
                             }
                         }
                     }

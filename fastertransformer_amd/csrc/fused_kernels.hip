@@ -244,6 +244,14 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
                          && ((uintptr_t)a->logits & 15u) == 0 && ((size_t)a->vocab_size_padded * elem) % 16 == 0
                          && (a->penalty_type == FTK_PENALTY_NONE || a->penalties == nullptr
                              || a->step <= RW_HIST_U * RW_THREADS);
+    // A frequency penalty needs the counts of the history's ids, which only that kernel keeps (a table in LDS).
+    if (a->frequency_penalties != nullptr
+        && (a->penalties == nullptr || a->penalty_type != FTK_PENALTY_ADDITIVE || a->output_ids == nullptr)) {
+        return FTK_ERR_ARGUMENT;  // x - presence - frequency * count: the presence array comes with it
+    }
+    if (a->frequency_penalties != nullptr && (!rowwide || a->vocab_size_padded > FUSED_COUNT_MAX_VOCAB)) {
+        return FTK_ERR_UNSUPPORTED;
+    }
     const size_t   slot_bytes = lean_mode == 2 ? (size_t)lplan.splits * slot_u * LG_THREADS * sizeof(uint32_t) : 0;
     const size_t   lean_bytes =
         (size_t)(rows > 0 ? rows : 0)
@@ -290,6 +298,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
     p.bitmap_words       = bitmap_words;
     p.bitmaps_ready      = 0;
     p.lds_window         = 0;
+    p.frequencies        = (p.penalties != nullptr && a->step > 0) ? a->frequency_penalties : nullptr;
 
     char* ws = (char*)a->workspace;
     if (p.penalties != nullptr && a->step > 0) {

@@ -220,7 +220,7 @@ class FusedTopkArgs(C.Structure):
         ("input_lengths", _vp), ("output_ids", _vp), ("top_ks", _vp), ("top_ps", _vp), ("max_top_k", _i),
         ("skip_decode", _vp), ("rng_state", _vp), ("uniform_draws", _vp), ("ids", _vp), ("sequence_length", _vp),
         ("finished", _vp), ("cum_log_probs", _vp), ("output_log_probs", _vp), ("workspace", _vp),
-        ("workspace_size", _sz),
+        ("workspace_size", _sz), ("frequency_penalties", _vp),
     ]
 
 

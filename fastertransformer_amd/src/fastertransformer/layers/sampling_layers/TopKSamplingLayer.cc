@@ -153,15 +153,15 @@ void TopKSamplingLayer<T>::ensureWorkspace(int local_batch_size)
 }
 
 // One streaming pass over the logits for the whole penalty + mask + top-k pipeline - two passes when log-prob
-// outputs are requested, which need the probabilities of the whole row. Not taken with the frequency-penalty
-// extension, nor for the configurations the fused step reports as unsupported with log-probs, nor for log-probs
-// on small windows.
+// outputs are requested, which need the probabilities of the whole row. Not taken for the configurations the fused
+// step reports as unsupported (log-probs with a bias or a large k, the frequency-penalty extension outside the
+// one-launch step), nor for log-probs on small windows.
 template<typename T>
 bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_tensors)
 {
     float* cum_log_probs    = output_tensors->at("cum_log_probs", Tensor()).template getPtr<float>();
     float* output_log_probs = output_tensors->at("output_log_probs", Tensor()).template getPtr<float>();
-    if (fused_disabled_ || this->has_frequency_penalty_) {
+    if (fused_disabled_) {
         return false;
     }
     const int batch_size       = output_tensors->at("output_ids").shape[1];
@@ -198,6 +198,15 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
             a.penalty_type = toFtkPenalty(this->repetition_penalty_type_);
             a.penalties    = this->repetition_penalty_buf_ + off;
         }
+        if (this->has_frequency_penalty_) {
+            const float* fr = this->frequency_penalty_.data() + off;
+            if (!std::all_of(fr, fr + local_batch_size, [](float x) { return x == 0.0f; })) {
+                // (x - presence - frequency * count: the presence array goes along even when it is all zeros)
+                a.penalty_type        = FTK_PENALTY_ADDITIVE;
+                a.penalties           = this->repetition_penalty_buf_ + off;
+                a.frequency_penalties = this->frequency_penalty_buf_ + off;
+            }
+        }
     }
     const int  num_generated_tokens = step - max_input_length;
     const int* min_lengths          = this->min_lengths_.data() + off;
@@ -225,7 +234,8 @@ bool TopKSamplingLayer<T>::runFused(TensorMap* output_tensors, TensorMap* input_
     a.workspace = nullptr;
     const int query = ftk_fused_topk_step(&a, stream_);
     if (query == FTK_ERR_UNSUPPORTED) {
-        return false;  // log-probs with a bias, a large k or a tiny vocabulary: the kernel sequence
+        return false;  // log-probs with a bias, a large k or a tiny vocabulary, a frequency penalty outside the
+                       // one-launch step: the kernel sequence
     }
     check_ftk(query);
     if (a.workspace_size > sampling_workspace_size_) {

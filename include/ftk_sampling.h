@@ -231,6 +231,14 @@ typedef struct ftk_fused_topk_args {
     float* output_log_probs; /* [local] or NULL: the row of this step */
     void*  workspace;
     size_t workspace_size;
+    /* Frequency penalty, an extension without reference code: with it a column that occurs `count` times in the row's
+     * history gets x - penalties[b] - frequency_penalties[b] * count (penalty_type must be FTK_PENALTY_ADDITIVE and
+     * `penalties` hold the presence term, zeros if there is none). [local] or NULL. Covered where the step runs as one
+     * launch of one workgroup per row (no log-probs, no bias, largest k <= 192, rows on 16-byte boundaries, up to
+     * 256 rows of a small launch or nearly full rounds of 256 rows, history up to 4096 positions, vocabulary up to
+     * 2^18); anything else returns FTK_ERR_UNSUPPORTED: run ftk_invoke_batch_apply_frequency_penalty and the rest of
+     * the kernel sequence instead. */
+    const float* frequency_penalties;
 } ftk_fused_topk_args;
 
 /* workspace == NULL in args: writes the required size into args->workspace_size, launches nothing. */

@@ -84,7 +84,7 @@ def uniforms(rng, n):
     return u.astype(np.float32)
 
 
-def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=None):
+def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=None, ws_fill=None):
     """One fused decode step straight through the C ABI (temperature 0.8, repetition penalty 1.1 over `history`,
     top-k `k`, top-p 0.9, injected draws). entry: "caller" = ftk_fused_topk_step with a workspace of the queried
     size, "static" = ftk_fused_topk_step_static. Returns (ids, sequence_length, finished, rc, needed bytes, change of
@@ -120,6 +120,8 @@ def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finishe
         a.workspace = None
         ops.check(lib.ftk_fused_topk_step(C.addressof(a), stream), "size query")
         ws = torch.empty(a.workspace_size, dtype=torch.uint8, device=dev)
+        if ws_fill is not None:
+            ws.fill_(ws_fill)  # (nothing in the workspace has to start at zero)
         a.workspace = ws.data_ptr()
         rc = lib.ftk_fused_topk_step(C.addressof(a), stream)
         torch.cuda.synchronize()

@@ -136,3 +136,34 @@ def test_rowwide_kernel_is_what_these_shapes_take():
             hooks.ftk_test_set_fused_two_launches(0)
         for a, b in zip(one[:3], two[:3]):
             assert np.array_equal(a, b)
+
+
+def test_rowwide_rows_walked_again_do_not_depend_on_the_workspace():
+    """Rows whose list outgrows LDS are walked again by the four waves that are left of the workgroup, with the
+    history bitmap rebuilt in the workspace: constant rows with a few larger columns, some of them in the history
+    (so the penalty decides which win), a workspace full of ones. Same ids as the two-launch step."""
+    import torch
+    from fastertransformer_amd import ops
+    from helpers import run_fused_step
+    hooks = ops.ftk_hooks()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    B, V, H, k = 32, 149544, 300, 150
+    logits = torch.full((B, V), 0.75, device="cuda")
+    logits[:, ::997] = 1.0
+    history = torch.randint(0, V // 997, (H, B), generator=gen, device="cuda", dtype=torch.int32) * 997
+    draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
+    finished0 = torch.zeros(B, dtype=torch.bool, device="cuda")
+    seqlen0 = torch.full((B,), H - 1, dtype=torch.int32, device="cuda")
+    one = run_fused_step("caller", torch, O.F32, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks,
+                         ws_fill=0xFF)
+    assert one[3] == 0 and hooks.ftk_test_last_fused_path() == 3
+    hooks.ftk_test_set_fused_two_launches(1)
+    try:
+        two = run_fused_step("caller", torch, O.F32, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks,
+                             ws_fill=0xFF)
+    finally:
+        hooks.ftk_test_set_fused_two_launches(0)
+    for a, b in zip(one[:3], two[:3]):
+        assert np.array_equal(a, b)
+    assert (one[0] % 997 == 0).all()  # only the larger columns can be sampled (k = 150 of them, all tied)
