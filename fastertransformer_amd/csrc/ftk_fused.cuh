@@ -126,6 +126,7 @@ __device__ __forceinline__ void fused_count_insert(uint32_t* table, int id)
 {
     const uint32_t tag = (uint32_t)(id + 1) << FUSED_COUNT_BITS;
     uint32_t       h   = fused_count_hash(id);
+#pragma unroll 1
     for (int probe = 0; probe < FUSED_COUNT_SLOTS; ++probe) {
         const uint32_t old = atomicCAS(&table[h], 0u, tag | 1u);
         if (old == 0u) {
@@ -141,6 +142,7 @@ __device__ __forceinline__ void fused_count_insert(uint32_t* table, int id)
 __device__ __forceinline__ int fused_count_lookup(const uint32_t* table, int id)
 {
     uint32_t h = fused_count_hash(id);
+#pragma unroll 1
     for (int probe = 0; probe < FUSED_COUNT_SLOTS; ++probe) {
         const uint32_t e = table[h];
         if (e == 0u) {

@@ -45,13 +45,17 @@ struct RowwideShared {
     int      stage_first[RW_WAVES][RW_STAGE];
     uint32_t slot_key[RW_THREADS];
     uint32_t bound;
+    float    bound_hot;  // what a raw maximum times the multiplier must reach under that bound
+    int      late[3];    // the row's top_p, sequence length and end id, for the end of the kernel
     int      n_list[2];  // length of the row's list; the second counter takes over when the list is pruned
 };
 
 // The largest value P, to within its low sixteen bits, such that at least k of 256 keys are >= P (0 when fewer
 // than k are non-zero); slot i of the 256 is the largest of keys i, i + 256, i + 512, i + 768 of the workgroup, all
-// of them keys of distinct elements. The first wave finds it, every thread gets it. Two barriers.
-__device__ __forceinline__ uint32_t rowwide_bound(RowwideShared& s, uint32_t my_key, int k)
+// of them keys of distinct elements. The first wave finds it and what follows from it for the stream (hot_of(P), a
+// few dozen instructions that sixteen waves in lock-step would each pay for); every thread gets both. Two barriers.
+template<typename HotOf>
+__device__ __forceinline__ uint32_t rowwide_bound(RowwideShared& s, uint32_t my_key, int k, HotOf hot_of, float& hot)
 {
     s.slot_key[threadIdx.x] = my_key;
     lds_barrier();
@@ -73,11 +77,14 @@ __device__ __forceinline__ uint32_t rowwide_bound(RowwideShared& s, uint32_t my_
             }
             P = c >= k ? cand : P;
         }
+        const float h = hot_of(P);
         if (lane_id() == 0) {
-            s.bound = P;
+            s.bound     = P;
+            s.bound_hot = h;
         }
     }
     lds_barrier();
+    hot = uniform_f(s.bound_hot);
     return (uint32_t)__builtin_amdgcn_readfirstlane((int)s.bound);
 }
 
@@ -262,16 +269,38 @@ __device__ __forceinline__ int rowwide_rank_distinct(TopkShared& s, int n, int k
     return n_list;
 }
 
+// The kernel's arguments as one block, so that code that is rarely reached can read them again from the
+// kernel-argument segment instead of keeping some fifty scalar registers alive through the whole kernel for it.
+struct RowwideArgs {
+    FusedParams p;
+    FusedLaunch l;
+};
+typedef const __attribute__((address_space(4))) void* RowwideArgSegment;
+
 // What is left to the first four waves when a row's list is still longer than 256 entries after the cut (the
 // selection of topk_select_lds for long lists) or outgrew LDS (the whole row is walked again with the stream that
 // recovers from overfull tiles; rows it cannot bound either take the literal replay). Not inlined, so that the
-// kernel's registers are planned for its stream; the launch arguments are passed by value (a reference would move
-// the kernel's own copy from scalar registers to scratch memory).
+// kernel's registers are planned for its stream, and it takes the launch arguments and the row's own from memory
+// again (passed by reference they would move the kernel's copy from scalar registers to scratch memory; passed by
+// value they stay live, and spill, all the way through the kernel).
 template<int DT>
-__device__ __noinline__ void rowwide_rare(TopkShared& ts, const FusedParams p, const FusedLaunch l,
-                                          const FusedRowArgs args, int row, int n, uint32_t thr, int k, float tp,
-                                          float u, const TopkOutputs out, const uint32_t* count_table)
+__device__ __noinline__ void rowwide_rare(TopkShared& ts, RowwideArgSegment segment, int row, int n, uint32_t thr, int k,
+                                          float tp, float u, const uint32_t* count_table)
 {
+    RowwideArgs a;
+    __builtin_memcpy(&a, (const void*)segment, sizeof(a));
+    const FusedParams& p    = a.p;
+    const FusedLaunch& l    = a.l;
+    const FusedRowArgs args = fused_row_args(p, row);
+    TopkOutputs        out;
+    out.ids                = l.ids;
+    out.sequence_length    = l.sequence_length;
+    out.finished           = l.finished;
+    out.cum_log_probs      = nullptr;
+    out.output_log_probs   = nullptr;
+    out.sequence_length_in = l.sequence_length != nullptr ? l.sequence_length[row] : 0;  // (not written yet)
+    out.cum_log_prob_in    = 0.0f;
+    out.end_id_in          = args.end_id;
     TopkEntry*      row_entries = l.entries + (size_t)row * l.row_entries;
     FusedRow<DT, 0> r0(p, row, args);
     r0.team = TK_THREADS;  // (the other waves of the workgroup have left)
@@ -302,16 +331,18 @@ __device__ __forceinline__ void rowwide_pin(V& v)
 }
 
 template<int DT, int BMW>
-__global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedParams p_in, const FusedLaunch l_in)
+__global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideArgs a_in)
 {
-    FusedParams p = p_in;
-    FusedLaunch l = l_in;
+    const FusedLaunch& l_in = a_in.l;
+    FusedParams        p    = a_in.p;
+    FusedLaunch        l    = a_in.l;
     rowwide_pin(p.V);
     rowwide_pin(p.Vp);
     rowwide_pin(p.step);
     rowwide_pin(p.max_input_length);
     rowwide_pin(p.max_top_k);
     rowwide_pin(p.penalty_type);
+    rowwide_pin(p.col_offset);
     // (pointers that are only stored through, at the end: a pinned pointer is a generic one to the compiler)
     rowwide_pin(l.ids);
     rowwide_pin(l.sequence_length);
@@ -359,6 +390,9 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
     unsigned long long counter_addr = (unsigned long long)(l.rng != nullptr ? &l.rng[row].offset : nullptr);
     rowwide_pin(counter_addr);
     const bool         hist = p.bitmaps != nullptr && p.penalties != nullptr;
+    // (the instruction scheduler keeps the argument loads above in front of the vector loads below: requested behind
+    // them, they would also arrive behind them)
+    __builtin_amdgcn_sched_barrier(0);
     int                hist_ids[RW_HIST_U];
     {
         const int* column = hist ? p.output_ids + row : p.end_ids;  // (without a history: any valid address)
@@ -410,7 +444,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         }
         return;
     }
-    // the row's draw: taken once, by the rows that take part (like the reference's curand_uniform)
+    // The row's draw: taken once, by the rows that take part (like the reference's curand_uniform). With it, what
+    // only the end of the kernel needs of the row's arguments moves to LDS: values that stay in scalar registers from
+    // their load to the end are the first the register allocator spills, and a spill of a value that is still on
+    // its way waits for it - in front of the row's loads.
     if (t == 0) {
         float u = draw.injected;
         if (!injected) {
@@ -419,6 +456,9 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
             *(__attribute__((address_space(1))) uint64_t*)counter_addr = next;
         }
         ts.misc[0] = __float_as_int(u);
+        s.late[0]  = __float_as_int(tp);
+        s.late[1]  = seq_in;
+        s.late[2]  = args.end_id;
     }
     if (hist) {
 #pragma unroll
@@ -454,9 +494,13 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
     uint32_t thr     = KMIN;  // candidates are the elements with key >= thr
     float    thr_f   = key_to_float(thr);
     float    thr_hot = NEG_INF;  // (without a bound every vector is looked at exactly)
-    auto     set_threshold = [&](uint32_t key) {
+    auto     set_threshold = [&](uint32_t key, float hot) {
         thr     = key;
         thr_f   = key_to_float(key);
+        thr_hot = hot;
+    };
+    auto hot_of = [&](uint32_t key) -> float {
+        const float thr_f = key_to_float(key);
         // What the unrounded, unpenalised product of an element must reach for its final value to reach thr_f:
         // rounding to T can lift a product by half a unit of T, and a history penalty that raises values
         // (a multiplicative one below 1, a negative additive one) can lift it further.
@@ -484,7 +528,7 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
         if (!(h == h) || !(__builtin_fabsf(thr_f) < __builtin_inff())) {
             h = NEG_INF;
         }
-        thr_hot = uniform_f(h);
+        return h;
     };
 
     // flags of the vector that starts at column `first` (a multiple of EPV): one bit per column of the history
@@ -510,9 +554,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
             tmax              = __builtin_fmaxf(tmax, clean ? vm : NEG_INF);
         }
         tmax = all_hit ? NEG_INF : rowctx.fast(tmax);  // (the transform keeps the order)
-        const uint32_t P = rowwide_bound(s, order_key(tmax), k);
+        float          hot;
+        const uint32_t P = rowwide_bound(s, order_key(tmax), k, hot_of, hot);
         if (P >= KMIN) {
-            set_threshold(P);
+            set_threshold(P, hot);
         }
     }
 
@@ -647,9 +692,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
                     const uint32_t idx     = t < n_now ? ts.cand.idx[t] : 0u;
                     // the k-th largest of 256 disjoint groups of the list's entries; of the lanes' largest entries when
                     // the list is longer than the workgroup
-                    const uint32_t P = rowwide_bound(s, listed ? key : dmax, k);
+                    float          hot;
+                    const uint32_t P = rowwide_bound(s, listed ? key : dmax, k, hot_of, hot);
                     if (P > thr) {
-                        set_threshold(P);
+                        set_threshold(P, hot);
                         if (listed) {
                             // entries below the new bound (collected under an older one) leave the list
                             const bool               keep = key >= P;  // (P > 0: the slots past the list drop out)
@@ -704,9 +750,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
     out.finished           = l.finished;
     out.cum_log_probs      = nullptr;
     out.output_log_probs   = nullptr;
-    out.sequence_length_in = seq_in;
+    out.sequence_length_in = __builtin_amdgcn_readfirstlane(s.late[1]);
     out.cum_log_prob_in    = 0.0f;
-    out.end_id_in          = args.end_id;
+    out.end_id_in          = __builtin_amdgcn_readfirstlane(s.late[2]);
+    const float tp_late    = uniform_f(__int_as_float(s.late[0]));
     int         n = s.n_list[cur];
     const float u = __int_as_float(ts.misc[0]);
     if (n > k + k / 2 && n > 96 && n <= 4 * TK_THREADS) {
@@ -759,10 +806,11 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const FusedPar
 #ifdef FTK_RW_STAMPS
         if (threadIdx.x == 0) { stamps[9] = (unsigned long long)n; }
 #endif
-        topk_finish_list<DT>(ts, n_list, row, p.Vp, tp, false, u, p.end_ids, out);
+        topk_finish_list<DT>(ts, n_list, row, p.Vp, tp_late, false, u, p.end_ids, out);
     }
     else {
-        rowwide_rare<DT>(ts, p, l, args, row, n, thr, k, tp, u, out, counting ? s.count_table : nullptr);
+        rowwide_rare<DT>(ts, (RowwideArgSegment)__builtin_amdgcn_kernarg_segment_ptr(), row, n, thr, k, tp_late, u,
+                         counting ? s.count_table : nullptr);
     }
     RW_STAMP(6)
 }

@@ -95,12 +95,15 @@ int rowwide_launch_bf16
 #endif
     (int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start, hipEvent_t stop)
 {
+    RowwideArgs a;
+    a.p = p;
+    a.l = l;
     auto launch = [&](auto kernel) {
         if (start != nullptr) {
-            hipExtLaunchKernelGGL(kernel, dim3(rows), dim3(RW_THREADS), 0, st, start, stop, 0, p, l);
+            hipExtLaunchKernelGGL(kernel, dim3(rows), dim3(RW_THREADS), 0, st, start, stop, 0, a);
         }
         else {
-            hipLaunchKernelGGL(kernel, dim3(rows), dim3(RW_THREADS), 0, st, p, l);
+            hipLaunchKernelGGL(kernel, dim3(rows), dim3(RW_THREADS), 0, st, a);
         }
     };
     if (window == 2) {
