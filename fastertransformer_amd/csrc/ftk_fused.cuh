@@ -156,6 +156,15 @@ __device__ __forceinline__ int fused_count_lookup(const uint32_t* table, int id)
     return 0;
 }
 
+// What a FusedRow works out from the row's arguments, as ten 32-bit words: one wave can do the arithmetic and hand
+// the result to the others of a large workgroup.
+struct FusedRowDerived {
+    static constexpr int WORDS = 10;
+    float inv, fast_mul, penalty, frequency, up_mul_neg, up_mul_pos, up_add;
+    int   masked_end_id, input_length;
+    int   flags;  // bit 0: keep_pads, bit 1: up_ok
+};
+
 template<int DT, int BMW>
 struct FusedRow {
     static constexpr int  LDS_WORDS = BMW > 0 ? BMW : 1;
@@ -186,18 +195,65 @@ struct FusedRow {
     const uint32_t* count_table; // null: no frequency penalty
 
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row): FusedRow(p, row, fused_row_args(p, row)) {}
+    // what does not depend on the row's own arguments
+    __device__ __forceinline__ void from_launch(const FusedParams& p, int row)
+    {
+        rowp             = (const T*)p.logits + (size_t)row * p.Vp;
+        bias             = (const T*)p.bias;
+        V                = p.V;
+        Vp               = p.Vp;
+        temp_active      = p.temperatures != nullptr;
+        penalty_type     = p.penalties != nullptr ? p.penalty_type : 2;
+        global_bm        = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
+        global_ready     = p.bitmaps_ready != 0;
+        bm_mode          = (BMW == 0 && global_bm != nullptr && global_ready) ? 1 : 0;
+        bm_origin        = 0;
+        history          = p.output_ids != nullptr ? p.output_ids + row : nullptr;
+        batch_size       = p.batch_size;
+        step             = p.step;
+        max_input_length = p.max_input_length;
+        col_offset       = p.col_offset;
+        team             = (int)blockDim.x;
+        count_table      = nullptr;  // (the kernel that keeps the table sets it)
+    }
+    // from what another wave worked out with the constructor below (and derived())
+    __device__ __forceinline__ FusedRow(const FusedParams& p, int row, const FusedRowDerived& d)
+    {
+        from_launch(p, row);
+        inv           = d.inv;
+        fast_mul      = d.fast_mul;
+        penalty       = d.penalty;
+        frequency     = d.frequency;
+        up_mul_neg    = d.up_mul_neg;
+        up_mul_pos    = d.up_mul_pos;
+        up_add        = d.up_add;
+        masked_end_id = d.masked_end_id;
+        input_length  = d.input_length;
+        keep_pads     = (d.flags & 1) != 0;
+        up_ok         = (d.flags & 2) != 0;
+    }
+    __device__ __forceinline__ FusedRowDerived derived() const
+    {
+        FusedRowDerived d;
+        d.inv           = inv;
+        d.fast_mul      = fast_mul;
+        d.penalty       = penalty;
+        d.frequency     = frequency;
+        d.up_mul_neg    = up_mul_neg;
+        d.up_mul_pos    = up_mul_pos;
+        d.up_add        = up_add;
+        d.masked_end_id = masked_end_id;
+        d.input_length  = input_length;
+        d.flags         = (keep_pads ? 1 : 0) | (up_ok ? 2 : 0);
+        return d;
+    }
     __device__ __forceinline__ FusedRow(const FusedParams& p, int row, const FusedRowArgs& args)
     {
-        rowp        = (const T*)p.logits + (size_t)row * p.Vp;
-        bias        = (const T*)p.bias;
-        V           = p.V;
-        Vp          = p.Vp;
-        temp_active = p.temperatures != nullptr;
+        from_launch(p, row);
         const TemperatureCtx<DT> tc(args.temperature, V, Vp, false);
         inv           = tc.inv;
         fast_mul      = temp_active ? tc.inv : 1.0f;
         keep_pads     = tc.keep_pads;
-        penalty_type  = p.penalties != nullptr ? p.penalty_type : 2;
         penalty       = args.penalty;
         if (penalty_type == 0) {  // additive
             up_mul_neg = 1.0f;
@@ -211,14 +267,6 @@ struct FusedRow {
             up_mul_pos = up_ok ? (1.0f / penalty) * 1.00000095367431640625f : 0.0f;
             up_add     = 0.0f;
         }
-        global_bm     = (p.bitmaps != nullptr && penalty_type != 2) ? p.bitmaps + (size_t)row * p.bitmap_words : nullptr;
-        global_ready  = p.bitmaps_ready != 0;
-        bm_mode       = (BMW == 0 && global_bm != nullptr && global_ready) ? 1 : 0;
-        bm_origin     = 0;
-        history       = p.output_ids != nullptr ? p.output_ids + row : nullptr;
-        batch_size    = p.batch_size;
-        step          = p.step;
-        max_input_length = p.max_input_length;
         input_length  = args.input_length;
         // values that are the same for every lane of the workgroup but come out of floating-point
         // arithmetic: move them to scalar registers, they stay live for the whole kernel
@@ -228,10 +276,7 @@ struct FusedRow {
         up_mul_neg = uniform_f(up_mul_neg);
         up_mul_pos = uniform_f(up_mul_pos);
         up_add     = uniform_f(up_add);
-        col_offset    = p.col_offset;
-        team          = (int)blockDim.x;
         frequency     = uniform_f(args.frequency);
-        count_table   = nullptr;  // (the kernel that keeps the table sets it)
         masked_end_id = (p.min_lengths != nullptr
                          && min_length_masks(args.sequence_length, p.max_input_length, args.min_length)
                          && args.end_id >= p.col_offset) ?

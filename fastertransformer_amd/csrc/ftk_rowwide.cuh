@@ -1,13 +1,17 @@
-// The fused decode step in one launch for batches of about one row per compute unit: a 1024-thread workgroup owns
-// a whole row. It streams the row once like the lean gather of ftk_lean.cuh (same ring of sub-tiles, same
-// parking of vectors that may hold a candidate, same exact evaluation), but
-//   - the bound is one per row instead of one per share of a row: far fewer candidates (about 3 k instead of
-//     4 x 3 k at k = 64 over 128 Ki columns),
+// The fused decode step in one launch for batches of about one row per compute unit (and for any small launch): a
+// 1024-thread workgroup owns a whole row. It streams the row once like the lean gather of ftk_lean.cuh (a ring of
+// sub-tiles in registers, parking of the vectors that may hold a candidate, exact evaluation of what was parked), but
+//   - the bound is one per row instead of one per share of a row: the k-th largest of 256 maxima over the first
+//     sub-tile, raised once more two sub-tiles before the end from the list itself, which is pruned with it (about
+//     1.5 k candidates per row instead of 4 x 3 k at k = 64 over 128 Ki columns),
 //   - candidates go to a list in LDS, never to memory: no list headers, no second launch, no trip to memory between
 //     the read of the row and its selection,
-//   - the replay of the reference's tie orders (topk_stage1 / topk_stage2_sampling of
-//     src/fastertransformer/kernels/sampling_topk_kernels.cu:130-312) ranks the candidates with all sixteen waves.
-// Sixteen waves per compute unit are in flight, as with four 256-thread workgroups, and the same bytes per thread.
+//   - after the row's last column twelve of the sixteen waves leave; the first four (one per SIMD) cut the list to
+//     little more than k entries and replay the reference's tie orders (topk_stage1 / topk_stage2_sampling of
+//     src/fastertransformer/kernels/sampling_topk_kernels.cu:130-312) by counting, in one pass when all keys differ,
+//   - what is the same for the whole row (its arguments and what follows from them, its draw, every bound) is worked
+//     out by one wave and handed to the others through LDS: sixteen waves in lock-step pay sixteen issue slots for
+//     every instruction.
 // Rows the kernel cannot bound (a list that outgrows LDS) are walked again by the first four waves with the general
 // stream of ftk_topk.cuh, as the merging kernel of the lean gather does.
 #pragma once
@@ -46,7 +50,7 @@ struct RowwideShared {
     uint32_t slot_key[RW_THREADS];
     uint32_t bound;
     float    bound_hot;  // what a raw maximum times the multiplier must reach under that bound
-    int      late[3];    // the row's top_p, sequence length and end id, for the end of the kernel
+    int      setup[16];  // what the first wave made of the row's arguments, see the kernel
     int      n_list[2];  // length of the row's list; the second counter takes over when the list is pruned
 };
 
@@ -364,7 +368,6 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideA
 #else
 #define RW_STAMP(i)
 #endif
-    RW_STAMP(0)
 
     // the row's address, pinned as a number and used as a pointer to global memory
     typedef unsigned int                                  u4 __attribute__((ext_vector_type(4)));
@@ -374,25 +377,58 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideA
     const int nvec = p.V / EPV;  // whole vectors inside columns [0, V)
     const int    nsub = (nvec + RW_SUB_VECS - 1) / RW_SUB_VECS;
 
-    // ---- everything the row needs from memory is requested at once, in one block without control flow: the
-    // per-row arguments (scalar loads), the token history (time-major: every id is a cache line of its own; positions
-    // past the step re-read the last one), then the first sub-tiles of the row
-    const void*         safe   = p.end_ids + row;
-    const bool          skip   = row_flag_or(p.skip_decode, row, safe, false);
-    const bool          fin    = row_flag_or(p.finished_in, row, safe, false);
-    const int           k      = row_arg_or(p.top_ks, row, safe, p.max_top_k);
-    const float         tp     = row_arg_or(p.top_ps, row, safe, 1.0f);
-    const FusedRowArgs  args   = fused_row_args(p, row);
-    const int           seq_in = row_arg_or((const int*)l_in.sequence_length, row, safe, 0);  // (the unpinned copy: a
-                                                                    // load through a pointer known to be global)
-    const RowDrawSource draw   = row_draw_source(l.rng, l.uniforms, row, safe);
-    const bool         injected     = l.uniforms != nullptr;
-    unsigned long long counter_addr = (unsigned long long)(l.rng != nullptr ? &l.rng[row].offset : nullptr);
-    rowwide_pin(counter_addr);
-    const bool         hist = p.bitmaps != nullptr && p.penalties != nullptr;
+    // ---- Everything the row needs from memory is requested at once: the per-row arguments (scalar loads, ahead of
+    // everything else), the token history (time-major: every id is a cache line of its own; positions past the step
+    // re-read the last one), then the first sub-tile of the row. Sixteen waves in lock-step pay sixteen issue slots
+    // for every instruction, so what is the same for the whole row is worked out by one wave and handed to the others
+    // through LDS: the first wave takes the row's arguments and what follows from them, the second the row's draw.
+    const int           wv_s = __builtin_amdgcn_readfirstlane(wv);
+    const void*         safe = p.end_ids + row;
+    // (Only the loads themselves sit in the two branches: anything computed there from a loaded value would wait
+    // for it, in front of the wave's own loads of the history and the row.)
+    auto word_at = [&](const void* array, size_t offset) -> const uint32_t* {
+        return reinterpret_cast<const uint32_t*>(array != nullptr ? (const char*)array + offset : (const char*)safe);
+    };
+    auto flag_word_at = [&](const bool* flags) -> const uint32_t* {  // the aligned word that holds the row's flag
+        const char* flag = flags != nullptr ? (const char*)flags + row : (const char*)safe;
+        return reinterpret_cast<const uint32_t*>(flag - (reinterpret_cast<uintptr_t>(flag) & 3u));
+    };
+    auto flag_of = [&](const bool* flags, uint32_t word) -> bool {
+        const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(flags + row) & 3u);
+        return flags != nullptr && ((word >> (8u * mis)) & 0xFFu) != 0u;
+    };
+    const int* seq_from_array = p.min_lengths != nullptr ? p.sequence_length_in : nullptr;
+    uint32_t   w_skip = 0u, w_fin = 0u, w_k = 0u, w_tp = 0u, w_temp = 0u, w_pen = 0u, w_freq = 0u, w_in = 0u, w_min = 0u,
+             w_seq = 0u, w_end = 0u, w_seq_in = 0u;
+    RowDrawSource      draw         = {};
+    unsigned long long counter_addr = 0ull;
+    if (wv_s == 0) {
+        w_skip   = *flag_word_at(p.skip_decode);
+        w_fin    = *flag_word_at(p.finished_in);
+        w_k      = *word_at(p.top_ks, (size_t)row * 4);
+        w_tp     = *word_at(p.top_ps, (size_t)row * 4);
+        w_temp   = *word_at(p.temperatures, (size_t)row * 4);
+        w_pen    = *word_at(p.penalties, (size_t)row * 4);
+        w_freq   = *word_at(p.frequencies, (size_t)row * 4);
+        w_in     = *word_at(p.input_lengths, (size_t)row * 4);
+        w_min    = *word_at(p.min_lengths, (size_t)row * 4);
+        w_seq    = *word_at(seq_from_array, (size_t)row * 4);
+        w_end    = *word_at(p.end_ids, (size_t)row * 4);
+        w_seq_in = *word_at((const int*)l_in.sequence_length, (size_t)row * 4);  // (the unpinned copy: a load through
+                                                                                // a pointer known to be global)
+    }
+    else if (wv_s == 1) {
+        w_skip       = *flag_word_at(p.skip_decode);
+        w_fin        = *flag_word_at(p.finished_in);
+        draw         = row_draw_source(l.rng, l.uniforms, row, safe);
+        counter_addr = (unsigned long long)(l.rng != nullptr ? &l.rng[row].offset : nullptr);
+    }
+    const bool injected = l.uniforms != nullptr;
+    const bool hist     = p.bitmaps != nullptr && p.penalties != nullptr;
     // (the instruction scheduler keeps the argument loads above in front of the vector loads below: requested behind
     // them, they would also arrive behind them)
     __builtin_amdgcn_sched_barrier(0);
+    RW_STAMP(0)  // (behind the argument loads: a store in front of them would make vector loads of them)
     int                hist_ids[RW_HIST_U];
     {
         const int* column = hist ? p.output_ids + row : p.end_ids;  // (without a history: any valid address)
@@ -431,24 +467,43 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideA
             }
         }
     }
-    if (t == 0) {
-        s.n_list[0] = 0;
-        s.n_list[1] = 0;
-    }
-    lds_barrier();
-
-    FusedRow<DT, BMW> rowctx(p, row, args);
-    if (skip || fin) {
-        if (fin && !skip && t == 0) {
-            l.ids[row] = args.end_id;
+    // (a fixed point in the program: no arithmetic on the loaded words moves up from here into the branches above)
+    asm volatile("" : "+s"(w_skip), "+s"(w_fin), "+s"(w_temp), "+s"(w_pen), "+s"(w_freq), "+s"(w_k), "+s"(w_tp));
+    asm volatile("" : "+s"(w_in), "+s"(w_min), "+s"(w_seq), "+s"(w_end), "+s"(w_seq_in));
+    const bool skip01 = flag_of(p.skip_decode, w_skip), fin01 = flag_of(p.finished_in, w_fin);
+    if (wv_s == 0) {
+        FusedRowArgs args0;
+        args0.temperature     = p.temperatures != nullptr ? __uint_as_float(w_temp) : 1.0f;
+        args0.penalty         = p.penalties != nullptr ? __uint_as_float(w_pen) : 0.0f;
+        args0.frequency       = p.frequencies != nullptr ? __uint_as_float(w_freq) : 0.0f;
+        args0.input_length    = p.input_lengths != nullptr ? (int)w_in : p.max_input_length;
+        args0.min_length      = p.min_lengths != nullptr ? (int)w_min : 0;
+        args0.sequence_length = seq_from_array != nullptr ? (int)w_seq : 0;
+        args0.end_id          = (int)w_end;
+        const FusedRow<DT, BMW> first(p, row, args0);
+        const FusedRowDerived   d = first.derived();
+        if (lane == 0) {
+            s.n_list[0]  = 0;
+            s.n_list[1]  = 0;
+            s.setup[0]   = __float_as_int(d.inv);
+            s.setup[1]   = __float_as_int(d.fast_mul);
+            s.setup[2]   = __float_as_int(d.penalty);
+            s.setup[3]   = __float_as_int(d.frequency);
+            s.setup[4]   = __float_as_int(d.up_mul_neg);
+            s.setup[5]   = __float_as_int(d.up_mul_pos);
+            s.setup[6]   = __float_as_int(d.up_add);
+            s.setup[7]   = d.masked_end_id;
+            s.setup[8]   = d.input_length;
+            s.setup[9]   = d.flags;
+            s.setup[10]  = p.top_ks != nullptr ? (int)w_k : p.max_top_k;
+            s.setup[11]  = (skip01 ? 1 : 0) | (fin01 ? 2 : 0);
+            s.setup[12]  = p.top_ps != nullptr ? (int)w_tp : __float_as_int(1.0f);
+            s.setup[13]  = l_in.sequence_length != nullptr ? (int)w_seq_in : 0;
+            s.setup[14]  = (int)w_end;
         }
-        return;
     }
-    // The row's draw: taken once, by the rows that take part (like the reference's curand_uniform). With it, what
-    // only the end of the kernel needs of the row's arguments moves to LDS: values that stay in scalar registers from
-    // their load to the end are the first the register allocator spills, and a spill of a value that is still on
-    // its way waits for it - in front of the row's loads.
-    if (t == 0) {
+    // The row's draw: taken once, by the rows that take part (like the reference's curand_uniform).
+    if (wv_s == 1 && !(skip01 || fin01) && lane == 0) {
         float u = draw.injected;
         if (!injected) {
             uint64_t next;
@@ -456,9 +511,29 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideA
             *(__attribute__((address_space(1))) uint64_t*)counter_addr = next;
         }
         ts.misc[0] = __float_as_int(u);
-        s.late[0]  = __float_as_int(tp);
-        s.late[1]  = seq_in;
-        s.late[2]  = args.end_id;
+    }
+    lds_barrier();
+
+    const int       rec = s.setup[lane & 15];
+    FusedRowDerived d;
+    d.inv           = __int_as_float(__builtin_amdgcn_readlane(rec, 0));
+    d.fast_mul      = __int_as_float(__builtin_amdgcn_readlane(rec, 1));
+    d.penalty       = __int_as_float(__builtin_amdgcn_readlane(rec, 2));
+    d.frequency     = __int_as_float(__builtin_amdgcn_readlane(rec, 3));
+    d.up_mul_neg    = __int_as_float(__builtin_amdgcn_readlane(rec, 4));
+    d.up_mul_pos    = __int_as_float(__builtin_amdgcn_readlane(rec, 5));
+    d.up_add        = __int_as_float(__builtin_amdgcn_readlane(rec, 6));
+    d.masked_end_id = __builtin_amdgcn_readlane(rec, 7);
+    d.input_length  = __builtin_amdgcn_readlane(rec, 8);
+    d.flags         = __builtin_amdgcn_readlane(rec, 9);
+    const int  k    = __builtin_amdgcn_readlane(rec, 10);
+    const int  gone = __builtin_amdgcn_readlane(rec, 11);
+    FusedRow<DT, BMW> rowctx(p, row, d);
+    if (gone != 0) {  // the row is skipped or has finished
+        if (gone == 2 && t == 0) {
+            l.ids[row] = __builtin_amdgcn_readlane(rec, 14);
+        }
+        return;
     }
     if (hist) {
 #pragma unroll
@@ -750,10 +825,10 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideA
     out.finished           = l.finished;
     out.cum_log_probs      = nullptr;
     out.output_log_probs   = nullptr;
-    out.sequence_length_in = __builtin_amdgcn_readfirstlane(s.late[1]);
+    out.sequence_length_in = __builtin_amdgcn_readfirstlane(s.setup[13]);
     out.cum_log_prob_in    = 0.0f;
-    out.end_id_in          = __builtin_amdgcn_readfirstlane(s.late[2]);
-    const float tp_late    = uniform_f(__int_as_float(s.late[0]));
+    out.end_id_in          = __builtin_amdgcn_readfirstlane(s.setup[14]);
+    const float tp_late    = uniform_f(__int_as_float(s.setup[12]));
     int         n = s.n_list[cur];
     const float u = __int_as_float(ts.misc[0]);
     if (n > k + k / 2 && n > 96 && n <= 4 * TK_THREADS) {
