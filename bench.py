@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0
 PLAIN_READ = "plain_read_b256_v128256_f32"
 # HBM bytes per launch of the dominant kernel on the headline workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by a copy kernel of known size (summary under profiles/)
-TRAFFIC_BYTES_PER_LAUNCH = 132454502
+TRAFFIC_BYTES_PER_LAUNCH = 132478941
 
 WORKLOADS = {
     # the configuration the headline metric is quoted on

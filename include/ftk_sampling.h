@@ -298,7 +298,9 @@ int ftk_fused_topk_step_static(ftk_fused_topk_args* args, ftk_stream_t stream);
  * used) once with the launch shape and load instructions of the fused step's streaming kernel and nothing else
  * (one maximum per 16 bytes; one float per wave goes to `sink`, which needs at least 4096 floats). It is the
  * yardstick the streaming kernel's duration is compared with. elapsed_ms != NULL: the launch carries a pair of
- * events, the call waits for the kernel and returns its duration. */
+ * events, the call waits for the kernel and returns its duration. A measurement aid, not a serving entry point:
+ * with elapsed_ms it creates and destroys the two events (hipEventCreate, which may allocate) and blocks the
+ * calling thread, so it belongs neither under a graph capture nor in code that must not allocate. */
 int ftk_measure_plain_read(const void* data, size_t bytes, float* sink, size_t sink_floats, ftk_stream_t stream,
                            float* elapsed_ms);
 
@@ -425,8 +427,15 @@ int ftk_invoke_update_indir_cache(int* tgt_indir_cache, const int* src_indir_cac
  * utils/cuda_utils.h:247-258, utils/nvtx_utils.h:37-49) ------------------------------------------
  * ftk_profile_enable(n) makes the next n fused steps bracket each of their kernels with HIP events on
  * the caller's stream (n = 0 switches it off); ftk_profile_read sums them (it synchronises on the
- * events) and resets the count. kernel: 0 = history bitmap, 1 = gather (the streaming pass), 2 = select,
- * 3 = the first of two reads a launch with a large k makes (the maxima that bound the row's k-th largest). */
+ * events) and resets the count. kernel: 0 = history bitmap, 1 = gather (the streaming pass; the whole step where
+ * one launch does it), 2 = select, 3 = the first of two reads a launch with a large k makes (the maxima that bound
+ * the row's k-th largest).
+ * Measurement aids, not serving entry points: ftk_profile_enable destroys the events of the last call and creates
+ * 2 * n new ones per kernel slot (hipEventCreate, which may allocate); steps that run with profiling on launch
+ * with those events and do not belong under a graph capture; the
+ * event slots and counters are process-wide and unsynchronised, so ftk_profile_enable / ftk_profile_read and
+ * the steps they observe must not run concurrently from several threads. With profiling off (the default) the
+ * fused steps touch none of this. */
 int ftk_profile_enable(int max_launches);
 int ftk_profile_read(int kernel, double* total_ms, int* launches);
 
