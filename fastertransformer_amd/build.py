@@ -57,7 +57,7 @@ HIP_FLAGS = [
 
 
 HOOK_UNITS = [("fused_kernels.hip", "fused_kernels.o"), ("topp_kernels.hip", "topp_kernels.o"),
-              ("criteria_kernels.hip", "criteria_kernels.o")]
+              ("criteria_kernels.hip", "criteria_kernels.o"), ("beam_kernels.hip", "beam_kernels.o")]
 
 
 def _run(cmd):
@@ -102,7 +102,7 @@ def build(force=True, verbose=True, with_torch=True):
         list(pool.map(_run, jobs))
     kernels_so = os.path.join(LIB, "libftk_sampling.so")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", kernels_so] + objs)
-    # The hooks build for the test-suite (include/ftk_test_hooks.h): the three translation units that carry
+    # The hooks build for the test-suite (include/ftk_test_hooks.h): the translation units that carry
     # hooks are compiled again with -DFTK_TEST_HOOKS, everything else is shared with the product library.
     hook_objs = list(objs)
     hook_jobs = []

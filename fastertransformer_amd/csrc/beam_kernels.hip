@@ -19,6 +19,9 @@
 #include "ftk_device.cuh"
 #include "ftk_sampling.h"
 #include "ftk_transform.cuh"
+#ifdef FTK_TEST_HOOKS
+#include "ftk_test_hooks.h"
+#endif
 
 namespace ftk {
 
@@ -416,6 +419,160 @@ beam_row_kernel(const bool* __restrict__ finished, const int* __restrict__ end_i
     }
 }
 
+// The three kernels above in one launch: one 1024-thread workgroup per row finds the row's maximum, the sum of exponentials and every thread's largest
+// element, takes a bound from 256 (128, 64) joined thread maxima, collects what reaches it and leaves the row's 2K
+// best with their values. The passes over the row are the section kernels' with the whole row as the one section
+// (the second and third come from the caches); the bound is found by the first wave alone (a bisection with
+// ballots over the top 24 key bits: a floor at or below the 2K-th largest maximum, which is all the argument
+// needs) so that the other fifteen waves only wait at two barriers; after the last pass twelve waves leave and the
+// first four select with the code of the 256-thread kernels (a barrier counts the waves that are left).
+constexpr int BR_THREADS = 1024;
+constexpr int BR_WAVES   = BR_THREADS / WAVE;
+
+template<int DT>
+__global__ void __launch_bounds__(BR_THREADS)
+beam_rowwide_kernel(const typename Storage<DT>::T* __restrict__ x, const typename Storage<DT>::T* __restrict__ bias,
+                    const bool* __restrict__ finished, const int* __restrict__ end_ids,
+                    const float* __restrict__ cum_log_probs, int vocab, int K, int* __restrict__ cand_id,
+                    float* __restrict__ cand_val)
+{
+    typedef Storage<DT>   S;
+    __shared__ BeamSelect s;
+    __shared__ double     red[BR_WAVES];
+    __shared__ float      redf[BR_WAVES];
+    __shared__ double     row_sum;
+    __shared__ uint32_t   row_floor;
+    const int             row  = blockIdx.x;
+    const int             t    = threadIdx.x;
+    const int             N    = 2 * K;
+    const float           MAXT = S::max_t();
+    const float           cum  = cum_log_probs[row];
+    if (finished[row]) {
+        // MAX_T at the end id, -MAX_T elsewhere (:328-336): the end id first, then the lowest ids
+        const int  end_id = end_ids[row / K];
+        const bool inside = end_id >= 0 && end_id < vocab;
+        if (t < N) {
+            int   id;
+            float u;
+            if (inside) {
+                id = t == 0 ? end_id : (t - 1 < end_id ? t - 1 : t);
+                u  = t == 0 ? MAXT : -MAXT;
+            }
+            else {
+                id = t;
+                u  = -MAXT;
+            }
+            const float m    = inside ? MAXT : -MAXT;
+            const float logd = inside ? 0.0f : det_logf((float)vocab);
+            cand_id[(size_t)row * N + t]  = id + row * vocab;
+            cand_val[(size_t)row * N + t] = round_t<DT>((u - m - logd) + cum);
+        }
+        return;
+    }
+    const size_t rb = (size_t)row * vocab;
+    // first pass: the row's maximum
+    float m = -MAXT;
+    stream_columns<DT, BR_THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
+        const float e = beam_element_of<DT>(xv, bias, v);
+        m             = e > m ? e : m;
+    });
+    m = block_max<float, BR_WAVES>(m, redf, -MAXT);
+    // second pass: the sum, and every thread's largest element
+    double d    = 0.0;
+    float  fmax = -__builtin_inff();
+    stream_columns<DT, BR_THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
+        const float e = beam_element_of<DT>(xv, bias, v);
+        d += (double)det_expf_nonpos(e - m);
+        fmax = __builtin_fmaxf(fmax, e);
+    });
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        d += __shfl_xor(d, o, WAVE);
+    }
+    if (lane_id() == 0) {
+        red[wave_id()] = d;
+    }
+    // 2K <= 32 needs no more than 64 maxima to choose the 2K-th largest from, 2K <= 64 no more than 128
+    const int join    = N <= 32 ? 16 : N <= 64 ? 8 : 4;  // neighbouring threads that join their maxima
+    const int n_slots = BR_THREADS / join;
+    fmax              = __builtin_fmaxf(fmax, __shfl_xor(fmax, 1, WAVE));
+    fmax              = __builtin_fmaxf(fmax, __shfl_xor(fmax, 2, WAVE));
+    if (join >= 8) {
+        fmax = __builtin_fmaxf(fmax, __shfl_xor(fmax, 4, WAVE));
+    }
+    if (join == 16) {
+        fmax = __builtin_fmaxf(fmax, __shfl_xor(fmax, 8, WAVE));
+    }
+    uint32_t* slot_key = reinterpret_cast<uint32_t*>(s.slots);
+    if (t % join == 0) {
+        slot_key[t / join] = order_key(fmax);
+    }
+    if (t == 0) {
+        s.n_cand = 0;
+    }
+    __syncthreads();
+    if (wave_id() == 0) {
+        uint32_t kk[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int i = lane_id() + g * WAVE;
+            kk[g]       = i < n_slots ? slot_key[i] : 0u;
+        }
+        // The 2K-th largest of the maxima is an element with at least 2K elements at or above it: nothing below it
+        // can be among the 2K best; so is any value below that one. (A group that saw no element reports -inf.)
+        uint32_t P = 0u;
+        for (int bit = 31; bit >= 8; --bit) {
+            const uint32_t cand = P | (1u << bit);
+            int            c    = 0;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                c += (int)__builtin_popcountll(__ballot(kk[g] >= cand));
+            }
+            P = c >= N ? cand : P;
+        }
+        if (lane_id() == 0) {
+            double tot = 0.0;
+            for (int w = 0; w < BR_WAVES; ++w) {
+                tot += red[w];
+            }
+            row_sum   = tot;
+            row_floor = P;
+        }
+    }
+    __syncthreads();
+    const uint32_t floor_key = row_floor;
+    const float    floor_val = key_to_float(floor_key);
+    const bool     all_pass  = floor_key <= order_key(-__builtin_inff());  // then NaN columns are wanted too
+    stream_columns<DT, BR_THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
+        const float e = beam_element_of<DT>(xv, bias, v);
+        if (e >= floor_val || all_pass) {
+            const int at = atomicAdd(&s.n_cand, 1);
+            if (at < BM_CAP) {
+                s.cand[at] = beam_key(e, (uint32_t)v);
+            }
+        }
+    });
+    __syncthreads();
+    if (wave_id() >= BM_WAVES) {
+        return;  // the first four waves select
+    }
+    const int passed = s.n_cand;
+    const int take   = min(N, vocab);
+    if (passed <= BM_CAP) {
+        beam_select(s, [&](int i) { return s.cand[i]; }, passed, take);
+    }
+    else {
+        // (rows of many equal values) the selection runs over the row itself
+        beam_select(s, [&](int i) { return beam_key(beam_element<DT>(x, bias, rb, i), (uint32_t)i); }, vocab, take);
+    }
+    const float logd = det_logf((float)row_sum);
+    if (t < N) {
+        const unsigned long long k    = t < take ? s.out[t] : 0ull;
+        cand_id[(size_t)row * N + t]  = (int)beam_key_position(k) + row * vocab;
+        cand_val[(size_t)row * N + t] = round_t<DT>((beam_key_value(k) - m - logd) + cum);
+    }
+}
+
 struct BeamHypsDevice {
     int*         output_ids_tgt;
     int*         sequence_lengths_tgt;
@@ -728,6 +885,18 @@ __global__ void beam_indir_cache_kernel(int* __restrict__ tgt, const int* __rest
 
 using namespace ftk;
 
+constexpr int BR_SHORT_ROW = 65536;
+constexpr int BR_MANY_ROWS = 192;
+#ifdef FTK_TEST_HOOKS
+// Test hook (hooks build of the library only): 1 = sections of rows and three launches everywhere, 2 = one
+// workgroup per row everywhere, 0 = by the shape.
+static int g_beam_path = 0;
+extern "C" void ftk_test_set_beam_path(int v)
+{
+    g_beam_path = v;
+}
+#endif
+
 extern "C" {
 
 int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, const bool* finished,
@@ -808,17 +977,33 @@ int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, 
         h.early_stopping       = beam_hyps->early_stopping ? 1 : 0;
     }
     const dim3 sections(plan.parts, rows);
+    // One 1024-thread workgroup per row does the work of the first three launches, except where a few long rows
+    // would leave most compute units idle (measured on MI355X, f16: 32 rows of 128256 take 40 us that way and 34 us
+    // in sections; 64 rows of 50257 27 against 30 us, 256 rows 29 against 36 us, 512 rows of 152064 112 against
+    // 115 us).
+    bool one_per_row = vocab_size <= BR_SHORT_ROW || rows >= BR_MANY_ROWS;
+#ifdef FTK_TEST_HOOKS
+    one_per_row = g_beam_path == 0 ? one_per_row : g_beam_path == 2;
+#endif
     FTK_DISPATCH_DTYPE(dtype, {
         typedef Storage<DT>::T T;
-        beam_section_max_kernel<DT><<<sections, BM_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished,
-                                                                     vocab_size, plan.section, pmax);
-        FTK_LAUNCH_CHECK();
-        beam_section_kernel<DT><<<sections, BM_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished,
-                                                                 vocab_size, plan.section, N, pmax, psum, pkeys);
-        FTK_LAUNCH_CHECK();
-        beam_row_kernel<DT><<<rows, BM_THREADS, 0, st>>>(finished, end_ids, cum_log_probs, vocab_size, beam_width,
-                                                         plan.parts, pmax, psum, pkeys, cand_id, cand_val);
-        FTK_LAUNCH_CHECK();
+        if (one_per_row) {
+            beam_rowwide_kernel<DT><<<rows, BR_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished, end_ids,
+                                                                 cum_log_probs, vocab_size, beam_width, cand_id,
+                                                                 cand_val);
+            FTK_LAUNCH_CHECK();
+        }
+        else {
+            beam_section_max_kernel<DT><<<sections, BM_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished,
+                                                                         vocab_size, plan.section, pmax);
+            FTK_LAUNCH_CHECK();
+            beam_section_kernel<DT><<<sections, BM_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished,
+                                                                     vocab_size, plan.section, N, pmax, psum, pkeys);
+            FTK_LAUNCH_CHECK();
+            beam_row_kernel<DT><<<rows, BM_THREADS, 0, st>>>(finished, end_ids, cum_log_probs, vocab_size, beam_width,
+                                                             plan.parts, pmax, psum, pkeys, cand_id, cand_val);
+            FTK_LAUNCH_CHECK();
+        }
         beam_batch_kernel<DT><<<batch_size, BM_THREADS, 0, st>>>(cand_id, cand_val, ids, cum_log_probs,
                                                                  output_log_probs, finished, sequence_lengths, h,
                                                                  beam_width, 2 * max_k, vocab_size, length_penalty,

@@ -19,10 +19,11 @@ def _lib():
     return ops, ops.ftk()
 
 
-def _run_product(c, dt, batch, K, V, diversity, length_penalty, bias=None):
+def _run_product(c, dt, batch, K, V, diversity, length_penalty, bias=None, lib=None):
     """the step on the GPU; returns (ids, cum_log_probs, output_log_probs, hypotheses arrays) as numpy"""
     import torch
-    ops, lib = _lib()
+    ops, product = _lib()
+    lib = product if lib is None else lib
     d = {k: to_torch(c[k]) for k in ("finished", "sequence_lengths", "cum_log_probs", "end_ids", "ids",
                                      "output_log_probs")}
     d_x = to_torch(c["log_probs"], dt)
@@ -100,6 +101,50 @@ def test_beam_step_full_vocabularies_and_batches(dt):
     _one_case(rng, dt, 2, 8, 128256, True, 0.1, 0.0)
     _one_case(rng, dt, 300, 4, 3000, True, 0.0, 1.0)
     _one_case(rng, dt, 1, 2, 152064, False, 0.0, 0.0)
+
+
+@pytest.mark.parametrize("path", [1, 2], ids=["sections_three_launches", "one_workgroup_per_row"])
+def test_beam_step_both_forms_of_the_row_stage(path):
+    """The row stage has two forms, chosen by the shape: sections of rows in three launches, and one
+    1024-thread workgroup per row in one. The test build of the library forces either on the same cases: every
+    beam-width class, tiny and full vocabularies, more rows than compute units, rows of equal values (the bound
+    passes more than fits the list), rows masked to -inf, finished beams, NaN columns."""
+    from fastertransformer_amd import ops
+    hooks = ops.ftk_hooks()
+    rng = np.random.default_rng(77)
+    hooks.ftk_test_set_beam_path(path)
+    try:
+        for dt in DTYPES:
+            for batch, K, V in ((2, 2, 4), (3, 4, 9), (1, 64, 128), (2, 33, 1000), (4, 8, 50257), (1, 16, 152064),
+                                (90, 4, 2500), (2, 3, 20011)):
+                c = make_beam_case(rng, dt, batch, K, V, step=5, max_seq_len=12, with_hyps=True)
+                want = copy_beam_case(c)
+                assert O.topk_softmax(dt, want["log_probs"], None, want["finished"], want["sequence_lengths"],
+                                      want["cum_log_probs"], want["output_log_probs"], want["ids"], want["hyps"],
+                                      batch, K, V, want["end_ids"], 0.1, 0.7) == 0
+                print("beam form", path, DTYPE_NAMES[dt], batch, K, V, flush=True)
+                _compare(c, want, _run_product(c, dt, batch, K, V, 0.1, 0.7, lib=hooks), dt)
+        batch, K, V = 3, 4, 5000
+        for kind in range(4):
+            c = make_beam_case(rng, O.F32, batch, K, V, with_hyps=True, finished_frac=0.0)
+            if kind == 0:
+                c["log_probs"][:] = np.float32(1.5)
+                c["cum_log_probs"][:] = np.float32(-1.0)
+            elif kind == 1:
+                c["log_probs"][:] = -np.inf
+                c["log_probs"][:, rng.choice(V, 3 * K, replace=False)] = rng.standard_normal(3 * K).astype(np.float32)
+            elif kind == 2:
+                c["finished"][:] = True
+            else:
+                c["log_probs"][:, rng.choice(V, 40, replace=False)] = np.nan
+            want = copy_beam_case(c)
+            assert O.topk_softmax(O.F32, want["log_probs"], None, want["finished"], want["sequence_lengths"],
+                                  want["cum_log_probs"], want["output_log_probs"], want["ids"], want["hyps"], batch,
+                                  K, V, want["end_ids"], 0.0, 0.5) == 0
+            print("beam form", path, "degenerate kind", kind, flush=True)
+            _compare(c, want, _run_product(c, O.F32, batch, K, V, 0.0, 0.5, lib=hooks), O.F32)
+    finally:
+        hooks.ftk_test_set_beam_path(0)
 
 
 def test_beam_step_degenerate_rows():
