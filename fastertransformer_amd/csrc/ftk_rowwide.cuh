@@ -40,8 +40,6 @@ constexpr int RW_HIST_U     = 4;                    // history ids a thread requ
 constexpr int RW_FIRST_TIGHTEN = FTK_RW_T1;
 constexpr int RW_TAIL_GAP      = FTK_RW_GAP;
 constexpr int RW_MIN_SUBS   = 4;                    // shortest row that a batch of full rounds sends here, in sub-tiles
-constexpr int RW_SMALL_BYTES = 32 << 20;            // a launch that reads less than this takes the kernel at any
-                                                    // batch up to 256 rows: it is bound by latency, not bandwidth
 
 struct RowwideShared {
     uint32_t count_table[FUSED_COUNT_SLOTS];  // occurrences of the history's ids (rows with a frequency penalty)

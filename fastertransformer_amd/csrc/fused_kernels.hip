@@ -228,16 +228,16 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             || ((uintptr_t)a->logits % (uintptr_t)elem) != 0)) {
         return FTK_ERR_UNSUPPORTED;
     }
-    // About one row per compute unit (or a few rounds of that), a small k, long rows, no bias: a 1024-thread
-    // workgroup per row does the whole step in one launch (ftk_rowwide.cuh). It pays when the rounds of 256
-    // workgroups are nearly full and the row's history bitmap fits its LDS window.
-    // Small launches (a few megabytes of logits) are bound by latency: they take the same kernel at any batch up to
-    // 256 rows, one launch instead of two with lists through memory in between.
+    // Up to one row per compute unit, or a few nearly full rounds of that, a small k, no bias: a 1024-thread
+    // workgroup per row does the whole step in one launch (ftk_rowwide.cuh), provided the row's history bitmap fits
+    // its LDS window. With at most 256 rows it is the faster form at every size measured (MI355X, k = 64, one
+    // launch / gather + select in us: 96 x 128256 f32 24.5 / 33.1, 192 x 128256 f32 27.8 / 41.4, 160 x 152064 f16
+    // 25.7 / 33.7, 192 x 50264 f32 20.5 / 26.9; 16 to 64 rows, bound by latency either way, within 1 us); with more,
+    // it pays when the rounds of 256 workgroups are nearly full and the rows are long.
     const int  rw_rounds = (rows + 255) / 256;
     const bool rw_full   = rows * 5 >= rw_rounds * 256 * 4
                          && (size_t)a->vocab_size / (16 / elem) >= (size_t)RW_MIN_SUBS * RW_SUB_VECS;
-    const bool rw_small  = rows <= 256 && (size_t)rows * a->vocab_size_padded * elem <= (size_t)RW_SMALL_BYTES
-                          && a->vocab_size >= 1024;
+    const bool rw_small  = rows <= 256 && a->vocab_size >= 1024;
     const bool rowwide   = lean_mode == 1 && !want_log_probs && a->embedding_bias == nullptr && lplan.splits > 1
                          && g_fused_two_launches == 0 && (rw_full || rw_small)
                          && (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_LARGE

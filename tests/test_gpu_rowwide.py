@@ -1,7 +1,8 @@
 """The one-launch step for batches of about one row per compute unit (a 1024-thread workgroup per row,
 csrc/ftk_rowwide.cuh) against the CPU oracle, through DynamicDecodeLayer with injected draws: ids / finished /
-sequence_length bit-exact. The shapes are the ones the launcher sends to that kernel (205 to 1023 rows in nearly
-full rounds of 256, rows of at least 16384 16-byte vectors on 16-byte boundaries, k <= 192, no bias, no log-probs);
+sequence_length bit-exact. The shapes are the ones the launcher sends to that kernel (up to 256 rows, or up to 1023
+in nearly full rounds of 256 with rows of at least 16384 16-byte vectors; rows on 16-byte boundaries, k <= 192, no
+bias, no log-probs);
 the last test asks the test build of the library which kernel a launch of such a shape took."""
 import numpy as np
 import pytest
@@ -109,8 +110,8 @@ def test_rowwide_generated_draws_are_reproducible():
 
 def test_rowwide_kernel_is_what_these_shapes_take():
     """the test build of the library reports the path of its last fused step: 3 = one 1024-thread workgroup per row;
-    the same rows in two launches (hook) and a batch of 100 long rows do not take it, 100 short rows do (a launch
-    of a few megabytes is bound by latency), and all agree on the ids"""
+    the same rows in two launches (hook) do not take it, nor does a batch between one round of workgroups and a
+    nearly full second one (300 rows); any batch of up to 256 rows does; and all agree on the ids"""
     import torch
     from fastertransformer_amd import ops
     from helpers import run_fused_step
@@ -118,7 +119,7 @@ def test_rowwide_kernel_is_what_these_shapes_take():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(9)
     H, k = 16, 64
-    for B, V, want in ((256, 65600, 3), (100, 128256, 1), (100, 32000, 3)):  # (small launches take it at any batch)
+    for B, V, want in ((256, 65600, 3), (300, 65600, 1), (100, 128256, 3), (100, 32000, 3)):
         logits = torch.randn((B, V), generator=gen, device="cuda") * 2.0
         history = torch.randint(0, V, (H, B), generator=gen, device="cuda", dtype=torch.int32)
         draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
