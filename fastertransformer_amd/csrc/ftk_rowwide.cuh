@@ -724,9 +724,8 @@ __global__ void __launch_bounds__(RW_THREADS) rowwide_step_kernel(const RowwideA
         }
     };
 
-    // ---- the stream. The bound is raised again after 2, 4, 6, 8, 16, ... sub-tiles: the k-th largest of the largest
-    // candidates of disjoint groups of lanes bounds the k-th largest of everything seen so far. (The ring holds
-    // several microseconds of the compute unit's share of the bandwidth: memory does not wait for these pauses.)
+    // ---- the stream. The bound is raised again on the way (see below): the k-th largest of disjoint groups of
+    // the list's entries bounds the k-th largest of everything seen so far.
     int next_tighten = RW_FIRST_TIGHTEN;  // then twice that plus two, ...
     for (int q0 = 0; q0 < nsub; q0 += R) {
 #pragma unroll
