@@ -33,7 +33,8 @@ WORKLOADS = {
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=64, top_p=0.9, temperature=0.8,
         repetition_penalty=1.1, prompt=64, sigma=2.5),
     # secondary line (only with --workload): the top-p layer on Zipf-distributed rows, per-row top_p in
-    # [0.5, 0.99] with decay; the logits buffer is restored outside the timed events (softmax is in place)
+    # [0.5, 0.99] with decay; the logits buffer is restored outside the timed events (with
+    # FT_SAMPLING_DISABLE_FUSED=1 the layer turns it into probabilities in place, like the reference)
     "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9": dict(
         dtype="f32", batch=256, vocab=128256, vocab_padded=128256, top_k=0, top_p=(0.5, 0.99), top_p_decay=0.9,
         top_p_min=0.3, top_p_reset_id=13, zipf_s=1.1, noise=0.5, prompt=0),
@@ -229,8 +230,9 @@ def run_plain_read(steps, warmup, nbuf=4):
 
 
 def run_gpu_topp(name, w, steps, warmup, nbuf=3):
-    """Top-p layer steps; every step is bracketed by its own pair of events so that restoring the logits (the
-    layer turns them into probabilities in place) stays outside the measured time."""
+    """Top-p layer steps; every step is bracketed by its own pair of events so that restoring the logits (which the
+    layer turns into probabilities in place when it is asked for the reference's side effects) stays outside the
+    measured time."""
     import torch
     import fastertransformer_amd as fa
 

@@ -230,10 +230,11 @@ struct ToppRowMeta {
     unsigned long long best;   // (key << 32) | ~id of the arg-max (lowest id among equals)
     int                cut;    // lowest gathered bucket
     int                n;      // entries at or above the cut
-    int                n_pos;  // positive entries of the row
+    int                n_pos;  // positive entries of the row (0x7FFFFFFF: not known, some may lie below the cut)
     int                nseg;
     int                flags;
-    int                pad;
+    float              best_prob;  // the arg-max's probability (rows sampled straight from logits)
+    float              mx, denom;  // the row's softmax statistics (rows sampled straight from logits)
 };
 
 // Workspace sections (all offsets multiples of 256 bytes). `sorted` keeps the reference's shape of
@@ -487,7 +488,8 @@ topp_cut_kernel(int S, const uint32_t* __restrict__ part_cnt, const uint32_t* __
     m.cut = TPB_NB;
     m.n = m.n_pos = m.nseg = 0;
     m.flags = 0;
-    m.pad   = 0;
+    m.best_prob = 0.0f;
+    m.mx = m.denom = 0.0f;
     if (skip_decode != nullptr && skip_decode[row]) {
         if (t == 0) {
             m.flags   = TOPP_SKIP;
@@ -709,6 +711,438 @@ topp_gather_kernel(const typename Storage<DT>::T* __restrict__ probs, int vocab,
             }
         }
     });
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Sampling straight from logits (ftk_fused_topp_sample_step): the probabilities are never written. One 1024-thread
+// workgroup per row does what softmax, histogram, cut and gather do above, in three passes over the row:
+//   1. the maximum;
+//   2. the sum of e = T(exp(y - max)) in the reference's order and, on the way, the histogram - of e, not of the
+//      probability e / denominator, which is not known yet. The division is monotone, so buckets of e are ranges of
+//      probabilities too; the mass per bucket is kept in units of 2^-31 of e;
+//   3. once the denominator is there: the cut in the histogram (the draw scaled by the denominator), then the
+//      gather of what lies at or above the cut bucket, each entry with its exact probability T(e / denominator) as
+//      the key the segments are sorted by.
+// Two things differ from buckets of probabilities. Entries of different buckets can share a probability (numerators
+// a few units apart can round to one quotient): sorted segment by segment they may then stand in the wrong order of
+// ids across a segment boundary, which the pick kernel puts right for the entry it emits (topp_settle_ties). And an
+// e above zero can give a probability of zero: buckets that may hold such entries are never gathered (b0 below);
+// a draw that is not crossed above them sends the row to the exact fallback of the pick kernel.
+struct ToppRowValues {
+    // what the softmax sees of a row: y(v) as softmax_kernel's `masked`, rows without a bias
+    float MAXT;
+    bool  fin;
+    int   end_id, n;
+    __device__ __forceinline__ float masked(int v, float x) const
+    {
+        if (v >= n) {
+            return -MAXT;
+        }
+        if (fin) {
+            return v == end_id ? MAXT : -MAXT;
+        }
+        return x + 0.0f;
+    }
+};
+
+// the probability the softmax would store for an element with e = T(exp(y - max)), as a float
+template<int DT>
+__device__ __forceinline__ float topp_prob_of(float e, const RowDivisor& div, float denom)
+{
+    return round_t<DT>(div.ok ? div.divide(e) : e / denom);
+}
+
+constexpr int TPR_BAND = 16;  // numerators this many units of T below 1 may share the arg-max's probability
+
+template<int DT>
+__global__ void __launch_bounds__(SM_THREADS)
+topp_row_kernel(const typename Storage<DT>::T* __restrict__ logits, const int* __restrict__ end_ids,
+                const bool* __restrict__ finished, int n_padded, int n, const bool* __restrict__ skip_decode,
+                const RngState* rng, const float* __restrict__ uniforms, float top_p, const float* __restrict__ top_ps,
+                uint32_t* __restrict__ seg_ends, ToppRowMeta* __restrict__ meta, unsigned long long* __restrict__ sorted)
+{
+    typedef Storage<DT>           S;
+    constexpr int                 K = (TPB_NB + SM_THREADS - 1) / SM_THREADS;
+    __shared__ uint32_t           cnt[TPB_NB];
+    __shared__ uint32_t           off[TPB_NB];
+    __shared__ unsigned long long mass[TPB_NB];
+    __shared__ int                band[TPR_BAND + 1];
+    __shared__ float              sh[32];
+    __shared__ float              sh_bcast;
+    __shared__ uint32_t           wcnt[SM_THREADS / WAVE];
+    __shared__ unsigned long long wmass[SM_THREADS / WAVE];
+    __shared__ uint32_t           red32[16];
+    const int                     row = blockIdx.x;
+    const int                     t   = threadIdx.x;
+    ToppRowMeta                   m;
+    m.best      = 0ull;
+    m.cut       = TPB_NB;
+    m.n = m.n_pos = m.nseg = 0;
+    m.flags     = 0;
+    m.best_prob = 0.0f;
+    m.mx = m.denom = 0.0f;
+    if (skip_decode != nullptr && skip_decode[row]) {
+        if (t == 0) {
+            m.flags   = TOPP_SKIP;
+            meta[row] = m;
+        }
+        return;
+    }
+    ToppRowValues vals;
+    vals.MAXT   = S::max_t();
+    vals.fin    = finished != nullptr ? finished[row] : false;
+    vals.end_id = vals.fin ? end_ids[row] : -1;
+    vals.n      = n;
+    const typename S::T* rowp = logits + (size_t)row * n_padded;
+    const float          MAXT = vals.MAXT;
+
+    // ---- 1. the maximum (softmax_kernel's, in any order of the columns)
+    float mx = -3.402823466e+38f;
+    if (!vals.fin) {
+        stream_columns<DT, SM_THREADS>(rowp, 0, n, [&](int, float x) { mx = __builtin_fmaxf(mx, x + 0.0f); });
+        if (n_padded > n) {
+            mx = __builtin_fmaxf(mx, -MAXT);
+        }
+    }
+    else {
+        for (int v = t; v < n_padded; v += SM_THREADS) {
+            mx = __builtin_fmaxf(mx, vals.masked(v, 0.0f));
+        }
+    }
+    for (int b = t; b < TPB_NB; b += SM_THREADS) {
+        cnt[b] = 0u;
+    }
+    if (t <= TPR_BAND) {
+        band[t] = 0x7FFFFFFF;
+    }
+    mx = block_max<float, SM_THREADS / WAVE>(mx, sh, -3.402823466e+38f);  // (two barriers: the histogram is clear)
+
+    // ---- 2. the sum in the reference's order, the histogram of e on the way
+    constexpr uint32_t ONE_BITS  = 0x3F800000u;
+    constexpr int      UNIT_LOG2 = DT == DT_F32 ? 0 : DT == DT_F16 ? 13 : 16;  // a unit of T in fp32 mantissa bits
+    // (Only the entries are counted: a bucket's mass is taken as at least its count times its lower edge, which is
+    // within 1/64 of the truth and costs no second atomic per element.)
+    constexpr uint32_t BAND_LOW = (ONE_BITS - ((uint32_t)TPR_BAND << UNIT_LOG2)) | 0x80000000u;
+    auto tally = [&](int v, float e) {
+        const uint32_t k = order_key_nonneg(e);
+        if (k > ZERO_KEY) {
+            atomicAdd(&cnt[topp_bucket(k)], 1u);
+            if (k >= BAND_LOW) {  // within a few units of 1: rare
+                const uint32_t bits = k & 0x7FFFFFFFu;
+                if (bits <= ONE_BITS) {
+                    atomicMin(&band[(ONE_BITS - bits) >> UNIT_LOG2], v);
+                }
+            }
+        }
+    };
+    const float pad_e = round_t<DT>(det_expf_nonpos(-MAXT - mx));
+    float       sum   = 0.0f;
+    if (!vals.fin) {
+        constexpr int U = DT == DT_F32 ? 8 : 16;
+        int           v = t;
+        for (; v + (U - 1) * SM_THREADS < n; v += U * SM_THREADS) {
+            float x[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                x[u] = S::ld(rowp[v + u * SM_THREADS]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float e = round_t<DT>(det_expf_nonpos((x[u] + 0.0f) - mx));
+                sum += e;
+                tally(v + u * SM_THREADS, e);
+            }
+        }
+        for (; v < n; v += SM_THREADS) {
+            const float e = round_t<DT>(det_expf_nonpos((S::ld(rowp[v]) + 0.0f) - mx));
+            sum += e;
+            tally(v, e);
+        }
+        for (; v < n_padded; v += SM_THREADS) {
+            sum += pad_e;
+            tally(v, pad_e);
+        }
+    }
+    else {
+        for (int v = t; v < n_padded; v += SM_THREADS) {
+            const float e = round_t<DT>(det_expf_nonpos(vals.masked(v, 0.0f) - mx));
+            sum += e;
+            tally(v, e);
+        }
+    }
+#pragma unroll
+    for (int mm = 16; mm > 0; mm >>= 1) {
+        sum += __shfl_xor(sum, mm, 32);
+    }
+    if ((t & 31) == 0) {
+        sh[t >> 5] = sum;
+    }
+    __syncthreads();
+    if (t < 32) {
+        float v = sh[t];
+#pragma unroll
+        for (int mm = 16; mm > 0; mm >>= 1) {
+            v += __shfl_xor(v, mm, 32);
+        }
+        if (t == 0) {
+            sh_bcast = v;
+        }
+    }
+    __syncthreads();
+    const float      denom = sh_bcast + 1e-6f;
+    const RowDivisor div(denom);
+    m.mx    = mx;
+    m.denom = denom;
+    if (!(denom == denom)) {
+        // a NaN among the logits: every probability is a NaN, none is positive, nothing is gathered
+        if (t == 0) {
+            meta[row] = m;
+        }
+        return;
+    }
+
+    // ---- the arg-max: the lowest id among the entries that share the largest probability. The largest e is 1
+    // (the maximum's own); numerators a few units below 1 may round to the same quotient.
+    {
+        const float p_one = topp_prob_of<DT>(1.0f, div, denom);
+        int         best  = 0x7FFFFFFF;
+        for (int j = 0; j <= TPR_BAND; ++j) {
+            const float e_j = u2f(ONE_BITS - ((uint32_t)j << UNIT_LOG2));
+            if (topp_prob_of<DT>(e_j, div, denom) == p_one) {
+                best = min(best, band[j]);
+            }
+        }
+        if (best != 0x7FFFFFFF) {
+            m.best      = ((unsigned long long)order_key(p_one) << 32) | (uint32_t)(~(uint32_t)best);
+            m.best_prob = p_one;
+        }
+    }
+    const float p = top_ps != nullptr ? top_ps[row] : top_p;
+    if ((uint32_t)(m.best >> 32) != 0u && round_t<DT>(0.0f + m.best_prob) >= p) {
+        // arg-max shortcut of the reference (:842-849): nothing else of the row is needed
+        if (t == 0) {
+            m.flags   = TOPP_SHORTCUT;
+            meta[row] = m;
+        }
+        return;
+    }
+    const float rand_num = row_uniform_peek(rng, uniforms, row) * p;
+
+    // ---- 3a. the cut. Buckets up to b0 may hold numerators whose probability rounds to zero: never gathered.
+    uint32_t total = 0;
+    {
+        const float tiny   = DT == DT_F32 ? 1.0e-44f : DT == DT_F16 ? 1.2e-7f : 2.0e-40f;  // above two units of T at zero
+        const float e_zero = tiny * denom * 1.001f;
+        const int   b0     = topp_bucket(order_key_nonneg(__builtin_fminf(e_zero, 2.0f)));
+        // smallest mass (units of 2^-31 of e) that certainly covers the draw: the scan's own rounding, the rounding
+        // of every quotient to T (relative, and absolute where the probabilities are subnormal in T)
+        uint32_t lc = 0;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const int d = K * t + i;
+            if (d < TPB_NB) {
+                lc += cnt[TPB_NB - 1 - d];
+            }
+        }
+        // a bucket's mass in units of 2^-31 of e: at least its count times its lower edge (the lowest bucket holds
+        // everything under 2^-32 and counts for nothing, the highest one only values above 1, of which there are none)
+        auto mass_of = [&](int b) -> unsigned long long {
+            if (b <= 0 || b >= TPB_NB - 1) {
+                return 0ull;
+            }
+            const float edge_b = u2f((uint32_t)(b + (TPB_ONE - TPB_SPAN)) << TPB_SHIFT);
+            return (unsigned long long)cnt[b] * (unsigned long long)(edge_b * 2147483648.0f);
+        };
+        unsigned long long lm = 0;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const int d = K * t + i;
+            if (d < TPB_NB) {
+                mass[TPB_NB - 1 - d] = mass_of(TPB_NB - 1 - d);
+                lm += mass[TPB_NB - 1 - d];
+            }
+        }
+        uint32_t           ic = lc;
+        unsigned long long im = lm;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const uint32_t           uc = __shfl_up(ic, o, WAVE);
+            const unsigned long long um = __shfl_up(im, o, WAVE);
+            if (lane_id() >= o) {
+                ic += uc;
+                im += um;
+            }
+        }
+        if (lane_id() == WAVE - 1) {
+            wcnt[wave_id()]  = ic;
+            wmass[wave_id()] = im;
+        }
+        __syncthreads();
+        uint32_t           ec = ic - lc;
+        unsigned long long em = im - lm;
+        for (int w = 0; w < SM_THREADS / WAVE; ++w) {
+            if (w < wave_id()) {
+                ec += wcnt[w];
+                em += wmass[w];
+            }
+            total += wcnt[w];
+        }
+        const double half_unit = DT == DT_F32 ? 0.0 : DT == DT_F16 ? 2.98023223876953125e-08 : 4.6e-41;
+        const double slack     = DT == DT_BF16 ? 1.0 / 100.0 : 1.0 / 512.0;  // (half a unit of bfloat16 is 2^-9)
+        const double want      = ((double)rand_num * (1.0 + slack) + (double)total * half_unit) * (double)denom;
+        const unsigned long long target = (unsigned long long)(want * 2147483648.0) + 64ull;
+        uint32_t first = 0xFFFFFFFFu;  // first descending position where the suffix covers the target
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const int d = K * t + i;
+            if (d < TPB_NB) {
+                const int b = TPB_NB - 1 - d;
+                off[b]      = ec;
+                ec += cnt[b];
+                em += mass[b];
+                if (em >= target && first == 0xFFFFFFFFu) {
+                    first = (uint32_t)d;
+                }
+            }
+        }
+        first = block_min<uint32_t, SM_THREADS / WAVE>(first, red32, 0xFFFFFFFFu);
+        int cut = first == 0xFFFFFFFFu ? 0 : TPB_NB - 1 - (int)first;
+        cut     = max(cut, b0 + 1);
+        cut     = min(cut, TPB_NB - 1);
+        // Entries that share a probability are ordered by id in the reference, whatever their e: the prefix must
+        // hold all of them or none. The cut moves down while the two values of T either side of its lower edge give
+        // the same probability (equal probabilities have numerators within a few units of T: a few buckets at most).
+        bool splits = false;
+        for (int guard = 0; guard < 64; ++guard) {
+            if (cut >= TPB_NB - 1) {
+                break;
+            }
+            const float edge_at = u2f((uint32_t)(cut + (TPB_ONE - TPB_SPAN)) << TPB_SHIFT);
+            float       above, under;  // the smallest value of T at or above the edge, the largest below it
+            if constexpr (DT == DT_F32) {
+                above = edge_at;
+                under = u2f(f2u(edge_at) - 1u);
+            }
+            else {
+                const typename S::T r = S::st(edge_at);
+                const bool          up = S::ld(r) >= edge_at;
+                above                  = up ? S::ld(r) : S::ld((typename S::T)(r + 1));
+                under                  = up ? S::ld((typename S::T)(r - 1)) : S::ld(r);
+            }
+            splits = topp_prob_of<DT>(above, div, denom) == topp_prob_of<DT>(under, div, denom);
+            if (!splits || cut <= b0 + 1) {
+                break;
+            }
+            cut--;
+        }
+        m.cut   = cut;
+        m.n     = (int)(off[cut] + cnt[cut]);
+        // every positive entry is in the prefix exactly when nothing lies below the cut (then none of them is one
+        // of the numerators whose probability may be zero)
+        m.n_pos = (uint32_t)m.n == total ? (int)total : 0x7FFFFFFF;
+        if (splits && (uint32_t)m.n != total) {
+            // (the lowest bucket that may be gathered still shares a probability with what lies below it: the
+            // exact fallback of the pick kernel orders the whole row)
+            m.n     = 0;
+            m.n_pos = 0x7FFFFFFF;
+        }
+    }
+    const int cut = m.cut;
+
+    // segments of whole buckets, as topp_cut_kernel makes them
+    {
+        const uint32_t n_gathered = (uint32_t)m.n;
+        uint32_t       closes[K];
+        uint32_t       lclose = 0;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            const int d = K * t + i;
+            closes[i]   = 0u;
+            if (d < TPB_NB && TPB_NB - 1 - d >= cut) {
+                const int      b = TPB_NB - 1 - d;
+                const uint32_t o = off[b];
+                const uint32_t e = o + cnt[b];
+                if (cnt[b] != 0u && (e / TPS_SEG != o / TPS_SEG || e == n_gathered)) {
+                    closes[i] = e;
+                    lclose++;
+                }
+            }
+        }
+        uint32_t iclose = lclose;
+#pragma unroll
+        for (int o = 1; o < WAVE; o <<= 1) {
+            const uint32_t up = __shfl_up(iclose, o, WAVE);
+            if (lane_id() >= o) {
+                iclose += up;
+            }
+        }
+        __syncthreads();
+        if (lane_id() == WAVE - 1) {
+            wcnt[wave_id()] = iclose;
+        }
+        __syncthreads();
+        uint32_t at   = iclose - lclose;
+        uint32_t nseg = 0;
+        for (int w = 0; w < SM_THREADS / WAVE; ++w) {
+            at += w < wave_id() ? wcnt[w] : 0u;
+            nseg += wcnt[w];
+        }
+        uint32_t* ends = seg_ends + (size_t)row * TPB_NB;
+#pragma unroll
+        for (int i = 0; i < K; ++i) {
+            if (closes[i] != 0u) {
+                ends[at++] = closes[i];
+            }
+        }
+        m.nseg = (int)nseg;
+    }
+    if (t == 0) {
+        meta[row] = m;
+    }
+    if (m.n == 0) {
+        return;
+    }
+
+    // ---- 3b. the gather: every bucket's cursor starts at the bucket's place in the prefix
+    __syncthreads();
+    for (int b = t; b < TPB_NB; b += SM_THREADS) {
+        cnt[b] = off[b];
+    }
+    __syncthreads();
+    unsigned long long* A = sorted + (size_t)row * 2 * n_padded;
+    // Nothing whose y lies under this can reach the cut bucket: the y of half the bucket's lower edge, less a margin.
+    // (An exponential under half the edge stays under the edge when it is rounded to T, also where T is subnormal:
+    // the edge is at least two units of T there, see b0. The margin covers the errors of exponential and logarithm
+    // many times over.)
+    const float edge  = u2f((uint32_t)(cut + (TPB_ONE - TPB_SPAN)) << TPB_SHIFT);
+    const float y_cut = cut >= TPB_NB - 1 ? -3.402823466e+38f :
+                                            (mx + det_logf(edge)) - (0.75f + 1e-6f * __builtin_fabsf(mx));
+    auto place = [&](int v, float y) {
+        if (y < y_cut) {
+            return;
+        }
+        const float    e = round_t<DT>(det_expf_nonpos(y - mx));
+        const uint32_t k = order_key_nonneg(e);
+        if (k > ZERO_KEY) {
+            const int b = topp_bucket(k);
+            if (b >= cut) {
+                const uint32_t kp   = order_key(topp_prob_of<DT>(e, div, denom));
+                const uint32_t slot = atomicAdd(&cnt[b], 1u);
+                A[slot]             = ((unsigned long long)(~kp) << 32) | (uint32_t)v;
+            }
+        }
+    };
+    if (!vals.fin) {
+        stream_columns<DT, SM_THREADS>(rowp, 0, n, [&](int v, float x) { place(v, x + 0.0f); });
+        for (int v = n + t; v < n_padded; v += SM_THREADS) {
+            place(v, -MAXT);
+        }
+    }
+    else {
+        for (int v = t; v < n_padded; v += SM_THREADS) {
+            place(v, vals.masked(v, 0.0f));
+        }
+    }
 }
 
 // Scratch of the radix sort below.
@@ -1273,12 +1707,13 @@ __device__ int scan_sorted(TopPShared& s, const unsigned long long* __restrict__
 // id of the `nth` (0-based) entry with probability exactly zero, in ascending id order: what a
 // stable descending sort leaves behind the positive entries. Single thread; reached only when a
 // draw lands within rounding distance of the total mass.
-template<int DT>
-__device__ int nth_zero_entry(const typename Storage<DT>::T* __restrict__ rowp, int vocab, int nth)
+// the id of the nth entry (in id order) whose probability is not positive; prob(v) gives the probability of column v
+template<class P>
+__device__ int nth_zero_entry(P&& prob, int vocab, int nth)
 {
     int seen = 0, last = vocab - 1;
     for (int v = 0; v < vocab; ++v) {
-        if (order_key(Storage<DT>::ld(rowp[v])) <= ZERO_KEY) {
+        if (order_key(prob(v)) <= ZERO_KEY) {
             last = v;
             if (seen == nth) {
                 return v;
@@ -1289,14 +1724,109 @@ __device__ int nth_zero_entry(const typename Storage<DT>::T* __restrict__ rowp, 
     return last;
 }
 
-template<int DT>
+// Rows sampled straight from logits: the segments of the ordered prefix are ranges of e, not of the probability,
+// and entries of neighbouring segments can share a probability. Within a segment equal probabilities stand in
+// ascending order of id, as in the reference's stable sort of the whole row; across a boundary they may not. The
+// walk's sums do not depend on the order of equal values, only the emitted id does: the reference emits, of the
+// entries that share the probability at position `found`, the one with as many smaller ids as there are entries of
+// the run in front of `found`. Called by every thread of the workgroup; every thread gets the entry to emit.
+__device__ unsigned long long topp_settle_ties(TopPShared& s, const unsigned long long* __restrict__ A, int n, int found,
+                                               const uint32_t* __restrict__ ends, int nseg, int vocab)
+{
+    const int t = threadIdx.x;
+    if (t == 0) {
+        const unsigned long long here = A[found];
+        const uint32_t           key  = (uint32_t)(here >> 32);
+        // the prefix is in ascending order of this word as a whole (the division keeps the order of the segments)
+        int lo = 0, hi = found;  // first position of the run
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if ((uint32_t)(A[mid] >> 32) < key) {
+                lo = mid + 1;
+            }
+            else {
+                hi = mid;
+            }
+        }
+        const int a = lo;
+        lo = found;
+        hi = n - 1;  // last position of the run
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if ((uint32_t)(A[mid] >> 32) > key) {
+                hi = mid - 1;
+            }
+            else {
+                lo = mid;
+            }
+        }
+        const int b = lo;
+        // does a segment end inside (a, b]?
+        int slo = 0, shi = nseg - 1;
+        while (slo < shi) {
+            const int mid = (slo + shi) >> 1;
+            if ((int)ends[mid] > a) {
+                shi = mid;
+            }
+            else {
+                slo = mid + 1;
+            }
+        }
+        const bool crosses = (int)ends[slo] > a && (int)ends[slo] <= b;
+        s.misc[4] = a;
+        s.misc[5] = b;
+        s.misc[6] = crosses ? 1 : 0;
+    }
+    __syncthreads();
+    const int  a       = s.misc[4];
+    const int  b       = s.misc[5];
+    const bool crosses = s.misc[6] != 0;
+    if (!crosses) {
+        return A[found];  // the run lies inside one segment: already in the reference's order
+    }
+    // the id with exactly (found - a) smaller ids in the run: bisection over the ids, counting with all threads
+    const int want = found - a;
+    int       lo = 0, hi = vocab;  // the answer lies in [lo, hi)
+    while (hi - lo > 1) {
+        const int mid = lo + (hi - lo) / 2;
+        if (t == 0) {
+            s.misc[7] = 0;
+        }
+        __syncthreads();
+        int mine = 0;
+        for (int i = a + t; i <= b; i += TP_THREADS) {
+            mine += (int)(uint32_t)A[i] < mid ? 1 : 0;
+        }
+        mine = wave_sum_i(mine);
+        if (lane_id() == 0 && mine != 0) {
+            atomicAdd(&s.misc[7], mine);
+        }
+        __syncthreads();
+        const int below_mid = s.misc[7];
+        __syncthreads();
+        // ids are distinct: the answer is below mid exactly when more than `want` ids are
+        if (below_mid > want) {
+            hi = mid;
+        }
+        else {
+            lo = mid;
+        }
+    }
+    const uint32_t key = (uint32_t)(A[found] >> 32);
+    return ((unsigned long long)key << 32) | (uint32_t)lo;
+}
+
+// LOGITS: `probs` holds the row's logits (n of its `vocab` columns are the vocabulary proper) and every probability
+// that is needed is worked out from them with the row's statistics in `meta` (topp_row_kernel); `seg_ends` are the
+// segments of the ordered prefix.
+template<int DT, bool LOGITS>
 __device__ __forceinline__ void
 topp_pick_row(TopPShared& s, const typename Storage<DT>::T* __restrict__ probs, int* ids,
               int* __restrict__ sequence_length, bool* __restrict__ finished, float* __restrict__ cum_log_probs,
               float* __restrict__ output_log_probs, RngState* rng, const float* __restrict__ uniforms, int vocab,
               const int* __restrict__ end_ids, float top_p, const float* top_ps,
               const bool* __restrict__ skip_decode, unsigned long long* __restrict__ sorted,
-              const ToppRowMeta* __restrict__ meta, int force_deep)
+              const ToppRowMeta* __restrict__ meta, int force_deep, int n, const uint32_t* __restrict__ seg_ends)
 {
     typedef Storage<DT>   S;
     const int             row = blockIdx.x;
@@ -1311,7 +1841,23 @@ topp_pick_row(TopPShared& s, const typename Storage<DT>::T* __restrict__ probs, 
     if ((uint32_t)(m.best >> 32) == 0u) {
         best_id = 0;  // nothing comparable in the row (all NaN): the reference keeps index 0
     }
-    const float best_prob = S::ld(rowp[best_id]);
+    ToppRowValues vals;
+    vals.MAXT   = S::max_t();
+    vals.fin    = LOGITS && finished != nullptr ? finished[row] : false;  // (read before this kernel writes the flag)
+    vals.end_id = vals.fin ? end_ids[row] : -1;
+    vals.n      = n;
+    const RowDivisor div(LOGITS ? m.denom : 1.0f);
+    // the probability of column v as the sampler of the reference would read it from the softmax's output
+    auto prob_at = [&](int v) -> float {
+        if constexpr (LOGITS) {
+            const float y = vals.masked(v, v < n ? S::ld(rowp[v]) : 0.0f);
+            return topp_prob_of<DT>(round_t<DT>(det_expf_nonpos(y - m.mx)), div, m.denom);
+        }
+        else {
+            return S::ld(rowp[v]);
+        }
+    };
+    const float best_prob = LOGITS ? ((uint32_t)(m.best >> 32) == 0u ? prob_at(0) : m.best_prob) : S::ld(rowp[best_id]);
 
     if (t == 0) {
         const float u = row_uniform(rng, uniforms, row);  // drawn for every non-skipped row
@@ -1355,14 +1901,22 @@ topp_pick_row(TopPShared& s, const typename Storage<DT>::T* __restrict__ probs, 
         const bool all   = m.n == m.n_pos;
         const int  found = m.n > 0 ? scan_sorted(s, A, m.n, rand_num) : -1;
         if (found >= 0 && (found < m.n || all)) {
+            unsigned long long e = 0ull;
+            if (found < m.n) {
+                if constexpr (LOGITS) {
+                    e = topp_settle_ties(s, A, m.n, found, seg_ends + (size_t)row * TPB_NB, m.nseg, vocab);
+                }
+                else {
+                    e = A[found];
+                }
+            }
             if (t == 0) {
                 if (found < m.n) {
-                    const unsigned long long e = A[found];
                     emit((int)(uint32_t)e, key64_prob(e));
                 }
                 else {
-                    const int id = nth_zero_entry<DT>(rowp, vocab, found - m.n);
-                    emit(id, S::ld(rowp[id]));
+                    const int id = nth_zero_entry(prob_at, vocab, found - m.n);
+                    emit(id, prob_at(id));
                 }
             }
             return;
@@ -1379,7 +1933,7 @@ topp_pick_row(TopPShared& s, const typename Storage<DT>::T* __restrict__ probs, 
     __syncthreads();
     for (int base = 0; base < vocab; base += TP_THREADS) {
         const int                v    = base + t;
-        const uint32_t           k    = v < vocab ? order_key(S::ld(rowp[v])) : 0u;
+        const uint32_t           k    = v < vocab ? order_key(prob_at(v)) : 0u;
         const bool               keep = k > ZERO_KEY;
         const unsigned long long bal  = __ballot(keep);
         const int                below = __popcll(bal & ((1ull << lane_id()) - 1ull));
@@ -1404,20 +1958,20 @@ topp_pick_row(TopPShared& s, const typename Storage<DT>::T* __restrict__ probs, 
         }
         __syncthreads();
     }
-    const int n = s.misc[2];
+    const int n_all = s.misc[2];
     __threadfence_block();
     __syncthreads();
     RadixScratch              rs{reinterpret_cast<unsigned short*>(s.buf), s.wtot, s.red64};
-    const unsigned long long* src   = radix_sort_range(A, B, n, 32, rs);
-    const int                 found = n > 0 ? scan_sorted(s, src, n, rand_num) : -1;
+    const unsigned long long* src   = radix_sort_range(A, B, n_all, 32, rs);
+    const int                 found = n_all > 0 ? scan_sorted(s, src, n_all, rand_num) : -1;
     if (found >= 0 && t == 0) {
-        if (found < n) {
+        if (found < n_all) {
             const unsigned long long e = src[found];
             emit((int)(uint32_t)e, key64_prob(e));
         }
         else {
-            const int id = nth_zero_entry<DT>(rowp, vocab, found - n);
-            emit(id, S::ld(rowp[id]));
+            const int id = nth_zero_entry(prob_at, vocab, found - n_all);
+            emit(id, prob_at(id));
         }
     }
 }
@@ -1431,18 +1985,18 @@ struct ToppDecayArgs {
     const int32_t* reset_ids;
 };
 
-template<int DT>
+template<int DT, bool LOGITS>
 __global__ void __launch_bounds__(TP_THREADS)
 topp_pick_kernel(const typename Storage<DT>::T* __restrict__ probs, int* ids, int* __restrict__ sequence_length,
                  bool* __restrict__ finished, float* __restrict__ cum_log_probs, float* __restrict__ output_log_probs,
                  RngState* rng, const float* __restrict__ uniforms, int vocab, const int* __restrict__ end_ids,
                  float top_p, const float* top_ps, const bool* __restrict__ skip_decode,
                  unsigned long long* __restrict__ sorted, const ToppRowMeta* __restrict__ meta, int force_deep,
-                 ToppDecayArgs dec)
+                 ToppDecayArgs dec, int n, const uint32_t* __restrict__ seg_ends)
 {
     __shared__ TopPShared s;
-    topp_pick_row<DT>(s, probs, ids, sequence_length, finished, cum_log_probs, output_log_probs, rng, uniforms, vocab,
-                      end_ids, top_p, top_ps, skip_decode, sorted, meta, force_deep);
+    topp_pick_row<DT, LOGITS>(s, probs, ids, sequence_length, finished, cum_log_probs, output_log_probs, rng, uniforms,
+                              vocab, end_ids, top_p, top_ps, skip_decode, sorted, meta, force_deep, n, seg_ends);
     // thread 0 wrote the row's id itself (a skipped row keeps what an earlier kernel left there) and every
     // thread read the row's top_p before the first barrier of the pick
     if (dec.runtime_top_p != nullptr && threadIdx.x == 0) {
@@ -1541,7 +2095,7 @@ static int topp_sampling_launch(int dtype, void* workspace, size_t* workspace_si
                                 const float* uniform_draws, int batch_size, size_t vocab_size_padded,
                                 const int* end_ids, float max_top_p, const float* top_ps, hipStream_t st,
                                 const bool* skip_decode, bool softmax_first, const void* bias, int vocab_size,
-                                ToppDecayArgs dec)
+                                ToppDecayArgs dec, bool from_logits = false)
 {
     if (dtype < 0 || dtype > 2) {
         return FTK_ERR_DTYPE;
@@ -1588,6 +2142,23 @@ static int topp_sampling_launch(int dtype, void* workspace, size_t* workspace_si
     ToppRowMeta*        meta    = (ToppRowMeta*)(ws + plan.off_meta);
     const int           vocab   = (int)vocab_size_padded;
     const dim3          chunks(plan.splits, batch_size);
+    if (from_logits) {
+        // the probabilities are never written: three launches
+        FTK_DISPATCH_DTYPE(dtype, topp_row_kernel<DT><<<batch_size, SM_THREADS, 0, st>>>(
+                                      (const Storage<DT>::T*)log_probs, end_ids, finished, vocab, vocab_size,
+                                      skip_decode, (const RngState*)rng_state, uniform_draws, max_top_p, top_ps, segs,
+                                      meta, sorted));
+        FTK_LAUNCH_CHECK();
+        topp_sort_kernel<<<plan.sorters, TP_THREADS, 0, st>>>(sorted, segs, meta, vocab, batch_size);
+        FTK_LAUNCH_CHECK();
+        FTK_DISPATCH_DTYPE(dtype, (topp_pick_kernel<DT, true><<<batch_size, TP_THREADS, 0, st>>>(
+                                      (const Storage<DT>::T*)log_probs, output_ids, sequence_length, finished,
+                                      cum_log_probs, output_log_probs, (RngState*)rng_state, uniform_draws, vocab,
+                                      end_ids, max_top_p, top_ps, skip_decode, sorted, meta, g_topp_force_deep, dec,
+                                      vocab_size, segs)));
+        FTK_LAUNCH_CHECK();
+        return 0;
+    }
     if (softmax_first) {
         float2* stats = (float2*)(ws + off_stats);
         FTK_DISPATCH_DTYPE(dtype, (softmax_kernel<DT, true><<<batch_size, SM_THREADS, 0, st>>>(
@@ -1616,10 +2187,11 @@ static int topp_sampling_launch(int dtype, void* workspace, size_t* workspace_si
         topp_sort_kernel<<<plan.sorters, TP_THREADS, 0, st>>>(sorted, segs, meta, vocab, batch_size);
         FTK_LAUNCH_CHECK();
     }
-    FTK_DISPATCH_DTYPE(dtype, topp_pick_kernel<DT><<<batch_size, TP_THREADS, 0, st>>>(
+    FTK_DISPATCH_DTYPE(dtype, (topp_pick_kernel<DT, false><<<batch_size, TP_THREADS, 0, st>>>(
                                   (const Storage<DT>::T*)log_probs, output_ids, sequence_length, finished,
                                   cum_log_probs, output_log_probs, (RngState*)rng_state, uniform_draws, vocab,
-                                  end_ids, max_top_p, top_ps, skip_decode, sorted, meta, g_topp_force_deep, dec));
+                                  end_ids, max_top_p, top_ps, skip_decode, sorted, meta, g_topp_force_deep, dec, vocab,
+                                  segs)));
     FTK_LAUNCH_CHECK();
     return 0;
 }
@@ -1660,6 +2232,30 @@ int ftk_fused_topp_step(int dtype, void* workspace, size_t* workspace_size, void
                                 cum_log_probs, output_log_probs, logits, rng_state, uniform_draws, batch_size,
                                 vocab_size_padded, end_ids, max_top_p, runtime_top_p, (hipStream_t)stream,
                                 skip_decode, true, bias, vocab_size, dec);
+}
+
+int ftk_fused_topp_sample_step(int dtype, void* workspace, size_t* workspace_size, const void* logits,
+                               int vocab_size, size_t vocab_size_padded, int batch_size, const int* end_ids,
+                               bool* finished, int* sequence_length, int* output_ids, float* cum_log_probs,
+                               float* output_log_probs, ftk_rng_state* rng_state, const float* uniform_draws,
+                               float max_top_p, float* runtime_top_p, const float* initial_top_p,
+                               const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
+                               const bool* skip_decode, ftk_stream_t stream)
+{
+    if (vocab_size < SM_THREADS) {
+        return FTK_ERR_UNSUPPORTED;  // (the sum's order follows the softmax's block of min(n, 1024) threads)
+    }
+    ToppDecayArgs dec = {nullptr, nullptr, nullptr, nullptr, nullptr};
+    if (top_p_decay != nullptr) {
+        if (runtime_top_p == nullptr || initial_top_p == nullptr || top_p_min == nullptr || top_p_reset_ids == nullptr) {
+            return FTK_ERR_ARGUMENT;
+        }
+        dec = ToppDecayArgs{runtime_top_p, initial_top_p, top_p_decay, top_p_min, top_p_reset_ids};
+    }
+    return topp_sampling_launch(dtype, workspace, workspace_size, nullptr, output_ids, sequence_length, finished,
+                                cum_log_probs, output_log_probs, const_cast<void*>(logits), rng_state, uniform_draws,
+                                batch_size, vocab_size_padded, end_ids, max_top_p, runtime_top_p, (hipStream_t)stream,
+                                skip_decode, true, nullptr, vocab_size, dec, true);
 }
 
 int ftk_invoke_compute_topp_decay(float* runtime_top_p, const float* runtime_initial_top_p, const int* output_ids,

@@ -50,6 +50,8 @@ _SIGNATURES = {
     "ftk_invoke_compute_topp_decay": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp],
     "ftk_fused_topp_step": [_i, _vp, _vp, _vp, _vp, _i, _sz, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp,
                             _vp, _vp, _vp, _vp, _vp],
+    "ftk_fused_topp_sample_step": [_i, _vp, _vp, _vp, _i, _sz, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f, _vp, _vp,
+                                   _vp, _vp, _vp, _vp, _vp],
     "ftk_invoke_apply_temperature_penalty": [_i, _vp, _vp, _f, _i, _i, _i, _vp],
     "ftk_invoke_batch_apply_temperature_penalty": [_i, _vp, _vp, _vp, _i, _i, _i, _vp],
     "ftk_invoke_apply_repetition_penalty": [_i, _vp, _f, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp],

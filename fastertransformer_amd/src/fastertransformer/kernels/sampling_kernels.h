@@ -158,6 +158,30 @@ void invokeFusedTopPStep(void* workspace, size_t& workspace_size, T* logits, con
                                   stream));
 }
 
+// The same step for a caller that does not need the probabilities afterwards: `logits` is only read. False when
+// the step does not take this shape (fewer than 1024 columns): the caller then uses invokeFusedTopPStep. The
+// workspace is invokeFusedTopPStep's.
+template<typename T>
+bool invokeFusedTopPSampleStep(void* workspace, size_t workspace_size, const T* logits, const int vocab_size,
+                               const size_t vocab_size_padded, const int batch_size, const int* end_ids, bool* finished,
+                               int* sequence_length, int* output_ids, float* cum_log_probs, float* output_log_probs,
+                               curandState_t* curandstate, const float* uniform_draws, const float max_top_p,
+                               float* runtime_top_p, const float* initial_top_p, const float* top_p_decay,
+                               const float* top_p_min, const int32_t* top_p_reset_ids, const bool* skip_decode,
+                               hipStream_t stream)
+{
+    const int rc = ftk_fused_topp_sample_step(FtkDType<T>::value, workspace, &workspace_size, logits, vocab_size,
+                                              vocab_size_padded, batch_size, end_ids, finished, sequence_length,
+                                              output_ids, cum_log_probs, output_log_probs, curandstate, uniform_draws,
+                                              max_top_p, runtime_top_p, initial_top_p, top_p_decay, top_p_min,
+                                              top_p_reset_ids, skip_decode, stream);
+    if (rc == FTK_ERR_UNSUPPORTED) {
+        return false;
+    }
+    check_ftk(rc);
+    return true;
+}
+
 inline void invokeComputeToppDecay(float* runtime_top_p, const float* runtime_initial_top_p, const int* output_ids,
                                    const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
                                    const int local_batch_size, hipStream_t stream)

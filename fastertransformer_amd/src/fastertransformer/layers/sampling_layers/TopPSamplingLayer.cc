@@ -1,3 +1,4 @@
+#include <cstdlib>
 #include "src/fastertransformer/layers/sampling_layers/TopPSamplingLayer.h"
 
 #include <algorithm>
@@ -41,6 +42,14 @@ template<typename T>
 void TopPSamplingLayer<T>::setup(const size_t batch_size, const size_t beam_width, TensorMap* runtime_args)
 {
     BaseSamplingLayer<T>::setup(batch_size, beam_width, runtime_args);
+    {
+        // The reference leaves the probabilities in the logits buffer (TopPSamplingLayer.cu:287-297); nothing in its
+        // decode loop reads them again, so by default the step samples straight from the logits and leaves them
+        // alone. FT_SAMPLING_DISABLE_FUSED=1 (the switch that makes the top-k layer mutate the logits like the
+        // reference, read once per setup() as there) keeps that side effect.
+        const char* env     = std::getenv("FT_SAMPLING_DISABLE_FUSED");
+        keep_probabilities_ = env != nullptr && env[0] == '1';
+    }
     const Tensor runtime_top_p = runtime_args->isExist("runtime_top_p") ? runtime_args->at("runtime_top_p") : Tensor();
     const size_t runtime_top_p_size = runtime_top_p.size();
     if (runtime_top_p_size == 0) {
@@ -160,6 +169,18 @@ void TopPSamplingLayer<T>::runSampling(TensorMap* output_tensors, TensorMap* inp
     if (need > sampling_workspace_size_) {
         sampling_workspace_      = allocator_->reMalloc(sampling_workspace_, need, false);
         sampling_workspace_size_ = need;
+    }
+    if (!keep_probabilities_
+        && invokeFusedTopPSampleStep<T>(
+            sampling_workspace_, sampling_workspace_size_, logits, (int)vocab_size_, vocab_size_padded_,
+            local_batch_size, end_ids, finished,
+            output_tensors->at("sequence_length", Tensor()).template getPtr<int>(), ids, cum_log_probs,
+            output_log_probs, curandstate_buf_ + off,
+            input_tensors->at("uniform_draws", Tensor()).template getPtr<const float>(), runtime_max_top_p_,
+            runtime_top_p_buf_ + off, initial_top_p_buf_ + off, top_p_decay_buf_ + off, top_p_min_buf_ + off,
+            top_p_reset_ids_buf_ + off, skip_decode_buf_ + off, stream_)) {
+        sync_check_hip_error();
+        return;
     }
     invokeFusedTopPStep<T>(sampling_workspace_, sampling_workspace_size_, logits, (const T*)nullptr, (int)vocab_size_,
                            vocab_size_padded_, local_batch_size, end_ids, finished,

@@ -8,6 +8,7 @@ namespace fastertransformer {
 template<typename T>
 class TopPSamplingLayer: public BaseSamplingLayer<T> {
     float    runtime_max_top_p_   = 0.0f;
+    bool     keep_probabilities_  = false;  // FT_SAMPLING_DISABLE_FUSED=1, read once per setup()
     float*   initial_top_p_buf_   = nullptr;
     float*   top_p_decay_buf_     = nullptr;
     float*   top_p_min_buf_       = nullptr;

@@ -118,6 +118,21 @@ int ftk_fused_topp_step(int dtype, void* workspace, size_t* workspace_size, void
                         const float* initial_top_p, const float* top_p_decay, const float* top_p_min,
                         const int32_t* top_p_reset_ids, const bool* skip_decode, ftk_stream_t stream);
 
+/* ftk_fused_topp_step for callers that do not need the probabilities: same arguments without the bias, same ids,
+ * log-probs, lengths, finished flags and decayed top-p values, but `logits` is only read (the reference leaves the
+ * probabilities there, layers/sampling_layers/TopPSamplingLayer.cu:287-297; nothing in its decode loop reads them
+ * again). Every probability that is needed is worked out from the logits on the way, with the arithmetic of
+ * ftk_invoke_add_bias_softmax, so the row is read three times and never written. FTK_ERR_UNSUPPORTED (also from
+ * the size query) when vocab_size < 1024; a step with an embedding bias takes ftk_fused_topp_step.
+ * workspace == NULL: size query (ftk_fused_topp_step's). */
+int ftk_fused_topp_sample_step(int dtype, void* workspace, size_t* workspace_size, const void* logits,
+                               int vocab_size, size_t vocab_size_padded, int batch_size, const int* end_ids,
+                               bool* finished, int* sequence_length, int* output_ids, float* cum_log_probs,
+                               float* output_log_probs, ftk_rng_state* rng_state, const float* uniform_draws,
+                               float max_top_p, float* runtime_top_p, const float* initial_top_p,
+                               const float* top_p_decay, const float* top_p_min, const int32_t* top_p_reset_ids,
+                               const bool* skip_decode, ftk_stream_t stream);
+
 /* ---- kernels/sampling_penalty_kernels.h -------------------------------------------------- */
 
 /* invokeApplyTemperaturePenalty<T>, kernels/sampling_penalty_kernels.cu:75-99 */

@@ -855,6 +855,33 @@ def _fused_topp_cases(env, dt, rng, shapes):
         got = (to_numpy(d_ids), to_numpy(d_fin), to_numpy(d_seq), to_numpy(d_cum), to_numpy(d_out))
         _compare_topk(got, (w_ids, w_fin, w_seq, w_cum, w_out), dt)
         assert np.array_equal(to_numpy(d_p).view(np.uint32), w_p.view(np.uint32)), where
+        # the same step straight from the logits, which it leaves alone (no bias, at least a block's width of columns)
+        sample_sizes = (dt, None, C.addressof(ws_size), None, V, Vp, batch) + (None,) * 8 + (1.0,) + (None,) * 7
+        rc = lib.ftk_fused_topp_sample_step(*sample_sizes)
+        if V < 1024:
+            assert rc == ops.FTK_ERR_UNSUPPORTED, where
+            continue
+        ops.check(rc)
+        if bias is not None:
+            continue
+        ws = torch.empty(max(ws_size.value, 16), dtype=torch.uint8, device="cuda")
+        d_x = to_torch(logits, dt)
+        d_ids = torch.full((batch,), -7, dtype=torch.int32, device="cuda")
+        d_fin, d_seq = to_torch(finished), to_torch(seq)
+        d_cum = torch.zeros(batch, dtype=torch.float32, device="cuda")
+        d_out = torch.zeros(batch, dtype=torch.float32, device="cuda")
+        d_p = to_torch(p_arr)
+        ops.check(lib.ftk_fused_topp_sample_step(dt, ws.data_ptr(), C.addressof(ws_size), d_x.data_ptr(), V, Vp, batch,
+                                                 d_end.data_ptr(), d_fin.data_ptr(), d_seq.data_ptr(), d_ids.data_ptr(),
+                                                 d_cum.data_ptr(), d_out.data_ptr(), None, d_u.data_ptr(),
+                                                 float(p_arr.max()), d_p.data_ptr(), d_init.data_ptr(),
+                                                 d_decay.data_ptr() if with_decay else None, d_pmin.data_ptr(),
+                                                 d_reset.data_ptr(), d_skip.data_ptr(), ops.current_stream()))
+        _sync(torch)
+        assert np.array_equal(np.asarray(to_numpy(d_x)).view(np.uint8), np.asarray(logits).view(np.uint8)), where
+        got = (to_numpy(d_ids), to_numpy(d_fin), to_numpy(d_seq), to_numpy(d_cum), to_numpy(d_out))
+        _compare_topk(got, (w_ids, w_fin, w_seq, w_cum, w_out), dt)
+        assert np.array_equal(to_numpy(d_p).view(np.uint32), w_p.view(np.uint32)), where
 
 
 @pytest.mark.parametrize("dt", DTYPES, ids=lambda d: DTYPE_NAMES[d])
