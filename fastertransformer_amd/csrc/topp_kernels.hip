@@ -1094,7 +1094,7 @@ topp_row_kernel(const typename Storage<DT>::T* __restrict__ logits, const int* _
                 ends[at++] = closes[i];
             }
         }
-        m.nseg = (int)nseg;
+        m.nseg = m.n == 0 ? 0 : (int)nseg;  // (a row sent to the fallback has nothing to sort here)
     }
     if (t == 0) {
         meta[row] = m;
