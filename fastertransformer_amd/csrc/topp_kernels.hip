@@ -209,6 +209,8 @@ softmax_kernel(typename Storage<DT>::T* __restrict__ logits, const typename Stor
 //                sequential carry over tiles) and emits the token.
 // A row whose draw is not crossed inside its prefix (it cannot be unless the bound above fails)
 // falls back to a stable radix sort of all its positive entries.
+// Callers that do not need the probabilities afterwards take a second form of the step (topp_row_kernel below):
+// softmax statistics, histogram, cut and gather in one kernel that only reads the logits, then sort and pick.
 constexpr int      TP_THREADS = 1024;
 constexpr int      TP_TILE    = 256;          // the reference's scan tile
 constexpr int      TP_ROUND   = 1024;         // tiles whose totals are held in LDS at a time
