@@ -800,6 +800,21 @@ def test_fused_topp_step_against_the_three_calls_of_the_oracle(env, dt, seed):
     _fused_topp_cases(env, dt, rng, shapes)
 
 
+@pytest.mark.parametrize("seed", [253, 290, 345, 1628, 2213, 6951, 13587, 22768])
+def test_topp_sample_step_equal_probabilities_from_different_numerators(env, seed):
+    """Seeded cases (mostly bfloat16, where a probability has one or two numerators) in which entries that share a
+    probability come from different buckets of the numerator's histogram: the step that samples straight from the
+    logits must keep all of them or none in its ordered prefix and emit the id the reference's stable order of the
+    whole row puts at the sampled position."""
+    rng = np.random.default_rng(424200 + seed)
+    dt = int(rng.integers(0, 3))
+    V = int(rng.choice([1024, 1025, rng.integers(1026, 5000), rng.integers(5000, 40000), rng.integers(40000, 160000)]))
+    Vp = V + int(rng.choice([0, 0, 1, 7, 64]))
+    batch = int(rng.integers(1, 7))
+    kind = int(rng.integers(0, 3))
+    _fused_topp_cases(env, dt, rng, [(V, Vp, batch, kind)])
+
+
 def _fused_topp_cases(env, dt, rng, shapes):
     torch, lib, ops = env
     for case, (V, Vp, batch, kind) in enumerate(shapes):
