@@ -2127,6 +2127,10 @@ static int topp_sampling_launch(int dtype, void* workspace, size_t* workspace_si
     if (rng_state == nullptr && uniform_draws == nullptr) {
         return FTK_ERR_ARGUMENT;
     }
+    if (log_probs == nullptr || output_ids == nullptr
+        || (end_ids == nullptr && finished != nullptr && (sequence_length != nullptr || softmax_first))) {
+        return FTK_ERR_ARGUMENT;  // (the kernels read and write these unconditionally)
+    }
     if (vocab_size_padded > (size_t)65535 * TP_THREADS) {
         return FTK_ERR_ARGUMENT;
     }
