@@ -264,6 +264,60 @@ __device__ __forceinline__ bool lp_ties_bounded(float e_bound, float denom)
     return e_bound >= 2.0f * smallest_normal * denom;
 }
 
+// The end of a row, by TK_THREADS threads: the candidates in s.cand carry e = T(exp(y - max)) as their keys; they
+// become probabilities T(e / denom), the list is cut to little more than k entries and the reference's tie orders
+// are replayed on probabilities (topk_select_lds), which also samples and writes the row's outputs. `slot` is scratch
+// for TK_THREADS keys. Rows whose candidates cannot be trusted take the literal replay.
+template<int DT>
+__device__ __forceinline__ void lp_finish(TopkShared& s, uint32_t* slot, int n, bool valid, uint32_t thr, float denom,
+                                          float row_max, int k, float tp, float u, const FusedParams& p,
+                                          const FusedLaunch& l, int row, const TopkOutputs& out)
+{
+    const int      t    = threadIdx.x;
+    const uint32_t KMIN = min_valid_key<DT>();
+    // ---- candidates: e -> probability
+    if (n > TK_CCAP || !valid || !lp_ties_bounded<DT>(key_to_float(thr), denom)) {
+        // The list is incomplete, or fewer than k columns have a non-zero e (then columns of probability zero
+        // are picked too, by the reference's tie rules), or the k-th largest probability may be subnormal
+        // (ties without bound): the literal replay, on probabilities.
+        n = -1;
+    }
+    else {
+        int positive = 0;
+        for (int i = t; i < n; i += TK_THREADS) {
+            const uint32_t key = order_key(round_t<DT>(key_to_float(s.cand.key[i]) / denom));
+            s.cand.key[i]      = key;
+            positive += key > order_key(0.0f) ? 1 : 0;
+        }
+        positive = block_sum_i<TK_WAVES>(positive, (int*)s.red32);
+        if (positive < k) {
+            // probabilities that round to zero reach into the top k: they tie with every other zero of the row
+            n = -1;
+        }
+        else if (n > k + k / 2 && n <= 4 * TK_THREADS) {
+            // keep what reaches the k-th largest of 256 slot maxima (at least k candidates do, and everything
+            // that ties with the k-th largest probability does)
+            uint32_t mx = 0u;
+            for (int i = t; i < n; i += TK_THREADS) {
+                const uint32_t key = s.cand.key[i];
+                mx                 = key > mx ? key : mx;
+            }
+            slot[t] = mx;
+            lds_barrier();
+            const uint32_t P = lean_kth_of_slots(slot, k);
+            lds_barrier();
+            if (P > KMIN) {
+                n = topk_prune(s, n, P);
+            }
+        }
+    }
+    FusedRow<DT, 0> r0(p, row);
+    r0.team = TK_THREADS;  // (the workgroup may have had more threads: those have left)
+    ProbRow<DT>     prow{&r0, row_max, denom};
+    topk_select_lds<DT, ProbRow<DT>, true>(prow, s, n, KMIN, row, p.Vp, k, tp, p.max_top_k,
+                                           l.entries + (size_t)row * l.row_entries, true, u, p.end_ids, out);
+}
+
 template<int DT, int BMW>
 __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, FusedLaunch l, LogProbLaunch lp)
 {
@@ -617,48 +671,293 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
     }
     __syncthreads();
     const float denom = uniform_f(warp_sum[0] + 1e-6f);
-    int         n     = s.n_cand;
+    const int   n     = s.n_cand;
     __syncthreads();
-    // ---- candidates: e -> probability
-    if (n > TK_CCAP || !valid || !lp_ties_bounded<DT>(key_to_float(thr), denom)) {
-        // The list is incomplete, or fewer than k columns have a non-zero e (then columns of probability zero
-        // are picked too, by the reference's tie rules), or the k-th largest probability may be subnormal
-        // (ties without bound): the literal replay, on probabilities.
-        n = -1;
+    lp_finish<DT>(s, slot_key[par], n, valid, thr, denom, row_max, k, tp, u, p, l, row, out);
+}
+
+// ---- one launch: a workgroup per row reads it twice ---------------------------------------------------------------
+// With few rows lp_row_kernel's four waves per row are what bounds the step (about a microsecond per 1024 columns),
+// and most compute units idle. Here THREADS threads share a row, thread t owning summation chains t, t + THREADS, ...
+// of the reference's 1024, so the sum has the reference's order without any regrouping. First pass: the row's maximum
+// after temperature, penalties and masks, and every thread's own largest value, from which the bound of the candidates
+// follows (the k-th largest of 256 joined thread maxima, each of them a column of its own). Second pass (the row
+// comes from the caches this time): e = T(exp(y - max)) summed chain by chain, candidates collected on the way. Then
+// all waves but four leave and those finish like lp_row_kernel (lp_finish).
+// THREADS = 1024 for launches of at most one row per compute unit; with more rows, workgroups of fewer threads share a
+// compute unit and one's first pass (memory) runs beside another's second (arithmetic).
+constexpr int LPW_THREADS = 1024;
+
+template<int DT, int BMW, int THREADS>
+__global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLaunch l, LogProbLaunch lp)
+{
+    typedef Storage<DT>   S;
+    typedef typename S::T T;
+    constexpr int         CH = LP_BLOCK / THREADS;  // chains of a thread
+    constexpr int         U  = 8 / CH;              // rounds (1024 columns each) of a thread's batch: 8 columns
+    constexpr int         N  = U * CH;
+    static_assert(THREADS * CH == LP_BLOCK && U * CH == 8 && THREADS % 32 == 0 && THREADS >= TK_THREADS,
+                  "a workgroup owns all chains of its row");
+    __shared__ TopkShared s;
+    __shared__ uint32_t   wide_key[THREADS];
+    __shared__ uint32_t   slot_key[TK_THREADS];
+    __shared__ float      warp_sum[32];
+    __shared__ float      redf[THREADS / WAVE];
+    const int             t    = threadIdx.x;
+    const int             row  = blockIdx.x;
+    const T*              rowp = (const T*)p.logits + (size_t)row * p.Vp;
+    // slot j of a batch: round j / CH of the batch, chain (j % CH) * THREADS + t
+    auto offset_of = [](int j) { return (j / CH) * LP_BLOCK + (j % CH) * THREADS; };
+    // the first columns of the row are on their way before anything else is read
+    const int nfull = p.V / (U * LP_BLOCK);  // batches that every thread holds in full
+    T         buf[2][N];
+    auto      load = [&](T* raw, int b) {
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            raw[j] = rowp[b * U * LP_BLOCK + offset_of(j) + t];
+        }
+    };
+    if (nfull > 0) {
+        load(buf[0], 0);
     }
-    else {
-        int positive = 0;
-        for (int i = t; i < n; i += LP_THREADS) {
-            const uint32_t key = order_key(round_t<DT>(key_to_float(s.cand.key[i]) / denom));
-            s.cand.key[i]      = key;
-            positive += key > order_key(0.0f) ? 1 : 0;
+    const bool            skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
+    const bool            fin  = row_flag_or(l.finished, row, p.end_ids + row, false);
+    const int             k    = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
+    const float           tp   = row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f);
+    FusedRow<DT, BMW>     rowctx(p, row);
+    if (skip) {
+        return;
+    }
+    if (fin) {
+        if (t == 0) {
+            l.ids[row] = p.end_ids[row];  // a finished row emits its end id: no draw, no log-prob, no length update
         }
-        positive = block_sum_i<LP_THREADS / WAVE>(positive, (int*)s.red32);
-        if (positive < k) {
-            // probabilities that round to zero reach into the top k: they tie with every other zero of the row
-            n = -1;
+        return;
+    }
+    if (t == 0) {
+        s.n_cand  = 0;
+        s.misc[0] = __float_as_int(row_uniform(l.rng, l.uniforms, row));
+    }
+    const TopkOutputs out =
+        topk_outputs(l.ids, l.sequence_length, l.finished, lp.cum_log_probs, lp.output_log_probs, row, p.end_ids);
+    rowctx.prepare(0, p.V);  // the row's history bitmap in LDS (launches with a window and a history penalty)
+    __syncthreads();
+    const float    u       = __int_as_float(s.misc[0]);
+    const uint32_t KMIN    = min_valid_key<DT>();
+    const float    NEG_INF = -__builtin_inff();
+    // The values of a batch's columns (v0 = the first one's, t included) after temperature, history penalty and the
+    // min-length mask. A column's history flag is bit t % 32 of word v / 32 of the bitmap. The words of a batch are
+    // read together, and one look tells whether any of its columns needs more than the multiplication.
+    const bool bitsv = rowctx.has_vector_bits();
+    const int  bsh   = t & 31;
+    auto values = [&](int v0, const T* raw, float* y) {
+        uint32_t w[N];
+        uint32_t any = 0u;
+        if (bitsv) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                w[j] = rowctx.bm_word((v0 + offset_of(j)) >> 5);
+            }
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                any |= w[j];
+            }
+            any = (any >> bsh) & 1u;
         }
-        else if (n > k + k / 2 && n <= 4 * TK_THREADS) {
-            // keep what reaches the k-th largest of 256 slot maxima (at least k candidates do, and everything
-            // that ties with the k-th largest probability does)
-            uint32_t mx = 0u;
-            for (int i = t; i < n; i += TK_THREADS) {
-                const uint32_t key = s.cand.key[i];
-                mx                 = key > mx ? key : mx;
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            y[j] = rowctx.fast(S::ld(raw[j]));
+        }
+        const uint32_t to_end = (uint32_t)(rowctx.masked_end_id - v0);  // offset_of(j) for the masked end id at slot j
+        if (any != 0u || (to_end < (uint32_t)(U * LP_BLOCK) && (to_end & (THREADS - 1)) == 0u)) {  // rare
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                if (bitsv && ((w[j] >> bsh) & 1u)) {
+                    y[j] = rowctx.flagged(y[j], v0 + offset_of(j));
+                }
+                if (to_end == (uint32_t)offset_of(j)) {
+                    y[j] = -S::max_t();
+                }
             }
-            slot_key[par][t] = mx;
-            lds_barrier();
-            const uint32_t P = lean_kth_of_slots(slot_key[par], k);
-            lds_barrier();
-            if (P > KMIN) {
-                n = topk_prune(s, n, P);
+        }
+    };
+    // the same for one column
+    auto value = [&](int v, T raw) -> float {
+        float y = rowctx.fast(S::ld(raw));
+        if (bitsv && ((rowctx.bm_word(v >> 5) >> bsh) & 1u)) {
+            y = rowctx.flagged(y, v);
+        }
+        return v == rowctx.masked_end_id ? -S::max_t() : y;
+    };
+    // One pass over the row: whole batches with the next one's loads issued before the current one is used (the
+    // first is on its way already when `loaded`), then the columns behind them one by one, loaded together.
+    // use_batch(v0, y) takes a batch's values, use_one(j, v, y) the value of column v at slot j.
+    auto stream = [&](bool loaded, auto&& use_batch, auto&& use_one) {
+        if (nfull > 0 && !loaded) {
+            load(buf[0], 0);
+        }
+        auto batch = [&](const T* raw, int b) {
+            float     y[N];
+            const int v0 = b * U * LP_BLOCK + t;
+            values(v0, raw, y);
+            use_batch(v0, y);
+        };
+        // (every load is issued whatever the batch, one past the last fetches the last again, unused: with the same
+        // number of loads on every path the waits can name the older batch instead of everything in flight)
+        for (int b = 0; b < nfull; b += 2) {
+            load(buf[1], min(b + 1, nfull - 1));
+            batch(buf[0], b);
+            load(buf[0], min(b + 2, nfull - 1));
+            if (b + 1 < nfull) {
+                batch(buf[1], b + 1);
             }
+        }
+        const int v0 = nfull * U * LP_BLOCK + t;
+        if (v0 < p.V) {
+            T raw[N];
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                raw[j] = rowp[min(v0 + offset_of(j), p.V - 1)];
+            }
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                if (v0 + offset_of(j) < p.V) {
+                    use_one(j, v0 + offset_of(j), value(v0 + offset_of(j), raw[j]));
+                }
+            }
+        }
+    };
+
+    // ---- first pass: the maximum (pad columns count as -MAX_T), and the thread's own
+    float m = NEG_INF;
+    stream(
+        true,
+        [&](int, const float* y) {
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                m = __builtin_fmaxf(m, y[j]);
+            }
+        },
+        [&](int, int, float y) { m = __builtin_fmaxf(m, y); });
+    float row_max = block_max<float, THREADS / WAVE>(m, redf, NEG_INF);
+    row_max       = __builtin_fmaxf(-3.402823466e+38f, row_max);
+    if (p.V < p.Vp) {
+        row_max = __builtin_fmaxf(row_max, -S::max_t());
+    }
+    row_max = uniform_f(row_max);
+    // the bound: every thread's largest e belongs to a column of its own
+    wide_key[t] = order_key(round_t<DT>(det_expf_nonpos(m - row_max)));
+    __syncthreads();
+    if (t < TK_THREADS) {
+        uint32_t key = wide_key[t];
+#pragma unroll
+        for (int g = 1; g < THREADS / TK_THREADS; ++g) {
+            key = max(key, wide_key[t + g * TK_THREADS]);
+        }
+        slot_key[t] = key;
+    }
+    __syncthreads();
+    uint32_t       thr     = KMIN;
+    float          thr_low = key_to_float(KMIN);
+    bool           valid   = false;
+    const uint32_t P       = lean_kth_of_slots(slot_key, k);
+    if (P > order_key(0.0f)) {  // at least k columns with e > 0 at or above it
+        thr           = P;
+        const float e = key_to_float(P);
+        thr_low       = uniform_f(e - e * lp_tie_rel<DT>());
+        valid         = true;
+    }
+
+    // ---- second pass: the sum chain by chain, candidates on the way
+    float acc[CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        acc[c] = 0.0f;
+    }
+    auto push = [&](int v, float e) {
+        const int slot = atomicAdd(&s.n_cand, 1);
+        if (slot < TK_CCAP) {
+            s.cand.key[slot] = order_key(e);
+            s.cand.idx[slot] = (uint32_t)v;
+        }
+    };
+    stream(
+        false,
+        [&](int v0, const float* y) {
+            float d[N], e[N];
+            bool  number = true;  // one look for a NaN per pair of columns instead of one per column
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                d[j] = y[j] - row_max;
+            }
+#pragma unroll
+            for (int j = 0; j < N; j += 2) {
+                number = number && !__builtin_isunordered(d[j], d[j + 1]);
+            }
+            if (number) {
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    e[j] = round_t<DT>(det_expf_nonpos_number(d[j]));
+                }
+            }
+            else {
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    e[j] = round_t<DT>(det_expf_nonpos(d[j]));
+                }
+            }
+            float top = e[0];
+#pragma unroll
+            for (int j = 0; j < N; ++j) {
+                acc[j % CH] = acc[j % CH] + e[j];  // (slots of a chain in ascending order of their columns)
+                top         = __builtin_fmaxf(top, e[j]);
+            }
+            if (top >= thr_low) {  // (a NaN is no candidate, with or without the maximum)
+#pragma unroll
+                for (int j = 0; j < N; ++j) {
+                    if (e[j] >= thr_low) {
+                        push(v0 + offset_of(j), e[j]);
+                    }
+                }
+            }
+        },
+        [&](int j, int v, float y) {
+            const float e = round_t<DT>(det_expf_nonpos(y - row_max));
+            acc[j % CH]   = acc[j % CH] + e;
+            if (e >= thr_low) {
+                push(v, e);
+            }
+        });
+    // the reference's order: xor butterflies inside 32-chain groups, then over the 32 group sums
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+#pragma unroll
+        for (int o = 16; o >= 1; o >>= 1) {
+            acc[c] = acc[c] + __shfl_xor(acc[c], o, 32);
+        }
+        if ((t & 31) == 0) {
+            warp_sum[(c * THREADS + t) >> 5] = acc[c];
         }
     }
-    FusedRow<DT, 0> r0(p, row);
-    ProbRow<DT>     prow{&r0, row_max, denom};
-    topk_select_lds<DT, ProbRow<DT>, true>(prow, s, n, KMIN, row, p.Vp, k, tp, p.max_top_k,
-                                           l.entries + (size_t)row * l.row_entries, true, u, p.end_ids, out);
+    __syncthreads();
+    if (t < 32) {
+        float total = warp_sum[t];
+#pragma unroll
+        for (int o = 16; o >= 1; o >>= 1) {
+            total = total + __shfl_xor(total, o, 32);
+        }
+        if (t == 0) {
+            warp_sum[0] = total;
+        }
+    }
+    __syncthreads();
+    if (wave_id() >= TK_WAVES) {
+        return;  // the first four waves select
+    }
+    const float denom = uniform_f(warp_sum[0] + 1e-6f);
+    const int   n     = s.n_cand;
+    __syncthreads();
+    lp_finish<DT>(s, slot_key, n, valid, thr, denom, row_max, k, tp, u, p, l, row, out);
 }
 
 // Launchers, one translation unit per element type (logprob_kernels.hip built with FTK_LP_DT = 0, 1, 2).
@@ -675,5 +974,12 @@ int lp_row_launch_f16(int window, int rows, hipStream_t st, const FusedParams& p
                       const LogProbLaunch& lp);
 int lp_row_launch_bf16(int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
                        const LogProbLaunch& lp);
+// threads: 1024, 512 or 256 per row
+int lp_wide_launch_f32(int window, int threads, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                       const LogProbLaunch& lp);
+int lp_wide_launch_f16(int window, int threads, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                       const LogProbLaunch& lp);
+int lp_wide_launch_bf16(int window, int threads, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+                        const LogProbLaunch& lp);
 
 }  // namespace ftk

@@ -93,7 +93,11 @@ FTK_HD float det_expf(float x)
 // clamp keeps -inf out of the argument reduction; it would also turn a NaN into a number, hence the two forms.
 FTK_HD float det_expf_nonpos_number(float x)  // x is not a NaN (a NaN would come out as a number)
 {
-    x             = __builtin_fmaxf(x, -104.0f);  // one instruction on the device
+#if defined(__HIP_DEVICE_COMPILE__)
+    x = __builtin_amdgcn_fmed3f(x, -104.0f, 0.0f);  // the clamp in one instruction (x <= 0: the upper end is never taken)
+#else
+    x = __builtin_fmaxf(x, -104.0f);
+#endif
     const float n = __builtin_rintf(x * 1.44269502162933349609375f);
     float       r = fma_rn(n, -0.693145751953125f, x);
     r             = fma_rn(n, -1.428606765330187045e-06f, r);

@@ -160,6 +160,13 @@ extern "C" int ftk_profile_read(int kernel, double* total_ms, int* launches)
     return 0;
 }
 
+// Threads per row of a log-prob step in one launch (lp_wide_kernel); 0: two launches instead (lp_rowmax_kernel,
+// lp_row_kernel).
+static int lp_threads_per_row(int rows)
+{
+    return rows <= 256 ? 1024 : 512;
+}
+
 #ifdef FTK_TEST_HOOKS
 // Test hook (hooks build of the library only): non-zero sends every launch through the general stream, so
 // that it can be compared with the lean gather on the shapes the lean gather normally takes.
@@ -167,6 +174,13 @@ static int g_fused_force_general = 0;
 extern "C" void ftk_test_set_fused_force_general(int v)
 {
     g_fused_force_general = v;
+}
+// Test hook: the form of the log-prob step. 0: the product's choice, 1: two launches, 1024 / 512 / 256: one launch
+// with that many threads per row.
+static int g_lp_form = 0;
+extern "C" void ftk_test_set_lp_form(int v)
+{
+    g_lp_form = (v == 1 || v == 1024 || v == 512 || v == 256) ? v : 0;
 }
 // Test hook: non-zero keeps the selection in a launch of its own also where one workgroup per row could do both.
 static int g_fused_two_launches = 0;
@@ -185,6 +199,7 @@ extern "C" int ftk_test_last_fused_path(void)
 #else
 static constexpr int g_fused_force_general = 0;
 static constexpr int g_fused_two_launches  = 0;
+static constexpr int g_lp_form             = 0;
 #define FTK_NOTE_PATH(v) ((void)0)
 #endif
 
@@ -383,6 +398,20 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             lp.partial_max      = (float*)l.headers;  // one float per list header slot: the lists are not used
             lp.splits           = lplan.splits;
             hipEvent_t e0, e1;
+            const int lp_threads = g_lp_form == 0 ? lp_threads_per_row(rows) : (g_lp_form == 1 ? 0 : g_lp_form);
+            if (lp_threads != 0) {
+                take_events(1, &e0, &e1);
+                if (e0 != nullptr) {
+                    FTK_HIP_CHECK(hipEventRecord(e0, st));
+                }
+                rc = a->dtype == FTK_DTYPE_F32 ? lp_wide_launch_f32(window, lp_threads, rows, st, p, l, lp) :
+                     a->dtype == FTK_DTYPE_F16 ? lp_wide_launch_f16(window, lp_threads, rows, st, p, l, lp) :
+                                                 lp_wide_launch_bf16(window, lp_threads, rows, st, p, l, lp);
+                if (rc == 0 && e1 != nullptr) {
+                    FTK_HIP_CHECK(hipEventRecord(e1, st));
+                }
+                return rc;
+            }
             take_events(1, &e0, &e1);
             if (e0 != nullptr) {
                 FTK_HIP_CHECK(hipEventRecord(e0, st));

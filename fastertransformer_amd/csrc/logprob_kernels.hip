@@ -57,4 +57,39 @@ int lp_row_launch_bf16
     return (int)hipGetLastError();
 }
 
+#if FTK_LP_DT == 0
+int lp_wide_launch_f32
+#elif FTK_LP_DT == 1
+int lp_wide_launch_f16
+#else
+int lp_wide_launch_bf16
+#endif
+    (int window, int threads, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l,
+     const LogProbLaunch& lp)
+{
+    constexpr int DT = FTK_LP_DT;
+    auto launch = [&](auto words) {
+        constexpr int BMW = decltype(words)::value;
+        if (threads == 1024) {
+            hipLaunchKernelGGL((lp_wide_kernel<DT, BMW, 1024>), dim3(rows), dim3(1024), 0, st, p, l, lp);
+        }
+        else if (threads == 512) {
+            hipLaunchKernelGGL((lp_wide_kernel<DT, BMW, 512>), dim3(rows), dim3(512), 0, st, p, l, lp);
+        }
+        else {
+            hipLaunchKernelGGL((lp_wide_kernel<DT, BMW, 256>), dim3(rows), dim3(256), 0, st, p, l, lp);
+        }
+    };
+    if (window == 0) {
+        launch(std::integral_constant<int, FUSED_BITMAP_WORDS_GLOBAL>());
+    }
+    else if (window == 2) {
+        launch(std::integral_constant<int, FUSED_BITMAP_WORDS_LARGE>());
+    }
+    else {
+        launch(std::integral_constant<int, FUSED_BITMAP_WORDS_SMALL>());
+    }
+    return (int)hipGetLastError();
+}
+
 }  // namespace ftk

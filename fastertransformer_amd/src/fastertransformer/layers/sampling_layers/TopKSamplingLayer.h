@@ -10,7 +10,7 @@ class TopKSamplingLayer: public BaseSamplingLayer<T> {
     uint runtime_max_top_k_ = 1;
     // the two environment switches of the layer as setup() found them
     bool fused_disabled_           = false;
-    int  fused_log_probs_min_rows_ = 192;
+    int  fused_log_probs_min_rows_ = 0;
 
     void allocateBuffer() override;
     void allocateBuffer(size_t batch_size, Tensor top_k, Tensor top_p) override;

@@ -84,11 +84,14 @@ def uniforms(rng, n):
     return u.astype(np.float32)
 
 
-def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=None, ws_fill=None):
+def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=None, ws_fill=None,
+                   log_probs=None, Vp=None):
     """One fused decode step straight through the C ABI (temperature 0.8, repetition penalty 1.1 over `history`,
     top-k `k`, top-p 0.9, injected draws). entry: "caller" = ftk_fused_topk_step with a workspace of the queried
     size, "static" = ftk_fused_topk_step_static. Returns (ids, sequence_length, finished, rc, needed bytes, change of
-    the device's free memory across the static call)."""
+    the device's free memory across the static call). With a dict as `log_probs` the step also keeps log-probs:
+    cum_log_probs start at the dict's "cum" (zeros without it) and come back there, output_log_probs under "out".
+    `Vp` is the pitch of the logits' rows in elements when they are padded."""
     import ctypes as C
     import fastertransformer_amd as fa
     from fastertransformer_amd import ops
@@ -104,7 +107,8 @@ def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finishe
     top_ps = torch.full((B,), 0.9, device=dev)
     a = ops.FusedTopkArgs()
     a.dtype, a.logits, a.embedding_bias = dt, logits.data_ptr(), None
-    a.vocab_size = a.vocab_size_padded = V
+    a.vocab_size = V
+    a.vocab_size_padded = V if Vp is None else Vp
     a.batch_size = a.local_batch_size = B
     a.step, a.max_input_length = H, H
     a.temperatures, a.penalties, a.penalty_type = temps.data_ptr(), pens.data_ptr(), ops.PENALTY_MULTIPLICATIVE
@@ -113,6 +117,10 @@ def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finishe
     a.uniform_draws = draws.data_ptr()
     a.ids = out_ids.data_ptr() + 4 * H * B
     a.sequence_length, a.finished = seq.data_ptr(), finished.data_ptr()
+    if log_probs is not None:
+        cum = torch.zeros(B, device=dev) if "cum" not in log_probs else torch.as_tensor(log_probs["cum"]).to(dev)
+        olp = torch.zeros(B, device=dev)
+        a.cum_log_probs, a.output_log_probs = cum.data_ptr(), olp.data_ptr()
     lib = fa.ftk() if lib is None else lib
     stream = ops.current_stream()
     ws = None
@@ -133,6 +141,8 @@ def run_fused_step(entry, torch, dt, B, V, H, k, logits, history, draws, finishe
         rc = lib.ftk_fused_topk_step_static(C.addressof(a), stream)
         torch.cuda.synchronize()
         freed = torch.cuda.mem_get_info()[0] - free_before
+    if log_probs is not None:
+        log_probs["cum"], log_probs["out"] = cum.cpu().numpy(), olp.cpu().numpy()
     return out_ids[H].cpu().numpy(), seq.cpu().numpy(), finished.cpu().numpy(), rc, a.workspace_size, freed
 
 

@@ -438,14 +438,20 @@ def test_fused_step_with_log_probs_random_scenarios(dt, seed):
         _run_case(c, rng, 3, logits_fn, check_logits=False)
 
 
-def test_log_probs_on_small_windows_take_the_kernel_sequence(monkeypatch):
-    """Without the override of the test session, log-prob outputs send windows of fewer than 192 rows through the
-    kernel sequence (which writes the penalised logits and the probabilities back like the reference) and larger
-    ones through the fused step (which leaves the logits alone); the results are the reference's either way."""
-    monkeypatch.delenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS")
+@pytest.mark.parametrize("min_rows", [None, 100])
+def test_log_probs_take_the_fused_step_from_the_smallest_window_on(monkeypatch, min_rows):
+    """Without the environment's override, log-prob outputs send every window through the fused step (which leaves the
+    logits alone); with FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS=100 windows of fewer than 100 rows take the kernel
+    sequence instead (which writes the penalised logits and the probabilities back like the reference); the results
+    are the reference's either way."""
+    if min_rows is None:
+        monkeypatch.delenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS")
+    else:
+        monkeypatch.setenv("FT_SAMPLING_FUSED_LOGPROBS_MIN_ROWS", str(min_rows))
     rng = np.random.default_rng(7200)
     V = 2051
-    for B, mutated in ((8, True), (191, True), (192, False), (400, False)):
+    for B in (8, 99, 100, 400):
+        mutated = min_rows is not None and B < min_rows
         c = Case(O.F32, B, V, V, max_input_length=4, gen_len=2, runtime_top_k=[8], runtime_top_p=[0.9],
                  temperature=[0.7], repetition_penalty=[1.3], prompt=_history(rng, 4, B, V), with_cum=True,
                  with_out_lp=True)
