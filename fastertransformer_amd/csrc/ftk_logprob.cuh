@@ -46,6 +46,44 @@ struct LogProbLaunch {
     int    splits;            // workgroups per row of lp_rowmax_kernel
 };
 
+// The exact value of the largest element of a 16-byte vector whose first element is column `first` (`a` columns of
+// the row's first vector lie in front of the row): plain vectors through their raw maximum (rounding to T and a
+// positive multiplier keep the order), the others element by element.
+template<int DT, int BMW>
+__device__ __forceinline__ float lp_vector_max(const FusedRow<DT, BMW>& rowctx, const uint4& v, int first, int a,
+                                               bool bitsv, bool ordered)
+{
+    typedef Storage<DT> S;
+    constexpr int       EPV  = (int)(16 / sizeof(typename S::T));
+    uint32_t            bits = 0u;
+    if (bitsv) {
+        if (BMW > 0 && a == 0) {  // the flags of a vector never straddle a word of the bitmap
+            const int rel = first - rowctx.bm_origin;
+            bits          = (rowctx.bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
+        }
+        else {
+            bits = rowctx.vector_bits(first, EPV);
+        }
+    }
+    const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - first);
+    if (bits == 0u && rel_end >= (uint32_t)EPV && ordered) {
+        return rowctx.fast(lean_raw_max<DT>(v));
+    }
+    float vm = -__builtin_inff();
+#pragma unroll
+    for (int c = 0; c < EPV; ++c) {
+        float x = rowctx.fast(vector_element<DT>(v, c));
+        if ((bits >> c) & 1u) {
+            x = rowctx.flagged(x, first + c);
+        }
+        if ((uint32_t)c == rel_end) {
+            x = -S::max_t();
+        }
+        vm = __builtin_fmaxf(vm, x);
+    }
+    return vm;
+}
+
 // ---- pass 1 --------------------------------------------------------------------------------------------
 template<int DT, int BMW>
 __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(FusedParams p, FusedLaunch l, LogProbLaunch lp)
@@ -133,36 +171,8 @@ __global__ void __launch_bounds__(LG_THREADS, LG_OCCUPANCY) lp_rowmax_kernel(Fus
     const bool  ordered = mul > 0.0f && mul < __builtin_inff();  // the plain transform keeps the order
     const float NEG_INF = -__builtin_inff();
     float       m       = NEG_INF;
-    // the exact value of a vector's largest element: plain vectors through their raw maximum (rounding to T and
-    // a positive multiplier keep the order), the others element by element
     auto vector_max = [&](const uint4& v, int first) -> float {
-        uint32_t bits = 0u;
-        if (bitsv) {
-            if (BMW > 0 && a == 0) {  // the flags of a vector never straddle a word of the bitmap
-                const int rel = first - rowctx.bm_origin;
-                bits          = (rowctx.bm_word(rel >> 5) >> (rel & 31)) & ((1u << EPV) - 1u);
-            }
-            else {
-                bits = rowctx.vector_bits(first, EPV);
-            }
-        }
-        const uint32_t rel_end = (uint32_t)(rowctx.masked_end_id - first);
-        if (bits == 0u && rel_end >= (uint32_t)EPV && ordered) {
-            return rowctx.fast(lean_raw_max<DT>(v));
-        }
-        float vm = NEG_INF;
-#pragma unroll
-        for (int c = 0; c < EPV; ++c) {
-            float x = rowctx.fast(vector_element<DT>(v, c));
-            if ((bits >> c) & 1u) {
-                x = rowctx.flagged(x, first + c);
-            }
-            if ((uint32_t)c == rel_end) {
-                x = -S::max_t();
-            }
-            vm = __builtin_fmaxf(vm, x);
-        }
-        return vm;
+        return lp_vector_max<DT, BMW>(rowctx, v, first, a, bitsv, ordered);
     };
     for (int q0 = 0; q0 < nsub; q0 += R) {
 #pragma unroll
@@ -688,6 +698,12 @@ __global__ void __launch_bounds__(LP_THREADS) lp_row_kernel(FusedParams p, Fused
 // compute unit and one's first pass (memory) runs beside another's second (arithmetic).
 constexpr int LPW_THREADS = 1024;
 
+#ifdef FTK_LP_STAMPS  // development builds: wall-clock stamps of a row's phases in its candidate list area
+#define LPW_STAMP(i) if (threadIdx.x == 0) { reinterpret_cast<unsigned long long*>(l.entries + (size_t)blockIdx.x * l.row_entries)[i] = wall_clock64(); }
+#else
+#define LPW_STAMP(i)
+#endif
+
 template<int DT, int BMW, int THREADS>
 __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLaunch l, LogProbLaunch lp)
 {
@@ -708,7 +724,38 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
     const T*              rowp = (const T*)p.logits + (size_t)row * p.Vp;
     // slot j of a batch: round j / CH of the batch, chain (j % CH) * THREADS + t
     auto offset_of = [](int j) { return (j / CH) * LP_BLOCK + (j % CH) * THREADS; };
-    // the first columns of the row are on their way before anything else is read
+    // First pass, for the maximum only: the order of the columns does not matter, so the row comes in as the 16-byte
+    // vectors of the memory, thread t taking vectors vlo + t, vlo + t + THREADS, ... (`a` columns of the row's first
+    // vector lie in front of the row; what lies in front of vector vlo and behind vector vhi is looked at column by
+    // column). The first vectors are on their way before anything else is read.
+    constexpr int EPV   = (int)(16 / sizeof(T));
+    constexpr int R1    = 8;  // vectors a thread keeps in flight
+    const int     a     = (int)(((uintptr_t)rowp & 15u) / sizeof(T));
+    const uint4*  base  = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(rowp) - a * sizeof(T));
+    const int     vlo   = (a + EPV - 1) / EPV;
+    const int     vhi   = max(vlo + 1, (a + p.V) / EPV);  // (a row has at least 1024 columns)
+    const int     nvec  = vhi - vlo;
+    const int     turns = (nvec + THREADS - 1) / THREADS;
+    // (the history before them: its ids are scattered reads that nothing should queue behind)
+    constexpr int HU   = 2048 / THREADS;
+    const bool    hist = BMW > 0 && p.bitmaps != nullptr && p.penalties != nullptr;
+    int           hist_ids[HU];
+    if (hist) {
+#pragma unroll
+        for (int i = 0; i < HU; ++i) {
+            const int pos = t + i * THREADS;
+            hist_ids[i]   = pos < p.step ? p.output_ids[(size_t)pos * p.batch_size + row] : -1;
+        }
+    }
+    uint4         ring[R1];
+    // (every load is issued whatever the turn, one past the last fetches the last again, unused: with the same number
+    // of loads on every path the waits can name the oldest load instead of everything in flight)
+    auto vload = [&](int slot, int q) { ring[slot] = base[vlo + min(min(q, turns - 1) * THREADS + t, nvec - 1)]; };
+#pragma unroll
+    for (int r = 0; r < R1; ++r) {
+        vload(r, r);
+    }
+    // Second pass: thread t takes columns of its own chains, batches of N
     const int nfull = p.V / (U * LP_BLOCK);  // batches that every thread holds in full
     T         buf[2][N];
     auto      load = [&](T* raw, int b) {
@@ -717,14 +764,12 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
             raw[j] = rowp[b * U * LP_BLOCK + offset_of(j) + t];
         }
     };
-    if (nfull > 0) {
-        load(buf[0], 0);
-    }
     const bool            skip = row_flag_or(p.skip_decode, row, p.end_ids + row, false);
     const bool            fin  = row_flag_or(l.finished, row, p.end_ids + row, false);
     const int             k    = row_arg_or(p.top_ks, row, p.end_ids + row, p.max_top_k);
     const float           tp   = row_arg_or(p.top_ps, row, p.end_ids + row, 1.0f);
     FusedRow<DT, BMW>     rowctx(p, row);
+    LPW_STAMP(0)
     if (skip) {
         return;
     }
@@ -735,14 +780,38 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
         return;
     }
     if (t == 0) {
-        s.n_cand  = 0;
-        s.misc[0] = __float_as_int(row_uniform(l.rng, l.uniforms, row));
+        s.n_cand = 0;
     }
     const TopkOutputs out =
         topk_outputs(l.ids, l.sequence_length, l.finished, lp.cum_log_probs, lp.output_log_probs, row, p.end_ids);
-    rowctx.prepare(0, p.V);  // the row's history bitmap in LDS (launches with a window and a history penalty)
+    if (hist) {
+        // the row's history bitmap in LDS (launches with a window and a history penalty)
+        uint32_t* window = fused_lds_bitmap<FusedRow<DT, BMW>::LDS_WORDS>();
+        const int words  = min(FusedRow<DT, BMW>::LDS_WORDS, (p.V + 31) / 32 + 1);
+        for (int i = t; i < words; i += THREADS) {
+            window[i] = 0u;
+        }
+        __syncthreads();
+        auto mark = [&](int pos, int id) {
+            id -= p.col_offset;
+            if (id >= 0 && id < p.V && rowctx.history_position_counts(pos)) {
+                atomicOr(&window[id >> 5], 1u << (id & 31));
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < HU; ++i) {
+            if (hist_ids[i] >= 0) {
+                mark(t + i * THREADS, hist_ids[i]);
+            }
+        }
+        for (int pos = t + HU * THREADS; pos < p.step; pos += THREADS) {
+            mark(pos, p.output_ids[(size_t)pos * p.batch_size + row]);
+        }
+        rowctx.bm_mode   = 1;
+        rowctx.bm_origin = 0;
+    }
     __syncthreads();
-    const float    u       = __int_as_float(s.misc[0]);
+    LPW_STAMP(1)
     const uint32_t KMIN    = min_valid_key<DT>();
     const float    NEG_INF = -__builtin_inff();
     // The values of a batch's columns (v0 = the first one's, t included) after temperature, history penalty and the
@@ -784,16 +853,16 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
     // the same for one column
     auto value = [&](int v, T raw) -> float {
         float y = rowctx.fast(S::ld(raw));
-        if (bitsv && ((rowctx.bm_word(v >> 5) >> bsh) & 1u)) {
+        if (bitsv && ((rowctx.bm_word(v >> 5) >> (v & 31)) & 1u)) {
             y = rowctx.flagged(y, v);
         }
         return v == rowctx.masked_end_id ? -S::max_t() : y;
     };
-    // One pass over the row: whole batches with the next one's loads issued before the current one is used (the
-    // first is on its way already when `loaded`), then the columns behind them one by one, loaded together.
+    // The second pass over the row: whole batches with the next one's loads issued before the current one is used,
+    // then the columns behind them one by one, loaded together.
     // use_batch(v0, y) takes a batch's values, use_one(j, v, y) the value of column v at slot j.
-    auto stream = [&](bool loaded, auto&& use_batch, auto&& use_one) {
-        if (nfull > 0 && !loaded) {
+    auto stream = [&](auto&& use_batch, auto&& use_one) {
+        if (nfull > 0) {
             load(buf[0], 0);
         }
         auto batch = [&](const T* raw, int b) {
@@ -830,16 +899,36 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
 
     // ---- first pass: the maximum (pad columns count as -MAX_T), and the thread's own
     float m = NEG_INF;
-    stream(
-        true,
-        [&](int, const float* y) {
+    {
+        const float mul     = rowctx.fast_mul;
+        const bool  ordered = mul > 0.0f && mul < __builtin_inff();  // the plain transform keeps the order
+        for (int q0 = 0; q0 < turns; q0 += R1) {
 #pragma unroll
-            for (int j = 0; j < N; ++j) {
-                m = __builtin_fmaxf(m, y[j]);
+            for (int r = 0; r < R1; ++r) {
+                const int q = q0 + r;
+                if (q < turns) {
+                    const int   rel = q * THREADS + t;
+                    const float vm  = lp_vector_max<DT, BMW>(rowctx, ring[r], (vlo + min(rel, nvec - 1)) * EPV - a, a,
+                                                            bitsv, ordered);
+                    m               = __builtin_fmaxf(m, rel < nvec ? vm : NEG_INF);
+                }
+                vload(r, q + R1);
             }
-        },
-        [&](int, int, float y) { m = __builtin_fmaxf(m, y); });
+        }
+        // the columns in front of the first whole vector and behind the last
+        for (int v = t; v < min(p.V, vlo * EPV - a); v += THREADS) {
+            m = __builtin_fmaxf(m, value(v, rowp[v]));
+        }
+        for (int v = vhi * EPV - a + t; v < p.V; v += THREADS) {
+            m = __builtin_fmaxf(m, value(v, rowp[v]));
+        }
+    }
+    LPW_STAMP(2)
+    if (t == 0) {
+        s.misc[0] = __float_as_int(row_uniform(l.rng, l.uniforms, row));  // (read behind the barriers of the sum)
+    }
     float row_max = block_max<float, THREADS / WAVE>(m, redf, NEG_INF);
+    LPW_STAMP(3)
     row_max       = __builtin_fmaxf(-3.402823466e+38f, row_max);
     if (p.V < p.Vp) {
         row_max = __builtin_fmaxf(row_max, -S::max_t());
@@ -868,6 +957,7 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
         valid         = true;
     }
 
+    LPW_STAMP(4)
     // ---- second pass: the sum chain by chain, candidates on the way
     float acc[CH];
 #pragma unroll
@@ -882,7 +972,6 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
         }
     };
     stream(
-        false,
         [&](int v0, const float* y) {
             float d[N], e[N];
             bool  number = true;  // one look for a NaN per pair of columns instead of one per column
@@ -928,6 +1017,7 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
                 push(v, e);
             }
         });
+    LPW_STAMP(5)
     // the reference's order: xor butterflies inside 32-chain groups, then over the 32 group sums
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -956,8 +1046,11 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
     }
     const float denom = uniform_f(warp_sum[0] + 1e-6f);
     const int   n     = s.n_cand;
+    const float u     = __int_as_float(s.misc[0]);
     __syncthreads();
+    LPW_STAMP(6)
     lp_finish<DT>(s, slot_key, n, valid, thr, denom, row_max, k, tp, u, p, l, row, out);
+    LPW_STAMP(7)
 }
 
 // Launchers, one translation unit per element type (logprob_kernels.hip built with FTK_LP_DT = 0, 1, 2).

@@ -160,11 +160,18 @@ extern "C" int ftk_profile_read(int kernel, double* total_ms, int* launches)
     return 0;
 }
 
-// Threads per row of a log-prob step in one launch (lp_wide_kernel); 0: two launches instead (lp_rowmax_kernel,
-// lp_row_kernel).
-static int lp_threads_per_row(int rows)
+// Threads per row of a log-prob step in one launch (lp_wide_kernel). Measured on MI355X (k = 64, us per step with 1024
+// / 512 / 256 threads per row; the two-launch form in brackets): 256 x 152064 f16 59 / 66 / 96 (129); 512 x 152064 f16
+// 109 / 96 / 110 (153); 1024 x 152064 f16 209 / 174 / 200 (218); 1024 x 128256 f32 206 / 177 / 217 (219); 1024 x 50264
+// f32 114 / 89 / 88 (111); 1024 x 32000 bf16 94 / 72 / 64; 8 x 50264 f32 28 / 33 / 47 (58). One workgroup per compute
+// unit wants all sixteen waves on its row; with more rows than compute units, two workgroups of eight waves overlap
+// one's reading with the other's arithmetic; many short rows do best with four of four.
+static int lp_threads_per_row(int rows, int vocab_size)
 {
-    return rows <= 256 ? 1024 : 512;
+    if (rows <= 256) {
+        return 1024;
+    }
+    return rows >= 1024 && vocab_size <= 65536 ? 256 : 512;
 }
 
 #ifdef FTK_TEST_HOOKS
@@ -398,7 +405,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             lp.partial_max      = (float*)l.headers;  // one float per list header slot: the lists are not used
             lp.splits           = lplan.splits;
             hipEvent_t e0, e1;
-            const int lp_threads = g_lp_form == 0 ? lp_threads_per_row(rows) : (g_lp_form == 1 ? 0 : g_lp_form);
+            const int lp_threads = g_lp_form == 0 ? lp_threads_per_row(rows, a->vocab_size) : (g_lp_form == 1 ? 0 : g_lp_form);
             if (lp_threads != 0) {
                 take_events(1, &e0, &e1);
                 if (e0 != nullptr) {

@@ -29,8 +29,13 @@ def _case(torch, dt, B, V, Vp, H, k, seed, kind):
         x[2, 7] = float("inf")
         x[3, :] = float("-inf")
         x[3, 11] = 0.0
-    logits = x.to(tdt)
     history = torch.randint(0, V, (H, B), generator=gen, device="cuda", dtype=torch.int32)
+    if kind == "edges":  # the largest values in the row's first and last columns, all of them in the history
+        x[:, :8] += 20.0
+        x[:, V - 8:V] += 20.0
+        history[0:8] = torch.arange(8, dtype=torch.int32, device="cuda")[:, None]
+        history[8:16] = torch.arange(V - 8, V, dtype=torch.int32, device="cuda")[:, None]
+    logits = x.to(tdt)
     draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
     finished0 = torch.zeros(B, dtype=torch.bool, device="cuda")
     finished0[B // 3] = True
@@ -47,6 +52,9 @@ CASES = [
     (O.F16, 16, 16500, 16504, 2000, 64, "normal"),  # a long history
     (O.F32, 8, 30011, 30011, 32, 20, "flat"),       # rows the candidates' bound cannot separate, NaN, infinities
     (O.F16, 520, 152064, 152064, 64, 64, "normal"),  # two rounds of 512-thread workgroups
+    (O.BF16, 13, 1024, 1027, 16, 8, "edges"),       # rows off 16-byte boundaries whose maxima lie in the columns in
+    (O.F32, 11, 4999, 5001, 16, 30, "edges"),       # front of the first whole vector and behind the last
+    (O.F16, 19, 33001, 33003, 16, 64, "edges"),
 ]
 
 
