@@ -840,21 +840,38 @@ topp_row_kernel(const typename Storage<DT>::T* __restrict__ logits, const int* _
     const float pad_e = round_t<DT>(det_expf_nonpos(-MAXT - mx));
     float       sum   = 0.0f;
     if (!vals.fin) {
-        constexpr int U = DT == DT_F32 ? 8 : 16;
-        int           v = t;
-        for (; v + (U - 1) * SM_THREADS < n; v += U * SM_THREADS) {
-            float x[U];
+        // batches of U columns per thread, the next batch's loads issued before the current one is used (every load is
+        // issued whatever the batch, one past the last fetches the last again, unused: with the same number of loads
+        // on every path the waits can name the older batch instead of everything in flight)
+        constexpr int        U     = 8;
+        const int            nfull = n / (U * SM_THREADS);  // batches that every thread holds in full
+        typename S::T        buf[2][U];
+        auto                 load  = [&](typename S::T* raw, int b) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                x[u] = S::ld(rowp[v + u * SM_THREADS]);
+                raw[u] = rowp[(b * U + u) * SM_THREADS + t];
             }
+        };
+        auto batch = [&](const typename S::T* raw, int b) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const float e = round_t<DT>(det_expf_nonpos((x[u] + 0.0f) - mx));
+                const float e = round_t<DT>(det_expf_nonpos((S::ld(raw[u]) + 0.0f) - mx));
                 sum += e;
-                tally(v + u * SM_THREADS, e);
+                tally((b * U + u) * SM_THREADS + t, e);
+            }
+        };
+        if (nfull > 0) {
+            load(buf[0], 0);
+        }
+        for (int b = 0; b < nfull; b += 2) {
+            load(buf[1], min(b + 1, nfull - 1));
+            batch(buf[0], b);
+            load(buf[0], min(b + 2, nfull - 1));
+            if (b + 1 < nfull) {
+                batch(buf[1], b + 1);
             }
         }
+        int v = nfull * U * SM_THREADS + t;
         for (; v < n; v += SM_THREADS) {
             const float e = round_t<DT>(det_expf_nonpos((S::ld(rowp[v]) + 0.0f) - mx));
             sum += e;
