@@ -722,6 +722,12 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
     const int             t    = threadIdx.x;
     const int             row  = blockIdx.x;
     const T*              rowp = (const T*)p.logits + (size_t)row * p.Vp;
+    // A workgroup that shares its compute unit with others is served first while it waits for memory more than it
+    // computes (set-up, first pass, selection): its few instructions then do not queue behind the arithmetic of a
+    // neighbour's second pass, and its loads stay in flight.
+    if constexpr (THREADS < LPW_THREADS) {
+        __builtin_amdgcn_s_setprio(3);
+    }
     // slot j of a batch: round j / CH of the batch, chain (j % CH) * THREADS + t
     auto offset_of = [](int j) { return (j / CH) * LP_BLOCK + (j % CH) * THREADS; };
     // First pass, for the maximum only: the order of the columns does not matter, so the row comes in as the 16-byte
@@ -958,6 +964,9 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
     }
 
     LPW_STAMP(4)
+    if constexpr (THREADS < LPW_THREADS) {
+        __builtin_amdgcn_s_setprio(0);
+    }
     // ---- second pass: the sum chain by chain, candidates on the way
     float acc[CH];
 #pragma unroll
@@ -1018,6 +1027,9 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
             }
         });
     LPW_STAMP(5)
+    if constexpr (THREADS < LPW_THREADS) {
+        __builtin_amdgcn_s_setprio(3);
+    }
     // the reference's order: xor butterflies inside 32-chain groups, then over the 32 group sums
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
