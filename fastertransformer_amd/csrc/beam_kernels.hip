@@ -426,17 +426,20 @@ beam_row_kernel(const bool* __restrict__ finished, const int* __restrict__ end_i
 // ballots over the top 24 key bits: a floor at or below the 2K-th largest maximum, which is all the argument
 // needs) so that the other fifteen waves only wait at two barriers; after the last pass twelve waves leave and the
 // first four select with the code of the 256-thread kernels (a barrier counts the waves that are left).
+// With more rows than compute units the workgroups have 512 threads and two of them share a compute unit: one's reads
+// run beside the other's exponentials (64 x 8 beams x 152064 fp16: 120 -> 116 us).
 constexpr int BR_THREADS = 1024;
-constexpr int BR_WAVES   = BR_THREADS / WAVE;
 
-template<int DT>
-__global__ void __launch_bounds__(BR_THREADS)
+template<int DT, int THREADS>
+__global__ void __launch_bounds__(THREADS)
 beam_rowwide_kernel(const typename Storage<DT>::T* __restrict__ x, const typename Storage<DT>::T* __restrict__ bias,
                     const bool* __restrict__ finished, const int* __restrict__ end_ids,
                     const float* __restrict__ cum_log_probs, int vocab, int K, int* __restrict__ cand_id,
                     float* __restrict__ cand_val)
 {
     typedef Storage<DT>   S;
+    constexpr int         BR_WAVES = THREADS / WAVE;
+    static_assert(THREADS == 1024 || THREADS == 512, "256, 128 or 64 joined maxima");
     __shared__ BeamSelect s;
     __shared__ double     red[BR_WAVES];
     __shared__ float      redf[BR_WAVES];
@@ -472,7 +475,7 @@ beam_rowwide_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     const size_t rb = (size_t)row * vocab;
     // first pass: the row's maximum
     float m = -MAXT;
-    stream_columns<DT, BR_THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
+    stream_columns<DT, THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
         const float e = beam_element_of<DT>(xv, bias, v);
         m             = e > m ? e : m;
     });
@@ -480,7 +483,7 @@ beam_rowwide_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     // second pass: the sum, and every thread's largest element
     double d    = 0.0;
     float  fmax = -__builtin_inff();
-    stream_columns<DT, BR_THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
+    stream_columns<DT, THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
         const float e = beam_element_of<DT>(xv, bias, v);
         d += (double)det_expf_nonpos(e - m);
         fmax = __builtin_fmaxf(fmax, e);
@@ -493,10 +496,12 @@ beam_rowwide_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
         red[wave_id()] = d;
     }
     // 2K <= 32 needs no more than 64 maxima to choose the 2K-th largest from, 2K <= 64 no more than 128
-    const int join    = N <= 32 ? 16 : N <= 64 ? 8 : 4;  // neighbouring threads that join their maxima
-    const int n_slots = BR_THREADS / join;
+    const int n_slots = N <= 32 ? 64 : N <= 64 ? 128 : 256;
+    const int join    = THREADS / n_slots;  // neighbouring threads that join their maxima: 2 to 16
     fmax              = __builtin_fmaxf(fmax, __shfl_xor(fmax, 1, WAVE));
-    fmax              = __builtin_fmaxf(fmax, __shfl_xor(fmax, 2, WAVE));
+    if (join >= 4) {
+        fmax = __builtin_fmaxf(fmax, __shfl_xor(fmax, 2, WAVE));
+    }
     if (join >= 8) {
         fmax = __builtin_fmaxf(fmax, __shfl_xor(fmax, 4, WAVE));
     }
@@ -543,7 +548,7 @@ beam_rowwide_kernel(const typename Storage<DT>::T* __restrict__ x, const typenam
     const uint32_t floor_key = row_floor;
     const float    floor_val = key_to_float(floor_key);
     const bool     all_pass  = floor_key <= order_key(-__builtin_inff());  // then NaN columns are wanted too
-    stream_columns<DT, BR_THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
+    stream_columns<DT, THREADS>(x + rb, 0, vocab, [&](int v, float xv) {
         const float e = beam_element_of<DT>(xv, bias, v);
         if (e >= floor_val || all_pass) {
             const int at = atomicAdd(&s.n_cand, 1);
@@ -889,7 +894,7 @@ constexpr int BR_SHORT_ROW = 65536;
 constexpr int BR_MANY_ROWS = 192;
 #ifdef FTK_TEST_HOOKS
 // Test hook (hooks build of the library only): 1 = sections of rows and three launches everywhere, 2 = one
-// workgroup per row everywhere, 0 = by the shape.
+// 1024-thread workgroup per row everywhere, 3 = one 512-thread workgroup per row everywhere, 0 = by the shape.
 static int g_beam_path = 0;
 extern "C" void ftk_test_set_beam_path(int v)
 {
@@ -982,15 +987,23 @@ int ftk_invoke_topk_softmax(int dtype, const void* log_probs, const void* bias, 
     // in sections; 64 rows of 50257 27 against 30 us, 256 rows 29 against 36 us, 512 rows of 152064 112 against
     // 115 us).
     bool one_per_row = vocab_size <= BR_SHORT_ROW || rows >= BR_MANY_ROWS;
+    bool half_size   = rows > 256;  // two 512-thread workgroups per compute unit
 #ifdef FTK_TEST_HOOKS
-    one_per_row = g_beam_path == 0 ? one_per_row : g_beam_path == 2;
+    one_per_row = g_beam_path == 0 ? one_per_row : g_beam_path >= 2;
+    half_size   = g_beam_path <= 1 ? half_size : g_beam_path == 3;
 #endif
     FTK_DISPATCH_DTYPE(dtype, {
         typedef Storage<DT>::T T;
-        if (one_per_row) {
-            beam_rowwide_kernel<DT><<<rows, BR_THREADS, 0, st>>>((const T*)log_probs, (const T*)bias, finished, end_ids,
-                                                                 cum_log_probs, vocab_size, beam_width, cand_id,
-                                                                 cand_val);
+        if (one_per_row && half_size) {
+            beam_rowwide_kernel<DT, BR_THREADS / 2><<<rows, BR_THREADS / 2, 0, st>>>(
+                (const T*)log_probs, (const T*)bias, finished, end_ids, cum_log_probs, vocab_size, beam_width, cand_id,
+                cand_val);
+            FTK_LAUNCH_CHECK();
+        }
+        else if (one_per_row) {
+            beam_rowwide_kernel<DT, BR_THREADS><<<rows, BR_THREADS, 0, st>>>(
+                (const T*)log_probs, (const T*)bias, finished, end_ids, cum_log_probs, vocab_size, beam_width, cand_id,
+                cand_val);
             FTK_LAUNCH_CHECK();
         }
         else {

@@ -38,8 +38,9 @@ int ftk_test_last_fused_path(void);
 /* the form of the fused log-prob step: 0 the product's choice, 1 two launches (row maxima, then one 256-thread
    workgroup per row), 1024 / 512 / 256 one launch with that many threads per row; process-wide */
 void ftk_test_set_lp_form(int form);
-/* the beam-search step: 1 = sections of rows in three launches everywhere, 2 = one workgroup per row in one launch
-   everywhere, 0 = chosen by the shape (the product's behaviour); process-wide */
+/* the beam-search step: 1 = sections of rows in three launches everywhere, 2 = one 1024-thread workgroup per row in
+   one launch everywhere, 3 = the same with 512 threads, 0 = chosen by the shape (the product's behaviour);
+   process-wide */
 void ftk_test_set_beam_path(int path);
 
 #ifdef __cplusplus

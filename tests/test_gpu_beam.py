@@ -103,10 +103,11 @@ def test_beam_step_full_vocabularies_and_batches(dt):
     _one_case(rng, dt, 1, 2, 152064, False, 0.0, 0.0)
 
 
-@pytest.mark.parametrize("path", [1, 2], ids=["sections_three_launches", "one_workgroup_per_row"])
+@pytest.mark.parametrize("path", [1, 2, 3], ids=["sections_three_launches", "one_workgroup_per_row",
+                                                  "one_512_thread_workgroup_per_row"])
 def test_beam_step_both_forms_of_the_row_stage(path):
-    """The row stage has two forms, chosen by the shape: sections of rows in three launches, and one
-    1024-thread workgroup per row in one. The test build of the library forces either on the same cases: every
+    """The row stage has two forms, chosen by the shape: sections of rows in three launches, and one workgroup per row
+    in one launch (1024 threads, or 512 when there are more rows than compute units). The test build of the library forces either on the same cases: every
     beam-width class, tiny and full vocabularies, more rows than compute units, rows of equal values (the bound
     passes more than fits the list), rows masked to -inf, finished beams, NaN columns."""
     from fastertransformer_amd import ops
