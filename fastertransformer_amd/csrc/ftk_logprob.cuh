@@ -4,27 +4,29 @@
 // (src/fastertransformer/layers/sampling_layers/TopKSamplingLayer.cu:220-266: invokeAddBiasSoftMax, then the
 // top-k kernels on probabilities, whose log-prob outputs are log p and log p - log S). Its kernel sequence
 // moves the row nine times (temperature R+W, penalties, softmax 3R+3W, top-k k+2 R). Here the row is read
-// twice and never written:
-//   lp_rowmax_kernel - streams the row once (the launch shape of the lean gather), applies temperature,
-//                      history penalty and the min-length mask in registers and leaves the exact maximum of
-//                      every workgroup's share in the workspace;
-//   lp_row_kernel    - one workgroup per row streams it again, with the same arithmetic, and
-//                        * sums e_v = T(exp(y_v - max)) in the order of the reference's softmax
-//                          (sampling_topp_kernels.cu:1308-1344: thread t of 1024 adds columns t, t + 1024, ...
-//                          one after the other; reduce_kernel_utils.cuh:73-103: xor butterflies 16..1 inside
-//                          32-lane groups, then over the 32 group sums), so the sum has the reference's bits:
-//                          a thread owns four neighbouring chains and walks them with 16-byte (fp32) or 8-byte
-//                          (16-bit types) loads that are 1024 columns apart;
-//                        * gathers the candidates of the top-k selection by e_v, with a bound lowered by what
-//                          the division and rounding to T can merge, so that every column whose probability
-//                          ties with the k-th largest is among them;
-//                        * turns the candidates' e_v into probabilities T(e_v / (sum + 1e-6)), replays the
-//                          reference's tie orders on them and samples (topk_select_lds with probabilities in).
-// Rows it cannot bound take the literal replay on probabilities computed on the fly.
+// twice and never written. Both reads apply temperature, history penalty and the min-length mask in registers:
+//   1. the exact maximum of the row;
+//   2. e_v = T(exp(y_v - max)) summed in the order of the reference's softmax
+//      (sampling_topp_kernels.cu:1308-1344: thread t of 1024 adds columns t, t + 1024, ... one after the other;
+//      reduce_kernel_utils.cuh:73-103: xor butterflies 16..1 inside 32-lane groups, then over the 32 group sums),
+//      so the sum has the reference's bits; on the way the candidates of the top-k selection are gathered by e_v,
+//      with a bound lowered by what the division and rounding to T can merge, so that every column whose
+//      probability ties with the k-th largest is among them. The candidates' e_v then become probabilities
+//      T(e_v / (sum + 1e-6)), the reference's tie orders are replayed on them and the row is sampled
+//      (topk_select_lds with probabilities in). Rows it cannot bound take the literal replay on probabilities
+//      computed on the fly.
+// Two forms:
+//   lp_wide_kernel - the product's: one launch, one workgroup of 1024, 512 or 256 threads per row does both reads
+//                    (the second one comes from the caches), a thread owning 1, 2 or 4 whole summation chains;
+//   lp_rowmax_kernel + lp_row_kernel - two launches: the first streams the row in the launch shape of the lean
+//                    gather and leaves the maximum of every workgroup's share in the workspace, the second gives
+//                    a row to one 256-thread workgroup whose threads own four neighbouring chains each and walk
+//                    them with 16-byte (fp32) or 8-byte (16-bit types) loads that are 1024 columns apart. The test
+//                    build of the library can select it; the forms must agree bit for bit.
 // Preconditions (checked by the host, which otherwise reports FTK_ERR_UNSUPPORTED and the layer runs the kernel
 // sequence): no embedding bias, largest k <= 128, vocabulary >= 1024 (the reference's block is min(V, 1024)
-// threads). Rows may have any pitch and start on any element boundary: the loads are the aligned vectors of the
-// memory, and the few columns of the first one that lie in front of the row are masked.
+// threads). Rows may have any pitch and start on any element boundary: vector loads are the aligned vectors of the
+// memory, and the few columns of the first one that lie in front of the row are masked or looked at one by one.
 #pragma once
 #include <type_traits>
 
