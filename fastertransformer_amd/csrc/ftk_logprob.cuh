@@ -722,7 +722,9 @@ __global__ void __launch_bounds__(THREADS) lp_wide_kernel(FusedParams p, FusedLa
     __shared__ float      warp_sum[32];
     __shared__ float      redf[THREADS / WAVE];
     const int             t    = threadIdx.x;
-    const int             row  = blockIdx.x;
+    // The last rows first: whatever produced the logits wrote them shortly before this launch, and of a batch that is
+    // larger than the last-level cache the rows written last are the ones still in it.
+    const int             row  = (int)gridDim.x - 1 - (int)blockIdx.x;
     const T*              rowp = (const T*)p.logits + (size_t)row * p.Vp;
     // A workgroup that shares its compute unit with others is served first while it waits for memory more than it
     // computes (set-up, first pass, selection): its few instructions then do not queue behind the arithmetic of a
