@@ -168,11 +168,14 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     achieved = alg / (gather_ms * 1e-3) / 1e9 if gather_ms > 0 else 0.0
     # Which kernel streams the logits: one 1024-thread workgroup per row does the whole step in one launch where the
     # batch fills the chip in nearly full rounds of 256 rows (rowwide_step_kernel); otherwise the lean gather
-    # (largest k beyond 192: twice, maxima first) followed by a selection launch. Timer 1 carries either.
+    # (largest k beyond 192 on more than 256 rows: twice, maxima first) followed by a selection launch. Timer 1
+    # carries either.
     rounds = (B + 255) // 256
     rowwide = (not isinstance(w["top_k"], tuple) and w["top_k"] <= 192 and B < 1024 and B * 5 >= rounds * 256 * 4
                and V // (16 // (4 if w["dtype"] == "f32" else 2)) >= 4 * 4096)
-    dominant = "rowwide_step_kernel" if rowwide else "lean_gather_kernel"
+    # (a largest k beyond 192 on up to 256 rows: one 1024-thread workgroup per row makes the lists, in one launch)
+    largek = isinstance(w["top_k"], tuple) and max(w["top_k"]) > 192 and B <= 256
+    dominant = "rowwide_step_kernel" if rowwide else ("largek_gather_kernel" if largek else "lean_gather_kernel")
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,
         kernel_ms=dict(history_bitmap=kernel_ms[0], gather=kernel_ms[1], select=kernel_ms[2], maxima=kernel_ms[3]),

@@ -22,6 +22,7 @@
 #include "ftk_test_hooks.h"
 #endif
 #include "ftk_fused.cuh"
+#include "ftk_largek.cuh"
 #include "ftk_lean.cuh"
 #include "ftk_logprob.cuh"
 #include "ftk_rowwide.cuh"
@@ -189,6 +190,13 @@ extern "C" void ftk_test_set_lp_form(int v)
 {
     g_lp_form = (v == 1 || v == 1024 || v == 512 || v == 256) ? v : 0;
 }
+// Test hook: non-zero keeps launches with a large k on the two launches of the lean gather also where one
+// 1024-thread workgroup per row would make their lists in one.
+static int g_largek_two_launches = 0;
+extern "C" void ftk_test_set_largek_two_launches(int v)
+{
+    g_largek_two_launches = v;
+}
 // Test hook: non-zero keeps the selection in a launch of its own also where one workgroup per row could do both.
 static int g_fused_two_launches = 0;
 extern "C" void ftk_test_set_fused_two_launches(int v)
@@ -196,7 +204,8 @@ extern "C" void ftk_test_set_fused_two_launches(int v)
     g_fused_two_launches = v;
 }
 // Test hook: which kernels the last fused step launched. 0: general stream, 1: lean gather + select, 2: lean gather
-// that also selects (one 256-thread workgroup per row), 3: one 1024-thread workgroup per row, 4: log-prob step.
+// that also selects (one 256-thread workgroup per row), 3: one 1024-thread workgroup per row, 4: log-prob step,
+// 5: large-k lists in one launch + select.
 static int g_fused_last_path = -1;
 extern "C" int ftk_test_last_fused_path(void)
 {
@@ -206,6 +215,7 @@ extern "C" int ftk_test_last_fused_path(void)
 #else
 static constexpr int g_fused_force_general = 0;
 static constexpr int g_fused_two_launches  = 0;
+static constexpr int g_largek_two_launches = 0;
 static constexpr int g_lp_form             = 0;
 #define FTK_NOTE_PATH(v) ((void)0)
 #endif
@@ -266,6 +276,14 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
                          && ((uintptr_t)a->logits & 15u) == 0 && ((size_t)a->vocab_size_padded * elem) % 16 == 0
                          && (a->penalty_type == FTK_PENALTY_NONE || a->penalties == nullptr
                              || a->step <= RW_HIST_U * RW_THREADS);
+    // A large k (the launch reads twice) on up to one row per compute unit: one 1024-thread workgroup per row makes
+    // the row's list in one launch (ftk_largek.cuh) where the lean gather takes two launches of small workgroups
+    // (256 x 51200 fp16, k up to 1024: 28 us against 10 + 25 us).
+    const bool largek = lean_mode == 2 && !want_log_probs && a->embedding_bias == nullptr && rows <= 256
+                        && g_largek_two_launches == 0 && a->max_top_k <= 1024
+                        && (size_t)a->vocab_size / (16 / elem) >= (size_t)LK_GROUPS * LK_THREADS
+                        && (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_LARGE
+                        && ((uintptr_t)a->logits & 15u) == 0 && ((size_t)a->vocab_size_padded * elem) % 16 == 0;
     // A frequency penalty needs the counts of the history's ids, which only that kernel keeps (a table in LDS).
     if (a->frequency_penalties != nullptr
         && (a->penalties == nullptr || a->penalty_type != FTK_PENALTY_ADDITIVE || a->output_ids == nullptr)) {
@@ -336,7 +354,7 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
         const bool   local      = words <= (size_t)FUSED_BITMAP_WORDS_LARGE && (many == 0 || lean_mode != 0)
                            && ((lean_mode != 0 ? lplan.splits : plan.splits) == 1 && !want_log_probs
                                || a->step <= FUSED_SPLIT_BITMAP_MAX_STEP);
-        if (rowwide) {
+        if (rowwide || largek) {
             p.lds_window = (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_SMALL ? 1 : 2;
         }
         else if (local) {
@@ -452,6 +470,24 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
             return a->dtype == FTK_DTYPE_F32 ? rowwide_launch_f32(w, rows, st, p, l, e0, e1) :
                    a->dtype == FTK_DTYPE_F16 ? rowwide_launch_f16(w, rows, st, p, l, e0, e1) :
                                                rowwide_launch_bf16(w, rows, st, p, l, e0, e1);
+        }
+        if (largek) {
+            // one list per row from one launch, then the selection
+            FTK_NOTE_PATH(5);
+            l.splits = 1;
+            hipEvent_t e0, e1;
+            take_events(1, &e0, &e1);
+            const int w = p.lds_window == 2 ? 2 : 1;
+            rc = a->dtype == FTK_DTYPE_F32 ? largek_gather_launch_f32(w, rows, st, p, l, e0, e1) :
+                 a->dtype == FTK_DTYPE_F16 ? largek_gather_launch_f16(w, rows, st, p, l, e0, e1) :
+                                             largek_gather_launch_bf16(w, rows, st, p, l, e0, e1);
+            if (rc != 0) {
+                return rc;
+            }
+            take_events(2, &e0, &e1);
+            return a->dtype == FTK_DTYPE_F32 ? lean_select_launch_f32(rows, st, p, l, e0, e1) :
+                   a->dtype == FTK_DTYPE_F16 ? lean_select_launch_f16(rows, st, p, l, e0, e1) :
+                                               lean_select_launch_bf16(rows, st, p, l, e0, e1);
         }
         // one workgroup per row: it also orders and samples, the step is one launch
         const bool row_select =

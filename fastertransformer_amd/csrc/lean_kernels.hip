@@ -1,6 +1,7 @@
 // Instances of the lean gather (ftk_lean.cuh) for one element type: this file is compiled once per type with
 // -DFTK_LEAN_DT=0 (f32), 1 (f16), 2 (bf16), so that the three sets of kernels build side by side.
 #include "ftk_lean.cuh"
+#include "ftk_largek.cuh"
 #include "ftk_rowwide.cuh"
 #include "ftk_sampling.h"
 
@@ -111,6 +112,32 @@ int rowwide_launch_bf16
     }
     else {
         launch(rowwide_step_kernel<FTK_LEAN_DT, FUSED_BITMAP_WORDS_SMALL>);
+    }
+    return (int)hipGetLastError();
+}
+
+#if FTK_LEAN_DT == 0
+int largek_gather_launch_f32
+#elif FTK_LEAN_DT == 1
+int largek_gather_launch_f16
+#else
+int largek_gather_launch_bf16
+#endif
+    (int window, int rows, hipStream_t st, const FusedParams& p, const FusedLaunch& l, hipEvent_t start, hipEvent_t stop)
+{
+    auto launch = [&](auto kernel) {
+        if (start != nullptr) {
+            hipExtLaunchKernelGGL(kernel, dim3(rows), dim3(LK_THREADS), 0, st, start, stop, 0, p, l);
+        }
+        else {
+            hipLaunchKernelGGL(kernel, dim3(rows), dim3(LK_THREADS), 0, st, p, l);
+        }
+    };
+    if (window == 2) {
+        launch(largek_gather_kernel<FTK_LEAN_DT, FUSED_BITMAP_WORDS_LARGE>);
+    }
+    else {
+        launch(largek_gather_kernel<FTK_LEAN_DT, FUSED_BITMAP_WORDS_SMALL>);
     }
     return (int)hipGetLastError();
 }

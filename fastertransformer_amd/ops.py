@@ -93,12 +93,13 @@ _HOOK_SIGNATURES = {
     "ftk_test_last_fused_path": [],
     "ftk_test_set_beam_path": [_i],
     "ftk_test_set_lp_form": [_i],
+    "ftk_test_set_largek_two_launches": [_i],
     "ftk_host_philox4x32_10": [_vp, _vp, _vp],
 }
 _RESTYPES = {"ftk_host_expf": _f, "ftk_host_logf": _f, "ftk_error_string": C.c_char_p,
              "ftk_test_set_topp_force_deep": None, "ftk_test_set_fused_force_general": None,
              "ftk_test_set_fused_two_launches": None, "ftk_test_set_beam_path": None,
-             "ftk_test_set_lp_form": None,
+             "ftk_test_set_lp_form": None, "ftk_test_set_largek_two_launches": None,
              "ftk_host_philox4x32_10": None}
 
 

@@ -32,12 +32,15 @@ void ftk_test_set_fused_force_general(int enable);
    both in one; process-wide */
 void ftk_test_set_fused_two_launches(int enable);
 /* which kernels the last fused step of this process launched: 0 general stream, 1 lean gather + select, 2 lean gather
-   that also selects (one 256-thread workgroup per row), 3 one 1024-thread workgroup per row, 4 log-prob step;
+   that also selects (one 256-thread workgroup per row), 3 one 1024-thread workgroup per row, 4 log-prob step, 5 large-k lists in one launch + select;
    -1 before the first step */
 int ftk_test_last_fused_path(void);
 /* the form of the fused log-prob step: 0 the product's choice, 1 two launches (row maxima, then one 256-thread
    workgroup per row), 1024 / 512 / 256 one launch with that many threads per row; process-wide */
 void ftk_test_set_lp_form(int form);
+/* non-zero keeps launches with a large k (beyond 192) on the two launches of the lean gather also where one
+   1024-thread workgroup per row would make the rows' lists in one launch; process-wide */
+void ftk_test_set_largek_two_launches(int on);
 /* the beam-search step: 1 = sections of rows in three launches everywhere, 2 = one 1024-thread workgroup per row in
    one launch everywhere, 3 = the same with 512 threads, 0 = chosen by the shape (the product's behaviour);
    process-wide */

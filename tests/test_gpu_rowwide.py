@@ -168,3 +168,50 @@ def test_rowwide_rows_walked_again_do_not_depend_on_the_workspace():
     for a, b in zip(one[:3], two[:3]):
         assert np.array_equal(a, b)
     assert (one[0] % 997 == 0).all()  # only the larger columns can be sampled (k = 150 of them, all tied)
+
+
+def test_large_k_lists_in_one_launch_agree_with_the_two_launches():
+    """With a largest k beyond 192 and at most one row per compute unit, one 1024-thread workgroup per row makes the
+    row's candidate list in one launch (csrc/ftk_largek.cuh; path 5) where the lean gather takes two (maxima, then
+    gather); the test build can keep the two launches (path 1). Same ids, lengths and flags on rows of three types:
+    vocabularies that end inside a 16-byte vector, histories, rows with fewer valid columns than k, constant rows
+    (lists that overflow and send the row to the exact replay)."""
+    import torch
+    from fastertransformer_amd import ops
+    from helpers import run_fused_step
+    hooks = ops.ftk_hooks()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(21)
+    tdt = {O.F32: torch.float32, O.F16: torch.float16, O.BF16: torch.bfloat16}
+    for dt, B, V, Vp, H, k, kind in ((O.F16, 256, 50257, 51200, 64, 1024, "normal"), (O.F32, 40, 50261, 50264, 16, 700, "normal"),
+                                     (O.BF16, 100, 32000, 32000, 300, 300, "grid"), (O.F32, 24, 20000, 20000, 8, 1024, "sparse"),
+                                     (O.F16, 16, 40000, 40000, 8, 512, "flat")):
+        x = torch.randn((B, Vp), generator=gen, device="cuda") * 3.0
+        if kind == "grid":
+            x = torch.round(x * 2.0) / 2.0
+        elif kind == "sparse":  # fewer valid columns than k in some rows
+            x[::3] = float("-inf")
+            for b in range(0, B, 3):
+                cols = torch.randint(0, V, (200,), generator=gen, device="cuda")
+                x[b, cols] = torch.randn(200, generator=gen, device="cuda")
+        elif kind == "flat":
+            x[::2] = 0.5
+        logits = x.to(tdt[dt])
+        history = torch.randint(0, V, (H, B), generator=gen, device="cuda", dtype=torch.int32)
+        draws = torch.rand(B, generator=gen, device="cuda").clamp_(min=1e-6)
+        finished0 = torch.zeros(B, dtype=torch.bool, device="cuda")
+        finished0[1] = True
+        seqlen0 = torch.full((B,), H - 1, dtype=torch.int32, device="cuda")
+        one = run_fused_step("caller", torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks,
+                             Vp=Vp, ws_fill=0xFF)
+        assert one[3] == 0 and hooks.ftk_test_last_fused_path() == 5, (dt, B, V)
+        hooks.ftk_test_set_largek_two_launches(1)
+        try:
+            two = run_fused_step("caller", torch, dt, B, V, H, k, logits, history, draws, finished0, seqlen0, lib=hooks,
+                                 Vp=Vp, ws_fill=0xFF)
+            assert two[3] == 0 and hooks.ftk_test_last_fused_path() == 1
+        finally:
+            hooks.ftk_test_set_largek_two_launches(0)
+        for name, a, b in zip(("ids", "sequence_length", "finished"), one[:3], two[:3]):
+            assert np.array_equal(a, b), (name, DTYPE_NAMES[dt], B, V, kind)
+        assert ((one[0] >= 0) & (one[0] < V)).all()
