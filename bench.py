@@ -174,7 +174,8 @@ def run_gpu(name, w, steps, warmup, nbuf=4, check_oracle=False):
     rowwide = (not isinstance(w["top_k"], tuple) and w["top_k"] <= 192 and B < 1024 and B * 5 >= rounds * 256 * 4
                and V // (16 // (4 if w["dtype"] == "f32" else 2)) >= 4 * 4096)
     # (a largest k beyond 192 on up to 256 rows: one 1024-thread workgroup per row makes the lists, in one launch)
-    largek = isinstance(w["top_k"], tuple) and max(w["top_k"]) > 192 and B <= 256
+    largek = (isinstance(w["top_k"], tuple) and max(w["top_k"]) > 192 and B <= 256
+              and (B >= 128 or V * (4 if w["dtype"] == "f32" else 2) <= (128 << 10)))
     dominant = "rowwide_step_kernel" if rowwide else ("largek_gather_kernel" if largek else "lean_gather_kernel")
     return dict(
         tokens_per_s=B * steps / wall, ms_per_step=ms_per_step, gpu_ms_per_step=gpu_ms / steps,

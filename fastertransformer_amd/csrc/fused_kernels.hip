@@ -277,9 +277,13 @@ extern "C" int ftk_fused_topk_step(ftk_fused_topk_args* a, ftk_stream_t stream)
                          && (a->penalty_type == FTK_PENALTY_NONE || a->penalties == nullptr
                              || a->step <= RW_HIST_U * RW_THREADS);
     // A large k (the launch reads twice) on up to one row per compute unit: one 1024-thread workgroup per row makes
-    // the row's list in one launch (ftk_largek.cuh) where the lean gather takes two launches of small workgroups
-    // (256 x 51200 fp16, k up to 1024: 28 us against 10 + 25 us).
+    // the row's list in one launch (ftk_largek.cuh) where the lean gather takes two launches of small workgroups.
+    // Measured on MI355X with k = 1024 in every row, us per step, one launch / two: 256 x 51200 f16 70.7 / 79.3, 16 x
+    // 51200 f16 65 / 67, 256 x 128256 f32 94 / 100, 128 x 128256 f32 83 / 85, 160 x 152064 f16 87 / 96; a few long
+    // rows are better spread over several workgroups each (16 x 128256 f32 78 / 58, 96 x 152064 f16 85 / 78), and
+    // so is more than one round of rows (320 x 51200 f16 93 / 90, 320 x 152064 f16 130 / 116).
     const bool largek = lean_mode == 2 && !want_log_probs && a->embedding_bias == nullptr && rows <= 256
+                        && (rows >= 128 || (size_t)a->vocab_size * elem <= ((size_t)128 << 10))
                         && g_largek_two_launches == 0 && a->max_top_k <= 1024
                         && (size_t)a->vocab_size / (16 / elem) >= (size_t)LK_GROUPS * LK_THREADS
                         && (size_t)a->vocab_size / 32 + 4 <= (size_t)FUSED_BITMAP_WORDS_LARGE

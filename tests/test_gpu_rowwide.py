@@ -183,7 +183,7 @@ def test_large_k_lists_in_one_launch_agree_with_the_two_launches():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(21)
     tdt = {O.F32: torch.float32, O.F16: torch.float16, O.BF16: torch.bfloat16}
-    for dt, B, V, Vp, H, k, kind in ((O.F16, 256, 50257, 51200, 64, 1024, "normal"), (O.F32, 40, 50261, 50264, 16, 700, "normal"),
+    for dt, B, V, Vp, H, k, kind in ((O.F16, 256, 50257, 51200, 64, 1024, "normal"), (O.F32, 130, 50261, 50264, 16, 700, "normal"),
                                      (O.BF16, 100, 32000, 32000, 300, 300, "grid"), (O.F32, 24, 20000, 20000, 8, 1024, "sparse"),
                                      (O.F16, 16, 40000, 40000, 8, 512, "flat")):
         x = torch.randn((B, Vp), generator=gen, device="cuda") * 3.0
