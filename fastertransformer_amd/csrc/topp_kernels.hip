@@ -1756,11 +1756,28 @@ __device__ unsigned long long topp_settle_ties(TopPShared& s, const unsigned lon
     if (t == 0) {
         const unsigned long long here = A[found];
         const uint32_t           key  = (uint32_t)(here >> 32);
-        // the prefix is in ascending order of this word as a whole (the division keeps the order of the segments)
-        int lo = 0, hi = found;  // first position of the run
+        // The prefix is in ascending order of this word as a whole (the division keeps the order of the segments).
+        // Runs are short as a rule, and every probe is a dependent load: both ends are looked for outwards from
+        // `found` in doubling steps, then by bisection inside the last step.
+        auto high = [&](int i) { return (uint32_t)(A[i] >> 32); };
+        int  hi = found, lo = 0;  // first position of the run: in [lo, hi], A[hi] belongs to it
+        for (int step = 1;; step <<= 1) {
+            const int probe = hi - step;
+            if (probe < 0) {
+                lo = 0;
+                break;
+            }
+            if (high(probe) == key) {
+                hi = probe;
+            }
+            else {
+                lo = probe + 1;
+                break;
+            }
+        }
         while (lo < hi) {
             const int mid = (lo + hi) >> 1;
-            if ((uint32_t)(A[mid] >> 32) < key) {
+            if (high(mid) < key) {
                 lo = mid + 1;
             }
             else {
@@ -1769,10 +1786,24 @@ __device__ unsigned long long topp_settle_ties(TopPShared& s, const unsigned lon
         }
         const int a = lo;
         lo = found;
-        hi = n - 1;  // last position of the run
+        hi = n - 1;  // last position of the run: in [lo, hi], A[lo] belongs to it
+        for (int step = 1;; step <<= 1) {
+            const int probe = lo + step;
+            if (probe > n - 1) {
+                hi = n - 1;
+                break;
+            }
+            if (high(probe) == key) {
+                lo = probe;
+            }
+            else {
+                hi = probe - 1;
+                break;
+            }
+        }
         while (lo < hi) {
             const int mid = (lo + hi + 1) >> 1;
-            if ((uint32_t)(A[mid] >> 32) > key) {
+            if (high(mid) > key) {
                 hi = mid - 1;
             }
             else {
