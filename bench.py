@@ -448,7 +448,7 @@ def run_gpu_beam(name, w, steps, warmup):
                 ids_checksum=checksum)
 
 
-# ---- the other BASELINE configurations: short timed runs and a one-step oracle check each -------------------------
+# ---- the other benchmark configurations: short timed runs and a one-step oracle check each -------------------------
 
 SECONDARY = [
     "topp_step_b256_v128256_f32_zipf1.1_p0.5-0.99_decay0.9",
